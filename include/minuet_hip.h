@@ -1,0 +1,251 @@
+/*
+ * minuet_hip.h — C ABI of libminuet_hip.so: the sparse-convolution hot path
+ * (Map -> Gather -> grouped GEMM -> Scatter) as hand-written gfx950 HIP kernels.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream
+ * (passed as void*; NULL = the null stream).  Inputs are borrowed and never
+ * written; outputs are caller-allocated.  Temporaries come from the
+ * library's own per-stream scratch arena (mnt_buffer_* below).  All work is
+ * enqueued on the given stream; entry points that must read a scalar back
+ * (documented per function) synchronise that stream before returning.
+ *
+ * Return convention: 0 on success, non-zero on failure; the message of the
+ * last failure on the calling thread is returned by mnt_last_error().
+ *
+ * Each declaration cites the interface of the reference (paths relative to
+ * the reference checkout) that a binding would route to it.
+ */
+#ifndef MINUET_HIP_H_
+#define MINUET_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* integer element types of coordinate / index tensors */
+#define MNT_INT32 0
+#define MNT_INT64 1
+/* feature element types */
+#define MNT_FLOAT32 0
+#define MNT_FLOAT16 1
+#define MNT_BFLOAT16 2
+
+#define MNT_MAX_NDIM 4
+
+/* ---- library ----------------------------------------------------------- */
+
+/* ABI version of this header (bumped on any signature change). */
+int mnt_abi_version(void);
+
+/* Message of the last failed call on this thread ("" if none).
+ * Replaces MinuetException::what(), csrc/minuet/common/exception.h:9-21. */
+const char *mnt_last_error(void);
+
+/* ---- scratch arena (csrc/minuet/torch/cuda_memory_buffer.cu:6-47,
+ *      csrc/minuet/cuda/buffer_pool.cu:100-216) ----------------------------- */
+int mnt_buffer_preallocate(void *stream, size_t bytes);   /* cuda_preallocate_buffer */
+int mnt_buffer_free(void *stream);                        /* cuda_free_buffers (synchronises) */
+int mnt_buffer_set_growth(void *stream, float growth);    /* cuda_set_buffer_growth */
+int mnt_buffer_set_page_size(void *stream, size_t bytes); /* cuda_set_buffer_page_size */
+size_t mnt_buffer_total_size(void *stream);               /* cuda_buffer_total_size */
+size_t mnt_buffer_used_size(void *stream);                /* cuda_buffer_used_size */
+int mnt_reset_error(void);                                /* cuda_reset_error */
+
+/* ---- Map: coordinate sort ---------------------------------------------- */
+
+/* Stable lexicographic arg-sort of coords[n, ndim] (dimension 0 most
+ * significant); with batch_dims[num_batches+1] the result is batch-major.
+ * indices_out[n] has element type index_dtype (= the type of batch_dims when
+ * given).  sorted_coords_out (nullable) receives coords[indices_out].
+ * Synchronises once (coordinate bounds are read back to size the keys).
+ * Replaces cuda_arg_sort_coordinates / cuda_multi_arg_sort_coordinates,
+ * csrc/minuet/torch/cuda_arg_sort_coordinates.cu:8-70 and
+ * csrc/minuet/cuda/functions/arg_sort_coodrinates.cu:273-469. */
+int mnt_arg_sort_coordinates(const void *coords, int64_t n, int ndim, int coord_dtype,
+                             const void *batch_dims, int64_t num_batches, int index_dtype,
+                             void *indices_out, void *sorted_coords_out, void *stream);
+
+/* ---- Map: unique ------------------------------------------------------- */
+
+/* Run-end counting on SORTED coords: idx_out[0]=0, idx_out[i+1]=idx_out[i]+
+ * [row i is the last of its run or of its batch]; *num_unique_out = idx_out[n].
+ * Synchronises once.  Replaces the first half of cuda_unique_coordinates /
+ * cuda_multi_unique_coordinates, csrc/minuet/torch/cuda_unique_coordinates.cu:8-85
+ * (UniqueCoordinates::operator(), csrc/minuet/cuda/functions/unique_coordinates.cu:10-95). */
+int mnt_unique_coordinates(const void *sorted_coords, int64_t n, int ndim, int coord_dtype,
+                           const void *batch_dims, int64_t num_batches, int index_dtype,
+                           void *idx_out, int64_t *num_unique_out, void *stream);
+
+/* unique_out[idx[i]] = sorted_coords[i] wherever idx[i] != idx[i+1].
+ * Replaces FillUniqueCoordinates, csrc/minuet/cuda/functions/unique_coordinates.cu:97-102. */
+int mnt_fill_unique_coordinates(const void *sorted_coords, int64_t n, int ndim, int coord_dtype,
+                                const void *idx, int index_dtype, void *unique_out, void *stream);
+
+/* Target voxel set of a strided layer in one call: floor(c / stride) * stride,
+ * sort, unique.  Phase 1 returns the count (synchronises once) and keeps the
+ * sorted keys in the arena slot of this stream; phase 2 writes the coordinates
+ * and target_batch_dims_out[num_batches+1] (nullable, element type
+ * index_dtype).  Phase 2 must follow phase 1 on the same stream with no other
+ * library call in between.  Replaces the torch expression in
+ * KernelMapCache.get_target_coordinates, minuet/nn/convolutions.py:84-99. */
+int mnt_target_coordinates_count(const void *source_coords, int64_t n, int ndim, int coord_dtype,
+                                 const int64_t *target_stride, const void *batch_dims,
+                                 int64_t num_batches, int index_dtype,
+                                 int64_t *num_targets_out, void *stream);
+int mnt_target_coordinates_fill(void *target_coords_out, void *target_batch_dims_out,
+                                void *stream);
+
+/* ---- Map: query -------------------------------------------------------- */
+
+/* Dense kernel map: kernel_map_out[o*T + t] = j with sources[j] == targets[t] +
+ * offsets[o] (same batch), else -1.  sources/targets sorted; offsets[O, ndim]
+ * is a device array of coord_dtype.  batch dims (both or neither) have element
+ * type batch_dtype and num_batches+1 entries; kernel_map_out has out_dtype.
+ * Synchronises once (bounds).  Replaces cuda_query_sorted_index_with_offsets /
+ * cuda_multi_query_sorted_index_with_offsets,
+ * csrc/minuet/torch/cuda_sparse_convolution_mapping.cu:9-93. */
+int mnt_query_sorted_index_with_offsets(const void *sources, int64_t num_sources,
+                                        const void *targets, int64_t num_targets,
+                                        const void *offsets, int64_t num_offsets,
+                                        int ndim, int coord_dtype,
+                                        const void *source_batch_dims,
+                                        const void *target_batch_dims,
+                                        int64_t num_batches, int batch_dtype,
+                                        void *kernel_map_out, int out_dtype, void *stream);
+
+/* sizes_out[o] = #{t : kernel_map[o,t] != -1} (device, index_dtype).
+ * Replaces cuda_compute_kernel_map_sizes,
+ * csrc/minuet/torch/cuda_sparse_convolution_mapping.cu:95-121. */
+int mnt_compute_kernel_map_sizes(const void *kernel_map, int64_t num_offsets,
+                                 int64_t num_targets, int index_dtype, void *sizes_out,
+                                 void *stream);
+
+/* Rank tables: target_masks[o,t] = rank of the hit among the hits of row o in
+ * target order, source_masks[o, kernel_map[o,t]] = the same rank, -1 elsewhere.
+ * Replaces cuda_compute_kernel_map_masks,
+ * csrc/minuet/torch/cuda_sparse_convolution_mapping.cu:123-156. */
+int mnt_compute_kernel_map_masks(const void *kernel_map, int64_t num_offsets,
+                                 int64_t num_sources, int64_t num_targets, int index_dtype,
+                                 void *source_masks_out, void *target_masks_out, void *stream);
+
+/* Kernel-map build of KernelMapCache.get_kernel_map on a miss
+ * (minuet/nn/convolutions.py:147-170) in two calls with no intermediate
+ * tensors on the host side.
+ *
+ * mnt_kernel_map_query: dense map (kernel_map_out, int32 [O,T], rows in offset
+ * order), per-offset sizes and the stable ascending size order (reorder != 0;
+ * identity otherwise).  offsets_host[O*ndim] is a HOST array of int64.
+ * order_host_out[j] is the offset of output row j and sizes_host_out[j] its
+ * hit count.  Synchronises twice (bounds; sizes).
+ *
+ * mnt_kernel_map_emit: must directly follow the query on the same stream, with
+ * kernel_map_out still alive.  Writes any non-null output: the rank tables
+ * source_masks_out [O,S] / target_masks_out [O,T] (row j <-> offset order[j]),
+ * the pair lists in_idx_out / out_idx_out [nnz] (rows concatenated in output
+ * row order, hits in target order) and device copies of sizes / order.
+ * Does not synchronise.  Replaces the chain compute_kernel_map_sizes ->
+ * torch.sort -> kernel_map[order] -> compute_kernel_map_masks. */
+int mnt_kernel_map_query(const void *sources, int64_t num_sources,
+                         const void *targets, int64_t num_targets,
+                         const int64_t *offsets_host, int64_t num_offsets,
+                         int ndim, int coord_dtype,
+                         const void *source_batch_dims, const void *target_batch_dims,
+                         int64_t num_batches, int batch_dtype, int reorder,
+                         int32_t *kernel_map_out,
+                         int64_t *sizes_host_out, int64_t *order_host_out, void *stream);
+int mnt_kernel_map_emit(int32_t *source_masks_out, int32_t *target_masks_out,
+                        int32_t *in_idx_out, int32_t *out_idx_out,
+                        int32_t *sizes_dev_out, int32_t *order_dev_out, void *stream);
+
+/* Per-offset (in_idx, out_idx) pair lists from a dense int32 kernel map: for row
+ * o the hits in target order are written at list positions
+ * cumsum_host[o] .. cumsum_host[o]+sizes[o]-1 (cumsum_host[O+1], HOST, exclusive
+ * prefix of the row sizes, e.g. from mnt_compute_kernel_map_sizes).  This is
+ * the inverse of the two rank tables of mnt_compute_kernel_map_masks. */
+int mnt_kernel_map_pair_lists(const int32_t *kernel_map, int64_t num_offsets,
+                              int64_t num_targets, const int64_t *cumsum_host,
+                              int32_t *in_idx_out, int32_t *out_idx_out, void *stream);
+
+/* ---- GMaS: padding plan (host only) -------------------------------------- */
+
+/* Greedy contiguous grouping of size-ascending offsets: extend a bucket while
+ * (max*count - sum)/sum <= threshold; has_threshold == 0 -> one bucket,
+ * threshold < 0 -> singletons.  Writes boundaries (first 0, last O) and
+ * returns their count through num_boundaries_out (buckets_out holds O+1).
+ * Replaces GeneratePaddingBuckets,
+ * csrc/minuet/cuda/functions/sparse_convolution.cu:16-43. */
+int mnt_generate_padding_buckets(const int64_t *sizes_host, int64_t num_offsets,
+                                 int has_threshold, double threshold,
+                                 int64_t *buckets_out, int64_t *num_boundaries_out);
+
+/* Each offset of a bucket owns max-size-in-bucket rows; cumsum_out[O+1].
+ * Replaces ComputeCumsumKernelPaddedSizes, sparse_convolution.cu:272-292. */
+int mnt_cumsum_kernel_padded_sizes(const int64_t *sizes_host, int64_t num_offsets,
+                                   const int64_t *buckets, int64_t num_boundaries,
+                                   int64_t *cumsum_out);
+
+/* ---- GMaS: forward ------------------------------------------------------- */
+
+/* out[T, Cout] = sum over offsets of gather(sources) x weights[order[o]],
+ * scattered target-stationary in offset order with fp32 accumulation.
+ * sources[S, Cin], weights[O, Cin, Cout], out: float_dtype; masks [O,S] / [O,T],
+ * order (nullable) and sizes [O]: device arrays of index_dtype.
+ * sizes_host (nullable, int64[O]) spares the read-back of sizes; without it
+ * the call synchronises once.  gather_tile / scatter_tile are elements per
+ * lane (0 = pick automatically).  parallel is accepted for signature
+ * compatibility (all offsets run in one grouped launch).
+ * Replaces cuda_sparse_convolution_forward,
+ * csrc/minuet/torch/cuda_sparse_convolution_forward.cu:136-213 and
+ * SparseConvolutionForward::operator(),
+ * csrc/minuet/cuda/functions/sparse_convolution.cu:504-661. */
+int mnt_sparse_convolution_forward(int64_t gather_tile, int64_t scatter_tile,
+                                   int allow_shortcut_matmul, int64_t parallel,
+                                   int has_threshold, double threshold,
+                                   const void *sources, const void *weights,
+                                   const void *source_masks, const void *target_masks,
+                                   const void *kernel_map_order, const void *kernel_map_sizes,
+                                   const int64_t *sizes_host,
+                                   int64_t num_sources, int64_t num_targets,
+                                   int64_t num_offsets, int64_t num_source_features,
+                                   int64_t num_target_features,
+                                   int index_dtype, int float_dtype,
+                                   void *out, void *stream);
+
+/* Timers used by the autotuner: run the named stage once on scratch buffers and
+ * return the elapsed milliseconds through ms_out (synchronise).
+ * Replace cuda_time_gather / cuda_time_scatter / cuda_time_gemm,
+ * csrc/minuet/torch/cuda_sparse_convolution_forward.cu:7-134 (TimeGather,
+ * TimeScatter, TimeGEMM: csrc/minuet/cuda/functions/sparse_convolution.cu:294-502). */
+int mnt_time_gather(int64_t tile, int allow_shortcut_matmul, int has_threshold, double threshold,
+                    const void *source_masks, const void *kernel_map_sizes,
+                    int64_t num_sources, int64_t num_targets, int64_t num_offsets,
+                    int64_t num_source_features, int64_t num_target_features,
+                    int index_dtype, int float_dtype, float *ms_out, void *stream);
+int mnt_time_scatter(int64_t tile, int allow_shortcut_matmul, int has_threshold, double threshold,
+                     const void *target_masks, const void *kernel_map_sizes,
+                     int64_t num_sources, int64_t num_targets, int64_t num_offsets,
+                     int64_t num_source_features, int64_t num_target_features,
+                     int index_dtype, int float_dtype, float *ms_out, void *stream);
+int mnt_time_gemm(int allow_shortcut_matmul, int64_t parallel, int has_threshold, double threshold,
+                  const void *weights, const void *kernel_map_sizes,
+                  int64_t num_sources, int64_t num_targets, int64_t num_offsets,
+                  int64_t num_source_features, int64_t num_target_features,
+                  int index_dtype, int float_dtype, float *ms_out, void *stream);
+
+/* ---- stage timing of the last mnt_sparse_convolution_forward ------------- */
+
+/* When enabled, the forward call brackets weight-pack, gather, GEMM and
+ * scatter with events on its stream; mnt_profile_read synchronises and returns
+ * the four durations in milliseconds (order: pack, gather, gemm, scatter).
+ * No counterpart in the reference; used by the benchmark for per-kernel
+ * roofline figures. */
+int mnt_profile_enable(int on);
+int mnt_profile_read(float *ms4_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MINUET_HIP_H_ */

@@ -1,0 +1,903 @@
+// Gather -> grouped MFMA GEMM -> Scatter for gfx950, plus the host-side padding
+// plan, the forward driver and the autotuner's stage timers.
+//
+// Data flow and addressing follow SparseConvolutionForward::operator()
+// (csrc/minuet/cuda/functions/sparse_convolution.cu:504-661): row `rank` of
+// offset o lives at buffer row cumsum_padded[o] + rank; the gather is
+// source-stationary over source_masks[O,S]
+// (kernels/padded_gather_warp_optimized.cuh:43-59) and the scatter is
+// target-stationary over target_masks[O,T] with offsets summed in row order and
+// no atomics (kernels/padded_scatter_warp_optimized.cuh:33-62).  All offsets
+// are multiplied in ONE grouped launch whose tiles never cross an offset, so
+// padded rows are never computed.
+#include <algorithm>
+
+#include "device_utils.h"
+
+namespace mnt {
+
+typedef _Float16 half_t;
+typedef __bf16 bf16_t;
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// ------------------------------------------------------------ host plan ----
+
+static void padding_buckets(const int64_t *sizes, int64_t n, bool has_threshold, double threshold,
+                            std::vector<int64_t> &buckets) {
+  buckets.clear();
+  buckets.push_back(0);
+  int64_t i = 0;
+  while (i < n) {
+    const int64_t first = i;
+    uint64_t actual = static_cast<uint64_t>(sizes[i]);
+    uint64_t summit = actual;
+    while (i + 1 < n) {
+      actual += static_cast<uint64_t>(sizes[i + 1]);
+      summit = std::max<uint64_t>(summit, static_cast<uint64_t>(sizes[i + 1]));
+      const uint64_t padded = summit * static_cast<uint64_t>((i + 1) - first + 1);
+      if (has_threshold) {
+        if (threshold < 0) break;
+        // 0/0 is NaN in the reference and never exceeds the threshold
+        if (actual > 0 && static_cast<double>(padded - actual) / static_cast<double>(actual) > threshold) break;
+      }
+      ++i;
+    }
+    buckets.push_back(i + 1);
+    ++i;
+  }
+}
+
+static void cumsum_padded(const int64_t *sizes, int64_t n, const std::vector<int64_t> &buckets,
+                          std::vector<int64_t> &cum) {
+  cum.assign(n + 1, 0);
+  for (size_t b = 0; b + 1 < buckets.size(); ++b) {
+    int64_t summit = 0;
+    for (int64_t j = buckets[b]; j < buckets[b + 1]; ++j) summit = std::max(summit, sizes[j]);
+    for (int64_t j = buckets[b]; j < buckets[b + 1]; ++j) cum[j + 1] = cum[j] + summit;
+  }
+}
+
+// ------------------------------------------- small uploads through kernargs ----
+
+constexpr int kUploadInts = 512;
+struct IntChunk {
+  int v[kUploadInts];
+};
+
+__global__ __launch_bounds__(256) void upload_ints_kernel(IntChunk chunk, int count, int *__restrict__ dst) {
+  for (int i = threadIdx.x; i < count; i += blockDim.x) dst[i] = chunk.v[i];
+}
+
+// Copies a small host int array to device memory as kernel arguments: no
+// staging buffer to protect, no synchronisation, safe under stream capture.
+static void upload_ints(const std::vector<int> &host, int *dst, hipStream_t stream) {
+  for (size_t base = 0; base < host.size(); base += kUploadInts) {
+    IntChunk chunk;
+    const int count = static_cast<int>(std::min<size_t>(kUploadInts, host.size() - base));
+    memcpy(chunk.v, host.data() + base, sizeof(int) * count);
+    upload_ints_kernel<<<1, 256, 0, stream>>>(chunk, count, dst + base);
+    check_launch("upload_ints_kernel");
+  }
+}
+
+// --------------------------------------------------------- weight packing ----
+
+// wt[j][n][k] = w[order[j]][k][n], zero-padded to [Np][Kp]: the K-contiguous,
+// transposed form the GEMM stages into LDS.  Takes the place of PermuteWeights
+// (csrc/minuet/cuda/kernels/permute_weights.cuh:8-36).
+template <typename T, typename IT>
+__global__ __launch_bounds__(256) void pack_weights_kernel(const T *__restrict__ w,
+                                                           const IT *__restrict__ order,
+                                                           int num_offsets, int K, int N, int Kp,
+                                                           int Np, T *__restrict__ wt) {
+  const long long total = static_cast<long long>(num_offsets) * Np * Kp;
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int k = static_cast<int>(i % Kp);
+    const int n = static_cast<int>((i / Kp) % Np);
+    const int j = static_cast<int>(i / (static_cast<long long>(Kp) * Np));
+    T value = static_cast<T>(0.0f);
+    if (k < K && n < N) {
+      const long long src = order ? static_cast<long long>(order[j]) : j;
+      value = w[(src * K + k) * N + n];
+    }
+    wt[i] = value;
+  }
+}
+
+// ----------------------------------------------------------------- gather ----
+
+template <int VB>
+struct VecOf;
+template <>
+struct VecOf<16> { typedef uint4 type; };
+template <>
+struct VecOf<8> { typedef uint2 type; };
+template <>
+struct VecOf<4> { typedef unsigned type; };
+template <>
+struct VecOf<2> { typedef unsigned short type; };
+
+// One lane group per source row: the row is read once, then copied to the
+// buffer row of every offset that uses it.
+template <int VB, int NV, typename IT>
+__global__ __launch_bounds__(256) void gather_kernel(const unsigned char *__restrict__ sources,
+                                                     unsigned char *__restrict__ buffer,
+                                                     const IT *__restrict__ source_masks,
+                                                     const int *__restrict__ row_start,
+                                                     long long num_sources, int num_offsets,
+                                                     int row_bytes, int lanes_per_row) {
+  typedef typename VecOf<VB>::type V;
+  const long long gtid = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const long long s = gtid / lanes_per_row;
+  const int lr = static_cast<int>(gtid % lanes_per_row);
+  if (s >= num_sources) return;
+  V value[NV];
+  const unsigned char *src = sources + s * row_bytes;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) value[i] = *reinterpret_cast<const V *>(src + (lr + i * lanes_per_row) * VB);
+  for (int o = 0; o < num_offsets; ++o) {
+    const long long d = static_cast<long long>(source_masks[static_cast<long long>(o) * num_sources + s]);
+    if (d < 0) continue;
+    unsigned char *dst = buffer + (static_cast<long long>(row_start[o]) + d) * row_bytes;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) *reinterpret_cast<V *>(dst + (lr + i * lanes_per_row) * VB) = value[i];
+  }
+}
+
+// ---------------------------------------------------------------- scatter ----
+
+template <typename T>
+__device__ __forceinline__ float to_float(T v) { return static_cast<float>(v); }
+
+// One lane group per target row: sums its buffer rows in offset order in fp32
+// and writes the row once.  With `accumulate` the previous content of the row
+// (the centre-offset product written by the direct GEMM) is the initial value.
+template <typename T, int VB, int NV, typename IT>
+__global__ __launch_bounds__(256) void scatter_kernel(const unsigned char *__restrict__ buffer,
+                                                      unsigned char *__restrict__ targets,
+                                                      const IT *__restrict__ target_masks,
+                                                      const int *__restrict__ row_start,
+                                                      long long num_targets, int num_offsets,
+                                                      int row_bytes, int lanes_per_row,
+                                                      int accumulate) {
+  typedef typename VecOf<VB>::type V;
+  constexpr int E = VB / static_cast<int>(sizeof(T));
+  const long long gtid = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const long long t = gtid / lanes_per_row;
+  const int lr = static_cast<int>(gtid % lanes_per_row);
+  if (t >= num_targets) return;
+  float acc[NV][E];
+  unsigned char *dst = targets + t * row_bytes;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if (accumulate) {
+      V raw = *reinterpret_cast<const V *>(dst + (lr + i * lanes_per_row) * VB);
+      const T *e = reinterpret_cast<const T *>(&raw);
+#pragma unroll
+      for (int k = 0; k < E; ++k) acc[i][k] = to_float(e[k]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < E; ++k) acc[i][k] = 0.0f;
+    }
+  }
+  for (int o = 0; o < num_offsets; ++o) {
+    const long long d = static_cast<long long>(target_masks[static_cast<long long>(o) * num_targets + t]);
+    if (d < 0) continue;
+    const unsigned char *src = buffer + (static_cast<long long>(row_start[o]) + d) * row_bytes;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      V raw = *reinterpret_cast<const V *>(src + (lr + i * lanes_per_row) * VB);
+      const T *e = reinterpret_cast<const T *>(&raw);
+#pragma unroll
+      for (int k = 0; k < E; ++k) acc[i][k] += to_float(e[k]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    V raw;
+    T *e = reinterpret_cast<T *>(&raw);
+#pragma unroll
+    for (int k = 0; k < E; ++k) e[k] = static_cast<T>(acc[i][k]);
+    *reinterpret_cast<V *>(dst + (lr + i * lanes_per_row) * VB) = raw;
+  }
+}
+
+// ------------------------------------------------------------ grouped GEMM ----
+
+template <typename T>
+struct Mfma;
+template <>
+struct Mfma<half_t> {
+  __device__ static __forceinline__ floatx16 run(const uint4 &a, const uint4 &b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8 *>(&a),
+                                                  *reinterpret_cast<const half8 *>(&b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma<bf16_t> {
+  __device__ static __forceinline__ floatx16 run(const uint4 &a, const uint4 &b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8 *>(&a),
+                                                   *reinterpret_cast<const bf16x8 *>(&b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma<float> {
+  __device__ static __forceinline__ floatx16 run(const uint4 &a, const uint4 &b, floatx16 c) {
+    const float *fa = reinterpret_cast<const float *>(&a);
+    const float *fb = reinterpret_cast<const float *>(&b);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[i], c, 0, 0, 0);
+    return c;
+  }
+};
+
+constexpr int kGemmBlock = 256;
+constexpr int kGemmRows = 128;          // rows of A per workgroup (32 per wavefront)
+constexpr int kChunkBytes = 128;        // bytes of K staged per row and step
+constexpr int kLdsRowBytes = kChunkBytes + 16;
+
+// meta: [G | tile_prefix (G+1) | row_start (G+1) | rows (G) | weight (G)]
+//
+// out^T = W^T x A^T per tile: the first MFMA operand holds 32 output channels,
+// the second 32 data rows, so every lane ends up with 4 consecutive channels
+// of ONE data row per accumulator group and stores them as one vector.
+// The K order inside a 128-byte chunk is permuted identically for both
+// operands (lane half h of step kk reads bytes [32*kk + 16*h, +16) of the
+// row), which leaves the dot products unchanged.
+template <typename T, int TN, bool VEC>
+__global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
+    const T *__restrict__ a, T *__restrict__ c, const T *__restrict__ wt,
+    const int *__restrict__ meta, int K, int N, int Kp, int Np) {
+  constexpr int EPC = 16 / static_cast<int>(sizeof(T));        // elements per 16-byte piece
+  constexpr int KC = kChunkBytes / static_cast<int>(sizeof(T));
+  constexpr int NB = TN / 32;
+  __shared__ __align__(16) unsigned char a_lds[kGemmRows * kLdsRowBytes];
+  __shared__ __align__(16) unsigned char b_lds[TN * kLdsRowBytes];
+
+  const int G = meta[0];
+  const int *tile_prefix = meta + 1;
+  const int *row_start = tile_prefix + G + 1;
+  const int *rows = row_start + G + 1;
+  const int *weight = rows + G;
+
+  const int tile = blockIdx.x;
+  int lo = 0, hi = G - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (tile_prefix[mid] <= tile) {
+      lo = mid;
+    } else {
+      hi = mid - 1;
+    }
+  }
+  const int g = lo;
+  const int r0 = (tile - tile_prefix[g]) * kGemmRows;
+  const int valid = min(kGemmRows, rows[g] - r0);
+  const long long row_base = static_cast<long long>(row_start[g]) + r0;
+  const int n0 = blockIdx.y * TN;
+  const T *w_base = wt + (static_cast<long long>(weight[g]) * Np + n0) * Kp;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wv = tid >> 6;
+  const int r = lane & 31;
+  const int h = lane >> 5;
+
+  floatx16 acc[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[b][j] = 0.0f;
+  }
+
+  for (int k0 = 0; k0 < Kp; k0 += KC) {
+    // stage A: 128 rows x 8 pieces
+#pragma unroll
+    for (int i = 0; i < (kGemmRows * 8) / kGemmBlock; ++i) {
+      const int piece = tid + i * kGemmBlock;
+      const int row = piece >> 3;
+      const int q = piece & 7;
+      const int k = k0 + q * EPC;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (row < valid) {
+        const T *src = a + (row_base + row) * K + k;
+        if (VEC && k + EPC <= K) {
+          v = *reinterpret_cast<const uint4 *>(src);
+        } else {
+          T *e = reinterpret_cast<T *>(&v);
+#pragma unroll
+          for (int x = 0; x < EPC; ++x) {
+            if (k + x < K) e[x] = src[x];
+          }
+        }
+      }
+      *reinterpret_cast<uint4 *>(a_lds + row * kLdsRowBytes + q * 16) = v;
+    }
+    // stage W^T: TN channels x 8 pieces (always in bounds: padded to [Np][Kp])
+#pragma unroll
+    for (int i = 0; i < (TN * 8 + kGemmBlock - 1) / kGemmBlock; ++i) {
+      const int piece = tid + i * kGemmBlock;
+      if (piece < TN * 8) {
+        const int n = piece >> 3;
+        const int q = piece & 7;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (n0 + n < Np) v = *reinterpret_cast<const uint4 *>(w_base + static_cast<long long>(n) * Kp + k0 + q * EPC);
+        *reinterpret_cast<uint4 *>(b_lds + n * kLdsRowBytes + q * 16) = v;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < kChunkBytes / 32; ++kk) {
+      const int off = kk * 32 + h * 16;
+      const uint4 rows_frag = *reinterpret_cast<const uint4 *>(a_lds + (wv * 32 + r) * kLdsRowBytes + off);
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        const uint4 chan_frag = *reinterpret_cast<const uint4 *>(b_lds + (b * 32 + r) * kLdsRowBytes + off);
+        acc[b] = Mfma<T>::run(chan_frag, rows_frag, acc[b]);
+      }
+    }
+    __syncthreads();
+  }
+
+  const int row = wv * 32 + r;
+  if (row < valid) {
+    T *dst = c + (row_base + row) * N;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int ch = n0 + b * 32 + q * 8 + h * 4;
+        if (VEC && ch + 4 <= N) {
+          T out[4];
+#pragma unroll
+          for (int x = 0; x < 4; ++x) out[x] = static_cast<T>(acc[b][q * 4 + x]);
+          if (sizeof(T) == 2) {
+            *reinterpret_cast<uint2 *>(dst + ch) = *reinterpret_cast<const uint2 *>(out);
+          } else {
+            *reinterpret_cast<uint4 *>(dst + ch) = *reinterpret_cast<const uint4 *>(out);
+          }
+        } else {
+#pragma unroll
+          for (int x = 0; x < 4; ++x) {
+            if (ch + x < N) dst[ch + x] = static_cast<T>(acc[b][q * 4 + x]);
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------- host launchers ----
+
+static int pow2_vec(int64_t bytes_per_lane, int64_t row_bytes, const void *p0, const void *p1) {
+  const uintptr_t align = reinterpret_cast<uintptr_t>(p0) | reinterpret_cast<uintptr_t>(p1);
+  for (int vb = 16; vb >= 2; vb >>= 1) {
+    if (bytes_per_lane % vb == 0 && row_bytes % vb == 0 && align % vb == 0) return vb;
+  }
+  return 0;
+}
+
+struct LaneShape {
+  int vb;
+  int nv;
+  int lanes_per_row;
+};
+
+// Maps the reference's "tile size" (feature elements per thread, must divide
+// the channel count) to vector width and vectors per lane.  tile == 0 picks
+// 16 bytes per lane.
+static LaneShape lane_shape(int64_t tile, int64_t channels, int esize, const void *p0, const void *p1,
+                            const char *what) {
+  const int64_t row_bytes = channels * esize;
+  if (tile <= 0) {
+    tile = 16 / esize;
+    while (tile > 1 && channels % tile != 0) tile >>= 1;
+  }
+  MNT_CHECK(channels % tile == 0, "Unsupported %s = %lld with tile size = %lld", what,
+            static_cast<long long>(channels), static_cast<long long>(tile));
+  const int64_t bytes_per_lane = tile * esize;
+  LaneShape shape;
+  shape.vb = pow2_vec(bytes_per_lane, row_bytes, p0, p1);
+  MNT_CHECK(shape.vb >= esize && shape.vb > 0, "feature rows are not aligned to their element size");
+  shape.nv = static_cast<int>(bytes_per_lane / shape.vb);
+  MNT_CHECK(shape.nv >= 1 && shape.nv <= 8 && (shape.nv & (shape.nv - 1)) == 0,
+            "Unsupported %s = %lld with tile size = %lld", what, static_cast<long long>(channels),
+            static_cast<long long>(tile));
+  shape.lanes_per_row = static_cast<int>(row_bytes / bytes_per_lane);
+  return shape;
+}
+
+template <typename IT>
+static void launch_gather(const LaneShape &sh, const void *sources, void *buffer, const IT *masks,
+                          const int *row_start, int64_t num_sources, int num_offsets, int row_bytes,
+                          hipStream_t stream) {
+  if (num_sources == 0 || num_offsets == 0) return;
+  const unsigned grid = static_cast<unsigned>(div_ceil(num_sources * sh.lanes_per_row, 256));
+#define MNT_G(VB, NV)                                                                            \
+  gather_kernel<VB, NV, IT><<<grid, 256, 0, stream>>>(static_cast<const unsigned char *>(sources), \
+                                                      static_cast<unsigned char *>(buffer), masks,  \
+                                                      row_start, num_sources, num_offsets,          \
+                                                      row_bytes, sh.lanes_per_row)
+#define MNT_GV(VB)                 \
+  switch (sh.nv) {                 \
+    case 1: MNT_G(VB, 1); break;   \
+    case 2: MNT_G(VB, 2); break;   \
+    case 4: MNT_G(VB, 4); break;   \
+    default: MNT_G(VB, 8); break;  \
+  }
+  switch (sh.vb) {
+    case 16: MNT_GV(16); break;
+    case 8: MNT_GV(8); break;
+    case 4: MNT_GV(4); break;
+    default: MNT_GV(2); break;
+  }
+#undef MNT_GV
+#undef MNT_G
+  check_launch("gather_kernel");
+}
+
+template <typename T, typename IT>
+static void launch_scatter(const LaneShape &sh, const void *buffer, void *targets, const IT *masks,
+                           const int *row_start, int64_t num_targets, int num_offsets, int row_bytes,
+                           int accumulate, hipStream_t stream) {
+  if (num_targets == 0) return;
+  const unsigned grid = static_cast<unsigned>(div_ceil(num_targets * sh.lanes_per_row, 256));
+#define MNT_S(VB, NV)                                                                              \
+  scatter_kernel<T, VB, NV, IT><<<grid, 256, 0, stream>>>(static_cast<const unsigned char *>(buffer), \
+                                                          static_cast<unsigned char *>(targets), masks, \
+                                                          row_start, num_targets, num_offsets,        \
+                                                          row_bytes, sh.lanes_per_row, accumulate)
+#define MNT_SV(VB)                 \
+  switch (sh.nv) {                 \
+    case 1: MNT_S(VB, 1); break;   \
+    case 2: MNT_S(VB, 2); break;   \
+    case 4: MNT_S(VB, 4); break;   \
+    default: MNT_S(VB, 8); break;  \
+  }
+  if (sh.vb == 16) {
+    MNT_SV(16);
+  } else if (sh.vb == 8) {
+    MNT_SV(8);
+  } else if (sh.vb == 4) {
+    MNT_SV(4);
+  } else {
+    if constexpr (sizeof(T) == 2) {
+      MNT_SV(2);
+    } else {
+      MNT_FAIL("feature rows are not aligned to their element size");
+    }
+  }
+#undef MNT_SV
+#undef MNT_S
+  check_launch("scatter_kernel");
+}
+
+template <typename T>
+static void launch_gemm(const T *a, T *c, const T *wt, const int *meta, int num_tiles, int K, int N,
+                        int Kp, int Np, hipStream_t stream) {
+  if (num_tiles == 0) return;
+  const bool vec = (static_cast<int64_t>(K) * sizeof(T)) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(a) % 16 == 0 && N % 4 == 0 &&
+                   reinterpret_cast<uintptr_t>(c) % 16 == 0;
+  const int tn = Np >= 128 ? 128 : (Np >= 64 ? 64 : 32);
+  dim3 grid(num_tiles, static_cast<unsigned>(div_ceil(Np, tn)));
+#define MNT_MM(TN)                                                                              \
+  do {                                                                                          \
+    if (vec) {                                                                                  \
+      grouped_gemm_kernel<T, TN, true><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np);  \
+    } else {                                                                                    \
+      grouped_gemm_kernel<T, TN, false><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np); \
+    }                                                                                           \
+  } while (0)
+  if (tn == 128) {
+    MNT_MM(128);
+  } else if (tn == 64) {
+    MNT_MM(64);
+  } else {
+    MNT_MM(32);
+  }
+#undef MNT_MM
+  check_launch("grouped_gemm_kernel");
+}
+
+// --------------------------------------------------------------- profiling ----
+
+static bool g_profile = false;
+static hipEvent_t g_events[5];
+static bool g_events_ready = false;
+static bool g_events_recorded = false;
+
+static void profile_mark(int slot, hipStream_t stream) {
+  if (!g_profile) return;
+  if (!g_events_ready) {
+    for (auto &e : g_events) MNT_HIP(hipEventCreate(&e));
+    g_events_ready = true;
+  }
+  MNT_HIP(hipEventRecord(g_events[slot], stream));
+  if (slot == 4) g_events_recorded = true;
+}
+
+// ------------------------------------------------------------ forward plan ----
+
+struct ForwardPlan {
+  int64_t active_offsets;            // offsets that go through gather/GEMM/scatter
+  bool shortcut;
+  std::vector<int64_t> cum;          // padded row prefix, active_offsets + 1
+  std::vector<int> meta;             // grouped-GEMM meta (see kernel)
+  std::vector<int> row_start;        // int copy of cum for gather / scatter
+  int num_tiles;
+  int64_t total_rows;
+};
+
+static ForwardPlan make_forward_plan(const int64_t *sizes, int64_t num_offsets, int64_t num_sources,
+                                     int64_t num_targets, bool allow_shortcut, bool has_threshold,
+                                     double threshold) {
+  ForwardPlan plan;
+  plan.shortcut = allow_shortcut && num_offsets > 0 && sizes[num_offsets - 1] == num_targets &&
+                  sizes[num_offsets - 1] == num_sources;
+  plan.active_offsets = plan.shortcut ? num_offsets - 1 : num_offsets;
+  std::vector<int64_t> buckets;
+  padding_buckets(sizes, plan.active_offsets, has_threshold, threshold, buckets);
+  cumsum_padded(sizes, plan.active_offsets, buckets, plan.cum);
+  plan.total_rows = plan.cum[plan.active_offsets];
+  MNT_CHECK(plan.total_rows <= INT32_MAX, "gather buffer of %lld rows exceeds the 32-bit row index",
+            static_cast<long long>(plan.total_rows));
+  plan.row_start.resize(plan.active_offsets + 1);
+  for (int64_t j = 0; j <= plan.active_offsets; ++j) plan.row_start[j] = static_cast<int>(plan.cum[j]);
+  std::vector<int> groups;
+  for (int64_t j = 0; j < plan.active_offsets; ++j) {
+    if (sizes[j] > 0) groups.push_back(static_cast<int>(j));
+  }
+  const int G = static_cast<int>(groups.size());
+  plan.meta.assign(1 + (G + 1) + (G + 1) + G + G, 0);
+  plan.meta[0] = G;
+  int *tile_prefix = plan.meta.data() + 1;
+  int *row_start = tile_prefix + G + 1;
+  int *rows = row_start + G + 1;
+  int *weight = rows + G;
+  int tiles = 0;
+  for (int i = 0; i < G; ++i) {
+    const int j = groups[i];
+    tile_prefix[i] = tiles;
+    row_start[i] = static_cast<int>(plan.cum[j]);
+    rows[i] = static_cast<int>(sizes[j]);
+    weight[i] = j;
+    tiles += static_cast<int>(div_ceil(sizes[j], kGemmRows));
+  }
+  tile_prefix[G] = tiles;
+  row_start[G] = static_cast<int>(plan.total_rows);
+  plan.num_tiles = tiles;
+  return plan;
+}
+
+static std::vector<int> direct_meta(int64_t rows, int weight_index) {
+  // one group: all rows of the source tensor against one weight matrix
+  std::vector<int> meta = {1, 0, static_cast<int>(div_ceil(rows, kGemmRows)), 0, static_cast<int>(rows),
+                           static_cast<int>(rows), weight_index};
+  return meta;
+}
+
+static void read_sizes(const void *sizes_dev, int index_dtype, int64_t num_offsets,
+                       std::vector<int64_t> &out, hipStream_t stream) {
+  out.resize(num_offsets);
+  if (num_offsets == 0) return;
+  const int isz = int_size(index_dtype);
+  std::vector<unsigned char> raw(static_cast<size_t>(isz) * num_offsets);
+  MNT_HIP(hipMemcpyAsync(raw.data(), sizes_dev, raw.size(), hipMemcpyDeviceToHost, stream));
+  MNT_HIP(hipStreamSynchronize(stream));
+  for (int64_t j = 0; j < num_offsets; ++j) {
+    out[j] = isz == 4 ? static_cast<int64_t>(reinterpret_cast<int32_t *>(raw.data())[j])
+                      : reinterpret_cast<int64_t *>(raw.data())[j];
+  }
+}
+
+template <typename T, typename IT>
+static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const ForwardPlan &plan,
+                          const T *sources, const T *weights, const IT *source_masks,
+                          const IT *target_masks, const IT *order, int64_t S, int64_t Tn, int64_t O,
+                          int64_t K, int64_t N, T *out, hipStream_t stream) {
+  Scope scope(stream);
+  const int kc = kChunkBytes / static_cast<int>(sizeof(T));
+  const int Kp = static_cast<int>(div_ceil(K, kc) * kc);
+  const int Np = static_cast<int>(div_ceil(N, 32) * 32);
+  const int active = static_cast<int>(plan.active_offsets);
+
+  profile_mark(0, stream);
+  T *wt = scope.alloc<T>(static_cast<size_t>(O) * Np * Kp);
+  {
+    const long long total = static_cast<long long>(O) * Np * Kp;
+    pack_weights_kernel<T, IT><<<grid_for(total, 256, 4096), 256, 0, stream>>>(
+        weights, order, static_cast<int>(O), static_cast<int>(K), static_cast<int>(N), Kp, Np, wt);
+    check_launch("pack_weights_kernel");
+  }
+  int *d_row_start = scope.alloc<int>(plan.row_start.size());
+  upload_ints(plan.row_start, d_row_start, stream);
+  int *d_meta = scope.alloc<int>(plan.meta.size());
+  upload_ints(plan.meta, d_meta, stream);
+  profile_mark(1, stream);
+
+  const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
+  T *abuf = scope.alloc<T>(rows * K);
+  T *cbuf = scope.alloc<T>(rows * N);
+
+  const LaneShape gsh = lane_shape(gather_tile, K, sizeof(T), sources, abuf, "num_source_features");
+  launch_gather<IT>(gsh, sources, abuf, source_masks, d_row_start, S, active,
+                    static_cast<int>(K * sizeof(T)), stream);
+  profile_mark(2, stream);
+
+  launch_gemm<T>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
+  if (plan.shortcut) {
+    std::vector<int> meta = direct_meta(S, static_cast<int>(O - 1));
+    int *d_direct = scope.alloc<int>(meta.size());
+    upload_ints(meta, d_direct, stream);
+    launch_gemm<T>(sources, out, wt, d_direct, meta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
+  }
+  profile_mark(3, stream);
+
+  const LaneShape ssh = lane_shape(scatter_tile, N, sizeof(T), cbuf, out, "num_target_features");
+  launch_scatter<T, IT>(ssh, cbuf, out, target_masks, d_row_start, Tn, active,
+                        static_cast<int>(N * sizeof(T)), plan.shortcut ? 1 : 0, stream);
+  profile_mark(4, stream);
+}
+
+}  // namespace mnt
+
+using namespace mnt;
+
+extern "C" int mnt_generate_padding_buckets(const int64_t *sizes_host, int64_t num_offsets,
+                                            int has_threshold, double threshold,
+                                            int64_t *buckets_out, int64_t *num_boundaries_out) {
+  return guarded([&] {
+    MNT_CHECK(num_offsets >= 0 && buckets_out != nullptr && num_boundaries_out != nullptr, "bad argument");
+    std::vector<int64_t> buckets;
+    padding_buckets(sizes_host, num_offsets, has_threshold != 0, threshold, buckets);
+    MNT_CHECK(buckets.back() == num_offsets, "bucket boundaries do not cover all offsets");
+    for (size_t i = 0; i < buckets.size(); ++i) buckets_out[i] = buckets[i];
+    *num_boundaries_out = static_cast<int64_t>(buckets.size());
+  });
+}
+
+extern "C" int mnt_cumsum_kernel_padded_sizes(const int64_t *sizes_host, int64_t num_offsets,
+                                              const int64_t *buckets, int64_t num_boundaries,
+                                              int64_t *cumsum_out) {
+  return guarded([&] {
+    MNT_CHECK(num_offsets >= 0 && num_boundaries >= 1 && cumsum_out != nullptr, "bad argument");
+    std::vector<int64_t> b(buckets, buckets + num_boundaries), cum;
+    MNT_CHECK(b.front() == 0 && b.back() == num_offsets, "bucket boundaries must run from 0 to the number of offsets");
+    cumsum_padded(sizes_host, num_offsets, b, cum);
+    for (int64_t j = 0; j <= num_offsets; ++j) cumsum_out[j] = cum[j];
+  });
+}
+
+#define MNT_DISPATCH_FI(float_dtype, index_dtype, CALL)               \
+  do {                                                                \
+    const bool i32_ = index_dtype == MNT_INT32;                       \
+    if (float_dtype == MNT_FLOAT32) {                                 \
+      if (i32_) { CALL(float, int32_t); } else { CALL(float, int64_t); }       \
+    } else if (float_dtype == MNT_FLOAT16) {                          \
+      if (i32_) { CALL(half_t, int32_t); } else { CALL(half_t, int64_t); }     \
+    } else {                                                          \
+      if (i32_) { CALL(bf16_t, int32_t); } else { CALL(bf16_t, int64_t); }     \
+    }                                                                 \
+  } while (0)
+
+extern "C" int mnt_sparse_convolution_forward(
+    int64_t gather_tile, int64_t scatter_tile, int allow_shortcut_matmul, int64_t parallel,
+    int has_threshold, double threshold, const void *sources, const void *weights,
+    const void *source_masks, const void *target_masks, const void *kernel_map_order,
+    const void *kernel_map_sizes, const int64_t *sizes_host, int64_t S, int64_t T, int64_t O,
+    int64_t K, int64_t N, int index_dtype, int float_dtype, void *out, void *stream_) {
+  (void)parallel;
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    int_size(index_dtype);
+    float_size(float_dtype);
+    MNT_CHECK(S >= 0 && T >= 0 && O >= 0 && K >= 1 && N >= 1 && S <= INT32_MAX && T <= INT32_MAX &&
+                  O <= 65535 && K <= 65536 && N <= 65536,
+              "bad shape S=%lld T=%lld O=%lld Cin=%lld Cout=%lld", (long long)S, (long long)T,
+              (long long)O, (long long)K, (long long)N);
+    if (T == 0) return;
+    MNT_CHECK(out != nullptr, "out is null");
+    std::vector<int64_t> sizes;
+    if (sizes_host != nullptr) {
+      sizes.assign(sizes_host, sizes_host + O);
+    } else {
+      read_sizes(kernel_map_sizes, index_dtype, O, sizes, stream);
+    }
+    for (int64_t j = 0; j < O; ++j) {
+      MNT_CHECK(sizes[j] >= 0 && sizes[j] <= T,
+                "kernel map size %lld of offset %lld is out of range", (long long)sizes[j], (long long)j);
+    }
+    ForwardPlan plan = make_forward_plan(sizes.data(), O, S, T, allow_shortcut_matmul != 0,
+                                         has_threshold != 0, threshold);
+#define MNT_CALL(FT, IT)                                                                          \
+  forward_typed<FT, IT>(gather_tile, scatter_tile, plan, static_cast<const FT *>(sources),          \
+                        static_cast<const FT *>(weights), static_cast<const IT *>(source_masks),    \
+                        static_cast<const IT *>(target_masks), static_cast<const IT *>(kernel_map_order), \
+                        S, T, O, K, N, static_cast<FT *>(out), stream)
+    MNT_DISPATCH_FI(float_dtype, index_dtype, MNT_CALL);
+#undef MNT_CALL
+  });
+}
+
+// ---------------------------------------------------------- stage timers ----
+
+namespace mnt {
+
+struct TimerScope {
+  hipEvent_t start, stop;
+  hipStream_t stream;
+  explicit TimerScope(hipStream_t s) : stream(s) {
+    MNT_HIP(hipEventCreate(&start));
+    MNT_HIP(hipEventCreate(&stop));
+  }
+  ~TimerScope() {
+    (void)hipEventDestroy(start);
+    (void)hipEventDestroy(stop);
+  }
+  void begin() { MNT_HIP(hipEventRecord(start, stream)); }
+  float end() {
+    MNT_HIP(hipEventRecord(stop, stream));
+    MNT_HIP(hipEventSynchronize(stop));
+    float ms = 0.0f;
+    MNT_HIP(hipEventElapsedTime(&ms, start, stop));
+    return ms;
+  }
+};
+
+template <typename T, typename IT>
+static float time_gather_typed(int64_t tile, const ForwardPlan &plan, const IT *source_masks,
+                               int64_t S, int64_t K, hipStream_t stream) {
+  Scope scope(stream);
+  const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
+  T *sources = scope.alloc<T>(static_cast<size_t>(S > 0 ? S : 1) * K);
+  T *abuf = scope.alloc<T>(rows * K);
+  int *d_row_start = scope.alloc<int>(plan.row_start.size());
+  upload_ints(plan.row_start, d_row_start, stream);
+  const LaneShape sh = lane_shape(tile, K, sizeof(T), sources, abuf, "num_source_features");
+  TimerScope timer(stream);
+  timer.begin();
+  launch_gather<IT>(sh, sources, abuf, source_masks, d_row_start, S, static_cast<int>(plan.active_offsets),
+                    static_cast<int>(K * sizeof(T)), stream);
+  return timer.end();
+}
+
+template <typename T, typename IT>
+static float time_scatter_typed(int64_t tile, const ForwardPlan &plan, const IT *target_masks,
+                                int64_t Tn, int64_t N, hipStream_t stream) {
+  Scope scope(stream);
+  const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
+  T *cbuf = scope.alloc<T>(rows * N);
+  T *out = scope.alloc<T>(static_cast<size_t>(Tn > 0 ? Tn : 1) * N);
+  int *d_row_start = scope.alloc<int>(plan.row_start.size());
+  upload_ints(plan.row_start, d_row_start, stream);
+  const LaneShape sh = lane_shape(tile, N, sizeof(T), cbuf, out, "num_target_features");
+  TimerScope timer(stream);
+  timer.begin();
+  launch_scatter<T, IT>(sh, cbuf, out, target_masks, d_row_start, Tn, static_cast<int>(plan.active_offsets),
+                        static_cast<int>(N * sizeof(T)), 0, stream);
+  return timer.end();
+}
+
+template <typename T>
+static float time_gemm_typed(const ForwardPlan &plan, const T *weights, int64_t S, int64_t O, int64_t K,
+                             int64_t N, hipStream_t stream) {
+  Scope scope(stream);
+  const int kc = kChunkBytes / static_cast<int>(sizeof(T));
+  const int Kp = static_cast<int>(div_ceil(K, kc) * kc);
+  const int Np = static_cast<int>(div_ceil(N, 32) * 32);
+  const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
+  T *wt = scope.alloc<T>(static_cast<size_t>(O) * Np * Kp);
+  T *abuf = scope.alloc<T>(rows * K);
+  T *cbuf = scope.alloc<T>(rows * N);
+  T *direct_a = nullptr, *direct_c = nullptr;
+  int *d_direct = nullptr;
+  std::vector<int> dmeta;
+  if (plan.shortcut) {
+    direct_a = scope.alloc<T>(static_cast<size_t>(S) * K);
+    direct_c = scope.alloc<T>(static_cast<size_t>(S) * N);
+    dmeta = direct_meta(S, static_cast<int>(O - 1));
+    d_direct = scope.alloc<int>(dmeta.size());
+    upload_ints(dmeta, d_direct, stream);
+  }
+  const long long total = static_cast<long long>(O) * Np * Kp;
+  pack_weights_kernel<T, int32_t><<<grid_for(total, 256, 4096), 256, 0, stream>>>(
+      weights, nullptr, static_cast<int>(O), static_cast<int>(K), static_cast<int>(N), Kp, Np, wt);
+  check_launch("pack_weights_kernel");
+  // operands of a timing run are scratch: clear them so no NaN patterns slow or trap anything
+  MNT_HIP(hipMemsetAsync(abuf, 0, rows * K * sizeof(T), stream));
+  if (plan.shortcut) MNT_HIP(hipMemsetAsync(direct_a, 0, static_cast<size_t>(S) * K * sizeof(T), stream));
+  int *d_meta = scope.alloc<int>(plan.meta.size());
+  upload_ints(plan.meta, d_meta, stream);
+  TimerScope timer(stream);
+  timer.begin();
+  launch_gemm<T>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
+  if (plan.shortcut) {
+    launch_gemm<T>(direct_a, direct_c, wt, d_direct, dmeta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
+  }
+  return timer.end();
+}
+
+static ForwardPlan timer_plan(const void *sizes_dev, int index_dtype, int64_t S, int64_t T, int64_t O,
+                              int allow_shortcut, int has_threshold, double threshold,
+                              hipStream_t stream) {
+  std::vector<int64_t> sizes;
+  read_sizes(sizes_dev, index_dtype, O, sizes, stream);
+  return make_forward_plan(sizes.data(), O, S, T, allow_shortcut != 0, has_threshold != 0, threshold);
+}
+
+}  // namespace mnt
+
+extern "C" int mnt_time_gather(int64_t tile, int allow_shortcut_matmul, int has_threshold,
+                               double threshold, const void *source_masks,
+                               const void *kernel_map_sizes, int64_t S, int64_t T, int64_t O,
+                               int64_t K, int64_t N, int index_dtype, int float_dtype,
+                               float *ms_out, void *stream_) {
+  (void)N;
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    float_size(float_dtype);
+    ForwardPlan plan = timer_plan(kernel_map_sizes, index_dtype, S, T, O, allow_shortcut_matmul,
+                                  has_threshold, threshold, stream);
+#define MNT_CALL(FT, IT) \
+  *ms_out = time_gather_typed<FT, IT>(tile, plan, static_cast<const IT *>(source_masks), S, K, stream)
+    MNT_DISPATCH_FI(float_dtype, index_dtype, MNT_CALL);
+#undef MNT_CALL
+  });
+}
+
+extern "C" int mnt_time_scatter(int64_t tile, int allow_shortcut_matmul, int has_threshold,
+                                double threshold, const void *target_masks,
+                                const void *kernel_map_sizes, int64_t S, int64_t T, int64_t O,
+                                int64_t K, int64_t N, int index_dtype, int float_dtype,
+                                float *ms_out, void *stream_) {
+  (void)K;
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    float_size(float_dtype);
+    ForwardPlan plan = timer_plan(kernel_map_sizes, index_dtype, S, T, O, allow_shortcut_matmul,
+                                  has_threshold, threshold, stream);
+#define MNT_CALL(FT, IT) \
+  *ms_out = time_scatter_typed<FT, IT>(tile, plan, static_cast<const IT *>(target_masks), T, N, stream)
+    MNT_DISPATCH_FI(float_dtype, index_dtype, MNT_CALL);
+#undef MNT_CALL
+  });
+}
+
+extern "C" int mnt_time_gemm(int allow_shortcut_matmul, int64_t parallel, int has_threshold,
+                             double threshold, const void *weights, const void *kernel_map_sizes,
+                             int64_t S, int64_t T, int64_t O, int64_t K, int64_t N,
+                             int index_dtype, int float_dtype, float *ms_out, void *stream_) {
+  (void)parallel;
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    float_size(float_dtype);
+    ForwardPlan plan = timer_plan(kernel_map_sizes, index_dtype, S, T, O, allow_shortcut_matmul,
+                                  has_threshold, threshold, stream);
+    if (float_dtype == MNT_FLOAT32) {
+      *ms_out = time_gemm_typed<float>(plan, static_cast<const float *>(weights), S, O, K, N, stream);
+    } else if (float_dtype == MNT_FLOAT16) {
+      *ms_out = time_gemm_typed<half_t>(plan, static_cast<const half_t *>(weights), S, O, K, N, stream);
+    } else {
+      *ms_out = time_gemm_typed<bf16_t>(plan, static_cast<const bf16_t *>(weights), S, O, K, N, stream);
+    }
+  });
+}
+
+extern "C" int mnt_profile_enable(int on) {
+  g_profile = on != 0;
+  g_events_recorded = false;
+  return 0;
+}
+
+extern "C" int mnt_profile_read(float *ms4_out) {
+  return guarded([&] {
+    MNT_CHECK(g_profile && g_events_recorded, "no profiled forward call has been recorded");
+    MNT_HIP(hipEventSynchronize(g_events[4]));
+    for (int i = 0; i < 4; ++i) MNT_HIP(hipEventElapsedTime(&ms4_out[i], g_events[i], g_events[i + 1]));
+  });
+}

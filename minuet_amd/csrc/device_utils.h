@@ -1,0 +1,71 @@
+// Device-side helpers shared by the Map kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "common.h"
+
+namespace mnt {
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ unsigned lane_id() { return threadIdx.x & (kWave - 1); }
+
+__device__ __forceinline__ unsigned long long lanes_below() {
+  return (1ull << lane_id()) - 1ull;
+}
+
+// Batch of row i: the g with dims[g] <= i < dims[g+1] (dims has num_batches+1
+// entries).  Rows at or past dims[num_batches] land in the last batch.
+template <typename IT>
+__device__ __forceinline__ int batch_of(long long i, const IT *__restrict__ dims,
+                                        int num_batches) {
+  int lo = 0, hi = num_batches - 1;
+  while (lo < hi) {
+    int mid = (lo + hi) >> 1;
+    if (static_cast<long long>(dims[mid + 1]) > i) {
+      hi = mid;
+    } else {
+      lo = mid + 1;
+    }
+  }
+  return lo;
+}
+
+// Whether some batch ends exactly at row index `end` (exclusive end).
+template <typename IT>
+__device__ __forceinline__ bool is_batch_end(long long end, const IT *__restrict__ dims,
+                                             int num_batches) {
+  int lo = 0, hi = num_batches;
+  while (lo < hi) {
+    int mid = (lo + hi) >> 1;
+    if (static_cast<long long>(dims[mid]) < end) {
+      lo = mid + 1;
+    } else {
+      hi = mid;
+    }
+  }
+  return lo <= num_batches && static_cast<long long>(dims[lo]) == end;
+}
+
+// Key of one row under a Frame (see common.h).  `batch` is ignored when the
+// frame has no batch field.
+template <typename CT>
+__device__ __forceinline__ unsigned long long pack_row(const CT *__restrict__ row,
+                                                       const Frame &f, int batch) {
+  unsigned long long key = 0;
+#pragma unroll
+  for (int k = 0; k < MNT_MAX_NDIM; ++k) {
+    if (k < f.ndim) {
+      unsigned long long v = static_cast<unsigned long long>(static_cast<long long>(row[k])) -
+                             static_cast<unsigned long long>(f.lo[k]);
+      key |= v << f.shift[k];
+    }
+  }
+  if (f.batch_width > 0) key |= static_cast<unsigned long long>(batch) << f.batch_shift;
+  return key;
+}
+
+}  // namespace mnt

@@ -1,0 +1,707 @@
+// Map step, part 3: kernel-map query on packed voxel keys, per-offset sizes,
+// stable size order, rank tables (masks) and per-offset pair lists.
+//
+// The dense map has the meaning of QuerySortedIndexWithOffsets
+// (csrc/minuet/cuda/kernels/query_sorted_index_with_offsets.cuh:36-77, batched:
+// multi_query_sorted_index_with_offsets.cuh:38-91): M[o,t] = j iff
+// sources[j] == targets[t] + offsets[o] within one batch.  Sizes and rank
+// tables follow ComputeKernelMapSizes / ComputeKernelMapMasks
+// (csrc/minuet/cuda/functions/scan.cu:220-365).
+//
+// Layout of one query workgroup: 512 consecutive sorted targets.  Because the
+// targets are sorted, every shifted query of the tile lies between
+// key(first)+min_delta and key(last)+max_delta, so ONE window of the sorted
+// sources serves all offsets.  The window is packed to 64-bit keys and staged
+// in LDS (2048 keys at a time); every (offset, target) pair is then resolved
+// by a branch-free binary search in LDS, and hits are counted per offset with
+// wavefront ballots.
+#include "device_utils.h"
+#include "sort.h"
+
+namespace mnt {
+
+constexpr int kQueryBlock = 256;
+constexpr int kTargetsPerTile = 512;
+constexpr int kWindowChunk = 2048;
+
+template <typename CT, typename BT>
+struct KeyReader {
+  const CT *coords;
+  const BT *batch_dims;
+  int num_batches;
+  long long count;
+  __device__ __forceinline__ unsigned long long operator()(long long i, const Frame &f) const {
+    int b = 0;
+    if (f.batch_width > 0) b = batch_of<BT>(i, batch_dims, num_batches);
+    return pack_row<CT>(coords + i * f.ndim, f, b);
+  }
+};
+
+// First index in [0, count) whose key is >= q, found by one wavefront probing
+// 64 equally spaced rows per step.  All lanes must call with the same q.
+template <typename CT, typename BT>
+__device__ __forceinline__ long long wave_lower_bound(const KeyReader<CT, BT> &src, const Frame &f,
+                                                      unsigned long long q) {
+  long long lo = 0, hi = src.count;
+  const int lane = lane_id();
+  while (hi > lo) {
+    const long long len = hi - lo;
+    const long long step = (len + kWave - 1) / kWave;
+    const long long idx = lo + lane * step;
+    const bool less = idx < hi && src(idx, f) < q;
+    const int c = __popcll(__ballot(less));
+    if (c == 0) {
+      hi = lo;
+    } else {
+      const long long new_hi = lo + c * step;
+      lo = lo + (c - 1) * step + 1;
+      hi = new_hi < hi ? new_hi : hi;
+    }
+  }
+  return lo;
+}
+
+template <typename CT, typename BT, typename OT>
+__global__ __launch_bounds__(kQueryBlock) void query_kernel(
+    KeyReader<CT, BT> src, KeyReader<CT, BT> tgt, Frame frame,
+    const long long *__restrict__ deltas, int num_offsets, long long delta_min,
+    long long delta_max, OT *__restrict__ kernel_map, unsigned *__restrict__ tile_counts,
+    int num_tiles) {
+  extern __shared__ unsigned s_counts[];                 // [num_offsets]
+  __shared__ unsigned long long win[kWindowChunk];
+  __shared__ long long s_bounds[2];
+  __shared__ unsigned long long s_next_first;
+
+  const int tid = threadIdx.x;
+  const long long num_targets = tgt.count;
+  const long long t0 = static_cast<long long>(blockIdx.x) * kTargetsPerTile;
+  const long long t_end = t0 + kTargetsPerTile < num_targets ? t0 + kTargetsPerTile : num_targets;
+
+  for (int o = tid; o < num_offsets; o += kQueryBlock) s_counts[o] = 0;
+
+  // window of sources that can match any (offset, target) pair of this tile
+  const int w = tid >> 6;
+  if (w < 2) {
+    const unsigned long long edge = w == 0 ? tgt(t0, frame) + static_cast<unsigned long long>(delta_min)
+                                           : tgt(t_end - 1, frame) + static_cast<unsigned long long>(delta_max) + 1ull;
+    const long long pos = wave_lower_bound<CT, BT>(src, frame, edge);
+    if (lane_id() == 0) s_bounds[w] = pos;
+  }
+
+  long long tq[2];
+  unsigned long long tk[2];
+  bool tv[2];
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    tq[r] = t0 + r * kQueryBlock + tid;
+    tv[r] = tq[r] < t_end;
+    tk[r] = tv[r] ? tgt(tq[r], frame) : 0ull;
+  }
+  __syncthreads();
+  const long long w_lo = s_bounds[0];
+  const long long w_hi = s_bounds[1] > w_lo ? s_bounds[1] : w_lo;
+  const long long span = w_hi - w_lo;
+  const int num_chunks = span <= kWindowChunk ? 1 : static_cast<int>((span + kWindowChunk - 1) / kWindowChunk);
+
+  for (int c = 0; c < num_chunks; ++c) {
+    const long long c0 = w_lo + static_cast<long long>(c) * kWindowChunk;
+    const long long c1 = c0 + kWindowChunk < w_hi ? c0 + kWindowChunk : w_hi;
+    const int len = static_cast<int>(c1 - c0);
+    if (c > 0) __syncthreads();
+    for (int i = tid; i < kWindowChunk; i += kQueryBlock) {
+      win[i] = i < len ? src(c0 + i, frame) : ~0ull;
+    }
+    if (tid == 0) s_next_first = c1 < w_hi ? src(c1, frame) : ~0ull;
+    __syncthreads();
+    const unsigned long long first_key = win[0];
+    const unsigned long long next_first = s_next_first;
+    const bool is_first = c == 0;
+    const bool is_last = c == num_chunks - 1;
+    int top = 1;
+    while (top * 2 < len) top *= 2;      // highest power of two below len (>= 1)
+
+    for (int o = 0; o < num_offsets; ++o) {
+      const unsigned long long delta = static_cast<unsigned long long>(deltas[o]);
+      unsigned hits = 0;
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const unsigned long long q = tk[r] + delta;
+        const bool mine = tv[r] && (is_first || q >= first_key) && (is_last || q < next_first);
+        int pos = 0;
+        for (int step = top; step >= 1; step >>= 1) {
+          if (win[pos + step] <= q) pos += step;
+        }
+        const bool hit = mine && len > 0 && win[pos] == q;
+        if (mine) {
+          kernel_map[static_cast<long long>(o) * num_targets + tq[r]] =
+              hit ? static_cast<OT>(c0 + pos) : static_cast<OT>(-1);
+        }
+        hits += __popcll(__ballot(hit));
+      }
+      if (tile_counts != nullptr && hits != 0 && lane_id() == 0) atomicAdd(&s_counts[o], hits);
+    }
+  }
+  if (tile_counts != nullptr) {
+    __syncthreads();
+    for (int o = tid; o < num_offsets; o += kQueryBlock) {
+      tile_counts[static_cast<long long>(o) * num_tiles + blockIdx.x] = s_counts[o];
+    }
+  }
+}
+
+// Hit counts of every (row, tile of 512 targets) of an existing dense map.
+template <typename IT>
+__global__ __launch_bounds__(kQueryBlock) void count_tiles_kernel(
+    const IT *__restrict__ kernel_map, long long num_targets, unsigned *__restrict__ tile_counts,
+    int num_tiles) {
+  __shared__ unsigned s_sum;
+  const int o = blockIdx.y;
+  const long long t0 = static_cast<long long>(blockIdx.x) * kTargetsPerTile;
+  if (threadIdx.x == 0) s_sum = 0;
+  __syncthreads();
+  unsigned hits = 0;
+#pragma unroll
+  for (int r = 0; r < kTargetsPerTile / kQueryBlock; ++r) {
+    const long long t = t0 + r * kQueryBlock + threadIdx.x;
+    const bool hit = t < num_targets && kernel_map[static_cast<long long>(o) * num_targets + t] != static_cast<IT>(-1);
+    hits += __popcll(__ballot(hit));
+  }
+  if (lane_id() == 0 && hits) atomicAdd(&s_sum, hits);
+  __syncthreads();
+  if (threadIdx.x == 0) tile_counts[static_cast<long long>(o) * num_tiles + blockIdx.x] = s_sum;
+}
+
+// One workgroup per row: exclusive scan of its tile counts in place and the
+// row total.
+__global__ __launch_bounds__(256) void tile_scan_kernel(unsigned *__restrict__ tile_counts,
+                                                        int num_tiles,
+                                                        unsigned *__restrict__ row_sizes) {
+  __shared__ unsigned partial[256];
+  unsigned *row = tile_counts + static_cast<long long>(blockIdx.x) * num_tiles;
+  const int t = threadIdx.x;
+  const int chunk = (num_tiles + 255) / 256;
+  const int lo = t * chunk;
+  const int hi = lo + chunk < num_tiles ? lo + chunk : num_tiles;
+  unsigned sum = 0;
+  for (int i = lo; i < hi; ++i) sum += row[i];
+  partial[t] = sum;
+  __syncthreads();
+  for (int off = 1; off < 256; off <<= 1) {
+    unsigned v = t >= off ? partial[t - off] : 0;
+    __syncthreads();
+    partial[t] += v;
+    __syncthreads();
+  }
+  unsigned run = partial[t] - sum;
+  for (int i = lo; i < hi; ++i) {
+    unsigned v = row[i];
+    row[i] = run;
+    run += v;
+  }
+  if (t == 255) row_sizes[blockIdx.x] = partial[255];
+}
+
+// Stable ascending order of the rows by size (or identity), the inverse
+// permutation, the sizes in row order and their exclusive prefix.
+// plan layout (unsigned, 4 blocks of num_offsets (+1 for the prefix)):
+//   order[j] | position_of[o] | sorted_sizes[j] | prefix[j] (num_offsets+1)
+__global__ __launch_bounds__(256) void order_kernel(const unsigned *__restrict__ row_sizes,
+                                                    int num_offsets, int reorder,
+                                                    unsigned *__restrict__ plan) {
+  unsigned *order = plan;
+  unsigned *position_of = plan + num_offsets;
+  unsigned *sorted_sizes = plan + 2 * num_offsets;
+  unsigned *prefix = plan + 3 * num_offsets;
+  for (int o = threadIdx.x; o < num_offsets; o += blockDim.x) {
+    const unsigned mine = row_sizes[o];
+    int pos = o;
+    if (reorder) {
+      pos = 0;
+      for (int p = 0; p < num_offsets; ++p) {
+        const unsigned other = row_sizes[p];
+        pos += (other < mine || (other == mine && p < o)) ? 1 : 0;
+      }
+    }
+    order[pos] = o;
+    position_of[o] = pos;
+    sorted_sizes[pos] = mine;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned run = 0;
+    for (int j = 0; j < num_offsets; ++j) {
+      prefix[j] = run;
+      run += sorted_sizes[j];
+    }
+    prefix[num_offsets] = run;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void fill_kernel(T *__restrict__ data, long long n, T value) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
+    data[i] = value;
+  }
+}
+
+// One wavefront per (row, tile): walks the 512 targets of the tile in order and
+// ranks the hits.  Writes any of: target rank table, source rank table, pair
+// lists.  `position_of` maps an offset to its output row (null = identity) and
+// `row_base` gives the list position of the first hit of an output row.
+template <typename IT>
+__global__ __launch_bounds__(kQueryBlock) void emit_kernel(
+    const IT *__restrict__ kernel_map, long long num_sources, long long num_targets,
+    int num_offsets, const unsigned *__restrict__ tile_bases, int num_tiles,
+    const unsigned *__restrict__ position_of, const unsigned *__restrict__ row_base,
+    IT *__restrict__ source_masks, IT *__restrict__ target_masks, int *__restrict__ in_idx,
+    int *__restrict__ out_idx) {
+  const int o = blockIdx.y * (kQueryBlock / kWave) + (threadIdx.x >> 6);
+  if (o >= num_offsets) return;
+  const int lane = lane_id();
+  const long long row = position_of ? position_of[o] : o;
+  const long long t0 = static_cast<long long>(blockIdx.x) * kTargetsPerTile;
+  unsigned running = tile_bases[static_cast<long long>(o) * num_tiles + blockIdx.x];
+  const long long list_base = row_base ? static_cast<long long>(row_base[row]) : 0;
+  const unsigned long long below = (1ull << lane) - 1ull;
+#pragma unroll 2
+  for (int r = 0; r < kTargetsPerTile / kWave; ++r) {
+    const long long t = t0 + r * kWave + lane;
+    const bool valid = t < num_targets;
+    const IT m = valid ? kernel_map[static_cast<long long>(o) * num_targets + t] : static_cast<IT>(-1);
+    const bool hit = m != static_cast<IT>(-1);
+    const unsigned long long votes = __ballot(hit);
+    const unsigned rank = running + __popcll(votes & below);
+    if (valid && target_masks) target_masks[row * num_targets + t] = hit ? static_cast<IT>(rank) : static_cast<IT>(-1);
+    if (hit) {
+      if (source_masks) source_masks[row * num_sources + static_cast<long long>(m)] = static_cast<IT>(rank);
+      if (in_idx) {
+        in_idx[list_base + rank] = static_cast<int>(m);
+        out_idx[list_base + rank] = static_cast<int>(t);
+      }
+    }
+    running += __popcll(votes);
+  }
+}
+
+template <typename IT>
+__global__ __launch_bounds__(256) void export_sizes_kernel(const unsigned *__restrict__ sizes,
+                                                           int n, IT *__restrict__ out) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = static_cast<IT>(sizes[i]);
+}
+
+// ------------------------------------------------------------------ host ----
+
+static int width_of(unsigned long long range) {
+  return range == 0 ? 0 : 64 - __builtin_clzll(range);
+}
+
+struct QueryPlan {
+  Frame frame;
+  std::vector<long long> deltas;
+  long long delta_min, delta_max;
+};
+
+// Builds the packing frame from the coordinate bounds of sources and targets
+// (h_bounds: 8 slots each, min then max) and the kernel offsets.
+static QueryPlan make_plan(const long long *src_bounds, const long long *tgt_bounds,
+                           const int64_t *offsets, int64_t num_offsets, int ndim,
+                           int64_t num_batches) {
+  QueryPlan plan;
+  memset(&plan.frame, 0, sizeof(Frame));
+  Frame &f = plan.frame;
+  f.ndim = ndim;
+  int bits = 0;
+  for (int k = ndim - 1; k >= 0; --k) {
+    long long omin = 0, omax = 0;
+    for (int64_t o = 0; o < num_offsets; ++o) {
+      long long d = offsets[o * ndim + k];
+      omin = d < omin ? d : omin;
+      omax = d > omax ? d : omax;
+    }
+    __int128 lo = static_cast<__int128>(tgt_bounds[k]) + omin;
+    __int128 hi = static_cast<__int128>(tgt_bounds[MNT_MAX_NDIM + k]) + omax;
+    if (src_bounds[k] < lo) lo = src_bounds[k];
+    if (src_bounds[MNT_MAX_NDIM + k] > hi) hi = src_bounds[MNT_MAX_NDIM + k];
+    __int128 range = hi - lo;
+    MNT_CHECK(range >= 0 && range < (static_cast<__int128>(1) << 63) &&
+                  lo >= INT64_MIN && lo <= INT64_MAX,
+              "coordinate range of dimension %d is too large to pack into a voxel key", k);
+    f.lo[k] = static_cast<long long>(lo);
+    f.width[k] = width_of(static_cast<unsigned long long>(range));
+    f.shift[k] = bits < 63 ? bits : 63;
+    bits += f.width[k];
+  }
+  f.batch_width = num_batches > 1 ? width_of(static_cast<unsigned long long>(num_batches - 1)) : 0;
+  f.batch_shift = bits < 63 ? bits : 63;
+  bits += f.batch_width;
+  f.total_bits = bits;
+  MNT_CHECK(bits <= 63,
+            "voxel keys need %d bits (coordinate ranges plus kernel reach plus batch id); at most "
+            "63 are supported",
+            bits);
+  plan.deltas.resize(num_offsets);
+  plan.delta_min = 0;
+  plan.delta_max = 0;
+  for (int64_t o = 0; o < num_offsets; ++o) {
+    long long d = 0;
+    for (int k = 0; k < ndim; ++k) {
+      d += static_cast<long long>(static_cast<unsigned long long>(offsets[o * ndim + k]) << f.shift[k]);
+    }
+    plan.deltas[o] = d;
+    if (o == 0 || d < plan.delta_min) plan.delta_min = d;
+    if (o == 0 || d > plan.delta_max) plan.delta_max = d;
+  }
+  return plan;
+}
+
+struct QueryArgs {
+  const void *sources;
+  int64_t num_sources;
+  const void *targets;
+  int64_t num_targets;
+  int ndim;
+  int coord_dtype;
+  const void *source_batch_dims;
+  const void *target_batch_dims;
+  int64_t num_batches;
+  int batch_dtype;
+};
+
+static void check_query_args(const QueryArgs &a, int64_t num_offsets) {
+  MNT_CHECK(a.ndim >= 1 && a.ndim <= MNT_MAX_NDIM, "ndim must be in [1, %d] but found %d",
+            MNT_MAX_NDIM, a.ndim);
+  MNT_CHECK(a.num_sources >= 0 && a.num_sources <= INT32_MAX && a.num_targets >= 0 &&
+                a.num_targets <= INT32_MAX,
+            "number of sources / targets out of range");
+  MNT_CHECK(num_offsets >= 0 && num_offsets <= 65535, "number of offsets %lld out of range",
+            static_cast<long long>(num_offsets));
+  MNT_CHECK((a.source_batch_dims == nullptr) == (a.target_batch_dims == nullptr),
+            "source_batch_dims and target_batch_dims must be both provided or neither provided");
+  int_size(a.coord_dtype);
+  if (a.source_batch_dims) {
+    int_size(a.batch_dtype);
+    MNT_CHECK(a.num_batches >= 1, "batch dims must have at least 2 entries");
+  }
+}
+
+template <typename CT, typename BT, typename OT>
+static void launch_query(const QueryArgs &a, const QueryPlan &plan, const long long *d_deltas,
+                         int num_offsets, OT *kernel_map, unsigned *tile_counts, int num_tiles,
+                         hipStream_t stream) {
+  KeyReader<CT, BT> src{static_cast<const CT *>(a.sources), static_cast<const BT *>(a.source_batch_dims),
+                        static_cast<int>(a.num_batches), a.num_sources};
+  KeyReader<CT, BT> tgt{static_cast<const CT *>(a.targets), static_cast<const BT *>(a.target_batch_dims),
+                        static_cast<int>(a.num_batches), a.num_targets};
+  const size_t dyn = sizeof(unsigned) * static_cast<size_t>(num_offsets > 0 ? num_offsets : 1);
+  query_kernel<CT, BT, OT><<<num_tiles, kQueryBlock, dyn, stream>>>(
+      src, tgt, plan.frame, d_deltas, num_offsets, plan.delta_min, plan.delta_max, kernel_map,
+      tile_counts, num_tiles);
+  check_launch("query_kernel");
+}
+
+// Runs the query into kernel_map (element size out_size) and, when tile_counts
+// is given, the per-(offset, tile) hit counts.  offsets_host: int64 [O, ndim].
+static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t num_offsets,
+                      void *kernel_map, int out_dtype, unsigned *tile_counts, Scope &scope,
+                      hipStream_t stream) {
+  const int num_tiles = static_cast<int>(div_ceil(a.num_targets, kTargetsPerTile));
+  const bool batched = a.source_batch_dims != nullptr && a.num_batches > 1;
+  long long *d_bounds = scope.alloc<long long>(4 * MNT_MAX_NDIM);
+  enqueue_bounds(a.sources, a.num_sources, a.ndim, a.coord_dtype, d_bounds, true, stream);
+  enqueue_bounds(a.targets, a.num_targets, a.ndim, a.coord_dtype, d_bounds + 2 * MNT_MAX_NDIM, true, stream);
+  long long *h_bounds = static_cast<long long *>(scope.arena().pinned());
+  MNT_HIP(hipMemcpyAsync(h_bounds, d_bounds, sizeof(long long) * 4 * MNT_MAX_NDIM,
+                         hipMemcpyDeviceToHost, stream));
+  MNT_HIP(hipStreamSynchronize(stream));
+  QueryPlan plan = make_plan(h_bounds, h_bounds + 2 * MNT_MAX_NDIM, offsets_host, num_offsets,
+                             a.ndim, batched ? a.num_batches : 1);
+  // Upload the packed offsets through the pinned block (past the bounds
+  // slots).  The stream was synchronised above, so no earlier copy still
+  // reads this block.
+  MNT_CHECK(sizeof(long long) * num_offsets + 512 <= Arena::kPinnedBytes,
+            "too many kernel offsets (%lld)", static_cast<long long>(num_offsets));
+  long long *h_deltas = reinterpret_cast<long long *>(static_cast<char *>(scope.arena().pinned()) + 512);
+  memcpy(h_deltas, plan.deltas.data(), sizeof(long long) * num_offsets);
+  long long *d_deltas = scope.alloc<long long>(num_offsets);
+  MNT_HIP(hipMemcpyAsync(d_deltas, h_deltas, sizeof(long long) * num_offsets,
+                         hipMemcpyHostToDevice, stream));
+  QueryArgs b = a;
+  if (!batched) {
+    b.source_batch_dims = nullptr;
+    b.target_batch_dims = nullptr;
+    b.num_batches = 1;
+  }
+  const bool c32 = a.coord_dtype == MNT_INT32;
+  const bool b32 = !batched || a.batch_dtype == MNT_INT32;
+  const bool o32 = out_dtype == MNT_INT32;
+  const int no = static_cast<int>(num_offsets);
+#define MNT_Q(CT, BT, OT) \
+  launch_query<CT, BT, OT>(b, plan, d_deltas, no, static_cast<OT *>(kernel_map), tile_counts, num_tiles, stream)
+  if (c32 && b32 && o32) MNT_Q(int32_t, int32_t, int32_t);
+  else if (c32 && b32) MNT_Q(int32_t, int32_t, int64_t);
+  else if (c32 && o32) MNT_Q(int32_t, int64_t, int32_t);
+  else if (c32) MNT_Q(int32_t, int64_t, int64_t);
+  else if (b32 && o32) MNT_Q(int64_t, int32_t, int32_t);
+  else if (b32) MNT_Q(int64_t, int32_t, int64_t);
+  else if (o32) MNT_Q(int64_t, int64_t, int32_t);
+  else MNT_Q(int64_t, int64_t, int64_t);
+#undef MNT_Q
+}
+
+template <typename T>
+static void enqueue_fill(T *data, int64_t n, T value, hipStream_t stream) {
+  if (n <= 0) return;
+  fill_kernel<T><<<grid_for(n, 256 * 4, 8192), 256, 0, stream>>>(data, n, value);
+  check_launch("fill_kernel");
+}
+
+static void enqueue_count_tiles(const void *kernel_map, int index_dtype, int64_t num_offsets,
+                                int64_t num_targets, unsigned *tile_counts, int num_tiles,
+                                hipStream_t stream) {
+  dim3 grid(num_tiles, static_cast<unsigned>(num_offsets));
+  if (index_dtype == MNT_INT32) {
+    count_tiles_kernel<int32_t><<<grid, kQueryBlock, 0, stream>>>(
+        static_cast<const int32_t *>(kernel_map), num_targets, tile_counts, num_tiles);
+  } else {
+    count_tiles_kernel<int64_t><<<grid, kQueryBlock, 0, stream>>>(
+        static_cast<const int64_t *>(kernel_map), num_targets, tile_counts, num_tiles);
+  }
+  check_launch("count_tiles_kernel");
+}
+
+template <typename IT>
+static void enqueue_emit(const IT *kernel_map, int64_t num_sources, int64_t num_targets,
+                         int num_offsets, const unsigned *tile_bases, int num_tiles,
+                         const unsigned *position_of, const unsigned *row_base, IT *source_masks,
+                         IT *target_masks, int *in_idx, int *out_idx, hipStream_t stream) {
+  if (source_masks) enqueue_fill<IT>(source_masks, static_cast<int64_t>(num_offsets) * num_sources, static_cast<IT>(-1), stream);
+  if (num_targets == 0 || num_offsets == 0) return;
+  dim3 grid(num_tiles, static_cast<unsigned>(div_ceil(num_offsets, kQueryBlock / kWave)));
+  emit_kernel<IT><<<grid, kQueryBlock, 0, stream>>>(kernel_map, num_sources, num_targets, num_offsets,
+                                                   tile_bases, num_tiles, position_of, row_base,
+                                                   source_masks, target_masks, in_idx, out_idx);
+  check_launch("emit_kernel");
+}
+
+// persistent-state header of the two-phase kernel-map build
+struct MapState {
+  int64_t num_sources, num_targets, num_offsets;
+  int num_tiles;
+  int reorder;
+  const void *kernel_map;
+};
+
+}  // namespace mnt
+
+using namespace mnt;
+
+extern "C" int mnt_query_sorted_index_with_offsets(
+    const void *sources, int64_t num_sources, const void *targets, int64_t num_targets,
+    const void *offsets, int64_t num_offsets, int ndim, int coord_dtype,
+    const void *source_batch_dims, const void *target_batch_dims, int64_t num_batches,
+    int batch_dtype, void *kernel_map_out, int out_dtype, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    QueryArgs a{sources, num_sources, targets, num_targets, ndim, coord_dtype,
+                source_batch_dims, target_batch_dims, num_batches, batch_dtype};
+    check_query_args(a, num_offsets);
+    const int osz = int_size(out_dtype);
+    if (num_targets == 0 || num_offsets == 0) return;
+    MNT_CHECK(kernel_map_out != nullptr && offsets != nullptr, "null argument");
+    if (num_sources == 0) {
+      MNT_HIP(hipMemsetAsync(kernel_map_out, 0xFF, static_cast<size_t>(osz) * num_offsets * num_targets, stream));
+      return;
+    }
+    Scope scope(stream);
+    // offsets live on the device in the reference interface: bring them over
+    const int csz = int_size(coord_dtype);
+    std::vector<unsigned char> raw(static_cast<size_t>(csz) * num_offsets * ndim);
+    MNT_HIP(hipMemcpyAsync(raw.data(), offsets, raw.size(), hipMemcpyDeviceToHost, stream));
+    MNT_HIP(hipStreamSynchronize(stream));
+    std::vector<int64_t> host_offsets(static_cast<size_t>(num_offsets) * ndim);
+    for (size_t i = 0; i < host_offsets.size(); ++i) {
+      host_offsets[i] = csz == 4 ? static_cast<int64_t>(reinterpret_cast<int32_t *>(raw.data())[i])
+                                 : reinterpret_cast<int64_t *>(raw.data())[i];
+    }
+    run_query(a, host_offsets.data(), num_offsets, kernel_map_out, out_dtype, nullptr, scope, stream);
+  });
+}
+
+extern "C" int mnt_compute_kernel_map_sizes(const void *kernel_map, int64_t num_offsets,
+                                            int64_t num_targets, int index_dtype,
+                                            void *sizes_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int isz = int_size(index_dtype);
+    MNT_CHECK(num_offsets >= 0 && num_targets >= 0 && num_targets <= INT32_MAX, "bad shape");
+    if (num_offsets == 0) return;
+    if (num_targets == 0) {
+      MNT_HIP(hipMemsetAsync(sizes_out, 0, static_cast<size_t>(isz) * num_offsets, stream));
+      return;
+    }
+    Scope scope(stream);
+    const int num_tiles = static_cast<int>(div_ceil(num_targets, kTargetsPerTile));
+    unsigned *tile_counts = scope.alloc<unsigned>(static_cast<size_t>(num_offsets) * num_tiles);
+    unsigned *row_sizes = scope.alloc<unsigned>(num_offsets);
+    enqueue_count_tiles(kernel_map, index_dtype, num_offsets, num_targets, tile_counts, num_tiles, stream);
+    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes);
+    check_launch("tile_scan_kernel");
+    const unsigned grid = grid_for(num_offsets, 256);
+    if (index_dtype == MNT_INT32) {
+      export_sizes_kernel<int32_t><<<grid, 256, 0, stream>>>(row_sizes, static_cast<int>(num_offsets), static_cast<int32_t *>(sizes_out));
+    } else {
+      export_sizes_kernel<int64_t><<<grid, 256, 0, stream>>>(row_sizes, static_cast<int>(num_offsets), static_cast<int64_t *>(sizes_out));
+    }
+    check_launch("export_sizes_kernel");
+  });
+}
+
+extern "C" int mnt_compute_kernel_map_masks(const void *kernel_map, int64_t num_offsets,
+                                            int64_t num_sources, int64_t num_targets,
+                                            int index_dtype, void *source_masks_out,
+                                            void *target_masks_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    int_size(index_dtype);
+    MNT_CHECK(num_offsets >= 0 && num_offsets <= 65535 && num_targets >= 0 && num_targets <= INT32_MAX &&
+                  num_sources >= 0 && num_sources <= INT32_MAX,
+              "bad shape");
+    if (num_offsets == 0) return;
+    Scope scope(stream);
+    const int num_tiles = static_cast<int>(div_ceil(num_targets > 0 ? num_targets : 1, kTargetsPerTile));
+    unsigned *tile_counts = scope.alloc<unsigned>(static_cast<size_t>(num_offsets) * num_tiles);
+    unsigned *row_sizes = scope.alloc<unsigned>(num_offsets);
+    if (num_targets > 0) {
+      enqueue_count_tiles(kernel_map, index_dtype, num_offsets, num_targets, tile_counts, num_tiles, stream);
+      tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes);
+      check_launch("tile_scan_kernel");
+    }
+    if (index_dtype == MNT_INT32) {
+      enqueue_emit<int32_t>(static_cast<const int32_t *>(kernel_map), num_sources, num_targets,
+                            static_cast<int>(num_offsets), tile_counts, num_tiles, nullptr, nullptr,
+                            static_cast<int32_t *>(source_masks_out),
+                            static_cast<int32_t *>(target_masks_out), nullptr, nullptr, stream);
+    } else {
+      enqueue_emit<int64_t>(static_cast<const int64_t *>(kernel_map), num_sources, num_targets,
+                            static_cast<int>(num_offsets), tile_counts, num_tiles, nullptr, nullptr,
+                            static_cast<int64_t *>(source_masks_out),
+                            static_cast<int64_t *>(target_masks_out), nullptr, nullptr, stream);
+    }
+  });
+}
+
+extern "C" int mnt_kernel_map_pair_lists(const int32_t *kernel_map, int64_t num_offsets,
+                                         int64_t num_targets, const int64_t *cumsum_host,
+                                         int32_t *in_idx_out, int32_t *out_idx_out,
+                                         void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MNT_CHECK(num_offsets >= 0 && num_offsets <= 65535 && num_targets >= 0 && num_targets <= INT32_MAX, "bad shape");
+    if (num_offsets == 0 || num_targets == 0) return;
+    MNT_CHECK(cumsum_host != nullptr && in_idx_out != nullptr && out_idx_out != nullptr, "null argument");
+    Scope scope(stream);
+    const int num_tiles = static_cast<int>(div_ceil(num_targets, kTargetsPerTile));
+    unsigned *tile_counts = scope.alloc<unsigned>(static_cast<size_t>(num_offsets) * num_tiles);
+    unsigned *row_sizes = scope.alloc<unsigned>(num_offsets);
+    unsigned *row_base = scope.alloc<unsigned>(num_offsets + 1);
+    std::vector<unsigned> base(num_offsets + 1);
+    for (int64_t o = 0; o <= num_offsets; ++o) base[o] = static_cast<unsigned>(cumsum_host[o]);
+    MNT_HIP(hipMemcpyAsync(row_base, base.data(), sizeof(unsigned) * (num_offsets + 1), hipMemcpyHostToDevice, stream));
+    enqueue_count_tiles(kernel_map, MNT_INT32, num_offsets, num_targets, tile_counts, num_tiles, stream);
+    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes);
+    check_launch("tile_scan_kernel");
+    enqueue_emit<int32_t>(kernel_map, 0, num_targets, static_cast<int>(num_offsets), tile_counts,
+                          num_tiles, nullptr, row_base, nullptr, nullptr, in_idx_out, out_idx_out, stream);
+    MNT_HIP(hipStreamSynchronize(stream));   // `base` is pageable host memory
+  });
+}
+
+extern "C" int mnt_kernel_map_query(const void *sources, int64_t num_sources, const void *targets,
+                                    int64_t num_targets, const int64_t *offsets_host,
+                                    int64_t num_offsets, int ndim, int coord_dtype,
+                                    const void *source_batch_dims, const void *target_batch_dims,
+                                    int64_t num_batches, int batch_dtype, int reorder,
+                                    int32_t *kernel_map_out, int64_t *sizes_host_out,
+                                    int64_t *order_host_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    QueryArgs a{sources, num_sources, targets, num_targets, ndim, coord_dtype,
+                source_batch_dims, target_batch_dims, num_batches, batch_dtype};
+    check_query_args(a, num_offsets);
+    MNT_CHECK(offsets_host != nullptr && sizes_host_out != nullptr && order_host_out != nullptr, "null argument");
+    Arena &arena = Arena::of(stream);
+    const int num_tiles = static_cast<int>(div_ceil(num_targets > 0 ? num_targets : 1, kTargetsPerTile));
+    // persistent block: MapState | tile bases [O*tiles] | row sizes [O] | plan [4*O+1]
+    const size_t words = static_cast<size_t>(num_offsets) * num_tiles + num_offsets + 4 * num_offsets + 1;
+    char *keep = static_cast<char *>(arena.persistent(1, 256 + words * sizeof(unsigned)));
+    unsigned *tile_counts = reinterpret_cast<unsigned *>(keep + 256);
+    unsigned *row_sizes = tile_counts + static_cast<size_t>(num_offsets) * num_tiles;
+    unsigned *plan = row_sizes + num_offsets;
+    MapState state{num_sources, num_targets, num_offsets, num_tiles, reorder, kernel_map_out};
+    arena.map_state_valid = false;
+    if (num_offsets == 0) {
+      memcpy(arena.map_state, &state, sizeof(state));
+      arena.map_state_valid = true;
+      return;
+    }
+    if (num_targets == 0 || num_sources == 0) {
+      if (num_targets > 0) {
+        MNT_CHECK(kernel_map_out != nullptr, "kernel_map_out is null");
+        MNT_HIP(hipMemsetAsync(kernel_map_out, 0xFF, sizeof(int32_t) * num_offsets * num_targets, stream));
+      }
+      MNT_HIP(hipMemsetAsync(tile_counts, 0, words * sizeof(unsigned), stream));
+    } else {
+      MNT_CHECK(kernel_map_out != nullptr, "kernel_map_out is null");
+      Scope scope(stream);
+      run_query(a, offsets_host, num_offsets, kernel_map_out, MNT_INT32, tile_counts, scope, stream);
+    }
+    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes);
+    check_launch("tile_scan_kernel");
+    order_kernel<<<1, 256, 0, stream>>>(row_sizes, static_cast<int>(num_offsets), reorder, plan);
+    check_launch("order_kernel");
+    std::vector<unsigned> host(3 * num_offsets);
+    MNT_HIP(hipMemcpyAsync(host.data(), plan, sizeof(unsigned) * 3 * num_offsets, hipMemcpyDeviceToHost, stream));
+    MNT_HIP(hipStreamSynchronize(stream));
+    for (int64_t j = 0; j < num_offsets; ++j) {
+      order_host_out[j] = host[j];
+      sizes_host_out[j] = host[2 * num_offsets + j];
+    }
+    memcpy(arena.map_state, &state, sizeof(state));
+    arena.map_state_valid = true;
+  });
+}
+
+extern "C" int mnt_kernel_map_emit(int32_t *source_masks_out, int32_t *target_masks_out,
+                                   int32_t *in_idx_out, int32_t *out_idx_out,
+                                   int32_t *sizes_dev_out, int32_t *order_dev_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    Arena &arena = Arena::of(stream);
+    MNT_CHECK(arena.map_state_valid, "mnt_kernel_map_emit called without a preceding mnt_kernel_map_query");
+    MapState state;
+    memcpy(&state, arena.map_state, sizeof(state));
+    arena.map_state_valid = false;
+    MNT_CHECK((in_idx_out == nullptr) == (out_idx_out == nullptr), "in_idx_out and out_idx_out go together");
+    if (state.num_offsets == 0) return;
+    char *keep = static_cast<char *>(arena.persistent(1, 0));
+    unsigned *tile_bases = reinterpret_cast<unsigned *>(keep + 256);
+    unsigned *row_sizes = tile_bases + static_cast<size_t>(state.num_offsets) * state.num_tiles;
+    unsigned *plan = row_sizes + state.num_offsets;
+    const int no = static_cast<int>(state.num_offsets);
+    enqueue_emit<int32_t>(static_cast<const int32_t *>(state.kernel_map), state.num_sources,
+                          state.num_targets, no, tile_bases, state.num_tiles, plan + no,
+                          plan + 3 * no, source_masks_out, target_masks_out, in_idx_out, out_idx_out,
+                          stream);
+    const unsigned grid = grid_for(no, 256);
+    if (sizes_dev_out) {
+      export_sizes_kernel<int32_t><<<grid, 256, 0, stream>>>(plan + 2 * no, no, sizes_dev_out);
+      check_launch("export_sizes_kernel");
+    }
+    if (order_dev_out) {
+      export_sizes_kernel<int32_t><<<grid, 256, 0, stream>>>(plan, no, order_dev_out);
+      check_launch("export_sizes_kernel");
+    }
+  });
+}

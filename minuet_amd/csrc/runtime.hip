@@ -1,0 +1,163 @@
+// Library plumbing: last-error slot, per-stream scratch arena, buffer knobs.
+#include <map>
+#include <mutex>
+
+#include "common.h"
+
+namespace mnt {
+
+static thread_local std::string g_last_error;
+
+void set_last_error(const std::string &message) { g_last_error = message; }
+
+static std::mutex g_arena_mutex;
+static std::map<std::pair<int, hipStream_t>, Arena *> g_arenas;
+
+Arena &Arena::of(hipStream_t stream) {
+  int device = 0;
+  MNT_HIP(hipGetDevice(&device));
+  std::lock_guard<std::mutex> lock(g_arena_mutex);
+  auto key = std::make_pair(device, stream);
+  auto it = g_arenas.find(key);
+  if (it == g_arenas.end()) it = g_arenas.emplace(key, new Arena(stream)).first;
+  return *it->second;
+}
+
+static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+void Arena::add_page(size_t bytes) {
+  Page page;
+  page.size = align_up(bytes, 256);
+  page.used = 0;
+  MNT_HIP(hipMalloc(reinterpret_cast<void **>(&page.base), page.size));
+  pages_.push_back(page);
+}
+
+void *Arena::alloc(size_t bytes) {
+  bytes = align_up(bytes ? bytes : 1, 256);
+  for (size_t p = cursor_; p < pages_.size(); ++p) {
+    if (p != cursor_) pages_[p].used = 0;
+    if (pages_[p].used + bytes <= pages_[p].size) {
+      void *ptr = pages_[p].base + pages_[p].used;
+      pages_[p].used += bytes;
+      cursor_ = p;
+      return ptr;
+    }
+  }
+  size_t want = static_cast<size_t>(static_cast<double>(bytes) * (1.0 + (growth_ > 0 ? growth_ : 0)));
+  size_t pages = (want + page_size_ - 1) / page_size_;
+  add_page(pages * page_size_);
+  cursor_ = pages_.size() - 1;
+  pages_[cursor_].used = bytes;
+  return pages_[cursor_].base;
+}
+
+Arena::Mark Arena::mark() const {
+  if (pages_.empty()) return Mark{0, 0};
+  return Mark{cursor_, pages_[cursor_].used};
+}
+
+void Arena::release(const Mark &m) {
+  if (pages_.empty()) return;
+  for (size_t p = m.page + 1; p < pages_.size(); ++p) pages_[p].used = 0;
+  cursor_ = m.page;
+  if (cursor_ < pages_.size()) pages_[cursor_].used = m.used;
+}
+
+void Arena::preallocate(size_t bytes) {
+  size_t have = 0;
+  for (const auto &p : pages_) have = p.size > have ? p.size : have;
+  if (have >= bytes) return;
+  add_page(align_up(bytes, page_size_));
+}
+
+void Arena::free_all() {
+  MNT_HIP(hipStreamSynchronize(stream_));
+  for (auto &p : pages_) MNT_HIP(hipFree(p.base));
+  pages_.clear();
+  cursor_ = 0;
+  for (int slot = 0; slot < 2; ++slot) {
+    if (persistent_[slot]) {
+      MNT_HIP(hipFree(persistent_[slot]));
+      persistent_[slot] = nullptr;
+      persistent_size_[slot] = 0;
+    }
+  }
+  pending.valid = false;
+  map_state_valid = false;
+}
+
+size_t Arena::total() const {
+  size_t t = 0;
+  for (const auto &p : pages_) t += p.size;
+  return t;
+}
+
+size_t Arena::used() const {
+  size_t t = 0;
+  for (size_t p = 0; p < pages_.size() && p <= cursor_; ++p) t += pages_[p].used;
+  return t;
+}
+
+void *Arena::pinned() {
+  if (!pinned_) MNT_HIP(hipHostMalloc(&pinned_, kPinnedBytes, hipHostMallocDefault));
+  return pinned_;
+}
+
+void *Arena::persistent(int slot, size_t bytes) {
+  if (bytes > persistent_size_[slot]) {
+    if (persistent_[slot]) {
+      MNT_HIP(hipStreamSynchronize(stream_));
+      MNT_HIP(hipFree(persistent_[slot]));
+    }
+    persistent_size_[slot] = align_up(bytes + bytes / 4, 1 << 20);
+    MNT_HIP(hipMalloc(&persistent_[slot], persistent_size_[slot]));
+  }
+  return persistent_[slot];
+}
+
+}  // namespace mnt
+
+using namespace mnt;
+
+extern "C" {
+
+int mnt_abi_version(void) { return 1; }
+
+const char *mnt_last_error(void) { return g_last_error.c_str(); }
+
+int mnt_buffer_preallocate(void *stream, size_t bytes) {
+  return guarded([&] { Arena::of(static_cast<hipStream_t>(stream)).preallocate(bytes); });
+}
+
+int mnt_buffer_free(void *stream) {
+  return guarded([&] { Arena::of(static_cast<hipStream_t>(stream)).free_all(); });
+}
+
+int mnt_buffer_set_growth(void *stream, float growth) {
+  return guarded([&] { Arena::of(static_cast<hipStream_t>(stream)).set_growth(growth); });
+}
+
+int mnt_buffer_set_page_size(void *stream, size_t bytes) {
+  return guarded([&] { Arena::of(static_cast<hipStream_t>(stream)).set_page_size(bytes); });
+}
+
+size_t mnt_buffer_total_size(void *stream) {
+  size_t value = 0;
+  guarded([&] { value = Arena::of(static_cast<hipStream_t>(stream)).total(); });
+  return value;
+}
+
+size_t mnt_buffer_used_size(void *stream) {
+  size_t value = 0;
+  guarded([&] { value = Arena::of(static_cast<hipStream_t>(stream)).used(); });
+  return value;
+}
+
+int mnt_reset_error(void) {
+  (void)hipGetLastError();
+  g_last_error.clear();
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,469 @@
+// Map step, part 2: run-length unique of sorted coordinates and the fused
+// target-coordinate generation of strided layers (floor, sort, unique).
+//
+// Semantics follow UniqueCoordinates / MultiUniqueCoordinates /
+// FillUniqueCoordinates (csrc/minuet/cuda/functions/unique_coordinates.cu:10-102,
+// csrc/minuet/cuda/kernels/fill_unique_coordinate.cuh:8-22) and
+// KernelMapCache.get_target_coordinates (minuet/nn/convolutions.py:84-99).
+#include "device_utils.h"
+#include "sort.h"
+
+namespace mnt {
+
+constexpr int kScanBlock = 256;
+constexpr int kScanItems = 8;
+constexpr int kScanTile = kScanBlock * kScanItems;
+
+// Row i closes a run: it is the last row, differs from row i+1, or a batch
+// ends right after it.
+template <typename CT, typename IT>
+__device__ __forceinline__ bool row_ends_run(const CT *__restrict__ coords, long long i,
+                                             long long n, int ndim,
+                                             const IT *__restrict__ batch_dims, int num_batches) {
+  if (i + 1 >= n) return true;
+  bool same = true;
+  for (int k = 0; k < ndim; ++k) same &= coords[i * ndim + k] == coords[(i + 1) * ndim + k];
+  if (!same) return true;
+  if (batch_dims != nullptr) return is_batch_end<IT>(i + 1, batch_dims, num_batches);
+  return false;
+}
+
+// Exclusive scan of `flag` over the workgroup; returns this thread's exclusive
+// prefix and the workgroup total through *total.
+__device__ __forceinline__ unsigned block_exclusive_scan(unsigned value, unsigned *total) {
+  __shared__ unsigned wave_sums[kScanBlock / kWave];
+  unsigned inclusive = value;
+  for (int off = 1; off < kWave; off <<= 1) {
+    unsigned v = __shfl_up(inclusive, off);
+    if (static_cast<int>(lane_id()) >= off) inclusive += v;
+  }
+  const int w = threadIdx.x >> 6;
+  if (lane_id() == kWave - 1) wave_sums[w] = inclusive;
+  __syncthreads();
+  unsigned base = 0, sum = 0;
+  for (int ww = 0; ww < kScanBlock / kWave; ++ww) {
+    if (ww < w) base += wave_sums[ww];
+    sum += wave_sums[ww];
+  }
+  __syncthreads();
+  *total = sum;
+  return base + inclusive - value;
+}
+
+template <typename CT, typename IT>
+__global__ __launch_bounds__(kScanBlock) void unique_tile_sums_kernel(
+    const CT *__restrict__ coords, long long n, int ndim, const IT *__restrict__ batch_dims,
+    int num_batches, unsigned *__restrict__ tile_sums) {
+  const long long base = static_cast<long long>(blockIdx.x) * kScanTile + threadIdx.x * kScanItems;
+  unsigned count = 0;
+#pragma unroll
+  for (int r = 0; r < kScanItems; ++r) {
+    long long i = base + r;
+    if (i < n) count += row_ends_run<CT, IT>(coords, i, n, ndim, batch_dims, num_batches) ? 1u : 0u;
+  }
+  unsigned total;
+  block_exclusive_scan(count, &total);
+  if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+}
+
+template <typename CT, typename IT>
+__global__ __launch_bounds__(kScanBlock) void unique_write_kernel(
+    const CT *__restrict__ coords, long long n, int ndim, const IT *__restrict__ batch_dims,
+    int num_batches, const unsigned *__restrict__ tile_bases, IT *__restrict__ idx_out) {
+  const long long base = static_cast<long long>(blockIdx.x) * kScanTile + threadIdx.x * kScanItems;
+  bool flags[kScanItems];
+  unsigned count = 0;
+#pragma unroll
+  for (int r = 0; r < kScanItems; ++r) {
+    long long i = base + r;
+    flags[r] = i < n && row_ends_run<CT, IT>(coords, i, n, ndim, batch_dims, num_batches);
+    count += flags[r] ? 1u : 0u;
+  }
+  unsigned total;
+  unsigned run = block_exclusive_scan(count, &total) + tile_bases[blockIdx.x];
+  if (blockIdx.x == 0 && threadIdx.x == 0) idx_out[0] = 0;
+#pragma unroll
+  for (int r = 0; r < kScanItems; ++r) {
+    long long i = base + r;
+    run += flags[r] ? 1u : 0u;
+    if (i < n) idx_out[i + 1] = static_cast<IT>(run);
+  }
+}
+
+template <typename CT, typename IT>
+__global__ __launch_bounds__(256) void fill_unique_kernel(const CT *__restrict__ coords,
+                                                          long long n, int ndim,
+                                                          const IT *__restrict__ idx,
+                                                          CT *__restrict__ out) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += stride) {
+    const IT a = idx[i];
+    if (a != idx[i + 1]) {
+      for (int k = 0; k < ndim; ++k) out[static_cast<long long>(a) * ndim + k] = coords[i * ndim + k];
+    }
+  }
+}
+
+template <typename CT, typename IT>
+static void unique_typed(const CT *coords, int64_t n, int ndim, const IT *batch_dims,
+                         int64_t num_batches, IT *idx_out, int64_t *num_unique_out,
+                         hipStream_t stream) {
+  Scope scope(stream);
+  const int tiles = static_cast<int>(div_ceil(n, kScanTile));
+  unsigned *tile_sums = scope.alloc<unsigned>(tiles);
+  unique_tile_sums_kernel<CT, IT><<<tiles, kScanBlock, 0, stream>>>(
+      coords, n, ndim, batch_dims, static_cast<int>(num_batches), tile_sums);
+  check_launch("unique_tile_sums_kernel");
+  enqueue_exclusive_scan(tile_sums, tiles, stream);
+  unique_write_kernel<CT, IT><<<tiles, kScanBlock, 0, stream>>>(
+      coords, n, ndim, batch_dims, static_cast<int>(num_batches), tile_sums, idx_out);
+  check_launch("unique_write_kernel");
+  IT *h = static_cast<IT *>(scope.arena().pinned());
+  MNT_HIP(hipMemcpyAsync(h, idx_out + n, sizeof(IT), hipMemcpyDeviceToHost, stream));
+  MNT_HIP(hipStreamSynchronize(stream));
+  *num_unique_out = static_cast<int64_t>(*h);
+}
+
+// ------------------------------------------------- fused target coordinates ----
+
+struct TargetSpec {
+  long long base[MNT_MAX_NDIM];     // floor(min / stride) per dimension
+  long long stride[MNT_MAX_NDIM];
+  int shift[MNT_MAX_NDIM];
+  unsigned long long mask[MNT_MAX_NDIM];
+  int batch_shift;
+  int ndim;
+  int num_batches;                  // 0 when there is no batch field
+};
+
+__device__ __forceinline__ long long floor_div(long long a, long long b) {
+  long long q = a / b;
+  return (a % b != 0 && ((a < 0) != (b < 0))) ? q - 1 : q;
+}
+
+template <typename CT, typename IT>
+__global__ __launch_bounds__(256) void pack_target_keys_kernel(
+    const CT *__restrict__ coords, long long n, TargetSpec spec,
+    const IT *__restrict__ batch_dims, unsigned long long *__restrict__ keys,
+    unsigned *__restrict__ vals) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += stride) {
+    unsigned long long key = 0;
+#pragma unroll
+    for (int k = 0; k < MNT_MAX_NDIM; ++k) {
+      if (k < spec.ndim) {
+        long long cell = floor_div(static_cast<long long>(coords[i * spec.ndim + k]), spec.stride[k]);
+        key |= (static_cast<unsigned long long>(cell - spec.base[k]) & spec.mask[k]) << spec.shift[k];
+      }
+    }
+    if (spec.num_batches > 0) {
+      key |= static_cast<unsigned long long>(batch_of<IT>(i, batch_dims, spec.num_batches))
+             << spec.batch_shift;
+    }
+    keys[i] = key;
+    vals[i] = static_cast<unsigned>(i);
+  }
+}
+
+__global__ __launch_bounds__(kScanBlock) void key_tile_sums_kernel(
+    const unsigned long long *__restrict__ keys, long long n, unsigned *__restrict__ tile_sums) {
+  const long long base = static_cast<long long>(blockIdx.x) * kScanTile + threadIdx.x * kScanItems;
+  unsigned count = 0;
+#pragma unroll
+  for (int r = 0; r < kScanItems; ++r) {
+    long long i = base + r;
+    if (i < n) count += (i + 1 >= n || keys[i] != keys[i + 1]) ? 1u : 0u;
+  }
+  unsigned total;
+  block_exclusive_scan(count, &total);
+  if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+}
+
+// Writes the exclusive run index of every sorted key: rank[i] = number of runs
+// that end before position i (rank[n] = number of runs).
+__global__ __launch_bounds__(kScanBlock) void key_rank_kernel(
+    const unsigned long long *__restrict__ keys, long long n,
+    const unsigned *__restrict__ tile_bases, unsigned *__restrict__ rank) {
+  const long long base = static_cast<long long>(blockIdx.x) * kScanTile + threadIdx.x * kScanItems;
+  bool flags[kScanItems];
+  unsigned count = 0;
+#pragma unroll
+  for (int r = 0; r < kScanItems; ++r) {
+    long long i = base + r;
+    flags[r] = i < n && (i + 1 >= n || keys[i] != keys[i + 1]);
+    count += flags[r] ? 1u : 0u;
+  }
+  unsigned total;
+  unsigned run = block_exclusive_scan(count, &total) + tile_bases[blockIdx.x];
+  if (blockIdx.x == 0 && threadIdx.x == 0) rank[0] = 0;
+#pragma unroll
+  for (int r = 0; r < kScanItems; ++r) {
+    long long i = base + r;
+    run += flags[r] ? 1u : 0u;
+    if (i < n) rank[i + 1] = run;
+  }
+}
+
+template <typename CT, typename IT>
+__global__ __launch_bounds__(256) void emit_targets_kernel(
+    const unsigned long long *__restrict__ keys, const unsigned *__restrict__ rank, long long n,
+    TargetSpec spec, const IT *__restrict__ batch_dims_in, CT *__restrict__ out,
+    IT *__restrict__ batch_dims_out) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  const long long first = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  for (long long i = first; i < n; i += stride) {
+    const unsigned a = rank[i];
+    if (a != rank[i + 1]) {
+      const unsigned long long key = keys[i];
+#pragma unroll
+      for (int k = 0; k < MNT_MAX_NDIM; ++k) {
+        if (k < spec.ndim) {
+          long long cell = static_cast<long long>((key >> spec.shift[k]) & spec.mask[k]) + spec.base[k];
+          out[static_cast<long long>(a) * spec.ndim + k] = static_cast<CT>(cell * spec.stride[k]);
+        }
+      }
+    }
+  }
+  // Sorted keys are batch-major, so the rows of batch g occupy the same index
+  // range as in the input and rank[dims[g]] is the new boundary.
+  if (batch_dims_out != nullptr) {
+    for (long long g = first; g <= spec.num_batches; g += stride) {
+      batch_dims_out[g] = static_cast<IT>(rank[static_cast<long long>(batch_dims_in[g])]);
+    }
+  }
+}
+
+static int bit_width64(unsigned long long range) {
+  return range == 0 ? 0 : 64 - __builtin_clzll(range);
+}
+
+template <typename CT, typename IT>
+static void target_count_typed(const CT *coords, int64_t n, int ndim, const int64_t *target_stride,
+                               const IT *batch_dims, int64_t num_batches, int64_t *count_out,
+                               hipStream_t stream) {
+  Arena &arena = Arena::of(stream);
+  arena.pending.valid = false;
+  const bool batched = batch_dims != nullptr && num_batches > 1;
+  TargetSpec spec;
+  memset(&spec, 0, sizeof(spec));
+  {
+    Scope scope(stream);
+    long long *d_bounds = scope.alloc<long long>(2 * MNT_MAX_NDIM);
+    enqueue_bounds(coords, n, ndim, sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64, d_bounds, true, stream);
+    long long *h_bounds = static_cast<long long *>(arena.pinned());
+    MNT_HIP(hipMemcpyAsync(h_bounds, d_bounds, sizeof(long long) * 2 * MNT_MAX_NDIM,
+                           hipMemcpyDeviceToHost, stream));
+    MNT_HIP(hipStreamSynchronize(stream));
+    int bits = 0;
+    spec.ndim = ndim;
+    for (int k = ndim - 1; k >= 0; --k) {
+      MNT_CHECK(target_stride[k] > 0, "target stride must be positive but found %lld",
+                static_cast<long long>(target_stride[k]));
+      auto fdiv = [](long long a, long long b) {
+        long long q = a / b;
+        return (a % b != 0 && ((a < 0) != (b < 0))) ? q - 1 : q;
+      };
+      long long lo = fdiv(h_bounds[k], target_stride[k]);
+      long long hi = fdiv(h_bounds[MNT_MAX_NDIM + k], target_stride[k]);
+      int width = bit_width64(static_cast<unsigned long long>(hi) - static_cast<unsigned long long>(lo));
+      spec.base[k] = lo;
+      spec.stride[k] = target_stride[k];
+      spec.shift[k] = bits < 64 ? bits : 63;
+      spec.mask[k] = width >= 64 ? ~0ull : ((1ull << width) - 1ull);
+      bits += width;
+    }
+    int batch_width = batched ? bit_width64(static_cast<unsigned long long>(num_batches - 1)) : 0;
+    spec.batch_shift = bits < 64 ? bits : 63;
+    spec.num_batches = batched ? static_cast<int>(num_batches) : 0;
+    bits += batch_width;
+    MNT_CHECK(bits <= 64,
+              "coordinate range needs %d key bits; strided target generation supports at most 64",
+              bits);
+
+    // persistent block: sorted keys [n] then ranks [n+1]
+    size_t key_bytes = (static_cast<size_t>(n) * 8 + 255) / 256 * 256;
+    char *keep = static_cast<char *>(arena.persistent(0, key_bytes + (static_cast<size_t>(n) + 1) * 4));
+    unsigned long long *keys = scope.alloc<unsigned long long>(n);
+    unsigned long long *keys_alt = scope.alloc<unsigned long long>(n);
+    unsigned *vals = scope.alloc<unsigned>(n);
+    unsigned *vals_alt = scope.alloc<unsigned>(n);
+    unsigned *counts = scope.alloc<unsigned>(radix_counts_len(n));
+    const unsigned grid = grid_for(n, 256, 4096);
+    pack_target_keys_kernel<CT, IT><<<grid, 256, 0, stream>>>(coords, n, spec, batch_dims, keys, vals);
+    check_launch("pack_target_keys_kernel");
+    radix_sort_pairs(keys, vals, keys_alt, vals_alt, n, bits, counts, stream);
+    MNT_HIP(hipMemcpyAsync(keep, keys, static_cast<size_t>(n) * 8, hipMemcpyDeviceToDevice, stream));
+    unsigned long long *kept_keys = reinterpret_cast<unsigned long long *>(keep);
+    unsigned *rank = reinterpret_cast<unsigned *>(keep + key_bytes);
+    const int tiles = static_cast<int>(div_ceil(n, kScanTile));
+    unsigned *tile_sums = scope.alloc<unsigned>(tiles);
+    key_tile_sums_kernel<<<tiles, kScanBlock, 0, stream>>>(kept_keys, n, tile_sums);
+    check_launch("key_tile_sums_kernel");
+    enqueue_exclusive_scan(tile_sums, tiles, stream);
+    key_rank_kernel<<<tiles, kScanBlock, 0, stream>>>(kept_keys, n, tile_sums, rank);
+    check_launch("key_rank_kernel");
+    unsigned *h = static_cast<unsigned *>(arena.pinned());
+    MNT_HIP(hipMemcpyAsync(h, rank + n, sizeof(unsigned), hipMemcpyDeviceToHost, stream));
+    MNT_HIP(hipStreamSynchronize(stream));
+    *count_out = static_cast<int64_t>(*h);
+  }
+  auto &p = arena.pending;
+  p.valid = true;
+  p.count = *count_out;
+  p.n = n;
+  p.num_batches = batched ? num_batches : 0;
+  p.ndim = ndim;
+  p.coord_dtype = sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64;
+  p.index_dtype = sizeof(IT) == 4 ? MNT_INT32 : MNT_INT64;
+  static_assert(sizeof(TargetSpec) <= sizeof(p.blob), "pending blob too small");
+  memcpy(p.blob, &spec, sizeof(spec));
+  p.batch_dims = batch_dims;
+}
+
+template <typename CT, typename IT>
+static void target_fill_typed(CT *out, IT *batch_dims_out, hipStream_t stream) {
+  Arena &arena = Arena::of(stream);
+  auto &p = arena.pending;
+  TargetSpec spec;
+  memcpy(&spec, p.blob, sizeof(spec));
+  const int64_t n = p.n;
+  size_t key_bytes = (static_cast<size_t>(n) * 8 + 255) / 256 * 256;
+  char *keep = static_cast<char *>(arena.persistent(0, 0));
+  const unsigned long long *keys = reinterpret_cast<const unsigned long long *>(keep);
+  const unsigned *rank = reinterpret_cast<const unsigned *>(keep + key_bytes);
+  const unsigned grid = grid_for(n, 256, 4096);
+  emit_targets_kernel<CT, IT><<<grid, 256, 0, stream>>>(
+      keys, rank, n, spec, static_cast<const IT *>(p.batch_dims), out,
+      p.num_batches > 0 ? batch_dims_out : nullptr);
+  check_launch("emit_targets_kernel");
+  p.valid = false;
+}
+
+}  // namespace mnt
+
+using namespace mnt;
+
+#define MNT_DISPATCH_CI(coord_dtype, index_dtype, CALL) \
+  do {                                                  \
+    if (coord_dtype == MNT_INT32 && index_dtype == MNT_INT32) { \
+      CALL(int32_t, int32_t);                           \
+    } else if (coord_dtype == MNT_INT32) {              \
+      CALL(int32_t, int64_t);                           \
+    } else if (index_dtype == MNT_INT32) {              \
+      CALL(int64_t, int32_t);                           \
+    } else {                                            \
+      CALL(int64_t, int64_t);                           \
+    }                                                   \
+  } while (0)
+
+extern "C" int mnt_unique_coordinates(const void *sorted_coords, int64_t n, int ndim,
+                                      int coord_dtype, const void *batch_dims,
+                                      int64_t num_batches, int index_dtype, void *idx_out,
+                                      int64_t *num_unique_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MNT_CHECK(ndim >= 1 && ndim <= MNT_MAX_NDIM, "ndim must be in [1, %d] but found %d",
+              MNT_MAX_NDIM, ndim);
+    MNT_CHECK(n >= 0 && n <= INT32_MAX, "number of coordinates %lld out of range",
+              static_cast<long long>(n));
+    MNT_CHECK(idx_out != nullptr && num_unique_out != nullptr, "null output");
+    int_size(coord_dtype);
+    const int isz = int_size(index_dtype);
+    if (n == 0) {
+      MNT_HIP(hipMemsetAsync(idx_out, 0, isz, stream));
+      *num_unique_out = 0;
+      return;
+    }
+    if (batch_dims == nullptr) num_batches = 1;
+#define MNT_CALL(CT, IT)                                                                      \
+  unique_typed<CT, IT>(static_cast<const CT *>(sorted_coords), n, ndim,                         \
+                       static_cast<const IT *>(batch_dims), num_batches,                        \
+                       static_cast<IT *>(idx_out), num_unique_out, stream)
+    MNT_DISPATCH_CI(coord_dtype, index_dtype, MNT_CALL);
+#undef MNT_CALL
+  });
+}
+
+extern "C" int mnt_fill_unique_coordinates(const void *sorted_coords, int64_t n, int ndim,
+                                           int coord_dtype, const void *idx, int index_dtype,
+                                           void *unique_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MNT_CHECK(ndim >= 1 && ndim <= MNT_MAX_NDIM, "ndim must be in [1, %d] but found %d",
+              MNT_MAX_NDIM, ndim);
+    int_size(coord_dtype);
+    int_size(index_dtype);
+    if (n == 0) return;
+    const unsigned grid = grid_for(n, 256, 4096);
+#define MNT_CALL(CT, IT)                                                                  \
+  fill_unique_kernel<CT, IT><<<grid, 256, 0, stream>>>(static_cast<const CT *>(sorted_coords), \
+                                                       n, ndim, static_cast<const IT *>(idx),   \
+                                                       static_cast<CT *>(unique_out))
+    MNT_DISPATCH_CI(coord_dtype, index_dtype, MNT_CALL);
+#undef MNT_CALL
+    check_launch("fill_unique_kernel");
+  });
+}
+
+extern "C" int mnt_target_coordinates_count(const void *source_coords, int64_t n, int ndim,
+                                            int coord_dtype, const int64_t *target_stride,
+                                            const void *batch_dims, int64_t num_batches,
+                                            int index_dtype, int64_t *num_targets_out,
+                                            void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MNT_CHECK(ndim >= 1 && ndim <= MNT_MAX_NDIM, "ndim must be in [1, %d] but found %d",
+              MNT_MAX_NDIM, ndim);
+    MNT_CHECK(n >= 0 && n <= INT32_MAX, "number of coordinates %lld out of range",
+              static_cast<long long>(n));
+    MNT_CHECK(target_stride != nullptr && num_targets_out != nullptr, "null argument");
+    int_size(coord_dtype);
+    int_size(index_dtype);
+    if (n == 0) {
+      Arena &arena = Arena::of(stream);
+      arena.pending = Arena::Pending();
+      arena.pending.valid = true;
+      arena.pending.coord_dtype = coord_dtype;
+      arena.pending.index_dtype = index_dtype;
+      arena.pending.ndim = ndim;
+      arena.pending.num_batches = (batch_dims && num_batches > 1) ? num_batches : 0;
+      arena.pending.batch_dims = batch_dims;
+      *num_targets_out = 0;
+      return;
+    }
+    if (batch_dims == nullptr) num_batches = 1;
+#define MNT_CALL(CT, IT)                                                                        \
+  target_count_typed<CT, IT>(static_cast<const CT *>(source_coords), n, ndim, target_stride,      \
+                             static_cast<const IT *>(batch_dims), num_batches, num_targets_out,   \
+                             stream)
+    MNT_DISPATCH_CI(coord_dtype, index_dtype, MNT_CALL);
+#undef MNT_CALL
+  });
+}
+
+extern "C" int mnt_target_coordinates_fill(void *target_coords_out, void *target_batch_dims_out,
+                                           void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    Arena &arena = Arena::of(stream);
+    MNT_CHECK(arena.pending.valid,
+              "mnt_target_coordinates_fill called without a preceding mnt_target_coordinates_count");
+    const int coord_dtype = arena.pending.coord_dtype;
+    const int index_dtype = arena.pending.index_dtype;
+    if (arena.pending.n == 0) {
+      if (arena.pending.num_batches > 0 && target_batch_dims_out != nullptr) {
+        MNT_HIP(hipMemsetAsync(target_batch_dims_out, 0,
+                               int_size(index_dtype) * (arena.pending.num_batches + 1), stream));
+      }
+      arena.pending.valid = false;
+      return;
+    }
+#define MNT_CALL(CT, IT)                                                          \
+  target_fill_typed<CT, IT>(static_cast<CT *>(target_coords_out),                  \
+                            static_cast<IT *>(target_batch_dims_out), stream)
+    MNT_DISPATCH_CI(coord_dtype, index_dtype, MNT_CALL);
+#undef MNT_CALL
+  });
+}

@@ -1,0 +1,5 @@
+from . import functional
+from .convolutions import *
+from .activations import *
+from .normalizations import *
+from .pooling import *

@@ -1,0 +1,316 @@
+"""``SparseConv`` / ``SparseConv3d`` and the ``KernelMapCache`` they share
+(mirrors minuet/nn/convolutions.py of the reference).
+
+The cache builds target coordinates and kernel maps with fused library calls
+(``_C.target_coordinates``, ``_C.kernel_map_build``) instead of chains of
+tensor expressions, keeps a host copy of the per-offset sizes so that the
+forward pass never reads them back from the device, and orders offsets by
+size with a STABLE sort (the reference's device sort is unstable, so its tie
+order is not reproducible)."""
+import contextlib
+import functools
+import operator
+from typing import Any, Dict, Optional, Union
+
+import numpy as np
+import torch
+from torch.nn import Module
+
+from minuet_amd.nn import functional as F
+from minuet_amd.nn.functional import _C
+from minuet_amd.tensors import SparseTensor
+from minuet_amd.utils.helpers import as_tuple, generate_kernel_offsets
+
+__all__ = ["SparseConv", "SparseConv3d", "KernelMapCache"]
+
+_TRANSPOSED_FIRST = ("Layer must transpose=True must have its corresponding non-transposed layer "
+                     "before its execution")
+
+
+class KernelMapCache(object):
+    """Shares target coordinates and kernel maps between the layers of a network.
+
+    Coordinates are cached per tensor stride (first writer wins), kernel maps
+    per ``(source stride, target stride, kernel size, dilation)``; a transposed
+    layer looks up the map of its forward twin and swaps the two rank tables.
+    ``reset()`` must be called before every new input
+    (reference: convolutions.py:18-173)."""
+
+    def __init__(self, ndim: int, dtype: torch.dtype, device: Union[str, torch.device],
+                 layout: str = "minuet", disable_reordering: bool = False):
+        self._ndim = ndim
+        self._dtype = dtype
+        self._device = device
+        self._layout = layout
+        self._disable_reordering = disable_reordering
+        self._kernel_maps_cache = dict()
+        self._coordinates_cache = dict()
+        self.num_map_builds = 0
+        self.num_coordinate_builds = 0
+
+    @functools.lru_cache(maxsize=None)
+    def _kernel_offsets(self, source_stride, kernel_size, kernel_dilation) -> np.ndarray:
+        return np.ascontiguousarray(
+            generate_kernel_offsets(ndim=self._ndim, kernel_size=kernel_size,
+                                    source_stride=source_stride, dilation=kernel_dilation,
+                                    layout=self._layout), dtype=np.int64)
+
+    def reset(self):
+        self._coordinates_cache.clear()
+        self._kernel_maps_cache.clear()
+
+    def get_target_coordinates(self, source_coordinates: torch.Tensor,
+                               source_batch_dims: Optional[torch.Tensor],
+                               source_stride, kernel_stride, transposed: bool = False):
+        """Coordinates, stride and batch_dims of a layer's output
+        (reference: convolutions.py:58-100)."""
+        ndim = source_coordinates.shape[1]
+        source_stride = as_tuple(source_stride, size=ndim, name="source_stride")
+        kernel_stride = as_tuple(kernel_stride, size=ndim, name="kernel_stride")
+        self._coordinates_cache.setdefault(
+            source_stride, (source_coordinates, source_stride, source_batch_dims))
+        combine = operator.floordiv if transposed else operator.mul
+        target_stride = tuple(combine(a, b) for a, b in zip(source_stride, kernel_stride))
+        hit = self._coordinates_cache.get(target_stride)
+        if hit is not None:
+            return hit
+        if transposed:
+            raise RuntimeError(_TRANSPOSED_FIRST)
+        coords, batch_dims = _C.target_coordinates(source_coordinates.contiguous(),
+                                                   source_batch_dims, target_stride)
+        self.num_coordinate_builds += 1
+        entry = (coords, target_stride, batch_dims)
+        self._coordinates_cache[target_stride] = entry
+        return entry
+
+    def get_kernel_map(self, source_coordinates: torch.Tensor, source_stride,
+                       source_batch_dims: Optional[torch.Tensor],
+                       target_coordinates: torch.Tensor, target_stride,
+                       target_batch_dims: Optional[torch.Tensor], kernel_size, kernel_dilation,
+                       disable_reordering: bool = False, transposed: bool = False):
+        """``(source_masks, target_masks, kernel_map_order, kernel_map_sizes)`` of
+        a layer (reference: convolutions.py:102-173)."""
+        ndim = source_coordinates.shape[1]
+        source_stride = as_tuple(source_stride, size=ndim, name="source_stride")
+        target_stride = as_tuple(target_stride, size=ndim, name="target_stride")
+        kernel_size = as_tuple(kernel_size, size=ndim, name="kernel_size")
+        kernel_dilation = as_tuple(kernel_dilation, size=ndim, name="kernel_dilation")
+        strides = (target_stride, source_stride) if transposed else (source_stride, target_stride)
+        key = strides + (kernel_size, kernel_dilation)
+        hit = self._kernel_maps_cache.get(key)
+        if hit is not None:
+            source_masks, target_masks, order, sizes = hit
+            if transposed:
+                source_masks, target_masks = target_masks, source_masks
+            return source_masks, target_masks, order, sizes
+        if transposed:
+            raise RuntimeError(_TRANSPOSED_FIRST)
+
+        offsets = self._kernel_offsets(source_stride, kernel_size, kernel_dilation)
+        reorder = not self._disable_reordering and not disable_reordering
+        built = _C.kernel_map_build(source_coordinates.contiguous(),
+                                    target_coordinates.contiguous(), offsets,
+                                    source_batch_dims, target_batch_dims, reorder=reorder)
+        self.num_map_builds += 1
+        index_dtype = (source_coordinates.dtype if source_batch_dims is None
+                       else source_batch_dims.dtype)
+        cast = (lambda t: t) if index_dtype == torch.int32 else (lambda t: t.to(index_dtype))
+        sizes = cast(built["sizes"])
+        sizes.host_sizes = tuple(int(v) for v in built["sizes_host"])
+        order = cast(built["order"]) if reorder else None
+        entry = (cast(built["source_masks"]), cast(built["target_masks"]), order, sizes)
+        self._kernel_maps_cache[key] = entry
+        return entry
+
+
+class SparseConv(Module):
+    r"""Sparse convolution over a :class:`SparseTensor`.
+
+    With input points :math:`\mathcal{P}` and stride :math:`s` the output points
+    are :math:`\mathcal{Q} = \{\lfloor p / s \rfloor s : p \in \mathcal{P}\}`
+    (elementwise) and
+
+    .. math:: F^{\mathcal{Q}}_i = \sum_j \sum_k
+              [p_j = q_i + \delta_k] \, F^{\mathcal{P}}_j W_k
+
+    with the offsets :math:`\delta_k` from
+    :func:`~minuet_amd.utils.helpers.generate_kernel_offsets`.  Parameters are
+    ``kernel`` ``[K^D, C_in, C_out]`` and optionally ``bias`` ``[C_out]``.  A
+    transposed layer maps back to the coordinates its forward twin started from
+    and therefore has to run after it (reference: convolutions.py:176-499).
+    """
+
+    __AVAILABLE_THRESHOLD__ = [-1, *list(np.linspace(0, 2, num=50)), None]
+    __NUM_TUNING_ROUNDS__ = 10
+
+    def __init__(self, ndim: int, in_channels: int, out_channels: int, kernel_size,
+                 stride=1, dilation=1, bias: bool = False, transposed: bool = False,
+                 dtype: Optional[torch.dtype] = None,
+                 device: Optional[torch.device] = None):
+        super().__init__()
+        self.ndim = ndim
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.kernel_size = as_tuple(kernel_size, size=ndim, name="kernel_size")
+        self.stride = as_tuple(stride, size=ndim, name="stride")
+        self.dilation = as_tuple(dilation, size=ndim, name="dilation")
+        self.transposed = transposed
+        factory = {"device": device, "dtype": dtype}
+        volume = int(np.prod(self.kernel_size))
+        self.kernel = torch.nn.Parameter(torch.empty(volume, in_channels, out_channels, **factory))
+        if bias:
+            self.bias = torch.nn.Parameter(torch.empty(out_channels, **factory))
+        else:
+            self.register_parameter("bias", None)
+        self.reset_parameters()
+        self._kernel_map_cache: Optional[KernelMapCache] = None
+        self._tunable_config = {"threshold": -1,
+                                "gather_tile_size": min(in_channels, 1),
+                                "scatter_tile_size": min(out_channels, 1)}
+        self._tuning_data = None
+
+    @property
+    def _allow_shortcut_matmul(self) -> bool:
+        return (all(x == 1 for x in self.dilation) and all(x == 1 for x in self.stride)
+                and not self._kernel_map_cache._disable_reordering)
+
+    @property
+    def tunable_config(self) -> Dict[str, Any]:
+        """Padding threshold and gather / scatter tile sizes of this layer."""
+        return self._tunable_config
+
+    @property
+    def is_trivial(self) -> bool:
+        return all(x == 1 for x in self.stride + self.dilation + self.kernel_size)
+
+    def extra_repr(self) -> str:
+        parts = [f"{self.in_channels}, {self.out_channels}, kernel_size={self.kernel_size}"]
+        if any(x != 1 for x in self.stride):
+            parts.append(f"stride={self.stride}")
+        if any(x != 1 for x in self.dilation):
+            parts.append(f"dilation={self.dilation}")
+        if self.bias is None:
+            parts.append("bias=False")
+        if self.transposed:
+            parts.append("transposed=True")
+        return ", ".join(parts)
+
+    def reset_parameters(self):
+        """Uniform init in ``+-1/sqrt(C * K^D)`` with ``C`` the input (transposed:
+        output) channel count (reference: convolutions.py:311-319)."""
+        fan = self.out_channels if self.transposed else self.in_channels
+        bound = 1.0 / np.sqrt(fan * len(self.kernel))
+        self.kernel.data.uniform_(-bound, bound)
+        if self.bias is not None:
+            self.bias.data.uniform_(-bound, bound)
+
+    def set_kernel_map_cache(self, cache: KernelMapCache):
+        self._kernel_map_cache = cache
+
+    # ------------------------------------------------------------ autotune ----
+    def _score(self, timer, **kwargs):
+        times = []
+        for _ in range(self.__NUM_TUNING_ROUNDS__):
+            for source_masks, target_masks, sizes in self._tuning_data:
+                times.append(timer(weights=self.kernel, source_masks=source_masks,
+                                   target_masks=target_masks, kernel_map_sizes=sizes,
+                                   allow_shortcut_matmul=self._allow_shortcut_matmul, **kwargs))
+        return float(np.average(times)) if times else float("inf")
+
+    @contextlib.contextmanager
+    def autotune(self, free_buffers: bool = True):
+        """Context that records the kernel maps of every forward call made inside
+        it and, on exit, picks the fastest padding threshold, gather tile and
+        scatter tile for them (reference: convolutions.py:337-444)::
+
+            with conv.autotune():
+                for x in samples:
+                    conv(x)
+        """
+        try:
+            self._tuning_data = list()
+            if free_buffers:
+                F.cuda_free_buffers()
+            yield
+            if free_buffers:
+                F.cuda_free_buffers()
+            if self.is_trivial or not self._tuning_data:
+                return
+            best = None
+            for threshold in self.__AVAILABLE_THRESHOLD__:
+                try:
+                    score = self._score(F.cuda_time_gemm, threshold=threshold)
+                except RuntimeError:
+                    F.cuda_reset_error()
+                    print(f"Threshold {threshold} overflows memory exiting tuning")
+                    print(f"optimal={self._tunable_config['threshold']}")
+                    break
+                if best is None or score < best:
+                    best = score
+                    self._tunable_config["threshold"] = threshold
+            if free_buffers:
+                F.cuda_free_buffers()
+            for key, timer, channels in (("gather_tile_size", F.cuda_time_gather, self.in_channels),
+                                         ("scatter_tile_size", F.cuda_time_scatter, self.out_channels)):
+                best = None
+                for tile in range(1, channels + 1):
+                    if channels % tile != 0:
+                        continue
+                    try:
+                        score = self._score(timer, tile_size=tile,
+                                            threshold=self._tunable_config["threshold"])
+                    except RuntimeError:
+                        F.cuda_reset_error()      # tile shape this build does not offer
+                        continue
+                    if best is None or score < best:
+                        best = score
+                        self._tunable_config[key] = tile
+                if free_buffers:
+                    F.cuda_free_buffers()
+        finally:
+            self._tuning_data = None
+
+    # ------------------------------------------------------------- forward ----
+    def forward(self, inputs: SparseTensor) -> SparseTensor:
+        if self.is_trivial:
+            features = torch.mm(inputs.F, self.kernel.view(self.in_channels, self.out_channels))
+            coordinates, stride, batch_dims = inputs.C, inputs.stride, inputs.batch_dims
+        else:
+            cache = self._kernel_map_cache
+            if cache is None:
+                raise ValueError("Kernel map cache must be specified")
+            coordinates, stride, batch_dims = cache.get_target_coordinates(
+                transposed=self.transposed, source_coordinates=inputs.C,
+                source_batch_dims=inputs.batch_dims, source_stride=inputs.stride,
+                kernel_stride=self.stride)
+            source_masks, target_masks, order, sizes = cache.get_kernel_map(
+                transposed=self.transposed, source_coordinates=inputs.C,
+                source_stride=inputs.stride, source_batch_dims=inputs.batch_dims,
+                target_coordinates=coordinates, target_stride=stride,
+                target_batch_dims=batch_dims, kernel_size=self.kernel_size,
+                kernel_dilation=self.dilation)
+            if self._tuning_data is not None:
+                self._tuning_data.append((source_masks, target_masks, sizes))
+            features = F.sparse_convolution_forward(
+                sources=inputs.F, weights=self.kernel, source_masks=source_masks,
+                target_masks=target_masks, kernel_map_order=order, kernel_map_sizes=sizes,
+                gather_tile_size=self._tunable_config["gather_tile_size"],
+                scatter_tile_size=self._tunable_config["scatter_tile_size"],
+                allow_shortcut_matmul=self._allow_shortcut_matmul,
+                threshold=self._tunable_config["threshold"])
+        if self.bias is not None:
+            features += self.bias
+        return SparseTensor(features=features, coordinates=coordinates, stride=stride,
+                            batch_dims=batch_dims)
+
+
+class SparseConv3d(SparseConv):
+    """:class:`SparseConv` for 3-D point clouds; never transposed
+    (reference: convolutions.py:502-527)."""
+
+    def __init__(self, in_channels: int, out_channels: int, kernel_size, stride=1, dilation=1,
+                 bias: bool = False, dtype: Optional[torch.dtype] = None,
+                 device: Optional[torch.device] = None):
+        super().__init__(ndim=3, in_channels=in_channels, out_channels=out_channels,
+                         kernel_size=kernel_size, stride=stride, dilation=dilation, bias=bias,
+                         transposed=False, dtype=dtype, device=device)

@@ -1,0 +1,622 @@
+"""Bridge between torch tensors and libminuet_hip.so (ctypes, C ABI).
+
+Mirrors the function table of the reference's pybind module
+``minuet.nn.functional._C`` (registered with MINUET_TORCH_REGISTER in
+csrc/minuet/torch/*.cu): same names, same argument order, same result shapes
+and dtypes, same validation.  Every function here allocates its outputs with
+torch, hands raw device pointers plus torch's current stream to the library
+and raises ``RuntimeError`` with the library's message when a call fails.
+There is no CPU or eager fallback: without the built library nothing works.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))),
+                         "lib", "libminuet_hip.so")
+_lib = None
+
+_INT = {torch.int32: 0, torch.int64: 1}
+_FLOAT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+_c = ctypes
+_vp, _i64, _int, _dbl, _sz = _c.c_void_p, _c.c_int64, _c.c_int, _c.c_double, _c.c_size_t
+_pi64 = _c.POINTER(_c.c_int64)
+_pf = _c.POINTER(_c.c_float)
+
+# name -> (restype, argtypes); the single place that states the ABI on the
+# Python side.  tests/test_abi.py checks it against include/minuet_hip.h.
+SIGNATURES = {
+    "mnt_abi_version": (_int, []),
+    "mnt_last_error": (_c.c_char_p, []),
+    "mnt_buffer_preallocate": (_int, [_vp, _sz]),
+    "mnt_buffer_free": (_int, [_vp]),
+    "mnt_buffer_set_growth": (_int, [_vp, _c.c_float]),
+    "mnt_buffer_set_page_size": (_int, [_vp, _sz]),
+    "mnt_buffer_total_size": (_sz, [_vp]),
+    "mnt_buffer_used_size": (_sz, [_vp]),
+    "mnt_reset_error": (_int, []),
+    "mnt_arg_sort_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _vp, _vp]),
+    "mnt_unique_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _pi64, _vp]),
+    "mnt_fill_unique_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _int, _vp, _vp]),
+    "mnt_target_coordinates_count": (_int, [_vp, _i64, _int, _int, _pi64, _vp, _i64, _int, _pi64, _vp]),
+    "mnt_target_coordinates_fill": (_int, [_vp, _vp, _vp]),
+    "mnt_query_sorted_index_with_offsets": (_int, [_vp, _i64, _vp, _i64, _vp, _i64, _int, _int,
+                                                   _vp, _vp, _i64, _int, _vp, _int, _vp]),
+    "mnt_compute_kernel_map_sizes": (_int, [_vp, _i64, _i64, _int, _vp, _vp]),
+    "mnt_compute_kernel_map_masks": (_int, [_vp, _i64, _i64, _i64, _int, _vp, _vp, _vp]),
+    "mnt_kernel_map_query": (_int, [_vp, _i64, _vp, _i64, _pi64, _i64, _int, _int, _vp, _vp, _i64,
+                                    _int, _int, _vp, _pi64, _pi64, _vp]),
+    "mnt_kernel_map_emit": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "mnt_kernel_map_pair_lists": (_int, [_vp, _i64, _i64, _pi64, _vp, _vp, _vp]),
+    "mnt_generate_padding_buckets": (_int, [_pi64, _i64, _int, _dbl, _pi64, _pi64]),
+    "mnt_cumsum_kernel_padded_sizes": (_int, [_pi64, _i64, _pi64, _i64, _pi64]),
+    "mnt_sparse_convolution_forward": (_int, [_i64, _i64, _int, _i64, _int, _dbl, _vp, _vp, _vp, _vp,
+                                              _vp, _vp, _pi64, _i64, _i64, _i64, _i64, _i64, _int,
+                                              _int, _vp, _vp]),
+    "mnt_time_gather": (_int, [_i64, _int, _int, _dbl, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
+                               _int, _pf, _vp]),
+    "mnt_time_scatter": (_int, [_i64, _int, _int, _dbl, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
+                                _int, _pf, _vp]),
+    "mnt_time_gemm": (_int, [_int, _i64, _int, _dbl, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
+                             _int, _pf, _vp]),
+    "mnt_profile_enable": (_int, [_int]),
+    "mnt_profile_read": (_int, [_pf]),
+}
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def load_library():
+    """Load (once) the HIP library; build it first only when no build exists."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        from minuet_amd.build import build_library
+        build_library(verbose=False)
+    lib = ctypes.CDLL(_LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def _check(status: int):
+    if status != 0:
+        message = load_library().mnt_last_error().decode("utf-8", "replace")
+        raise RuntimeError(message or f"[Minuet] native call failed with status {status}")
+
+
+def _fail(message: str):
+    raise RuntimeError(f"[Minuet] {message}")
+
+
+def _ptr(tensor: Optional[torch.Tensor]):
+    if tensor is None or tensor.numel() == 0:
+        return None if tensor is None else ctypes.c_void_p(tensor.data_ptr())
+    return ctypes.c_void_p(tensor.data_ptr())
+
+
+def _stream(device: torch.device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _ensure_ndim(name: str, tensor: torch.Tensor, ndim: int):
+    if tensor.dim() != ndim:
+        _fail(f"Tensor {name} is expected to have {ndim} dimension(s) but found "
+              f"{tensor.dim()} dimension(s)")
+
+
+def _ensure_dim(name: str, tensor: torch.Tensor, dim: int, size: int):
+    if tensor.size(dim) != size:
+        _fail(f"The dimension {dim} of Tensor {name} is expected to be {size} but found "
+              f"{tensor.size(dim)}")
+
+
+def _common_device(tensors: Sequence[torch.Tensor]) -> torch.device:
+    device = tensors[0].device
+    for t in tensors:
+        if t.device != device:
+            _fail(f"Found tensors on two different device ({device} != {t.device})")
+    if device.type != "cuda":
+        _fail(f"tensors must live on a GPU but found device {device}")
+    return device
+
+
+def _common_dtype(tensors: Sequence[torch.Tensor]) -> torch.dtype:
+    dtype = tensors[0].dtype
+    for t in tensors:
+        if t.dtype != dtype:
+            _fail(f"Found tensors with two different scalar types ({dtype} != {t.dtype})")
+    return dtype
+
+
+def _int_code(dtype: torch.dtype, what: str, fn: str) -> int:
+    if dtype not in _INT:
+        _fail(f"Cannot find implementation of {fn} for {what} data type {dtype}")
+    return _INT[dtype]
+
+
+def _float_code(dtype: torch.dtype, fn: str) -> int:
+    if dtype not in _FLOAT:
+        _fail(f"Cannot find implementation of {fn} for feature data type {dtype}")
+    return _FLOAT[dtype]
+
+
+def _check_ndim_supported(ndim: int, fn: str, dtype):
+    if not 1 <= ndim <= 4:
+        _fail(f"Cannot find implementation of {fn} for coordinate data type {dtype} of with ndim={ndim}")
+
+
+# ----------------------------------------------------------------- sorting ----
+
+def cuda_arg_sort_coordinates(coordinates: torch.Tensor, enable_flattening: bool = True) -> torch.Tensor:
+    """csrc/minuet/torch/cuda_arg_sort_coordinates.cu:8-34.  ``enable_flattening``
+    only selects an algorithm in the reference; the result is the same either way."""
+    _ensure_ndim("coordinates", coordinates, 2)
+    device = _common_device([coordinates])
+    n, ndim = coordinates.shape
+    ccode = _int_code(coordinates.dtype, "coordinate", "CUDAArgSortCoordinates")
+    _check_ndim_supported(ndim, "CUDAArgSortCoordinates", coordinates.dtype)
+    itype = torch.int32 if n <= 2 ** 31 - 1 else torch.int64
+    indices = torch.empty((n,), dtype=itype, device=device)
+    with torch.cuda.device(device):
+        _check(load_library().mnt_arg_sort_coordinates(
+            _ptr(coordinates), n, ndim, ccode, None, 1, _INT[itype], _ptr(indices), None,
+            _stream(device)))
+    return indices
+
+
+def cuda_multi_arg_sort_coordinates(coordinates: torch.Tensor, batch_dims: torch.Tensor,
+                                    enable_flattening: bool = True) -> torch.Tensor:
+    """csrc/minuet/torch/cuda_arg_sort_coordinates.cu:36-66."""
+    _ensure_ndim("coordinates", coordinates, 2)
+    _ensure_ndim("batch_dims", batch_dims, 1)
+    device = _common_device([coordinates, batch_dims])
+    n, ndim = coordinates.shape
+    ccode = _int_code(coordinates.dtype, "coordinate", "CUDAMultiArgSortCoordinates")
+    icode = _int_code(batch_dims.dtype, "index", "CUDAMultiArgSortCoordinates")
+    _check_ndim_supported(ndim, "CUDAMultiArgSortCoordinates", coordinates.dtype)
+    indices = torch.empty((n,), dtype=batch_dims.dtype, device=device)
+    with torch.cuda.device(device):
+        _check(load_library().mnt_arg_sort_coordinates(
+            _ptr(coordinates), n, ndim, ccode, _ptr(batch_dims), batch_dims.numel() - 1, icode,
+            _ptr(indices), None, _stream(device)))
+    return indices
+
+
+def sort_coordinates(coordinates: torch.Tensor, batch_dims: Optional[torch.Tensor] = None
+                     ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Arg-sort and the sorted rows in one library call (int32 indices)."""
+    _ensure_ndim("coordinates", coordinates, 2)
+    device = _common_device([coordinates] + ([batch_dims] if batch_dims is not None else []))
+    n, ndim = coordinates.shape
+    ccode = _int_code(coordinates.dtype, "coordinate", "sort_coordinates")
+    itype = batch_dims.dtype if batch_dims is not None else torch.int32
+    indices = torch.empty((n,), dtype=itype, device=device)
+    out = torch.empty_like(coordinates)
+    with torch.cuda.device(device):
+        _check(load_library().mnt_arg_sort_coordinates(
+            _ptr(coordinates), n, ndim, ccode, _ptr(batch_dims),
+            batch_dims.numel() - 1 if batch_dims is not None else 1, _INT[itype], _ptr(indices),
+            _ptr(out), _stream(device)))
+    return indices, out
+
+
+# ------------------------------------------------------------------ unique ----
+
+def _unique(coordinates: torch.Tensor, batch_dims: Optional[torch.Tensor], fn: str):
+    _ensure_ndim("coordinates", coordinates, 2)
+    if batch_dims is not None:
+        _ensure_ndim("batch_dims", batch_dims, 1)
+    device = _common_device([coordinates] + ([batch_dims] if batch_dims is not None else []))
+    n, ndim = coordinates.shape
+    ccode = _int_code(coordinates.dtype, "coordinate", fn)
+    _check_ndim_supported(ndim, fn, coordinates.dtype)
+    itype = torch.int64 if batch_dims is None else batch_dims.dtype
+    icode = _int_code(itype, "index", fn)
+    indices = torch.empty((n + 1,), dtype=itype, device=device)
+    count = ctypes.c_int64(0)
+    lib = load_library()
+    with torch.cuda.device(device):
+        # the reference passes len(batch_dims) as the batch count
+        # (cuda_unique_coordinates.cu:51); results are the same with B
+        _check(lib.mnt_unique_coordinates(
+            _ptr(coordinates), n, ndim, ccode, _ptr(batch_dims),
+            batch_dims.numel() - 1 if batch_dims is not None else 1, icode, _ptr(indices),
+            ctypes.byref(count), _stream(device)))
+        targets = torch.empty((count.value, ndim), dtype=coordinates.dtype, device=device)
+        _check(lib.mnt_fill_unique_coordinates(
+            _ptr(coordinates), n, ndim, ccode, _ptr(indices), icode, _ptr(targets), _stream(device)))
+    return targets, indices
+
+
+def cuda_unique_coordinates(coordinates: torch.Tensor):
+    """csrc/minuet/torch/cuda_unique_coordinates.cu:8-43 -> (unique rows, idx[N+1] int64)."""
+    return _unique(coordinates, None, "CUDAUniqueCoordinates")
+
+
+def cuda_multi_unique_coordinates(coordinates: torch.Tensor, batch_dims: torch.Tensor):
+    """csrc/minuet/torch/cuda_unique_coordinates.cu:45-81 -> (unique rows, idx[N+1])."""
+    return _unique(coordinates, batch_dims, "CUDAMultiUniqueCoordinates")
+
+
+def target_coordinates(coordinates: torch.Tensor, batch_dims: Optional[torch.Tensor],
+                       target_stride: Sequence[int]):
+    """floor(c / stride) * stride, sorted and unique, plus the new batch
+    boundaries — the tensor expression of minuet/nn/convolutions.py:84-99 as two
+    library calls."""
+    _ensure_ndim("coordinates", coordinates, 2)
+    device = _common_device([coordinates] + ([batch_dims] if batch_dims is not None else []))
+    n, ndim = coordinates.shape
+    ccode = _int_code(coordinates.dtype, "coordinate", "target_coordinates")
+    itype = batch_dims.dtype if batch_dims is not None else torch.int32
+    icode = _int_code(itype, "index", "target_coordinates")
+    stride = (ctypes.c_int64 * ndim)(*[int(s) for s in target_stride])
+    count = ctypes.c_int64(0)
+    lib = load_library()
+    with torch.cuda.device(device):
+        _check(lib.mnt_target_coordinates_count(
+            _ptr(coordinates), n, ndim, ccode, stride, _ptr(batch_dims),
+            batch_dims.numel() - 1 if batch_dims is not None else 1, icode, ctypes.byref(count),
+            _stream(device)))
+        out = torch.empty((count.value, ndim), dtype=coordinates.dtype, device=device)
+        out_dims = torch.empty_like(batch_dims) if batch_dims is not None else None
+        _check(lib.mnt_target_coordinates_fill(_ptr(out), _ptr(out_dims), _stream(device)))
+    return out, out_dims
+
+
+# ------------------------------------------------------------------- query ----
+
+def cuda_query_sorted_index_with_offsets(sources: torch.Tensor, targets: torch.Tensor,
+                                         offsets: torch.Tensor) -> torch.Tensor:
+    """csrc/minuet/torch/cuda_sparse_convolution_mapping.cu:9-47 -> M[O,T] of the
+    coordinate dtype."""
+    fn = "CUDAQuerySortedIndexWithOffsets"
+    _ensure_ndim("sources", sources, 2)
+    _ensure_ndim("targets", targets, 2)
+    _ensure_ndim("offsets", offsets, 2)
+    ndim = offsets.size(1)
+    _ensure_dim("sources", sources, 1, ndim)
+    _ensure_dim("targets", targets, 1, ndim)
+    ctype = _common_dtype([sources, targets, offsets])
+    device = _common_device([sources, targets, offsets])
+    ccode = _int_code(ctype, "coordinate", fn)
+    _check_ndim_supported(ndim, fn, ctype)
+    out = torch.empty((offsets.size(0), targets.size(0)), dtype=ctype, device=device)
+    with torch.cuda.device(device):
+        _check(load_library().mnt_query_sorted_index_with_offsets(
+            _ptr(sources), sources.size(0), _ptr(targets), targets.size(0), _ptr(offsets),
+            offsets.size(0), ndim, ccode, None, None, 1, 0, _ptr(out), ccode, _stream(device)))
+    return out
+
+
+def cuda_multi_query_sorted_index_with_offsets(source_batch_dims: torch.Tensor,
+                                               target_batch_dims: torch.Tensor,
+                                               sources: torch.Tensor, targets: torch.Tensor,
+                                               offsets: torch.Tensor) -> torch.Tensor:
+    """csrc/minuet/torch/cuda_sparse_convolution_mapping.cu:49-93 -> M[O,T] of the
+    batch_dims dtype."""
+    fn = "CUDAMultiQuerySortedIndexWithOffsets"
+    _ensure_ndim("sources", sources, 2)
+    _ensure_ndim("targets", targets, 2)
+    _ensure_ndim("offsets", offsets, 2)
+    _ensure_ndim("source_batch_dims", source_batch_dims, 1)
+    _ensure_ndim("target_batch_dims", target_batch_dims, 1)
+    ndim = offsets.size(1)
+    _ensure_dim("sources", sources, 1, ndim)
+    _ensure_dim("targets", targets, 1, ndim)
+    ctype = _common_dtype([sources, targets, offsets])
+    itype = _common_dtype([source_batch_dims, target_batch_dims])
+    if source_batch_dims.size(0) <= 1:
+        _fail(f"Tensor source_batch_dims should be at least length 2 but found "
+              f"{source_batch_dims.size(0)} <= 1")
+    if target_batch_dims.size(0) != source_batch_dims.size(0):
+        _fail(f"Tensor target_batch_dims must have the same length as source_batch_dims but found "
+              f"{target_batch_dims.size(0)} != {source_batch_dims.size(0)}")
+    device = _common_device([sources, targets, offsets, source_batch_dims, target_batch_dims])
+    ccode = _int_code(ctype, "coordinate", fn)
+    icode = _int_code(itype, "index", fn)
+    _check_ndim_supported(ndim, fn, ctype)
+    out = torch.empty((offsets.size(0), targets.size(0)), dtype=itype, device=device)
+    with torch.cuda.device(device):
+        _check(load_library().mnt_query_sorted_index_with_offsets(
+            _ptr(sources), sources.size(0), _ptr(targets), targets.size(0), _ptr(offsets),
+            offsets.size(0), ndim, ccode, _ptr(source_batch_dims), _ptr(target_batch_dims),
+            source_batch_dims.size(0) - 1, icode, _ptr(out), icode, _stream(device)))
+    return out
+
+
+def cuda_compute_kernel_map_sizes(kernel_map: torch.Tensor) -> torch.Tensor:
+    """csrc/minuet/torch/cuda_sparse_convolution_mapping.cu:95-121."""
+    _ensure_ndim("kernel_map", kernel_map, 2)
+    device = _common_device([kernel_map])
+    icode = _int_code(kernel_map.dtype, "tensor", "CUDAComputeKernelMapSizes")
+    sizes = torch.empty((kernel_map.size(0),), dtype=kernel_map.dtype, device=device)
+    with torch.cuda.device(device):
+        _check(load_library().mnt_compute_kernel_map_sizes(
+            _ptr(kernel_map), kernel_map.size(0), kernel_map.size(1), icode, _ptr(sizes),
+            _stream(device)))
+    return sizes
+
+
+def cuda_compute_kernel_map_masks(num_sources: int, kernel_map: torch.Tensor,
+                                  kernel_map_sizes: torch.Tensor):
+    """csrc/minuet/torch/cuda_sparse_convolution_mapping.cu:123-156.  The ranks are
+    recomputed from ``kernel_map``; ``kernel_map_sizes`` is only validated."""
+    _ensure_ndim("kernel_map", kernel_map, 2)
+    device = _common_device([kernel_map, kernel_map_sizes])
+    icode = _int_code(kernel_map.dtype, "tensor", "CUDAComputeKernelMapMasks")
+    num_offsets, num_targets = kernel_map.shape
+    source_masks = torch.empty((num_offsets, num_sources), dtype=kernel_map.dtype, device=device)
+    target_masks = torch.empty((num_offsets, num_targets), dtype=kernel_map.dtype, device=device)
+    with torch.cuda.device(device):
+        _check(load_library().mnt_compute_kernel_map_masks(
+            _ptr(kernel_map), num_offsets, int(num_sources), num_targets, icode,
+            _ptr(source_masks), _ptr(target_masks), _stream(device)))
+    return source_masks, target_masks
+
+
+def kernel_map_build(sources: torch.Tensor, targets: torch.Tensor, offsets_host: np.ndarray,
+                     source_batch_dims: Optional[torch.Tensor],
+                     target_batch_dims: Optional[torch.Tensor], reorder: bool,
+                     want_masks: bool = True, want_lists: bool = False,
+                     want_dense: bool = False):
+    """Fused kernel-map build: query + sizes + stable size order + rank tables
+    and/or per-offset pair lists.  Returns a dict with ``sizes_host``,
+    ``order_host`` (numpy int64), ``sizes``/``order`` (int32 device) and the
+    requested tensors (``source_masks``, ``target_masks``, ``in_idx``,
+    ``out_idx``, ``kernel_map``)."""
+    _ensure_ndim("sources", sources, 2)
+    _ensure_ndim("targets", targets, 2)
+    ndim = sources.size(1)
+    _ensure_dim("targets", targets, 1, ndim)
+    ctype = _common_dtype([sources, targets])
+    tensors = [sources, targets]
+    if (source_batch_dims is None) != (target_batch_dims is None):
+        raise ValueError("source_batch_dims and target_batch_dims must be both provided or "
+                         "neither provided")
+    bcode = 0
+    if source_batch_dims is not None:
+        tensors += [source_batch_dims, target_batch_dims]
+        bcode = _int_code(_common_dtype([source_batch_dims, target_batch_dims]), "index",
+                          "kernel_map_build")
+    device = _common_device(tensors)
+    ccode = _int_code(ctype, "coordinate", "kernel_map_build")
+    offs = np.ascontiguousarray(np.asarray(offsets_host, dtype=np.int64).reshape(-1, ndim))
+    num_offsets = offs.shape[0]
+    num_sources, num_targets = sources.size(0), targets.size(0)
+    dense = torch.empty((num_offsets, num_targets), dtype=torch.int32, device=device)
+    sizes_host = np.zeros(num_offsets, dtype=np.int64)
+    order_host = np.zeros(num_offsets, dtype=np.int64)
+    lib = load_library()
+    result = {}
+    with torch.cuda.device(device):
+        stream = _stream(device)
+        _check(lib.mnt_kernel_map_query(
+            _ptr(sources), num_sources, _ptr(targets), num_targets,
+            offs.ctypes.data_as(_pi64), num_offsets, ndim, ccode, _ptr(source_batch_dims),
+            _ptr(target_batch_dims),
+            source_batch_dims.numel() - 1 if source_batch_dims is not None else 1, bcode,
+            1 if reorder else 0, _ptr(dense), sizes_host.ctypes.data_as(_pi64),
+            order_host.ctypes.data_as(_pi64), stream))
+        smask = tmask = in_idx = out_idx = None
+        if want_masks:
+            smask = torch.empty((num_offsets, num_sources), dtype=torch.int32, device=device)
+            tmask = torch.empty((num_offsets, num_targets), dtype=torch.int32, device=device)
+        if want_lists:
+            nnz = int(sizes_host.sum())
+            in_idx = torch.empty((nnz,), dtype=torch.int32, device=device)
+            out_idx = torch.empty((nnz,), dtype=torch.int32, device=device)
+        sizes_dev = torch.empty((num_offsets,), dtype=torch.int32, device=device)
+        order_dev = torch.empty((num_offsets,), dtype=torch.int32, device=device)
+        _check(lib.mnt_kernel_map_emit(_ptr(smask), _ptr(tmask), _ptr(in_idx), _ptr(out_idx),
+                                       _ptr(sizes_dev), _ptr(order_dev), stream))
+    result.update(sizes_host=sizes_host, order_host=order_host, sizes=sizes_dev, order=order_dev,
+                  source_masks=smask, target_masks=tmask, in_idx=in_idx, out_idx=out_idx)
+    if want_dense:
+        result["kernel_map"] = dense
+    return result
+
+
+def kernel_map_pair_lists(kernel_map: torch.Tensor, sizes_host: Sequence[int]):
+    """Per-offset (in_idx, out_idx) lists of an int32 dense kernel map."""
+    _ensure_ndim("kernel_map", kernel_map, 2)
+    device = _common_device([kernel_map])
+    if kernel_map.dtype != torch.int32:
+        _fail("kernel_map_pair_lists expects an int32 kernel map")
+    num_offsets, num_targets = kernel_map.shape
+    cum = np.zeros(num_offsets + 1, dtype=np.int64)
+    cum[1:] = np.cumsum(np.asarray(sizes_host, dtype=np.int64))
+    in_idx = torch.empty((int(cum[-1]),), dtype=torch.int32, device=device)
+    out_idx = torch.empty_like(in_idx)
+    with torch.cuda.device(device):
+        _check(load_library().mnt_kernel_map_pair_lists(
+            _ptr(kernel_map), num_offsets, num_targets, cum.ctypes.data_as(_pi64), _ptr(in_idx),
+            _ptr(out_idx), _stream(device)))
+    return in_idx, out_idx
+
+
+# ------------------------------------------------------------ padding plan ----
+
+def generate_padding_buckets(sizes: Sequence[int], threshold: Optional[float]):
+    """GeneratePaddingBuckets, csrc/minuet/cuda/functions/sparse_convolution.cu:16-43."""
+    arr = np.ascontiguousarray(np.asarray(sizes, dtype=np.int64))
+    out = np.zeros(arr.shape[0] + 1, dtype=np.int64)
+    count = ctypes.c_int64(0)
+    _check(load_library().mnt_generate_padding_buckets(
+        arr.ctypes.data_as(_pi64), arr.shape[0], 0 if threshold is None else 1,
+        0.0 if threshold is None else float(threshold), out.ctypes.data_as(_pi64),
+        ctypes.byref(count)))
+    return out[:count.value].tolist()
+
+
+def cumsum_kernel_padded_sizes(sizes: Sequence[int], buckets: Sequence[int]):
+    """ComputeCumsumKernelPaddedSizes, sparse_convolution.cu:272-292."""
+    arr = np.ascontiguousarray(np.asarray(sizes, dtype=np.int64))
+    bks = np.ascontiguousarray(np.asarray(buckets, dtype=np.int64))
+    out = np.zeros(arr.shape[0] + 1, dtype=np.int64)
+    _check(load_library().mnt_cumsum_kernel_padded_sizes(
+        arr.ctypes.data_as(_pi64), arr.shape[0], bks.ctypes.data_as(_pi64), bks.shape[0],
+        out.ctypes.data_as(_pi64)))
+    return out.tolist()
+
+
+# ----------------------------------------------------------------- forward ----
+
+def _conv_shapes(weights, source_masks, target_masks, kernel_map_sizes):
+    _ensure_ndim("weights", weights, 3)
+    _ensure_ndim("source_masks", source_masks, 2)
+    _ensure_ndim("target_masks", target_masks, 2)
+    _ensure_ndim("kernel_map_sizes", kernel_map_sizes, 1)
+    num_offsets = target_masks.size(0)
+    _ensure_dim("kernel_map_sizes", kernel_map_sizes, 0, num_offsets)
+    _ensure_dim("source_masks", source_masks, 0, num_offsets)
+    return (source_masks.size(1), target_masks.size(1), num_offsets, weights.size(1),
+            weights.size(2))
+
+
+def _host_sizes_arg(sizes_host, num_offsets):
+    if sizes_host is None:
+        return None, None
+    arr = np.ascontiguousarray(np.asarray(sizes_host, dtype=np.int64))
+    if arr.shape[0] != num_offsets:
+        _fail("host copy of kernel_map_sizes has the wrong length")
+    return arr, arr.ctypes.data_as(_pi64)
+
+
+def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: int,
+                                    allow_shortcut_matmul: bool, parallel: int,
+                                    threshold: Optional[float], sources: torch.Tensor,
+                                    weights: torch.Tensor, source_masks: torch.Tensor,
+                                    target_masks: torch.Tensor,
+                                    kernel_map_order: Optional[torch.Tensor],
+                                    kernel_map_sizes: torch.Tensor,
+                                    kernel_map_sizes_host=None) -> torch.Tensor:
+    """csrc/minuet/torch/cuda_sparse_convolution_forward.cu:136-213.  The extra
+    ``kernel_map_sizes_host`` spares the device read-back of the sizes."""
+    fn = "CUDASparseConvolutionForward"
+    _ensure_ndim("sources", sources, 2)
+    S, T, O, K, N = _conv_shapes(weights, source_masks, target_masks, kernel_map_sizes)
+    if kernel_map_order is not None:
+        _ensure_dim("kernel_map_order", kernel_map_order, 0, O)
+    _ensure_dim("weights", weights, 0, O)
+    _ensure_dim("sources", sources, 1, K)
+    _ensure_dim("sources", sources, 0, S)
+    index_tensors = [source_masks, target_masks, kernel_map_sizes]
+    if kernel_map_order is not None:
+        index_tensors.append(kernel_map_order)
+    device = _common_device([sources, weights] + index_tensors)
+    itype = _common_dtype(index_tensors)
+    if sources.dtype != weights.dtype:
+        _fail(f"Found tensors with two different scalar types ({sources.dtype} != {weights.dtype})")
+    fcode = _float_code(weights.dtype, fn)
+    icode = _int_code(itype, "index", fn)
+    out = torch.empty((T, N), dtype=weights.dtype, device=device)
+    keep, sizes_ptr = _host_sizes_arg(kernel_map_sizes_host, O)
+    with torch.cuda.device(device):
+        _check(load_library().mnt_sparse_convolution_forward(
+            int(gather_tile_size), int(scatter_tile_size), 1 if allow_shortcut_matmul else 0,
+            int(parallel), 0 if threshold is None else 1,
+            0.0 if threshold is None else float(threshold), _ptr(sources), _ptr(weights),
+            _ptr(source_masks), _ptr(target_masks), _ptr(kernel_map_order),
+            _ptr(kernel_map_sizes), sizes_ptr, S, T, O, K, N, icode, fcode, _ptr(out),
+            _stream(device)))
+    del keep
+    return out
+
+
+def _time_stage(name, lead_args, threshold, mask, weights, source_masks, target_masks,
+                kernel_map_sizes, pass_weights):
+    S, T, O, K, N = _conv_shapes(weights, source_masks, target_masks, kernel_map_sizes)
+    device = _common_device([weights, source_masks, target_masks, kernel_map_sizes])
+    itype = _common_dtype([source_masks, target_masks, kernel_map_sizes])
+    fcode = _float_code(weights.dtype, name)
+    icode = _int_code(itype, "index", name)
+    ms = ctypes.c_float(0.0)
+    first = weights if pass_weights else mask
+    with torch.cuda.device(device):
+        _check(getattr(load_library(), name)(
+            *lead_args, 0 if threshold is None else 1,
+            0.0 if threshold is None else float(threshold), _ptr(first), _ptr(kernel_map_sizes),
+            S, T, O, K, N, icode, fcode, ctypes.byref(ms), _stream(device)))
+    return float(ms.value)
+
+
+def cuda_time_gather(tile_size, allow_shortcut_matmul, threshold, weights, source_masks,
+                     target_masks, kernel_map_sizes) -> float:
+    """csrc/minuet/torch/cuda_sparse_convolution_forward.cu:50-91."""
+    return _time_stage("mnt_time_gather", (int(tile_size), 1 if allow_shortcut_matmul else 0),
+                       threshold, source_masks, weights, source_masks, target_masks,
+                       kernel_map_sizes, False)
+
+
+def cuda_time_scatter(tile_size, allow_shortcut_matmul, threshold, weights, source_masks,
+                      target_masks, kernel_map_sizes) -> float:
+    """csrc/minuet/torch/cuda_sparse_convolution_forward.cu:93-134."""
+    return _time_stage("mnt_time_scatter", (int(tile_size), 1 if allow_shortcut_matmul else 0),
+                       threshold, target_masks, weights, source_masks, target_masks,
+                       kernel_map_sizes, False)
+
+
+def cuda_time_gemm(allow_shortcut_matmul, parallel, threshold, weights, source_masks,
+                   target_masks, kernel_map_sizes) -> float:
+    """csrc/minuet/torch/cuda_sparse_convolution_forward.cu:7-48."""
+    return _time_stage("mnt_time_gemm", (1 if allow_shortcut_matmul else 0, int(parallel)),
+                       threshold, None, weights, source_masks, target_masks, kernel_map_sizes, True)
+
+
+# ------------------------------------------------------------------ memory ----
+
+def _current_stream():
+    if not torch.cuda.is_available():
+        _fail("no GPU is available")
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def cuda_preallocate_buffer(size: int):
+    _check(load_library().mnt_buffer_preallocate(_current_stream(), int(size)))
+
+
+def cuda_free_buffers():
+    _check(load_library().mnt_buffer_free(_current_stream()))
+
+
+def cuda_set_buffer_growth(growth: float):
+    _check(load_library().mnt_buffer_set_growth(_current_stream(), float(growth)))
+
+
+def cuda_set_buffer_page_size(page_size: int):
+    _check(load_library().mnt_buffer_set_page_size(_current_stream(), int(page_size)))
+
+
+def cuda_buffer_used_size() -> int:
+    return int(load_library().mnt_buffer_used_size(_current_stream()))
+
+
+def cuda_buffer_total_size() -> int:
+    return int(load_library().mnt_buffer_total_size(_current_stream()))
+
+
+def cuda_reset_error():
+    load_library().mnt_reset_error()
+
+
+def profile_enable(on: bool):
+    load_library().mnt_profile_enable(1 if on else 0)
+
+
+def profile_read():
+    ms = (ctypes.c_float * 4)()
+    _check(load_library().mnt_profile_read(ms))
+    return {"pack": ms[0], "gather": ms[1], "gemm": ms[2], "scatter": ms[3]}

@@ -1,0 +1,75 @@
+"""Gather-GEMM-Scatter forward and its stage timers (mirrors
+minuet/nn/functional/convolution.py)."""
+from typing import Optional
+
+import torch
+
+from . import _C
+
+__all__ = ["cuda_time_gather", "cuda_time_scatter", "sparse_convolution_forward",
+           "cuda_time_gemm", "set_gemm_parallel_level"]
+
+GEMM_PARALLEL_LEVEL = 4
+
+
+def set_gemm_parallel_level(level: int):
+    """Kept for compatibility (reference: convolution.py:15-25).  The reference
+    spreads per-bucket GEMMs over this many streams; here all offsets run in
+    one grouped launch, so the value has no effect."""
+    global GEMM_PARALLEL_LEVEL
+    GEMM_PARALLEL_LEVEL = level
+
+
+def cuda_time_gather(weights: torch.Tensor, source_masks: torch.Tensor,
+                     target_masks: torch.Tensor, kernel_map_sizes: torch.Tensor,
+                     tile_size: int, allow_shortcut_matmul: bool = False,
+                     threshold: Optional[float] = 0) -> float:
+    """Milliseconds of one Gather with ``tile_size`` feature elements per lane
+    (reference: convolution.py:28-53)."""
+    return _C.cuda_time_gather(tile_size, allow_shortcut_matmul, threshold, weights,
+                               source_masks, target_masks, kernel_map_sizes)
+
+
+def cuda_time_scatter(weights: torch.Tensor, source_masks: torch.Tensor,
+                      target_masks: torch.Tensor, kernel_map_sizes: torch.Tensor,
+                      tile_size: int, allow_shortcut_matmul: bool = False,
+                      threshold: Optional[float] = 0) -> float:
+    """Milliseconds of one Scatter (reference: convolution.py:56-81)."""
+    return _C.cuda_time_scatter(tile_size, allow_shortcut_matmul, threshold, weights,
+                                source_masks, target_masks, kernel_map_sizes)
+
+
+def cuda_time_gemm(weights: torch.Tensor, source_masks: torch.Tensor,
+                   target_masks: torch.Tensor, kernel_map_sizes: torch.Tensor,
+                   allow_shortcut_matmul: bool = False, parallel: Optional[int] = None,
+                   threshold: Optional[float] = 0) -> float:
+    """Milliseconds of the grouped GEMM (reference: convolution.py:84-107)."""
+    if parallel is None:
+        parallel = GEMM_PARALLEL_LEVEL
+    return _C.cuda_time_gemm(allow_shortcut_matmul, parallel, threshold, weights, source_masks,
+                             target_masks, kernel_map_sizes)
+
+
+def sparse_convolution_forward(sources: torch.Tensor, weights: torch.Tensor,
+                               source_masks: torch.Tensor, target_masks: torch.Tensor,
+                               kernel_map_order: Optional[torch.Tensor],
+                               kernel_map_sizes: torch.Tensor, gather_tile_size: int,
+                               scatter_tile_size: int, allow_shortcut_matmul: bool = False,
+                               parallel: Optional[int] = None,
+                               threshold: Optional[float] = 0) -> torch.Tensor:
+    """Output features ``[N_out, C_out]`` of one sparse convolution given the rank
+    tables of its kernel map (reference: convolution.py:110-155).  A host copy
+    of the sizes attached to ``kernel_map_sizes`` as attribute ``host_sizes``
+    (``KernelMapCache`` does that) avoids a device read-back per call."""
+    if not sources.is_cuda:
+        raise NotImplementedError
+    if parallel is None:
+        parallel = GEMM_PARALLEL_LEVEL
+    host_sizes = getattr(kernel_map_sizes, "host_sizes", None)
+    if kernel_map_order is not None:
+        kernel_map_order = kernel_map_order.contiguous()
+    return _C.cuda_sparse_convolution_forward(
+        gather_tile_size, scatter_tile_size, allow_shortcut_matmul, parallel, threshold,
+        sources.contiguous(), weights.contiguous(), source_masks.contiguous(),
+        target_masks.contiguous(), kernel_map_order, kernel_map_sizes.contiguous(),
+        kernel_map_sizes_host=host_sizes)

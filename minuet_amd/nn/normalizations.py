@@ -1,0 +1,15 @@
+"""Batch normalisation on the features of a SparseTensor (mirrors
+minuet/nn/normalizations.py)."""
+import torch
+
+from minuet_amd.tensors import SparseTensor
+
+__all__ = ["BatchNorm"]
+
+
+class BatchNorm(torch.nn.BatchNorm1d):
+    """:class:`torch.nn.BatchNorm1d` over the ``[N, C]`` feature tensor."""
+
+    def forward(self, x: SparseTensor) -> SparseTensor:
+        return SparseTensor(features=super().forward(x.F), coordinates=x.C, stride=x.stride,
+                            batch_dims=x.batch_dims)

@@ -1,0 +1,181 @@
+"""GPU parity of the Map step against the CPU oracle (bit-exact)."""
+import numpy as np
+import pytest
+import torch
+
+import minuet_oracle as orc
+from helpers import dev, host, random_cloud, sorted_unique
+from minuet_amd.nn import functional as F
+from minuet_amd.nn.functional import _C
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n,extent,lo,cdtype", [
+    (1, 5, 0, np.int32), (2, 1, 3, np.int32), (1000, 6, -3, np.int32), (5000, 300, -150, np.int32),
+    (70000, 2000, -1000, np.int32), (3000, 50, -20, np.int64),
+    (4000, 2 ** 30, -2 ** 29, np.int32), (4000, 2 ** 40, -2 ** 39, np.int64),
+])
+def test_arg_sort_single(n, extent, lo, cdtype):
+    c = random_cloud(n, extent, seed=n, lo=lo, duplicates=0.2, dtype=cdtype)
+    got = F.arg_sort_coordinates(dev(c))
+    assert got.dtype == torch.int32
+    np.testing.assert_array_equal(host(got).astype(np.int64), orc.arg_sort_coordinates(c))
+
+
+def test_arg_sort_wide_range_multi_round():
+    # 4 dims of int64 spanning ~2^62 each: keys cannot be packed in 64 bits
+    rng = np.random.default_rng(5)
+    c = rng.integers(-2 ** 61, 2 ** 61, size=(3000, 4)).astype(np.int64)
+    c[rng.integers(0, 3000, 500)] = c[rng.integers(0, 3000, 500)]
+    c[:, 0] = rng.integers(-2, 2, size=3000)          # many ties on the leading dimension
+    got = F.arg_sort_coordinates(dev(c))
+    np.testing.assert_array_equal(host(got).astype(np.int64), orc.arg_sort_coordinates(c))
+
+
+@pytest.mark.parametrize("ndim", [1, 2, 3, 4])
+@pytest.mark.parametrize("idtype", [np.int32, np.int64])
+def test_arg_sort_batched(ndim, idtype):
+    sizes = [700, 0, 1300, 1, 999]
+    bd = np.concatenate([[0], np.cumsum(sizes)]).astype(idtype)
+    c = random_cloud(int(bd[-1]), 9, seed=ndim, ndim=ndim, lo=-4, duplicates=0.3)
+    got = F.arg_sort_coordinates(dev(c), batch_dims=dev(bd))
+    assert got.dtype == (torch.int32 if idtype == np.int32 else torch.int64)
+    np.testing.assert_array_equal(host(got).astype(np.int64), orc.arg_sort_coordinates(c, bd))
+    got64 = F.build_sorted_index(dev(c), batch_dims=dev(bd))
+    assert got64.dtype == torch.int64
+
+
+def test_arg_sort_large_two_item_paths():
+    c = random_cloud(1_300_000, 1500, seed=9, lo=-700)
+    got = F.arg_sort_coordinates(dev(c))
+    np.testing.assert_array_equal(host(got).astype(np.int64), orc.arg_sort_coordinates(c))
+
+
+@pytest.mark.parametrize("batched", [False, True])
+def test_unique(batched):
+    bd = np.array([0, 2500, 2500, 6000], dtype=np.int32) if batched else None
+    c = random_cloud(6000, 7, seed=3, lo=-3, duplicates=0.1)
+    c = c[orc.arg_sort_coordinates(c, bd)]
+    u, idx = F.unique_coordinates(dev(c), batch_dims=dev(bd))
+    eu, eidx = orc.unique_coordinates(c, bd)
+    np.testing.assert_array_equal(host(u), eu)
+    np.testing.assert_array_equal(host(idx).astype(np.int64), eidx)
+    assert idx.dtype == (torch.int32 if batched else torch.int64)
+
+
+def test_unique_empty_and_single():
+    u, idx = F.unique_coordinates(dev(np.zeros((0, 3), dtype=np.int32)))
+    assert u.shape == (0, 3) and host(idx).tolist() == [0]
+    u, idx = F.unique_coordinates(dev(np.array([[1, 2, 3]], dtype=np.int32)))
+    assert host(u).tolist() == [[1, 2, 3]] and host(idx).tolist() == [0, 1]
+
+
+@pytest.mark.parametrize("stride", [(2, 2, 2), (4, 2, 1), (3, 3, 3)])
+@pytest.mark.parametrize("batched", [False, True])
+def test_target_coordinates(stride, batched):
+    bd = np.array([0, 4000, 9000], dtype=np.int32) if batched else None
+    c = random_cloud(9000, 40, seed=11, lo=-20)
+    c, bd = sorted_unique(c, bd)
+    got, got_bd = _C.target_coordinates(dev(c), dev(bd), stride)
+    exp, exp_bd = orc.target_coordinates(c, bd, stride)
+    np.testing.assert_array_equal(host(got), exp)
+    if batched:
+        np.testing.assert_array_equal(host(got_bd), exp_bd)
+    else:
+        assert got_bd is None
+
+
+def _query_case(seed, n, extent, lo, kernel, stride=1, batched=False, cdtype=np.int32, idtype=np.int32):
+    bd = None
+    if batched:
+        bd = np.array([0, n // 3, n // 3, n], dtype=idtype)
+    c = random_cloud(n, extent, seed=seed, lo=lo, dtype=cdtype)
+    src, sbd = sorted_unique(c, bd)
+    if stride == 1:
+        tgt, tbd = src, sbd
+    else:
+        tgt, tbd = orc.target_coordinates(src, sbd, stride)
+    off = orc.generate_kernel_offsets(3, kernel, 1, 1).astype(cdtype)
+    return src, sbd, tgt, tbd, off
+
+
+@pytest.mark.parametrize("kernel,stride,n,extent", [
+    (3, 1, 1, 4), (3, 1, 600, 7), (3, 1, 30000, 60), (2, 2, 30000, 60), (5, 1, 20000, 40),
+    (3, 1, 200000, 400), ((3, 1, 2), 1, 5000, 20),
+])
+def test_query_single(kernel, stride, n, extent):
+    src, _, tgt, _, off = _query_case(1, n, extent, -extent // 2, kernel, stride)
+    got = F.query_sorted_index_with_offsets(dev(src), dev(tgt), dev(off))
+    assert got.dtype == torch.int32 and got.shape == (off.shape[0], tgt.shape[0])
+    np.testing.assert_array_equal(host(got), orc.query_sorted_index_with_offsets(src, tgt, off))
+
+
+def test_query_dense_block_many_chunks():
+    # a fully occupied block: the source window of a tile spans several LDS chunks
+    g = np.stack(np.meshgrid(np.arange(6), np.arange(40), np.arange(40), indexing="ij"), -1)
+    src = g.reshape(-1, 3).astype(np.int32)
+    off = orc.generate_kernel_offsets(3, 5, 1, 1).astype(np.int32)
+    got = F.query_sorted_index_with_offsets(dev(src), dev(src), dev(off))
+    np.testing.assert_array_equal(host(got), orc.query_sorted_index_with_offsets(src, src, off))
+
+
+@pytest.mark.parametrize("cdtype,idtype", [(np.int32, np.int32), (np.int32, np.int64), (np.int64, np.int32)])
+@pytest.mark.parametrize("stride", [1, 2])
+def test_query_batched(cdtype, idtype, stride):
+    src, sbd, tgt, tbd, off = _query_case(2, 20000, 30, -15, 3 if stride == 1 else 2, stride,
+                                          batched=True, cdtype=cdtype, idtype=idtype)
+    got = F.query_sorted_index_with_offsets(dev(src), dev(tgt), dev(off), dev(sbd), dev(tbd))
+    exp = orc.query_sorted_index_with_offsets(src, tgt, off, sbd, tbd)
+    assert got.dtype == (torch.int32 if idtype == np.int32 else torch.int64)
+    np.testing.assert_array_equal(host(got), exp)
+
+
+def test_query_empty_inputs():
+    src = np.zeros((0, 3), dtype=np.int32)
+    tgt = random_cloud(50, 4, seed=1)
+    off = orc.generate_kernel_offsets(3, 3, 1, 1).astype(np.int32)
+    got = F.query_sorted_index_with_offsets(dev(src), dev(tgt), dev(off))
+    assert (host(got) == -1).all()
+    got = F.query_sorted_index_with_offsets(dev(tgt), dev(src), dev(off))
+    assert got.shape == (27, 0)
+
+
+@pytest.mark.parametrize("idtype", [np.int32, np.int64])
+def test_sizes_and_masks(idtype):
+    src, _, tgt, _, off = _query_case(4, 25000, 50, 0, 2, 2)
+    m = orc.query_sorted_index_with_offsets(src, tgt, off, dtype=idtype)
+    sizes = F.compute_kernel_map_sizes(dev(m))
+    np.testing.assert_array_equal(host(sizes), orc.compute_kernel_map_sizes(m))
+    sm, tm = F.compute_kernel_map_masks(src.shape[0], dev(m), sizes)
+    esm, etm = orc.compute_kernel_map_masks(src.shape[0], m)
+    np.testing.assert_array_equal(host(sm), esm)
+    np.testing.assert_array_equal(host(tm), etm)
+
+
+@pytest.mark.parametrize("reorder", [True, False])
+@pytest.mark.parametrize("kernel,stride,batched", [(3, 1, False), (2, 2, True), (5, 1, False)])
+def test_kernel_map_build(reorder, kernel, stride, batched):
+    src, sbd, tgt, tbd, off = _query_case(7, 30000, 45, -10, kernel, stride, batched=batched)
+    built = _C.kernel_map_build(dev(src), dev(tgt), off.astype(np.int64), dev(sbd), dev(tbd),
+                                reorder=reorder, want_masks=True, want_lists=True, want_dense=True)
+    esm, etm, eorder, esizes, em = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=reorder)
+    dense = orc.query_sorted_index_with_offsets(src, tgt, off, sbd, tbd, dtype=np.int32)
+    np.testing.assert_array_equal(host(built["kernel_map"]), dense)
+    np.testing.assert_array_equal(built["sizes_host"], esizes.astype(np.int64))
+    np.testing.assert_array_equal(host(built["sizes"]), esizes)
+    if reorder:
+        np.testing.assert_array_equal(built["order_host"], eorder.astype(np.int64))
+        np.testing.assert_array_equal(host(built["order"]), eorder)
+    else:
+        np.testing.assert_array_equal(built["order_host"], np.arange(off.shape[0]))
+    np.testing.assert_array_equal(host(built["source_masks"]), esm)
+    np.testing.assert_array_equal(host(built["target_masks"]), etm)
+    ein, eout, _ = orc.kernel_map_pair_lists(em)
+    np.testing.assert_array_equal(host(built["in_idx"]), ein)
+    np.testing.assert_array_equal(host(built["out_idx"]), eout)
+    # the stand-alone list builder agrees as well
+    in2, out2 = _C.kernel_map_pair_lists(dev(dense), orc.compute_kernel_map_sizes(dense))
+    e2in, e2out, _ = orc.kernel_map_pair_lists(dense)
+    np.testing.assert_array_equal(host(in2), e2in)
+    np.testing.assert_array_equal(host(out2), e2out)
