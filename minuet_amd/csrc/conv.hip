@@ -154,24 +154,30 @@ template <typename T>
 __device__ __forceinline__ float to_float(T v) { return static_cast<float>(v); }
 
 // One lane group per target row: sums its buffer rows in offset order in fp32
-// and writes the row once.  With `accumulate` the previous content of the row
-// (the centre-offset product written by the direct GEMM) is the initial value.
-template <typename T, int VB, int NV, typename IT>
-__global__ __launch_bounds__(256) void scatter_kernel(const unsigned char *__restrict__ buffer,
+// and writes the row once.  The buffer holds elements of type TB (the output
+// type, or fp32 when the output type is too coarse to round partial products
+// to), the output elements of type T.  With `accumulate` the previous content
+// of the row (the centre-offset product written by the direct GEMM) is the
+// initial value.
+template <typename TB, typename T, int VB, int NV, typename IT>
+__global__ __launch_bounds__(256) void scatter_kernel(const TB *__restrict__ buffer,
                                                       unsigned char *__restrict__ targets,
                                                       const IT *__restrict__ target_masks,
                                                       const int *__restrict__ row_start,
                                                       long long num_targets, int num_offsets,
-                                                      int row_bytes, int lanes_per_row,
+                                                      int channels, int lanes_per_row,
                                                       int accumulate) {
   typedef typename VecOf<VB>::type V;
   constexpr int E = VB / static_cast<int>(sizeof(T));
+  constexpr int BB = E * static_cast<int>(sizeof(TB));          // buffer bytes per vector
+  typedef typename VecOf<(BB > 16 ? 16 : BB)>::type BV;
+  constexpr int NBV = BB > 16 ? BB / 16 : 1;
   const long long gtid = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
   const long long t = gtid / lanes_per_row;
   const int lr = static_cast<int>(gtid % lanes_per_row);
   if (t >= num_targets) return;
   float acc[NV][E];
-  unsigned char *dst = targets + t * row_bytes;
+  unsigned char *dst = targets + t * channels * static_cast<long long>(sizeof(T));
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     if (accumulate) {
@@ -187,11 +193,14 @@ __global__ __launch_bounds__(256) void scatter_kernel(const unsigned char *__res
   for (int o = 0; o < num_offsets; ++o) {
     const long long d = static_cast<long long>(target_masks[static_cast<long long>(o) * num_targets + t]);
     if (d < 0) continue;
-    const unsigned char *src = buffer + (static_cast<long long>(row_start[o]) + d) * row_bytes;
+    const TB *src = buffer + (static_cast<long long>(row_start[o]) + d) * channels;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      V raw = *reinterpret_cast<const V *>(src + (lr + i * lanes_per_row) * VB);
-      const T *e = reinterpret_cast<const T *>(&raw);
+      const TB *piece = src + (lr + i * lanes_per_row) * E;
+      BV raw[NBV];
+#pragma unroll
+      for (int v = 0; v < NBV; ++v) raw[v] = reinterpret_cast<const BV *>(piece)[v];
+      const TB *e = reinterpret_cast<const TB *>(raw);
 #pragma unroll
       for (int k = 0; k < E; ++k) acc[i][k] += to_float(e[k]);
     }
@@ -205,6 +214,14 @@ __global__ __launch_bounds__(256) void scatter_kernel(const unsigned char *__res
     *reinterpret_cast<V *>(dst + (lr + i * lanes_per_row) * VB) = raw;
   }
 }
+
+// Element type of the GEMM-output / scatter-input buffer for feature type T.
+// bfloat16 keeps only 8 significant bits, so rounding every partial product
+// to it would cost more accuracy than the output rounding itself.
+template <typename T>
+struct BufferOf { typedef T type; };
+template <>
+struct BufferOf<bf16_t> { typedef float type; };
 
 // ------------------------------------------------------------ grouped GEMM ----
 
@@ -248,9 +265,9 @@ constexpr int kLdsRowBytes = kChunkBytes + 16;
 // The K order inside a 128-byte chunk is permuted identically for both
 // operands (lane half h of step kk reads bytes [32*kk + 16*h, +16) of the
 // row), which leaves the dot products unchanged.
-template <typename T, int TN, bool VEC>
+template <typename T, typename TC, int TN, bool VEC>
 __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
-    const T *__restrict__ a, T *__restrict__ c, const T *__restrict__ wt,
+    const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt,
     const int *__restrict__ meta, int K, int N, int Kp, int Np) {
   constexpr int EPC = 16 / static_cast<int>(sizeof(T));        // elements per 16-byte piece
   constexpr int KC = kChunkBytes / static_cast<int>(sizeof(T));
@@ -345,17 +362,17 @@ __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
 
   const int row = wv * 32 + r;
   if (row < valid) {
-    T *dst = c + (row_base + row) * N;
+    TC *dst = c + (row_base + row) * N;
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int ch = n0 + b * 32 + q * 8 + h * 4;
         if (VEC && ch + 4 <= N) {
-          T out[4];
+          TC out[4];
 #pragma unroll
-          for (int x = 0; x < 4; ++x) out[x] = static_cast<T>(acc[b][q * 4 + x]);
-          if (sizeof(T) == 2) {
+          for (int x = 0; x < 4; ++x) out[x] = static_cast<TC>(acc[b][q * 4 + x]);
+          if (sizeof(TC) == 2) {
             *reinterpret_cast<uint2 *>(dst + ch) = *reinterpret_cast<const uint2 *>(out);
           } else {
             *reinterpret_cast<uint4 *>(dst + ch) = *reinterpret_cast<const uint4 *>(out);
@@ -363,7 +380,7 @@ __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
         } else {
 #pragma unroll
           for (int x = 0; x < 4; ++x) {
-            if (ch + x < N) dst[ch + x] = static_cast<T>(acc[b][q * 4 + x]);
+            if (ch + x < N) dst[ch + x] = static_cast<TC>(acc[b][q * 4 + x]);
           }
         }
       }
@@ -440,17 +457,17 @@ static void launch_gather(const LaneShape &sh, const void *sources, void *buffer
   check_launch("gather_kernel");
 }
 
-template <typename T, typename IT>
-static void launch_scatter(const LaneShape &sh, const void *buffer, void *targets, const IT *masks,
-                           const int *row_start, int64_t num_targets, int num_offsets, int row_bytes,
+template <typename TB, typename T, typename IT>
+static void launch_scatter(const LaneShape &sh, const TB *buffer, void *targets, const IT *masks,
+                           const int *row_start, int64_t num_targets, int num_offsets, int channels,
                            int accumulate, hipStream_t stream) {
   if (num_targets == 0) return;
   const unsigned grid = static_cast<unsigned>(div_ceil(num_targets * sh.lanes_per_row, 256));
 #define MNT_S(VB, NV)                                                                              \
-  scatter_kernel<T, VB, NV, IT><<<grid, 256, 0, stream>>>(static_cast<const unsigned char *>(buffer), \
+  scatter_kernel<TB, T, VB, NV, IT><<<grid, 256, 0, stream>>>(buffer,                              \
                                                           static_cast<unsigned char *>(targets), masks, \
                                                           row_start, num_targets, num_offsets,        \
-                                                          row_bytes, sh.lanes_per_row, accumulate)
+                                                          channels, sh.lanes_per_row, accumulate)
 #define MNT_SV(VB)                 \
   switch (sh.nv) {                 \
     case 1: MNT_S(VB, 1); break;   \
@@ -476,8 +493,8 @@ static void launch_scatter(const LaneShape &sh, const void *buffer, void *target
   check_launch("scatter_kernel");
 }
 
-template <typename T>
-static void launch_gemm(const T *a, T *c, const T *wt, const int *meta, int num_tiles, int K, int N,
+template <typename T, typename TC>
+static void launch_gemm(const T *a, TC *c, const T *wt, const int *meta, int num_tiles, int K, int N,
                         int Kp, int Np, hipStream_t stream) {
   if (num_tiles == 0) return;
   const bool vec = (static_cast<int64_t>(K) * sizeof(T)) % 16 == 0 &&
@@ -488,9 +505,9 @@ static void launch_gemm(const T *a, T *c, const T *wt, const int *meta, int num_
 #define MNT_MM(TN)                                                                              \
   do {                                                                                          \
     if (vec) {                                                                                  \
-      grouped_gemm_kernel<T, TN, true><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np);  \
+      grouped_gemm_kernel<T, TC, TN, true><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np);  \
     } else {                                                                                    \
-      grouped_gemm_kernel<T, TN, false><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np); \
+      grouped_gemm_kernel<T, TC, TN, false><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np); \
     }                                                                                           \
   } while (0)
   if (tn == 128) {
@@ -621,26 +638,27 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
   profile_mark(1, stream);
 
   const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
+  typedef typename BufferOf<T>::type TB;
   T *abuf = scope.alloc<T>(rows * K);
-  T *cbuf = scope.alloc<T>(rows * N);
+  TB *cbuf = scope.alloc<TB>(rows * N);
 
   const LaneShape gsh = lane_shape(gather_tile, K, sizeof(T), sources, abuf, "num_source_features");
   launch_gather<IT>(gsh, sources, abuf, source_masks, d_row_start, S, active,
                     static_cast<int>(K * sizeof(T)), stream);
   profile_mark(2, stream);
 
-  launch_gemm<T>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
+  launch_gemm<T, TB>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
   if (plan.shortcut) {
     std::vector<int> meta = direct_meta(S, static_cast<int>(O - 1));
     int *d_direct = scope.alloc<int>(meta.size());
     upload_ints(meta, d_direct, stream);
-    launch_gemm<T>(sources, out, wt, d_direct, meta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
+    launch_gemm<T, T>(sources, out, wt, d_direct, meta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
   }
   profile_mark(3, stream);
 
   const LaneShape ssh = lane_shape(scatter_tile, N, sizeof(T), cbuf, out, "num_target_features");
-  launch_scatter<T, IT>(ssh, cbuf, out, target_masks, d_row_start, Tn, active,
-                        static_cast<int>(N * sizeof(T)), plan.shortcut ? 1 : 0, stream);
+  launch_scatter<TB, T, IT>(ssh, cbuf, out, target_masks, d_row_start, Tn, active,
+                            static_cast<int>(N), plan.shortcut ? 1 : 0, stream);
   profile_mark(4, stream);
 }
 
@@ -771,15 +789,16 @@ static float time_scatter_typed(int64_t tile, const ForwardPlan &plan, const IT 
                                 int64_t Tn, int64_t N, hipStream_t stream) {
   Scope scope(stream);
   const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
-  T *cbuf = scope.alloc<T>(rows * N);
+  typedef typename BufferOf<T>::type TB;
+  TB *cbuf = scope.alloc<TB>(rows * N);
   T *out = scope.alloc<T>(static_cast<size_t>(Tn > 0 ? Tn : 1) * N);
   int *d_row_start = scope.alloc<int>(plan.row_start.size());
   upload_ints(plan.row_start, d_row_start, stream);
   const LaneShape sh = lane_shape(tile, N, sizeof(T), cbuf, out, "num_target_features");
   TimerScope timer(stream);
   timer.begin();
-  launch_scatter<T, IT>(sh, cbuf, out, target_masks, d_row_start, Tn, static_cast<int>(plan.active_offsets),
-                        static_cast<int>(N * sizeof(T)), 0, stream);
+  launch_scatter<TB, T, IT>(sh, cbuf, out, target_masks, d_row_start, Tn,
+                            static_cast<int>(plan.active_offsets), static_cast<int>(N), 0, stream);
   return timer.end();
 }
 
@@ -791,9 +810,10 @@ static float time_gemm_typed(const ForwardPlan &plan, const T *weights, int64_t 
   const int Kp = static_cast<int>(div_ceil(K, kc) * kc);
   const int Np = static_cast<int>(div_ceil(N, 32) * 32);
   const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
+  typedef typename BufferOf<T>::type TB;
   T *wt = scope.alloc<T>(static_cast<size_t>(O) * Np * Kp);
   T *abuf = scope.alloc<T>(rows * K);
-  T *cbuf = scope.alloc<T>(rows * N);
+  TB *cbuf = scope.alloc<TB>(rows * N);
   T *direct_a = nullptr, *direct_c = nullptr;
   int *d_direct = nullptr;
   std::vector<int> dmeta;
@@ -815,9 +835,9 @@ static float time_gemm_typed(const ForwardPlan &plan, const T *weights, int64_t 
   upload_ints(plan.meta, d_meta, stream);
   TimerScope timer(stream);
   timer.begin();
-  launch_gemm<T>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
+  launch_gemm<T, TB>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
   if (plan.shortcut) {
-    launch_gemm<T>(direct_a, direct_c, wt, d_direct, dmeta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
+    launch_gemm<T, T>(direct_a, direct_c, wt, d_direct, dmeta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
   }
   return timer.end();
 }

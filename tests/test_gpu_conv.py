@@ -1,0 +1,196 @@
+"""GPU parity of Gather -> grouped GEMM -> Scatter and of the module API
+against the CPU oracle (fp64).  Tolerances (from the task statement):
+fp32: max-abs error <= 1e-5 x max|reference| (relative 1e-5);
+fp16 / bf16: max-abs error <= 2e-2 x RMS(reference)."""
+import numpy as np
+import pytest
+import torch
+
+import minuet_oracle as orc
+from helpers import dev, host, random_cloud, sorted_unique
+import minuet_amd as minuet
+from minuet_amd.nn import functional as F
+from minuet_amd.nn.functional import _C
+
+pytestmark = pytest.mark.gpu
+
+TORCH = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}
+
+
+def assert_features_close(got, ref, kind):
+    got = host(got.float()).astype(np.float64)
+    err = np.abs(got - ref).max() if ref.size else 0.0
+    if kind == "fp32":
+        bound = 1e-5 * max(np.abs(ref).max(), 1e-30)
+    else:
+        bound = 2e-2 * max(np.sqrt(np.mean(ref ** 2)), 1e-30)
+    assert err <= bound, f"{kind}: max-abs error {err:.3e} exceeds {bound:.3e}"
+
+
+def quantise(array, kind):
+    """Round inputs to the feature dtype first so the oracle sees what the GPU sees."""
+    return host(torch.from_numpy(array).to(TORCH[kind]).float()).astype(np.float64)
+
+
+def make_layer_case(seed, n, extent, kernel, cin, cout, kind, stride=1, batched=False):
+    rng = np.random.default_rng(seed)
+    bd = np.array([0, n // 2, n], dtype=np.int32) if batched else None
+    src, sbd = sorted_unique(random_cloud(n, extent, seed=seed, lo=-extent // 2), bd)
+    if stride == 1:
+        tgt, tbd = src, sbd
+    else:
+        tgt, tbd = orc.target_coordinates(src, sbd, stride)
+    off = orc.generate_kernel_offsets(3, kernel, 1, 1)
+    feats = quantise(rng.normal(size=(src.shape[0], cin)), kind)
+    k3 = off.shape[0]
+    weights = quantise(rng.normal(size=(k3, cin, cout)) / np.sqrt(k3 * cin), kind)
+    return src, sbd, tgt, tbd, off, feats, weights
+
+
+@pytest.mark.parametrize("kind", ["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("kernel,stride,cin,cout,n,extent", [
+    (3, 1, 32, 32, 20000, 60), (3, 1, 64, 64, 6000, 25), (2, 2, 64, 128, 20000, 50),
+    (3, 1, 4, 32, 5000, 20), (3, 1, 96, 48, 4000, 20), (5, 1, 16, 16, 3000, 16),
+    (3, 1, 256, 256, 3000, 16), (3, 1, 24, 40, 2000, 12), (3, 1, 3, 5, 2000, 12),
+])
+def test_forward_functional(kind, kernel, stride, cin, cout, n, extent):
+    src, sbd, tgt, tbd, off, feats, weights = make_layer_case(3, n, extent, kernel, cin, cout, kind, stride)
+    esm, etm, eorder, esizes, _ = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=True)
+    ref = orc.sparse_convolution_forward(feats, weights, esm, etm, eorder, esizes)
+    dtype = TORCH[kind]
+    for shortcut in (False, True):
+        for threshold in (-1, 0.3, None):
+            out = F.sparse_convolution_forward(
+                sources=dev(feats).to(dtype), weights=dev(weights).to(dtype),
+                source_masks=dev(esm), target_masks=dev(etm), kernel_map_order=dev(eorder),
+                kernel_map_sizes=dev(esizes), gather_tile_size=0, scatter_tile_size=0,
+                allow_shortcut_matmul=shortcut and stride == 1, threshold=threshold)
+            assert out.dtype == dtype and out.shape == (tgt.shape[0], cout)
+            assert_features_close(out, ref, kind)
+
+
+@pytest.mark.parametrize("tile", [1, 2, 4, 8, 16, 32])
+def test_forward_tile_sizes(tile):
+    src, sbd, tgt, tbd, off, feats, weights = make_layer_case(5, 5000, 20, 3, 32, 64, "fp16")
+    esm, etm, eorder, esizes, _ = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=True)
+    ref = orc.sparse_convolution_forward(feats, weights, esm, etm, eorder, esizes)
+    out = F.sparse_convolution_forward(
+        sources=dev(feats).half(), weights=dev(weights).half(), source_masks=dev(esm),
+        target_masks=dev(etm), kernel_map_order=dev(eorder), kernel_map_sizes=dev(esizes),
+        gather_tile_size=tile, scatter_tile_size=tile, allow_shortcut_matmul=True, threshold=-1)
+    assert_features_close(out, ref, "fp16")
+
+
+def test_forward_rejects_bad_tile():
+    src, sbd, tgt, tbd, off, feats, weights = make_layer_case(5, 500, 8, 3, 32, 32, "fp32")
+    esm, etm, eorder, esizes, _ = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=True)
+    with pytest.raises(RuntimeError, match="Unsupported num_source_features"):
+        F.sparse_convolution_forward(
+            sources=dev(feats).float(), weights=dev(weights).float(), source_masks=dev(esm),
+            target_masks=dev(etm), kernel_map_order=dev(eorder), kernel_map_sizes=dev(esizes),
+            gather_tile_size=5, scatter_tile_size=1)
+
+
+def test_forward_no_reorder_int64_index():
+    src, sbd, tgt, tbd, off, feats, weights = make_layer_case(8, 4000, 18, 3, 32, 32, "fp32")
+    esm, etm, _, esizes, _ = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=False,
+                                                  index_dtype=np.int64)
+    ref = orc.sparse_convolution_forward(feats, weights, esm, etm, None, esizes)
+    out = F.sparse_convolution_forward(
+        sources=dev(feats).float(), weights=dev(weights).float(), source_masks=dev(esm),
+        target_masks=dev(etm), kernel_map_order=None, kernel_map_sizes=dev(esizes),
+        gather_tile_size=4, scatter_tile_size=4, threshold=0)
+    assert_features_close(out, ref, "fp32")
+
+
+def _as_sparse(coords, bd, feats, dtype):
+    return minuet.SparseTensor(dev(feats).to(dtype), dev(coords), batch_dims=dev(bd))
+
+
+@pytest.mark.parametrize("kind", ["fp32", "fp16"])
+@pytest.mark.parametrize("batched", [False, True])
+def test_module_down_sub_up(kind, batched):
+    """stride-2 conv -> submanifold conv -> transposed conv sharing one cache."""
+    dtype = TORCH[kind]
+    rng = np.random.default_rng(2)
+    bd = np.array([0, 7000, 15000], dtype=np.int32) if batched else None
+    c, bd = sorted_unique(random_cloud(15000, 40, seed=4, lo=-20), bd)
+    feats = quantise(rng.normal(size=(c.shape[0], 16)), kind)
+    cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+    down = minuet.nn.SparseConv3d(16, 32, 2, stride=2, bias=True, dtype=dtype, device="cuda")
+    sub = minuet.nn.SparseConv3d(32, 32, 3, dtype=dtype, device="cuda")
+    up = minuet.nn.SparseConv(3, 32, 16, 2, stride=2, transposed=True, dtype=dtype, device="cuda")
+    net = torch.nn.Sequential(down, sub, up)
+    minuet.set_kernel_map_cache(net, cache)
+    x = _as_sparse(c, bd, feats, dtype)
+    with torch.no_grad():
+        y1 = down(x)
+        y2 = sub(y1)
+        y3 = up(y2)
+    assert cache.num_map_builds == 2 and cache.num_coordinate_builds == 1
+    w = lambda conv: host(conv.kernel.detach().float()).astype(np.float64)
+    r1, c1, bd1, s1 = orc.conv_layer(c, bd, feats, w(down), 2, stride=2,
+                                     bias=host(down.bias.detach().float()).astype(np.float64))
+    np.testing.assert_array_equal(host(y1.C), c1)
+    assert y1.stride == (2, 2, 2) and s1 == (2, 2, 2)
+    if batched:
+        np.testing.assert_array_equal(host(y1.batch_dims), bd1)
+    assert_features_close(y1.F, r1, kind)
+    r1q = quantise(host(y1.F.float()).astype(np.float64), kind)
+    r2, c2, bd2, s2 = orc.conv_layer(c1, bd1, r1q, w(sub), 3, source_stride=2)
+    np.testing.assert_array_equal(host(y2.C), c2)
+    assert_features_close(y2.F, r2, kind)
+    r2q = quantise(host(y2.F.float()).astype(np.float64), kind)
+    r3, c3, bd3, s3 = orc.conv_layer(c2, bd2, r2q, w(up), 2, stride=2, source_stride=2,
+                                     transposed_from=(c, bd, 1))
+    np.testing.assert_array_equal(host(y3.C), c)
+    assert y3.stride == (1, 1, 1)
+    assert_features_close(y3.F, r3, kind)
+
+
+def test_module_errors_and_trivial():
+    cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+    c, _ = sorted_unique(random_cloud(500, 8, seed=1))
+    x = minuet.SparseTensor(torch.randn(c.shape[0], 8, device="cuda"), dev(c))
+    conv = minuet.nn.SparseConv3d(8, 8, 3, device="cuda")
+    with pytest.raises(ValueError, match="Kernel map cache must be specified"):
+        conv(x)
+    up = minuet.nn.SparseConv(3, 8, 8, 2, stride=2, transposed=True, device="cuda")
+    up.set_kernel_map_cache(cache)
+    x2 = minuet.SparseTensor(x.F, x.C, stride=2)
+    with pytest.raises(RuntimeError, match="non-transposed layer"):
+        up(x2)
+    one = minuet.nn.SparseConv3d(8, 4, 1, device="cuda")
+    with torch.no_grad():
+        y = one(x)
+    torch.testing.assert_close(y.F, x.F @ one.kernel.view(8, 4))
+    with pytest.raises(NotImplementedError):
+        F.arg_sort_coordinates(torch.zeros((3, 3), dtype=torch.int32))
+
+
+def test_autotune_and_timers(tmp_path):
+    c, _ = sorted_unique(random_cloud(6000, 24, seed=6))
+    x = minuet.SparseTensor(torch.randn(c.shape[0], 32, device="cuda").half(), dev(c))
+    cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+    net = torch.nn.Sequential(minuet.nn.SparseConv3d(32, 64, 3, dtype=torch.float16, device="cuda"),
+                              minuet.nn.ReLU(),
+                              minuet.nn.SparseConv3d(64, 32, 3, dtype=torch.float16, device="cuda"))
+    minuet.set_kernel_map_cache(net, cache)
+    minuet.nn.SparseConv.__NUM_TUNING_ROUNDS__ = 1
+    minuet.nn.SparseConv.__AVAILABLE_THRESHOLD__ = [-1, 0.5, None]
+    path = str(tmp_path / "tuned" / "config.json")
+    with torch.no_grad():
+        before = net(x).F.clone()
+        minuet.autotune(net, cache, [x], cache_path=path)
+        cache.reset()
+        after = net(x).F
+    cfg = minuet.dump_tunable_config(net)
+    assert set(cfg["0"].keys()) == {"threshold", "gather_tile_size", "scatter_tile_size"}
+    assert 32 % cfg["0"]["gather_tile_size"] == 0 and 64 % cfg["0"]["scatter_tile_size"] == 0
+    torch.testing.assert_close(before, after, rtol=0, atol=0)
+    import json, os
+    assert os.path.exists(path)
+    with open(path) as fh:
+        saved = json.load(fh)
+    assert saved["0"]["gather_tile_size"] == cfg["0"]["gather_tile_size"]
+    assert F.cuda_buffer_total_size() >= F.cuda_buffer_used_size() >= 0
