@@ -235,15 +235,20 @@ int mnt_time_gemm(int allow_shortcut_matmul, int64_t parallel, int has_threshold
                   int64_t num_source_features, int64_t num_target_features,
                   int index_dtype, int float_dtype, float *ms_out, void *stream);
 
-/* ---- stage timing of the last mnt_sparse_convolution_forward ------------- */
+/* ---- stage timing -------------------------------------------------------- */
 
-/* When enabled, the forward call brackets weight-pack, gather, GEMM and
- * scatter with events on its stream; mnt_profile_read synchronises and returns
- * the four durations in milliseconds (order: pack, gather, gemm, scatter).
- * No counterpart in the reference; used by the benchmark for per-kernel
- * roofline figures. */
+/* mnt_profile_enable(1) makes the instrumented entry points (sort, query, emit,
+ * forward) record a timestamp event on their stream after every stage; (0)
+ * turns that off.  Either call discards what was recorded so far.
+ * mnt_profile_read waits for the last event and returns up to `capacity`
+ * intervals between consecutive marks, in recording order: ms_out[i] and the
+ * NUL-terminated stage name at labels_out + i*label_stride.  Intervals named
+ * "enter:*" are the gaps between two entry points (host time).  Reading clears
+ * the record.  No counterpart in the reference; used by the benchmark for
+ * per-kernel roofline figures. */
 int mnt_profile_enable(int on);
-int mnt_profile_read(float *ms4_out);
+int mnt_profile_read(int capacity, float *ms_out, char *labels_out, int label_stride,
+                     int *count_out);
 
 #ifdef __cplusplus
 }

@@ -143,6 +143,13 @@ class Scope {
   Arena::Mark mark_;
 };
 
+// ------------------------------------------------------------- profiling ----
+
+// Records a timestamp event on `stream` when stage profiling is on (see
+// mnt_profile_enable); the interval since the previous mark is reported under
+// `label`, which must be a string literal.
+void profile_mark(const char *label, hipStream_t stream);
+
 // ---------------------------------------------------------------- launch ----
 
 inline int64_t div_ceil(int64_t a, int64_t b) { return (a + b - 1) / b; }

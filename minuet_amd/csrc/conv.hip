@@ -521,23 +521,6 @@ static void launch_gemm(const T *a, TC *c, const T *wt, const int *meta, int num
   check_launch("grouped_gemm_kernel");
 }
 
-// --------------------------------------------------------------- profiling ----
-
-static bool g_profile = false;
-static hipEvent_t g_events[5];
-static bool g_events_ready = false;
-static bool g_events_recorded = false;
-
-static void profile_mark(int slot, hipStream_t stream) {
-  if (!g_profile) return;
-  if (!g_events_ready) {
-    for (auto &e : g_events) MNT_HIP(hipEventCreate(&e));
-    g_events_ready = true;
-  }
-  MNT_HIP(hipEventRecord(g_events[slot], stream));
-  if (slot == 4) g_events_recorded = true;
-}
-
 // ------------------------------------------------------------ forward plan ----
 
 struct ForwardPlan {
@@ -623,7 +606,7 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
   const int Np = static_cast<int>(div_ceil(N, 32) * 32);
   const int active = static_cast<int>(plan.active_offsets);
 
-  profile_mark(0, stream);
+  profile_mark("enter:forward", stream);
   T *wt = scope.alloc<T>(static_cast<size_t>(O) * Np * Kp);
   {
     const long long total = static_cast<long long>(O) * Np * Kp;
@@ -635,7 +618,7 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
   upload_ints(plan.row_start, d_row_start, stream);
   int *d_meta = scope.alloc<int>(plan.meta.size());
   upload_ints(plan.meta, d_meta, stream);
-  profile_mark(1, stream);
+  profile_mark("pack_weights", stream);
 
   const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
   typedef typename BufferOf<T>::type TB;
@@ -645,7 +628,7 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
   const LaneShape gsh = lane_shape(gather_tile, K, sizeof(T), sources, abuf, "num_source_features");
   launch_gather<IT>(gsh, sources, abuf, source_masks, d_row_start, S, active,
                     static_cast<int>(K * sizeof(T)), stream);
-  profile_mark(2, stream);
+  profile_mark("gather", stream);
 
   launch_gemm<T, TB>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
   if (plan.shortcut) {
@@ -654,12 +637,12 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
     upload_ints(meta, d_direct, stream);
     launch_gemm<T, T>(sources, out, wt, d_direct, meta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
   }
-  profile_mark(3, stream);
+  profile_mark("gemm", stream);
 
   const LaneShape ssh = lane_shape(scatter_tile, N, sizeof(T), cbuf, out, "num_target_features");
   launch_scatter<TB, T, IT>(ssh, cbuf, out, target_masks, d_row_start, Tn, active,
                             static_cast<int>(N), plan.shortcut ? 1 : 0, stream);
-  profile_mark(4, stream);
+  profile_mark("scatter", stream);
 }
 
 }  // namespace mnt
@@ -905,19 +888,5 @@ extern "C" int mnt_time_gemm(int allow_shortcut_matmul, int64_t parallel, int ha
     } else {
       *ms_out = time_gemm_typed<bf16_t>(plan, static_cast<const bf16_t *>(weights), S, O, K, N, stream);
     }
-  });
-}
-
-extern "C" int mnt_profile_enable(int on) {
-  g_profile = on != 0;
-  g_events_recorded = false;
-  return 0;
-}
-
-extern "C" int mnt_profile_read(float *ms4_out) {
-  return guarded([&] {
-    MNT_CHECK(g_profile && g_events_recorded, "no profiled forward call has been recorded");
-    MNT_HIP(hipEventSynchronize(g_events[4]));
-    for (int i = 0; i < 4; ++i) MNT_HIP(hipEventElapsedTime(&ms4_out[i], g_events[i], g_events[i + 1]));
   });
 }

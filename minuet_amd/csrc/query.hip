@@ -408,6 +408,7 @@ static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t n
                       hipStream_t stream) {
   const int num_tiles = static_cast<int>(div_ceil(a.num_targets, kTargetsPerTile));
   const bool batched = a.source_batch_dims != nullptr && a.num_batches > 1;
+  profile_mark("enter:query", stream);
   long long *d_bounds = scope.alloc<long long>(4 * MNT_MAX_NDIM);
   enqueue_bounds(a.sources, a.num_sources, a.ndim, a.coord_dtype, d_bounds, true, stream);
   enqueue_bounds(a.targets, a.num_targets, a.ndim, a.coord_dtype, d_bounds + 2 * MNT_MAX_NDIM, true, stream);
@@ -415,6 +416,7 @@ static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t n
   MNT_HIP(hipMemcpyAsync(h_bounds, d_bounds, sizeof(long long) * 4 * MNT_MAX_NDIM,
                          hipMemcpyDeviceToHost, stream));
   MNT_HIP(hipStreamSynchronize(stream));
+  profile_mark("query_bounds+sync", stream);
   QueryPlan plan = make_plan(h_bounds, h_bounds + 2 * MNT_MAX_NDIM, offsets_host, num_offsets,
                              a.ndim, batched ? a.num_batches : 1);
   // Upload the packed offsets through the pinned block (past the bounds
@@ -448,6 +450,7 @@ static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t n
   else if (o32) MNT_Q(int64_t, int64_t, int32_t);
   else MNT_Q(int64_t, int64_t, int64_t);
 #undef MNT_Q
+  profile_mark("query", stream);
 }
 
 template <typename T>
@@ -664,6 +667,7 @@ extern "C" int mnt_kernel_map_query(const void *sources, int64_t num_sources, co
     std::vector<unsigned> host(3 * num_offsets);
     MNT_HIP(hipMemcpyAsync(host.data(), plan, sizeof(unsigned) * 3 * num_offsets, hipMemcpyDeviceToHost, stream));
     MNT_HIP(hipStreamSynchronize(stream));
+    profile_mark("map_sizes_order+sync", stream);
     for (int64_t j = 0; j < num_offsets; ++j) {
       order_host_out[j] = host[j];
       sizes_host_out[j] = host[2 * num_offsets + j];
@@ -690,10 +694,12 @@ extern "C" int mnt_kernel_map_emit(int32_t *source_masks_out, int32_t *target_ma
     unsigned *row_sizes = tile_bases + static_cast<size_t>(state.num_offsets) * state.num_tiles;
     unsigned *plan = row_sizes + state.num_offsets;
     const int no = static_cast<int>(state.num_offsets);
+    profile_mark("enter:emit", stream);
     enqueue_emit<int32_t>(static_cast<const int32_t *>(state.kernel_map), state.num_sources,
                           state.num_targets, no, tile_bases, state.num_tiles, plan + no,
                           plan + 3 * no, source_masks_out, target_masks_out, in_idx_out, out_idx_out,
                           stream);
+    profile_mark("map_emit", stream);
     const unsigned grid = grid_for(no, 256);
     if (sizes_dev_out) {
       export_sizes_kernel<int32_t><<<grid, 256, 0, stream>>>(plan + 2 * no, no, sizes_dev_out);

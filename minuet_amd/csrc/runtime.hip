@@ -116,6 +116,31 @@ void *Arena::persistent(int slot, size_t bytes) {
   return persistent_[slot];
 }
 
+// ---- stage profiler -------------------------------------------------------
+
+static bool g_profile_on = false;
+static std::vector<std::pair<const char *, hipEvent_t>> g_marks;
+static std::vector<hipEvent_t> g_event_pool;
+static constexpr size_t kMaxMarks = 4096;
+
+void profile_mark(const char *label, hipStream_t stream) {
+  if (!g_profile_on || g_marks.size() >= kMaxMarks) return;
+  hipEvent_t event;
+  if (!g_event_pool.empty()) {
+    event = g_event_pool.back();
+    g_event_pool.pop_back();
+  } else {
+    MNT_HIP(hipEventCreate(&event));
+  }
+  MNT_HIP(hipEventRecord(event, stream));
+  g_marks.emplace_back(label, event);
+}
+
+static void profile_clear() {
+  for (auto &m : g_marks) g_event_pool.push_back(m.second);
+  g_marks.clear();
+}
+
 }  // namespace mnt
 
 using namespace mnt;
@@ -152,6 +177,33 @@ size_t mnt_buffer_used_size(void *stream) {
   size_t value = 0;
   guarded([&] { value = Arena::of(static_cast<hipStream_t>(stream)).used(); });
   return value;
+}
+
+int mnt_profile_enable(int on) {
+  return guarded([&] {
+    profile_clear();
+    g_profile_on = on != 0;
+  });
+}
+
+int mnt_profile_read(int capacity, float *ms_out, char *labels_out, int label_stride,
+                     int *count_out) {
+  return guarded([&] {
+    MNT_CHECK(ms_out != nullptr && labels_out != nullptr && count_out != nullptr && label_stride > 1,
+              "bad argument");
+    int count = 0;
+    if (!g_marks.empty()) MNT_HIP(hipEventSynchronize(g_marks.back().second));
+    for (size_t i = 1; i < g_marks.size() && count < capacity; ++i) {
+      float ms = 0.0f;
+      MNT_HIP(hipEventElapsedTime(&ms, g_marks[i - 1].second, g_marks[i].second));
+      ms_out[count] = ms;
+      snprintf(labels_out + static_cast<size_t>(count) * label_stride, label_stride, "%s",
+               g_marks[i].first);
+      ++count;
+    }
+    *count_out = count;
+    profile_clear();
+  });
 }
 
 int mnt_reset_error(void) {

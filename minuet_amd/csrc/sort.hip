@@ -317,12 +317,14 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
   Scope scope(stream);
   const bool batched = batch_dims != nullptr && num_batches > 1;
 
+  profile_mark("enter:arg_sort", stream);
   long long *d_bounds = scope.alloc<long long>(2 * MNT_MAX_NDIM);
   enqueue_bounds(coords, n, ndim, sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64, d_bounds, true, stream);
   long long *h_bounds = static_cast<long long *>(scope.arena().pinned());
   MNT_HIP(hipMemcpyAsync(h_bounds, d_bounds, sizeof(long long) * 2 * MNT_MAX_NDIM,
                          hipMemcpyDeviceToHost, stream));
   MNT_HIP(hipStreamSynchronize(stream));
+  profile_mark("sort_bounds+sync", stream);
 
   // fields from least to most significant: dims ndim-1 .. 0, then the batch id
   int widths[MNT_MAX_NDIM + 1];
@@ -371,10 +373,13 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
                                                        first ? nullptr : vals, keys, vals);
     check_launch("pack_keys_kernel");
     first = false;
+    profile_mark("sort_pack", stream);
     radix_sort_pairs(keys, vals, keys_alt, vals_alt, n, bits, counts, stream);
+    profile_mark("sort_radix", stream);
   }
   emit_sorted_kernel<CT, IT><<<grid, 256, 0, stream>>>(coords, n, ndim, vals, indices_out, sorted_out);
   check_launch("emit_sorted_kernel");
+  profile_mark("sort_emit", stream);
 }
 
 }  // namespace mnt

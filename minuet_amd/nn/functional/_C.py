@@ -66,7 +66,7 @@ SIGNATURES = {
     "mnt_time_gemm": (_int, [_int, _i64, _int, _dbl, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
                              _int, _pf, _vp]),
     "mnt_profile_enable": (_int, [_int]),
-    "mnt_profile_read": (_int, [_pf]),
+    "mnt_profile_read": (_int, [_int, _pf, _c.c_char_p, _int, _c.POINTER(_c.c_int)]),
 }
 
 
@@ -617,6 +617,15 @@ def profile_enable(on: bool):
 
 
 def profile_read():
-    ms = (ctypes.c_float * 4)()
-    _check(load_library().mnt_profile_read(ms))
-    return {"pack": ms[0], "gather": ms[1], "gemm": ms[2], "scatter": ms[3]}
+    """Stage intervals recorded since the last read: list of (name, ms)."""
+    capacity, stride = 4096, 32
+    ms = (ctypes.c_float * capacity)()
+    labels = ctypes.create_string_buffer(capacity * stride)
+    count = ctypes.c_int(0)
+    _check(load_library().mnt_profile_read(capacity, ms, labels, stride, ctypes.byref(count)))
+    raw = labels.raw
+    out = []
+    for i in range(count.value):
+        name = raw[i * stride:(i + 1) * stride].split(b"\0", 1)[0].decode()
+        out.append((name, float(ms[i])))
+    return out
