@@ -21,9 +21,10 @@ HBM_PEAK_GBS = 8000.0
 
 
 def map_step(_C, coords_dev, offsets):
-    _, sorted_dev = _C.sort_coordinates(coords_dev)
+    _, sorted_dev, bounds = _C.sort_coordinates(coords_dev, return_bounds=True)
     built = _C.kernel_map_build(sorted_dev, sorted_dev, offsets, None, None, reorder=False,
-                                want_masks=False, want_lists=True)
+                                want_masks=False, want_lists=True, source_bounds=bounds,
+                                target_bounds=bounds)
     return sorted_dev, built
 
 

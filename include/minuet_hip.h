@@ -59,14 +59,17 @@ int mnt_reset_error(void);                                /* cuda_reset_error */
 /* Stable lexicographic arg-sort of coords[n, ndim] (dimension 0 most
  * significant); with batch_dims[num_batches+1] the result is batch-major.
  * indices_out[n] has element type index_dtype (= the type of batch_dims when
- * given).  sorted_coords_out (nullable) receives coords[indices_out].
+ * given).  sorted_coords_out (nullable) receives coords[indices_out] and
+ * bounds_host_out (nullable, HOST, 8 x int64) the per-dimension minima [0..3]
+ * and maxima [4..7] of the coordinates.
  * Synchronises once (coordinate bounds are read back to size the keys).
  * Replaces cuda_arg_sort_coordinates / cuda_multi_arg_sort_coordinates,
  * csrc/minuet/torch/cuda_arg_sort_coordinates.cu:8-70 and
  * csrc/minuet/cuda/functions/arg_sort_coodrinates.cu:273-469. */
 int mnt_arg_sort_coordinates(const void *coords, int64_t n, int ndim, int coord_dtype,
                              const void *batch_dims, int64_t num_batches, int index_dtype,
-                             void *indices_out, void *sorted_coords_out, void *stream);
+                             void *indices_out, void *sorted_coords_out,
+                             int64_t *bounds_host_out, void *stream);
 
 /* ---- Map: unique ------------------------------------------------------- */
 
@@ -139,7 +142,12 @@ int mnt_compute_kernel_map_masks(const void *kernel_map, int64_t num_offsets,
  * order), per-offset sizes and the stable ascending size order (reorder != 0;
  * identity otherwise).  offsets_host[O*ndim] is a HOST array of int64.
  * order_host_out[j] is the offset of output row j and sizes_host_out[j] its
- * hit count.  Synchronises twice (bounds; sizes).
+ * hit count.  source_bounds_host / target_bounds_host (nullable, 8 x int64:
+ * per-dimension minima in [0..3], maxima in [4..7]) are the coordinate bounds
+ * when the caller already knows them, e.g. from mnt_arg_sort_coordinates;
+ * whatever is missing is reduced on the device.  bounds_host_out (nullable,
+ * 16 x int64) receives the bounds used (sources then targets).  Synchronises
+ * once for the sizes and once more only when bounds had to be computed.
  *
  * mnt_kernel_map_emit: must directly follow the query on the same stream, with
  * kernel_map_out still alive.  Writes any non-null output: the rank tables
@@ -154,7 +162,8 @@ int mnt_kernel_map_query(const void *sources, int64_t num_sources,
                          int ndim, int coord_dtype,
                          const void *source_batch_dims, const void *target_batch_dims,
                          int64_t num_batches, int batch_dtype, int reorder,
-                         int32_t *kernel_map_out,
+                         const int64_t *source_bounds_host, const int64_t *target_bounds_host,
+                         int64_t *bounds_host_out, int32_t *kernel_map_out,
                          int64_t *sizes_host_out, int64_t *order_host_out, void *stream);
 int mnt_kernel_map_emit(int32_t *source_masks_out, int32_t *target_masks_out,
                         int32_t *in_idx_out, int32_t *out_idx_out,

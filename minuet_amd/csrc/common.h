@@ -89,6 +89,11 @@ class Arena {
   // Pinned host staging block (64 KiB) for small read-backs and uploads.
   static constexpr size_t kPinnedBytes = 64 * 1024;
   void *pinned();
+  // Device-side address of the same block (kernels may write results there).
+  void *pinned_device();
+  // 16 zero-initialised device counters for "last workgroup" tickets; every
+  // kernel that uses one leaves it at zero again.
+  unsigned *tickets();
   // Long-lived device blocks that survive scopes (state of the two-phase entry
   // points; slot 0: target coordinates, slot 1: kernel-map build).  Grows to
   // at least `bytes`; 0 returns the current block.
@@ -124,6 +129,8 @@ class Arena {
   size_t page_size_ = size_t(8) << 20;
   float growth_ = 1.0f;
   void *pinned_ = nullptr;
+  void *pinned_device_ = nullptr;
+  unsigned *tickets_ = nullptr;
   void *persistent_[2] = {nullptr, nullptr};
   size_t persistent_size_[2] = {0, 0};
 };

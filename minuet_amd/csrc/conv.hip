@@ -13,6 +13,7 @@
 #include <algorithm>
 
 #include "device_utils.h"
+#include "sort.h"
 
 namespace mnt {
 
@@ -57,29 +58,6 @@ static void cumsum_padded(const int64_t *sizes, int64_t n, const std::vector<int
     int64_t summit = 0;
     for (int64_t j = buckets[b]; j < buckets[b + 1]; ++j) summit = std::max(summit, sizes[j]);
     for (int64_t j = buckets[b]; j < buckets[b + 1]; ++j) cum[j + 1] = cum[j] + summit;
-  }
-}
-
-// ------------------------------------------- small uploads through kernargs ----
-
-constexpr int kUploadInts = 512;
-struct IntChunk {
-  int v[kUploadInts];
-};
-
-__global__ __launch_bounds__(256) void upload_ints_kernel(IntChunk chunk, int count, int *__restrict__ dst) {
-  for (int i = threadIdx.x; i < count; i += blockDim.x) dst[i] = chunk.v[i];
-}
-
-// Copies a small host int array to device memory as kernel arguments: no
-// staging buffer to protect, no synchronisation, safe under stream capture.
-static void upload_ints(const std::vector<int> &host, int *dst, hipStream_t stream) {
-  for (size_t base = 0; base < host.size(); base += kUploadInts) {
-    IntChunk chunk;
-    const int count = static_cast<int>(std::min<size_t>(kUploadInts, host.size() - base));
-    memcpy(chunk.v, host.data() + base, sizeof(int) * count);
-    upload_ints_kernel<<<1, 256, 0, stream>>>(chunk, count, dst + base);
-    check_launch("upload_ints_kernel");
   }
 }
 

@@ -8,21 +8,30 @@
 // tables follow ComputeKernelMapSizes / ComputeKernelMapMasks
 // (csrc/minuet/cuda/functions/scan.cu:220-365).
 //
-// Layout of one query workgroup: 512 consecutive sorted targets.  Because the
-// targets are sorted, every shifted query of the tile lies between
+// Layout of one query workgroup: 512 consecutive sorted targets, one per lane.
+// Because the targets are sorted, every shifted query of the tile lies between
 // key(first)+min_delta and key(last)+max_delta, so ONE window of the sorted
 // sources serves all offsets.  The window is packed to 64-bit keys and staged
-// in LDS (2048 keys at a time); every (offset, target) pair is then resolved
-// by a branch-free binary search in LDS, and hits are counted per offset with
-// wavefront ballots.
+// in LDS (2048 keys at a time).  Offsets are visited in ascending key order
+// and split into groups of near-adjacent deltas (e.g. the three z-neighbours
+// of one (dx,dy)): the first query of a group is located by a branch-free
+// binary search in LDS (three groups searched in lockstep for latency
+// hiding), the others by walking forward from there.  Hits are counted per
+// offset with wavefront ballots.
+#include <algorithm>
+
 #include "device_utils.h"
 #include "sort.h"
 
 namespace mnt {
 
-constexpr int kQueryBlock = 256;
+constexpr int kQueryBlock = 256;          // emit / count kernels
+constexpr int kQueryThreads = 512;        // query kernel: one target per lane
 constexpr int kTargetsPerTile = 512;
 constexpr int kWindowChunk = 2048;
+constexpr int kWindowPad = 64;            // sentinel keys behind a full chunk
+constexpr long long kMaxWalkGap = 4;      // largest key gap bridged by walking
+constexpr int kGroupsInFlight = 3;
 
 template <typename CT, typename BT>
 struct KeyReader {
@@ -61,14 +70,17 @@ __device__ __forceinline__ long long wave_lower_bound(const KeyReader<CT, BT> &s
   return lo;
 }
 
+// sorted_delta[i] / sorted_offset[i]: packed delta and original row of the i-th
+// offset in ascending key order; group_start[g] .. group_start[g+1] are the
+// offsets of walk group g.
 template <typename CT, typename BT, typename OT>
-__global__ __launch_bounds__(kQueryBlock) void query_kernel(
+__global__ __launch_bounds__(kQueryThreads) void query_kernel(
     KeyReader<CT, BT> src, KeyReader<CT, BT> tgt, Frame frame,
-    const long long *__restrict__ deltas, int num_offsets, long long delta_min,
-    long long delta_max, OT *__restrict__ kernel_map, unsigned *__restrict__ tile_counts,
-    int num_tiles) {
+    const long long *__restrict__ sorted_delta, const int *__restrict__ sorted_offset,
+    const int *__restrict__ group_start, int num_groups, int num_offsets,
+    OT *__restrict__ kernel_map, unsigned *__restrict__ tile_counts, int num_tiles) {
   extern __shared__ unsigned s_counts[];                 // [num_offsets]
-  __shared__ unsigned long long win[kWindowChunk];
+  __shared__ unsigned long long win[kWindowChunk + kWindowPad];
   __shared__ long long s_bounds[2];
   __shared__ unsigned long long s_next_first;
 
@@ -77,26 +89,20 @@ __global__ __launch_bounds__(kQueryBlock) void query_kernel(
   const long long t0 = static_cast<long long>(blockIdx.x) * kTargetsPerTile;
   const long long t_end = t0 + kTargetsPerTile < num_targets ? t0 + kTargetsPerTile : num_targets;
 
-  for (int o = tid; o < num_offsets; o += kQueryBlock) s_counts[o] = 0;
+  for (int o = tid; o < num_offsets; o += kQueryThreads) s_counts[o] = 0;
 
   // window of sources that can match any (offset, target) pair of this tile
   const int w = tid >> 6;
   if (w < 2) {
-    const unsigned long long edge = w == 0 ? tgt(t0, frame) + static_cast<unsigned long long>(delta_min)
-                                           : tgt(t_end - 1, frame) + static_cast<unsigned long long>(delta_max) + 1ull;
+    const unsigned long long edge =
+        w == 0 ? tgt(t0, frame) + static_cast<unsigned long long>(sorted_delta[0])
+               : tgt(t_end - 1, frame) + static_cast<unsigned long long>(sorted_delta[num_offsets - 1]) + 1ull;
     const long long pos = wave_lower_bound<CT, BT>(src, frame, edge);
     if (lane_id() == 0) s_bounds[w] = pos;
   }
-
-  long long tq[2];
-  unsigned long long tk[2];
-  bool tv[2];
-#pragma unroll
-  for (int r = 0; r < 2; ++r) {
-    tq[r] = t0 + r * kQueryBlock + tid;
-    tv[r] = tq[r] < t_end;
-    tk[r] = tv[r] ? tgt(tq[r], frame) : 0ull;
-  }
+  const long long t = t0 + tid;
+  const bool valid = t < t_end;
+  const unsigned long long key = valid ? tgt(t, frame) : 0ull;
   __syncthreads();
   const long long w_lo = s_bounds[0];
   const long long w_hi = s_bounds[1] > w_lo ? s_bounds[1] : w_lo;
@@ -108,7 +114,7 @@ __global__ __launch_bounds__(kQueryBlock) void query_kernel(
     const long long c1 = c0 + kWindowChunk < w_hi ? c0 + kWindowChunk : w_hi;
     const int len = static_cast<int>(c1 - c0);
     if (c > 0) __syncthreads();
-    for (int i = tid; i < kWindowChunk; i += kQueryBlock) {
+    for (int i = tid; i < kWindowChunk + kWindowPad; i += kQueryThreads) {
       win[i] = i < len ? src(c0 + i, frame) : ~0ull;
     }
     if (tid == 0) s_next_first = c1 < w_hi ? src(c1, frame) : ~0ull;
@@ -120,30 +126,47 @@ __global__ __launch_bounds__(kQueryBlock) void query_kernel(
     int top = 1;
     while (top * 2 < len) top *= 2;      // highest power of two below len (>= 1)
 
-    for (int o = 0; o < num_offsets; ++o) {
-      const unsigned long long delta = static_cast<unsigned long long>(deltas[o]);
-      unsigned hits = 0;
+    for (int g0 = 0; g0 < num_groups; g0 += kGroupsInFlight) {
+      // lower bound of the first query of up to three groups, in lockstep
+      unsigned long long q0[kGroupsInFlight];
+      int pos[kGroupsInFlight];
 #pragma unroll
-      for (int r = 0; r < 2; ++r) {
-        const unsigned long long q = tk[r] + delta;
-        const bool mine = tv[r] && (is_first || q >= first_key) && (is_last || q < next_first);
-        int pos = 0;
-        for (int step = top; step >= 1; step >>= 1) {
-          if (win[pos + step] <= q) pos += step;
-        }
-        const bool hit = mine && len > 0 && win[pos] == q;
-        if (mine) {
-          kernel_map[static_cast<long long>(o) * num_targets + tq[r]] =
-              hit ? static_cast<OT>(c0 + pos) : static_cast<OT>(-1);
-        }
-        hits += __popcll(__ballot(hit));
+      for (int j = 0; j < kGroupsInFlight; ++j) {
+        const int g = g0 + j < num_groups ? g0 + j : num_groups - 1;
+        q0[j] = key + static_cast<unsigned long long>(sorted_delta[group_start[g]]);
+        pos[j] = 0;
       }
-      if (tile_counts != nullptr && hits != 0 && lane_id() == 0) atomicAdd(&s_counts[o], hits);
+      for (int step = top; step >= 1; step >>= 1) {
+#pragma unroll
+        for (int j = 0; j < kGroupsInFlight; ++j) {
+          if (win[pos[j] + step - 1] < q0[j]) pos[j] += step;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kGroupsInFlight; ++j) {
+        if (g0 + j >= num_groups) continue;       // uniform across the workgroup
+        int p = pos[j];
+        p += win[p] < q0[j] ? 1 : 0;
+        const int i_end = group_start[g0 + j + 1];
+        for (int i = group_start[g0 + j]; i < i_end; ++i) {
+          const unsigned long long q = key + static_cast<unsigned long long>(sorted_delta[i]);
+          const bool mine = valid && (is_first || q >= first_key) && (is_last || q < next_first);
+          while (mine && win[p] < q) ++p;
+          const bool hit = mine && win[p] == q;
+          const int o = sorted_offset[i];
+          if (mine) {
+            kernel_map[static_cast<long long>(o) * num_targets + t] =
+                hit ? static_cast<OT>(c0 + p) : static_cast<OT>(-1);
+          }
+          const unsigned hits = __popcll(__ballot(hit));
+          if (tile_counts != nullptr && hits != 0 && lane_id() == 0) atomicAdd(&s_counts[o], hits);
+        }
+      }
     }
   }
   if (tile_counts != nullptr) {
     __syncthreads();
-    for (int o = tid; o < num_offsets; o += kQueryBlock) {
+    for (int o = tid; o < num_offsets; o += kQueryThreads) {
       tile_counts[static_cast<long long>(o) * num_tiles + blockIdx.x] = s_counts[o];
     }
   }
@@ -172,11 +195,18 @@ __global__ __launch_bounds__(kQueryBlock) void count_tiles_kernel(
 }
 
 // One workgroup per row: exclusive scan of its tile counts in place and the
-// row total.
+// row total.  With `plan` the last workgroup to finish (self-resetting
+// ticket) also derives the row order: stable ascending by size (reorder) or
+// identity, its inverse, the sizes in row order and their exclusive prefix.
+// plan layout (unsigned): order[O] | position_of[O] | sorted_sizes[O] | prefix[O+1];
+// the first three blocks are mirrored into plan_host (pinned host memory).
 __global__ __launch_bounds__(256) void tile_scan_kernel(unsigned *__restrict__ tile_counts,
-                                                        int num_tiles,
-                                                        unsigned *__restrict__ row_sizes) {
+                                                        int num_tiles, unsigned *row_sizes,
+                                                        int reorder, unsigned *__restrict__ plan,
+                                                        unsigned *__restrict__ plan_host,
+                                                        unsigned *ticket) {
   __shared__ unsigned partial[256];
+  __shared__ bool s_last;
   unsigned *row = tile_counts + static_cast<long long>(blockIdx.x) * num_tiles;
   const int t = threadIdx.x;
   const int chunk = (num_tiles + 255) / 256;
@@ -198,42 +228,48 @@ __global__ __launch_bounds__(256) void tile_scan_kernel(unsigned *__restrict__ t
     row[i] = run;
     run += v;
   }
-  if (t == 255) row_sizes[blockIdx.x] = partial[255];
-}
-
-// Stable ascending order of the rows by size (or identity), the inverse
-// permutation, the sizes in row order and their exclusive prefix.
-// plan layout (unsigned, 4 blocks of num_offsets (+1 for the prefix)):
-//   order[j] | position_of[o] | sorted_sizes[j] | prefix[j] (num_offsets+1)
-__global__ __launch_bounds__(256) void order_kernel(const unsigned *__restrict__ row_sizes,
-                                                    int num_offsets, int reorder,
-                                                    unsigned *__restrict__ plan) {
+  if (t == 255) {
+    __hip_atomic_store(&row_sizes[blockIdx.x], partial[255], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (plan == nullptr) return;
+  const int num_offsets = gridDim.x;
+  __threadfence();
+  __syncthreads();
+  if (t == 0) s_last = atomicInc(ticket, gridDim.x - 1) == gridDim.x - 1;
+  __syncthreads();
+  if (!s_last) return;
+  __threadfence();
   unsigned *order = plan;
   unsigned *position_of = plan + num_offsets;
   unsigned *sorted_sizes = plan + 2 * num_offsets;
   unsigned *prefix = plan + 3 * num_offsets;
-  for (int o = threadIdx.x; o < num_offsets; o += blockDim.x) {
-    const unsigned mine = row_sizes[o];
+  for (int o = t; o < num_offsets; o += 256) {
+    const unsigned mine = __hip_atomic_load(&row_sizes[o], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     int pos = o;
     if (reorder) {
       pos = 0;
       for (int p = 0; p < num_offsets; ++p) {
-        const unsigned other = row_sizes[p];
+        const unsigned other = __hip_atomic_load(&row_sizes[p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         pos += (other < mine || (other == mine && p < o)) ? 1 : 0;
       }
     }
     order[pos] = o;
     position_of[o] = pos;
     sorted_sizes[pos] = mine;
+    if (plan_host != nullptr) {
+      plan_host[pos] = o;
+      plan_host[num_offsets + o] = pos;
+      plan_host[2 * num_offsets + pos] = mine;
+    }
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    unsigned run = 0;
+  if (t == 0) {
+    unsigned total = 0;
     for (int j = 0; j < num_offsets; ++j) {
-      prefix[j] = run;
-      run += sorted_sizes[j];
+      prefix[j] = total;
+      total += sorted_sizes[j];
     }
-    prefix[num_offsets] = run;
+    prefix[num_offsets] = total;
   }
 }
 
@@ -255,7 +291,15 @@ __global__ __launch_bounds__(kQueryBlock) void emit_kernel(
     int num_offsets, const unsigned *__restrict__ tile_bases, int num_tiles,
     const unsigned *__restrict__ position_of, const unsigned *__restrict__ row_base,
     IT *__restrict__ source_masks, IT *__restrict__ target_masks, int *__restrict__ in_idx,
-    int *__restrict__ out_idx) {
+    int *__restrict__ out_idx, const unsigned *__restrict__ plan, int *__restrict__ sizes_out,
+    int *__restrict__ order_out) {
+  if (plan != nullptr && blockIdx.x == 0 && blockIdx.y == 0) {
+    // device copies of the row order and the sizes in row order
+    for (int j = threadIdx.x; j < num_offsets; j += kQueryBlock) {
+      if (order_out) order_out[j] = static_cast<int>(plan[j]);
+      if (sizes_out) sizes_out[j] = static_cast<int>(plan[2 * num_offsets + j]);
+    }
+  }
   const int o = blockIdx.y * (kQueryBlock / kWave) + (threadIdx.x >> 6);
   if (o >= num_offsets) return;
   const int lane = lane_id();
@@ -299,8 +343,9 @@ static int width_of(unsigned long long range) {
 
 struct QueryPlan {
   Frame frame;
-  std::vector<long long> deltas;
-  long long delta_min, delta_max;
+  std::vector<long long> sorted_delta;   // packed offsets in ascending order
+  std::vector<int> sorted_offset;        // original row of each
+  std::vector<int> group_start;          // walk groups over the sorted order
 };
 
 // Builds the packing frame from the coordinate bounds of sources and targets
@@ -341,18 +386,26 @@ static QueryPlan make_plan(const long long *src_bounds, const long long *tgt_bou
             "voxel keys need %d bits (coordinate ranges plus kernel reach plus batch id); at most "
             "63 are supported",
             bits);
-  plan.deltas.resize(num_offsets);
-  plan.delta_min = 0;
-  plan.delta_max = 0;
+  std::vector<std::pair<long long, int>> keyed(num_offsets);
   for (int64_t o = 0; o < num_offsets; ++o) {
     long long d = 0;
     for (int k = 0; k < ndim; ++k) {
       d += static_cast<long long>(static_cast<unsigned long long>(offsets[o * ndim + k]) << f.shift[k]);
     }
-    plan.deltas[o] = d;
-    if (o == 0 || d < plan.delta_min) plan.delta_min = d;
-    if (o == 0 || d > plan.delta_max) plan.delta_max = d;
+    keyed[o] = std::make_pair(d, static_cast<int>(o));
   }
+  std::stable_sort(keyed.begin(), keyed.end(),
+                   [](const std::pair<long long, int> &x, const std::pair<long long, int> &y) {
+                     return x.first < y.first;
+                   });
+  plan.sorted_delta.resize(num_offsets);
+  plan.sorted_offset.resize(num_offsets);
+  for (int64_t i = 0; i < num_offsets; ++i) {
+    plan.sorted_delta[i] = keyed[i].first;
+    plan.sorted_offset[i] = keyed[i].second;
+    if (i == 0 || keyed[i].first - keyed[i - 1].first > kMaxWalkGap) plan.group_start.push_back(static_cast<int>(i));
+  }
+  plan.group_start.push_back(static_cast<int>(num_offsets));
   return plan;
 }
 
@@ -387,48 +440,66 @@ static void check_query_args(const QueryArgs &a, int64_t num_offsets) {
 }
 
 template <typename CT, typename BT, typename OT>
-static void launch_query(const QueryArgs &a, const QueryPlan &plan, const long long *d_deltas,
-                         int num_offsets, OT *kernel_map, unsigned *tile_counts, int num_tiles,
-                         hipStream_t stream) {
+static void launch_query(const QueryArgs &a, const QueryPlan &plan, const long long *d_delta,
+                         const int *d_offset, const int *d_group, int num_offsets, OT *kernel_map,
+                         unsigned *tile_counts, int num_tiles, hipStream_t stream) {
   KeyReader<CT, BT> src{static_cast<const CT *>(a.sources), static_cast<const BT *>(a.source_batch_dims),
                         static_cast<int>(a.num_batches), a.num_sources};
   KeyReader<CT, BT> tgt{static_cast<const CT *>(a.targets), static_cast<const BT *>(a.target_batch_dims),
                         static_cast<int>(a.num_batches), a.num_targets};
   const size_t dyn = sizeof(unsigned) * static_cast<size_t>(num_offsets > 0 ? num_offsets : 1);
-  query_kernel<CT, BT, OT><<<num_tiles, kQueryBlock, dyn, stream>>>(
-      src, tgt, plan.frame, d_deltas, num_offsets, plan.delta_min, plan.delta_max, kernel_map,
-      tile_counts, num_tiles);
+  query_kernel<CT, BT, OT><<<num_tiles, kQueryThreads, dyn, stream>>>(
+      src, tgt, plan.frame, d_delta, d_offset, d_group, static_cast<int>(plan.group_start.size()) - 1,
+      num_offsets, kernel_map, tile_counts, num_tiles);
   check_launch("query_kernel");
 }
 
-// Runs the query into kernel_map (element size out_size) and, when tile_counts
+// Coordinate bounds of both operands: taken from the caller when given (8
+// values each: min[4], max[4]), otherwise reduced on the device (one launch
+// and one synchronisation).  bounds_out (nullable, 16 values) receives them.
+static void resolve_bounds(const QueryArgs &a, const int64_t *source_bounds, const int64_t *target_bounds,
+                           long long bounds[16], int64_t *bounds_out, Scope &scope, hipStream_t stream) {
+  const bool need_src = source_bounds == nullptr;
+  const bool need_tgt = target_bounds == nullptr;
+  if (need_src || need_tgt) {
+    long long fresh[16];
+    read_bounds(need_src ? a.sources : nullptr, need_src ? a.num_sources : 0,
+                need_tgt ? a.targets : nullptr, need_tgt ? a.num_targets : 0, a.ndim, a.coord_dtype,
+                fresh, scope, stream);
+    memcpy(bounds, fresh, sizeof(fresh));
+  }
+  if (!need_src) memcpy(bounds, source_bounds, sizeof(long long) * 8);
+  if (!need_tgt) memcpy(bounds + 8, target_bounds, sizeof(long long) * 8);
+  if (bounds_out != nullptr) memcpy(bounds_out, bounds, sizeof(long long) * 16);
+}
+
+// Runs the query into kernel_map (element type out_dtype) and, when tile_counts
 // is given, the per-(offset, tile) hit counts.  offsets_host: int64 [O, ndim].
 static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t num_offsets,
-                      void *kernel_map, int out_dtype, unsigned *tile_counts, Scope &scope,
-                      hipStream_t stream) {
+                      const int64_t *source_bounds, const int64_t *target_bounds,
+                      int64_t *bounds_out, void *kernel_map, int out_dtype, unsigned *tile_counts,
+                      Scope &scope, hipStream_t stream) {
   const int num_tiles = static_cast<int>(div_ceil(a.num_targets, kTargetsPerTile));
   const bool batched = a.source_batch_dims != nullptr && a.num_batches > 1;
   profile_mark("enter:query", stream);
-  long long *d_bounds = scope.alloc<long long>(4 * MNT_MAX_NDIM);
-  enqueue_bounds(a.sources, a.num_sources, a.ndim, a.coord_dtype, d_bounds, true, stream);
-  enqueue_bounds(a.targets, a.num_targets, a.ndim, a.coord_dtype, d_bounds + 2 * MNT_MAX_NDIM, true, stream);
-  long long *h_bounds = static_cast<long long *>(scope.arena().pinned());
-  MNT_HIP(hipMemcpyAsync(h_bounds, d_bounds, sizeof(long long) * 4 * MNT_MAX_NDIM,
-                         hipMemcpyDeviceToHost, stream));
-  MNT_HIP(hipStreamSynchronize(stream));
+  long long bounds[16];
+  resolve_bounds(a, source_bounds, target_bounds, bounds, bounds_out, scope, stream);
   profile_mark("query_bounds+sync", stream);
-  QueryPlan plan = make_plan(h_bounds, h_bounds + 2 * MNT_MAX_NDIM, offsets_host, num_offsets,
-                             a.ndim, batched ? a.num_batches : 1);
-  // Upload the packed offsets through the pinned block (past the bounds
-  // slots).  The stream was synchronised above, so no earlier copy still
-  // reads this block.
-  MNT_CHECK(sizeof(long long) * num_offsets + 512 <= Arena::kPinnedBytes,
-            "too many kernel offsets (%lld)", static_cast<long long>(num_offsets));
-  long long *h_deltas = reinterpret_cast<long long *>(static_cast<char *>(scope.arena().pinned()) + 512);
-  memcpy(h_deltas, plan.deltas.data(), sizeof(long long) * num_offsets);
-  long long *d_deltas = scope.alloc<long long>(num_offsets);
-  MNT_HIP(hipMemcpyAsync(d_deltas, h_deltas, sizeof(long long) * num_offsets,
-                         hipMemcpyHostToDevice, stream));
+  QueryPlan plan = make_plan(bounds, bounds + 8, offsets_host, num_offsets, a.ndim,
+                             batched ? a.num_batches : 1);
+  // Upload the plan as kernel arguments of a tiny copy kernel: nothing to
+  // keep alive on the host and no staging buffer another call could overwrite.
+  const int no = static_cast<int>(num_offsets);
+  const int ng = static_cast<int>(plan.group_start.size());
+  std::vector<int> words(2 * no + no + ng);
+  memcpy(words.data(), plan.sorted_delta.data(), sizeof(long long) * no);
+  memcpy(words.data() + 2 * no, plan.sorted_offset.data(), sizeof(int) * no);
+  memcpy(words.data() + 3 * no, plan.group_start.data(), sizeof(int) * ng);
+  int *d_words = scope.alloc<int>(words.size() + 2);
+  upload_ints(words, d_words, stream);
+  const long long *d_delta = reinterpret_cast<const long long *>(d_words);
+  const int *d_offset = d_words + 2 * no;
+  const int *d_group = d_words + 3 * no;
   QueryArgs b = a;
   if (!batched) {
     b.source_batch_dims = nullptr;
@@ -438,9 +509,9 @@ static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t n
   const bool c32 = a.coord_dtype == MNT_INT32;
   const bool b32 = !batched || a.batch_dtype == MNT_INT32;
   const bool o32 = out_dtype == MNT_INT32;
-  const int no = static_cast<int>(num_offsets);
-#define MNT_Q(CT, BT, OT) \
-  launch_query<CT, BT, OT>(b, plan, d_deltas, no, static_cast<OT *>(kernel_map), tile_counts, num_tiles, stream)
+#define MNT_Q(CT, BT, OT)                                                                        \
+  launch_query<CT, BT, OT>(b, plan, d_delta, d_offset, d_group, no, static_cast<OT *>(kernel_map), \
+                           tile_counts, num_tiles, stream)
   if (c32 && b32 && o32) MNT_Q(int32_t, int32_t, int32_t);
   else if (c32 && b32) MNT_Q(int32_t, int32_t, int64_t);
   else if (c32 && o32) MNT_Q(int32_t, int64_t, int32_t);
@@ -478,13 +549,16 @@ template <typename IT>
 static void enqueue_emit(const IT *kernel_map, int64_t num_sources, int64_t num_targets,
                          int num_offsets, const unsigned *tile_bases, int num_tiles,
                          const unsigned *position_of, const unsigned *row_base, IT *source_masks,
-                         IT *target_masks, int *in_idx, int *out_idx, hipStream_t stream) {
+                         IT *target_masks, int *in_idx, int *out_idx, hipStream_t stream,
+                         const unsigned *plan = nullptr, int *sizes_out = nullptr,
+                         int *order_out = nullptr) {
   if (source_masks) enqueue_fill<IT>(source_masks, static_cast<int64_t>(num_offsets) * num_sources, static_cast<IT>(-1), stream);
-  if (num_targets == 0 || num_offsets == 0) return;
-  dim3 grid(num_tiles, static_cast<unsigned>(div_ceil(num_offsets, kQueryBlock / kWave)));
+  if (num_offsets == 0) return;
+  dim3 grid(num_tiles > 0 ? num_tiles : 1, static_cast<unsigned>(div_ceil(num_offsets, kQueryBlock / kWave)));
   emit_kernel<IT><<<grid, kQueryBlock, 0, stream>>>(kernel_map, num_sources, num_targets, num_offsets,
                                                    tile_bases, num_tiles, position_of, row_base,
-                                                   source_masks, target_masks, in_idx, out_idx);
+                                                   source_masks, target_masks, in_idx, out_idx,
+                                                   plan, sizes_out, order_out);
   check_launch("emit_kernel");
 }
 
@@ -528,7 +602,7 @@ extern "C" int mnt_query_sorted_index_with_offsets(
       host_offsets[i] = csz == 4 ? static_cast<int64_t>(reinterpret_cast<int32_t *>(raw.data())[i])
                                  : reinterpret_cast<int64_t *>(raw.data())[i];
     }
-    run_query(a, host_offsets.data(), num_offsets, kernel_map_out, out_dtype, nullptr, scope, stream);
+    run_query(a, host_offsets.data(), num_offsets, nullptr, nullptr, nullptr, kernel_map_out, out_dtype, nullptr, scope, stream);
   });
 }
 
@@ -549,7 +623,7 @@ extern "C" int mnt_compute_kernel_map_sizes(const void *kernel_map, int64_t num_
     unsigned *tile_counts = scope.alloc<unsigned>(static_cast<size_t>(num_offsets) * num_tiles);
     unsigned *row_sizes = scope.alloc<unsigned>(num_offsets);
     enqueue_count_tiles(kernel_map, index_dtype, num_offsets, num_targets, tile_counts, num_tiles, stream);
-    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes);
+    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes, 0, nullptr, nullptr, nullptr);
     check_launch("tile_scan_kernel");
     const unsigned grid = grid_for(num_offsets, 256);
     if (index_dtype == MNT_INT32) {
@@ -578,7 +652,7 @@ extern "C" int mnt_compute_kernel_map_masks(const void *kernel_map, int64_t num_
     unsigned *row_sizes = scope.alloc<unsigned>(num_offsets);
     if (num_targets > 0) {
       enqueue_count_tiles(kernel_map, index_dtype, num_offsets, num_targets, tile_counts, num_tiles, stream);
-      tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes);
+      tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes, 0, nullptr, nullptr, nullptr);
       check_launch("tile_scan_kernel");
     }
     if (index_dtype == MNT_INT32) {
@@ -613,7 +687,7 @@ extern "C" int mnt_kernel_map_pair_lists(const int32_t *kernel_map, int64_t num_
     for (int64_t o = 0; o <= num_offsets; ++o) base[o] = static_cast<unsigned>(cumsum_host[o]);
     MNT_HIP(hipMemcpyAsync(row_base, base.data(), sizeof(unsigned) * (num_offsets + 1), hipMemcpyHostToDevice, stream));
     enqueue_count_tiles(kernel_map, MNT_INT32, num_offsets, num_targets, tile_counts, num_tiles, stream);
-    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes);
+    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes, 0, nullptr, nullptr, nullptr);
     check_launch("tile_scan_kernel");
     enqueue_emit<int32_t>(kernel_map, 0, num_targets, static_cast<int>(num_offsets), tile_counts,
                           num_tiles, nullptr, row_base, nullptr, nullptr, in_idx_out, out_idx_out, stream);
@@ -626,6 +700,8 @@ extern "C" int mnt_kernel_map_query(const void *sources, int64_t num_sources, co
                                     int64_t num_offsets, int ndim, int coord_dtype,
                                     const void *source_batch_dims, const void *target_batch_dims,
                                     int64_t num_batches, int batch_dtype, int reorder,
+                                    const int64_t *source_bounds_host,
+                                    const int64_t *target_bounds_host, int64_t *bounds_host_out,
                                     int32_t *kernel_map_out, int64_t *sizes_host_out,
                                     int64_t *order_host_out, void *stream_) {
   return guarded([&] {
@@ -644,11 +720,16 @@ extern "C" int mnt_kernel_map_query(const void *sources, int64_t num_sources, co
     unsigned *plan = row_sizes + num_offsets;
     MapState state{num_sources, num_targets, num_offsets, num_tiles, reorder, kernel_map_out};
     arena.map_state_valid = false;
+    if (bounds_host_out != nullptr) {
+      for (int i = 0; i < 16; ++i) bounds_host_out[i] = (i & 4) ? INT64_MIN : INT64_MAX;
+    }
     if (num_offsets == 0) {
       memcpy(arena.map_state, &state, sizeof(state));
       arena.map_state_valid = true;
       return;
     }
+    MNT_CHECK(sizeof(unsigned) * 3 * num_offsets + 1024 <= Arena::kPinnedBytes,
+              "too many kernel offsets (%lld)", static_cast<long long>(num_offsets));
     if (num_targets == 0 || num_sources == 0) {
       if (num_targets > 0) {
         MNT_CHECK(kernel_map_out != nullptr, "kernel_map_out is null");
@@ -658,19 +739,20 @@ extern "C" int mnt_kernel_map_query(const void *sources, int64_t num_sources, co
     } else {
       MNT_CHECK(kernel_map_out != nullptr, "kernel_map_out is null");
       Scope scope(stream);
-      run_query(a, offsets_host, num_offsets, kernel_map_out, MNT_INT32, tile_counts, scope, stream);
+      run_query(a, offsets_host, num_offsets, source_bounds_host, target_bounds_host, bounds_host_out,
+                kernel_map_out, MNT_INT32, tile_counts, scope, stream);
     }
-    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes);
+    // sizes + order, mirrored into pinned host memory (past the bounds slots)
+    unsigned *h_plan = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned()) + 1024);
+    unsigned *d_plan_host = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned_device()) + 1024);
+    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(
+        tile_counts, num_tiles, row_sizes, reorder, plan, d_plan_host, arena.tickets() + 1);
     check_launch("tile_scan_kernel");
-    order_kernel<<<1, 256, 0, stream>>>(row_sizes, static_cast<int>(num_offsets), reorder, plan);
-    check_launch("order_kernel");
-    std::vector<unsigned> host(3 * num_offsets);
-    MNT_HIP(hipMemcpyAsync(host.data(), plan, sizeof(unsigned) * 3 * num_offsets, hipMemcpyDeviceToHost, stream));
     MNT_HIP(hipStreamSynchronize(stream));
     profile_mark("map_sizes_order+sync", stream);
     for (int64_t j = 0; j < num_offsets; ++j) {
-      order_host_out[j] = host[j];
-      sizes_host_out[j] = host[2 * num_offsets + j];
+      order_host_out[j] = h_plan[j];
+      sizes_host_out[j] = h_plan[2 * num_offsets + j];
     }
     memcpy(arena.map_state, &state, sizeof(state));
     arena.map_state_valid = true;
@@ -698,16 +780,7 @@ extern "C" int mnt_kernel_map_emit(int32_t *source_masks_out, int32_t *target_ma
     enqueue_emit<int32_t>(static_cast<const int32_t *>(state.kernel_map), state.num_sources,
                           state.num_targets, no, tile_bases, state.num_tiles, plan + no,
                           plan + 3 * no, source_masks_out, target_masks_out, in_idx_out, out_idx_out,
-                          stream);
+                          stream, plan, sizes_dev_out, order_dev_out);
     profile_mark("map_emit", stream);
-    const unsigned grid = grid_for(no, 256);
-    if (sizes_dev_out) {
-      export_sizes_kernel<int32_t><<<grid, 256, 0, stream>>>(plan + 2 * no, no, sizes_dev_out);
-      check_launch("export_sizes_kernel");
-    }
-    if (order_dev_out) {
-      export_sizes_kernel<int32_t><<<grid, 256, 0, stream>>>(plan, no, order_dev_out);
-      check_launch("export_sizes_kernel");
-    }
   });
 }

@@ -100,8 +100,24 @@ size_t Arena::used() const {
 }
 
 void *Arena::pinned() {
-  if (!pinned_) MNT_HIP(hipHostMalloc(&pinned_, kPinnedBytes, hipHostMallocDefault));
+  if (!pinned_) {
+    MNT_HIP(hipHostMalloc(&pinned_, kPinnedBytes, hipHostMallocDefault));
+    MNT_HIP(hipHostGetDevicePointer(&pinned_device_, pinned_, 0));
+  }
   return pinned_;
+}
+
+void *Arena::pinned_device() {
+  pinned();
+  return pinned_device_;
+}
+
+unsigned *Arena::tickets() {
+  if (!tickets_) {
+    MNT_HIP(hipMalloc(reinterpret_cast<void **>(&tickets_), 16 * sizeof(unsigned)));
+    MNT_HIP(hipMemset(tickets_, 0, 16 * sizeof(unsigned)));
+  }
+  return tickets_;
 }
 
 void *Arena::persistent(int slot, size_t bytes) {

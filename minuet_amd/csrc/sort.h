@@ -5,11 +5,16 @@
 
 namespace mnt {
 
-// Per-dimension min (slots 0..3) and max (slots 4..7) of coords[n, ndim] into
-// d_bounds (8 x int64, device).  With init the slots are reset first; without
-// it the call folds into what is already there.
-void enqueue_bounds(const void *coords, int64_t n, int ndim, int coord_dtype, long long *d_bounds,
-                    bool init, hipStream_t stream);
+// Per-dimension min / max of coords a[na, ndim] and (optionally) b[nb, ndim]:
+// out[0..3] = min of a, out[4..7] = max of a, out[8..15] the same for b
+// (INT64_MAX / INT64_MIN for an empty array).  One launch, then a stream
+// synchronisation; the kernel writes its result into pinned host memory.
+void read_bounds(const void *a, int64_t na, const void *b, int64_t nb, int ndim, int coord_dtype,
+                 long long out[16], Scope &scope, hipStream_t stream);
+
+// Copies a small host int array to device memory as arguments of a tiny copy
+// kernel: no staging buffer to protect, no synchronisation.
+void upload_ints(const std::vector<int> &host, int *dst, hipStream_t stream);
 
 // In-place exclusive prefix sum of `total` 32-bit counters (one workgroup).
 void enqueue_exclusive_scan(unsigned *data, int64_t total, hipStream_t stream);

@@ -6,30 +6,40 @@
 // lexicographic with dimension 0 most significant, batch-major.
 #include "sort.h"
 
+#include <algorithm>
+#include <vector>
+
 #include "device_utils.h"
 
 namespace mnt {
 
 // ----------------------------------------------------------------- bounds ----
 
-__global__ void bounds_init_kernel(long long *bounds) {
-  int t = threadIdx.x;
-  if (t < MNT_MAX_NDIM) bounds[t] = INT64_MAX;
-  if (t >= MNT_MAX_NDIM && t < 2 * MNT_MAX_NDIM) bounds[t] = INT64_MIN;
-}
+constexpr int kBoundsBlock = 256;
+constexpr int kBoundsMaxBlocks = 256;
 
+// Per-dimension min / max of up to two coordinate arrays in ONE launch with no
+// pre-initialised memory: every workgroup publishes its partial result, the
+// last one to finish (self-resetting ticket) folds all partials and writes
+// the 16 results straight into pinned host memory:
+//   out[0..3] = min of a, out[4..7] = max of a, out[8..11] / out[12..15] = b.
 template <typename CT>
-__global__ __launch_bounds__(256) void bounds_kernel(const CT *__restrict__ coords, long long n,
-                                                     int ndim, long long *bounds) {
+__global__ __launch_bounds__(kBoundsBlock) void bounds_kernel(
+    const CT *__restrict__ a, long long na, int blocks_a, const CT *__restrict__ b, long long nb,
+    int ndim, long long *partial, unsigned *ticket, long long *out) {
+  const bool second = static_cast<int>(blockIdx.x) >= blocks_a;
+  const CT *coords = second ? b : a;
+  const long long n = second ? nb : na;
+  const int my_block = second ? blockIdx.x - blocks_a : blockIdx.x;
+  const int my_blocks = second ? gridDim.x - blocks_a : blocks_a;
   long long lo[MNT_MAX_NDIM], hi[MNT_MAX_NDIM];
 #pragma unroll
   for (int k = 0; k < MNT_MAX_NDIM; ++k) {
     lo[k] = INT64_MAX;
     hi[k] = INT64_MIN;
   }
-  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
-  for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
-       i += stride) {
+  const long long stride = static_cast<long long>(my_blocks) * kBoundsBlock;
+  for (long long i = static_cast<long long>(my_block) * kBoundsBlock + threadIdx.x; i < n; i += stride) {
 #pragma unroll
     for (int k = 0; k < MNT_MAX_NDIM; ++k) {
       if (k < ndim) {
@@ -39,14 +49,15 @@ __global__ __launch_bounds__(256) void bounds_kernel(const CT *__restrict__ coor
       }
     }
   }
-  __shared__ long long s_lo[4][MNT_MAX_NDIM], s_hi[4][MNT_MAX_NDIM];
+  __shared__ long long s_lo[kBoundsBlock / kWave][MNT_MAX_NDIM], s_hi[kBoundsBlock / kWave][MNT_MAX_NDIM];
+  __shared__ bool s_last;
 #pragma unroll
   for (int k = 0; k < MNT_MAX_NDIM; ++k) {
     for (int off = 32; off > 0; off >>= 1) {
-      long long a = __shfl_down(lo[k], off);
-      long long b = __shfl_down(hi[k], off);
-      lo[k] = a < lo[k] ? a : lo[k];
-      hi[k] = b > hi[k] ? b : hi[k];
+      long long x = __shfl_down(lo[k], off);
+      long long y = __shfl_down(hi[k], off);
+      lo[k] = x < lo[k] ? x : lo[k];
+      hi[k] = y > hi[k] ? y : hi[k];
     }
   }
   const int w = threadIdx.x >> 6;
@@ -58,34 +69,121 @@ __global__ __launch_bounds__(256) void bounds_kernel(const CT *__restrict__ coor
     }
   }
   __syncthreads();
-  if (threadIdx.x < ndim) {
-    int k = threadIdx.x;
-    long long a = s_lo[0][k], b = s_hi[0][k];
-    for (int ww = 1; ww < 4; ++ww) {
-      a = s_lo[ww][k] < a ? s_lo[ww][k] : a;
-      b = s_hi[ww][k] > b ? s_hi[ww][k] : b;
+  if (threadIdx.x < 2 * MNT_MAX_NDIM) {
+    const int k = threadIdx.x & (MNT_MAX_NDIM - 1);
+    const bool is_max = threadIdx.x >= MNT_MAX_NDIM;
+    long long v = is_max ? s_hi[0][k] : s_lo[0][k];
+    for (int ww = 1; ww < kBoundsBlock / kWave; ++ww) {
+      long long u = is_max ? s_hi[ww][k] : s_lo[ww][k];
+      v = is_max ? (u > v ? u : v) : (u < v ? u : v);
     }
-    atomicMin(&bounds[k], a);
-    atomicMax(&bounds[MNT_MAX_NDIM + k], b);
+    __hip_atomic_store(&partial[static_cast<long long>(blockIdx.x) * 8 + threadIdx.x], v,
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __threadfence();
+  __syncthreads();
+  if (threadIdx.x == 0) s_last = atomicInc(ticket, gridDim.x - 1) == gridDim.x - 1;
+  __syncthreads();
+  if (!s_last) return;
+  __threadfence();
+  // fold the partials: thread t takes workgroups t, t+256, ... of each array
+  long long fa[8], fb[8];
+#pragma unroll
+  for (int slot = 0; slot < 8; ++slot) {
+    fa[slot] = slot >= MNT_MAX_NDIM ? INT64_MIN : INT64_MAX;
+    fb[slot] = fa[slot];
+  }
+  for (int blk = threadIdx.x; blk < static_cast<int>(gridDim.x); blk += kBoundsBlock) {
+    const bool of_b = blk >= blocks_a;
+#pragma unroll
+    for (int slot = 0; slot < 8; ++slot) {
+      const long long u = __hip_atomic_load(&partial[static_cast<long long>(blk) * 8 + slot],
+                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      long long &dst = of_b ? fb[slot] : fa[slot];
+      dst = slot >= MNT_MAX_NDIM ? (u > dst ? u : dst) : (u < dst ? u : dst);
+    }
+  }
+  __shared__ long long s_fold[kBoundsBlock / kWave][16];
+#pragma unroll
+  for (int slot = 0; slot < 8; ++slot) {
+    for (int off = 32; off > 0; off >>= 1) {
+      const long long x = __shfl_down(fa[slot], off);
+      const long long y = __shfl_down(fb[slot], off);
+      if (slot >= MNT_MAX_NDIM) {
+        fa[slot] = x > fa[slot] ? x : fa[slot];
+        fb[slot] = y > fb[slot] ? y : fb[slot];
+      } else {
+        fa[slot] = x < fa[slot] ? x : fa[slot];
+        fb[slot] = y < fb[slot] ? y : fb[slot];
+      }
+    }
+  }
+  if (lane_id() == 0) {
+#pragma unroll
+    for (int slot = 0; slot < 8; ++slot) {
+      s_fold[w][slot] = fa[slot];
+      s_fold[w][8 + slot] = fb[slot];
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < 16) {
+    const bool is_max = (threadIdx.x & 7) >= MNT_MAX_NDIM;
+    long long v = s_fold[0][threadIdx.x];
+    for (int ww = 1; ww < kBoundsBlock / kWave; ++ww) {
+      const long long u = s_fold[ww][threadIdx.x];
+      v = is_max ? (u > v ? u : v) : (u < v ? u : v);
+    }
+    out[threadIdx.x] = v;
   }
 }
 
-void enqueue_bounds(const void *coords, int64_t n, int ndim, int coord_dtype, long long *d_bounds,
-                    bool init, hipStream_t stream) {
-  if (init) {
-    bounds_init_kernel<<<1, 64, 0, stream>>>(d_bounds);
-    check_launch("bounds_init_kernel");
-  }
-  if (n == 0) return;
-  unsigned grid = grid_for(n, 256 * 4, 1024);
+void read_bounds(const void *a, int64_t na, const void *b, int64_t nb, int ndim, int coord_dtype,
+                 long long out[16], Scope &scope, hipStream_t stream) {
+  for (int i = 0; i < 16; ++i) out[i] = (i & 4) ? INT64_MIN : INT64_MAX;
+  if (na <= 0 && nb <= 0) return;
+  const int blocks_a = na > 0 ? static_cast<int>(std::min<int64_t>(div_ceil(na, kBoundsBlock * 4), kBoundsMaxBlocks)) : 0;
+  const int blocks_b = nb > 0 ? static_cast<int>(std::min<int64_t>(div_ceil(nb, kBoundsBlock * 4), kBoundsMaxBlocks)) : 0;
+  const int grid = blocks_a + blocks_b;
+  long long *partial = scope.alloc<long long>(static_cast<size_t>(grid) * 8);
+  unsigned *ticket = scope.arena().tickets();
+  long long *h_out = static_cast<long long *>(scope.arena().pinned());
+  long long *d_out = static_cast<long long *>(scope.arena().pinned_device());
   if (coord_dtype == MNT_INT32) {
-    bounds_kernel<int32_t><<<grid, 256, 0, stream>>>(static_cast<const int32_t *>(coords), n,
-                                                      ndim, d_bounds);
+    bounds_kernel<int32_t><<<grid, kBoundsBlock, 0, stream>>>(
+        static_cast<const int32_t *>(a), na, blocks_a, static_cast<const int32_t *>(b), nb, ndim,
+        partial, ticket, d_out);
   } else {
-    bounds_kernel<int64_t><<<grid, 256, 0, stream>>>(static_cast<const int64_t *>(coords), n,
-                                                      ndim, d_bounds);
+    bounds_kernel<int64_t><<<grid, kBoundsBlock, 0, stream>>>(
+        static_cast<const int64_t *>(a), na, blocks_a, static_cast<const int64_t *>(b), nb, ndim,
+        partial, ticket, d_out);
   }
   check_launch("bounds_kernel");
+  MNT_HIP(hipStreamSynchronize(stream));
+  if (na > 0) memcpy(out, h_out, sizeof(long long) * 8);
+  if (nb > 0) memcpy(out + 8, h_out + 8, sizeof(long long) * 8);
+}
+
+// ------------------------------------------- small uploads through kernargs ----
+
+constexpr int kUploadInts = 512;
+struct IntChunk {
+  int v[kUploadInts];
+};
+
+__global__ __launch_bounds__(256) void upload_ints_kernel(IntChunk chunk, int count, int *__restrict__ dst) {
+  for (int i = threadIdx.x; i < count; i += blockDim.x) dst[i] = chunk.v[i];
+}
+
+// Copies a small host int array to device memory as kernel arguments: no
+// staging buffer to protect, no synchronisation, safe under stream capture.
+void upload_ints(const std::vector<int> &host, int *dst, hipStream_t stream) {
+  for (size_t base = 0; base < host.size(); base += kUploadInts) {
+    IntChunk chunk;
+    const int count = static_cast<int>(std::min<size_t>(kUploadInts, host.size() - base));
+    memcpy(chunk.v, host.data() + base, sizeof(int) * count);
+    upload_ints_kernel<<<1, 256, 0, stream>>>(chunk, count, dst + base);
+    check_launch("upload_ints_kernel");
+  }
 }
 
 // ------------------------------------------------------------------ pack ----
@@ -185,6 +283,44 @@ void enqueue_exclusive_scan(unsigned *data, int64_t total, hipStream_t stream) {
   check_launch("scan_counts_kernel");
 }
 
+// Per-digit exclusive prefix over the tiles (one workgroup per digit, counts
+// are digit-major) plus the digit totals; the scatter kernel turns the totals
+// into digit bases itself.
+__global__ __launch_bounds__(kSortBlock) void digit_scan_kernel(unsigned *__restrict__ counts,
+                                                                int num_tiles,
+                                                                unsigned *__restrict__ totals) {
+  __shared__ unsigned wave_sums[kSortBlock / kWave];
+  __shared__ unsigned carry_s;
+  unsigned *row = counts + static_cast<long long>(blockIdx.x) * num_tiles;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int w = tid >> 6;
+  if (tid == 0) carry_s = 0;
+  __syncthreads();
+  for (int base = 0; base < num_tiles; base += kSortBlock) {
+    const int i = base + tid;
+    const unsigned v = i < num_tiles ? row[i] : 0u;
+    unsigned inc = v;
+    for (int off = 1; off < kWave; off <<= 1) {
+      unsigned u = __shfl_up(inc, off);
+      if (lane >= off) inc += u;
+    }
+    if (lane == kWave - 1) wave_sums[w] = inc;
+    __syncthreads();
+    unsigned before = carry_s;
+    unsigned all = 0;
+    for (int ww = 0; ww < kSortBlock / kWave; ++ww) {
+      if (ww < w) before += wave_sums[ww];
+      all += wave_sums[ww];
+    }
+    if (i < num_tiles) row[i] = before + inc - v;
+    __syncthreads();
+    if (tid == 0) carry_s += all;
+    __syncthreads();
+  }
+  if (tid == 0) totals[blockIdx.x] = carry_s;
+}
+
 // Stable scatter of one tile.  Wave w owns the contiguous slice
 // [w*64*ITEMS, (w+1)*64*ITEMS) of the tile and walks it 64 items at a time, so
 // (wave, round, lane) order equals input order; ranks within a digit follow it.
@@ -192,9 +328,11 @@ template <int ITEMS>
 __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     const unsigned long long *__restrict__ keys_in, const unsigned *__restrict__ vals_in,
     unsigned long long *__restrict__ keys_out, unsigned *__restrict__ vals_out, long long n,
-    int shift, const unsigned *__restrict__ offsets, int num_tiles) {
+    int shift, const unsigned *__restrict__ offsets, const unsigned *__restrict__ totals,
+    int num_tiles) {
   constexpr int kWaves = kSortBlock / kWave;
   __shared__ volatile unsigned cnt[kWaves][kRadix];
+  __shared__ unsigned digit_wave_sums[kWaves];
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int w = tid >> 6;
@@ -228,9 +366,19 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     if (valid && below == 0) cnt[w][d] = prev + __popcll(peers);
     __builtin_amdgcn_wave_barrier();
   }
+  // digit bases: exclusive scan of the 256 digit totals (thread d <-> digit d)
+  const unsigned total_d = totals[tid];
+  unsigned inc_d = total_d;
+  for (int off = 1; off < kWave; off <<= 1) {
+    unsigned u = __shfl_up(inc_d, off);
+    if (lane >= off) inc_d += u;
+  }
+  if (lane == kWave - 1) digit_wave_sums[w] = inc_d;
   __syncthreads();
   {
-    unsigned run = offsets[static_cast<long long>(tid) * num_tiles + blockIdx.x];
+    unsigned run = inc_d - total_d;
+    for (int ww = 0; ww < w; ++ww) run += digit_wave_sums[ww];
+    run += offsets[static_cast<long long>(tid) * num_tiles + blockIdx.x];
 #pragma unroll
     for (int ww = 0; ww < kWaves; ++ww) {
       unsigned c = cnt[ww][tid];
@@ -261,10 +409,11 @@ static void radix_sort_impl(unsigned long long *&keys, unsigned *&vals, unsigned
     const int shift = p * kRadixBits;
     radix_hist_kernel<ITEMS><<<num_tiles, kSortBlock, 0, stream>>>(keys, n, shift, counts, num_tiles);
     check_launch("radix_hist_kernel");
-    scan_counts_kernel<<<1, 1024, 0, stream>>>(counts, static_cast<long long>(kRadix) * num_tiles);
-    check_launch("scan_counts_kernel");
-    radix_scatter_kernel<ITEMS><<<num_tiles, kSortBlock, 0, stream>>>(keys, vals, keys_alt, vals_alt,
-                                                                       n, shift, counts, num_tiles);
+    unsigned *totals = counts + static_cast<long long>(kRadix) * num_tiles;
+    digit_scan_kernel<<<kRadix, kSortBlock, 0, stream>>>(counts, num_tiles, totals);
+    check_launch("digit_scan_kernel");
+    radix_scatter_kernel<ITEMS><<<num_tiles, kSortBlock, 0, stream>>>(
+        keys, vals, keys_alt, vals_alt, n, shift, counts, totals, num_tiles);
     check_launch("radix_scatter_kernel");
     std::swap(keys, keys_alt);
     std::swap(vals, vals_alt);
@@ -273,7 +422,7 @@ static void radix_sort_impl(unsigned long long *&keys, unsigned *&vals, unsigned
 
 size_t radix_counts_len(int64_t n) {
   int items = n <= (int64_t(1) << 20) ? 4 : 16;
-  return static_cast<size_t>(kRadix) * static_cast<size_t>(div_ceil(n, kSortBlock * items));
+  return static_cast<size_t>(kRadix) * static_cast<size_t>(div_ceil(n, kSortBlock * items)) + kRadix;
 }
 
 void radix_sort_pairs(unsigned long long *&keys, unsigned *&vals, unsigned long long *&keys_alt,
@@ -313,17 +462,14 @@ static int bit_width(unsigned long long range) {
 template <typename CT, typename IT>
 static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batch_dims,
                            int64_t num_batches, IT *indices_out, CT *sorted_out,
-                           hipStream_t stream) {
+                           int64_t *bounds_host_out, hipStream_t stream) {
   Scope scope(stream);
   const bool batched = batch_dims != nullptr && num_batches > 1;
 
   profile_mark("enter:arg_sort", stream);
-  long long *d_bounds = scope.alloc<long long>(2 * MNT_MAX_NDIM);
-  enqueue_bounds(coords, n, ndim, sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64, d_bounds, true, stream);
-  long long *h_bounds = static_cast<long long *>(scope.arena().pinned());
-  MNT_HIP(hipMemcpyAsync(h_bounds, d_bounds, sizeof(long long) * 2 * MNT_MAX_NDIM,
-                         hipMemcpyDeviceToHost, stream));
-  MNT_HIP(hipStreamSynchronize(stream));
+  long long h_bounds[16];
+  read_bounds(coords, n, nullptr, 0, ndim, sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64, h_bounds, scope, stream);
+  if (bounds_host_out != nullptr) memcpy(bounds_host_out, h_bounds, sizeof(long long) * 8);
   profile_mark("sort_bounds+sync", stream);
 
   // fields from least to most significant: dims ndim-1 .. 0, then the batch id
@@ -389,7 +535,8 @@ using namespace mnt;
 extern "C" int mnt_arg_sort_coordinates(const void *coords, int64_t n, int ndim, int coord_dtype,
                                         const void *batch_dims, int64_t num_batches,
                                         int index_dtype, void *indices_out,
-                                        void *sorted_coords_out, void *stream_) {
+                                        void *sorted_coords_out, int64_t *bounds_host_out,
+                                        void *stream_) {
   return guarded([&] {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MNT_CHECK(ndim >= 1 && ndim <= MNT_MAX_NDIM, "ndim must be in [1, %d] but found %d",
@@ -398,6 +545,9 @@ extern "C" int mnt_arg_sort_coordinates(const void *coords, int64_t n, int ndim,
               static_cast<long long>(n));
     int_size(coord_dtype);
     int_size(index_dtype);
+    if (bounds_host_out != nullptr) {
+      for (int i = 0; i < 8; ++i) bounds_host_out[i] = (i & 4) ? INT64_MIN : INT64_MAX;
+    }
     if (n == 0) return;
     MNT_CHECK(coords != nullptr, "coords is null");
     if (batch_dims == nullptr) num_batches = 1;
@@ -405,7 +555,7 @@ extern "C" int mnt_arg_sort_coordinates(const void *coords, int64_t n, int ndim,
   arg_sort_typed<CT, IT>(static_cast<const CT *>(coords), n, ndim,                            \
                          static_cast<const IT *>(batch_dims), num_batches,                    \
                          static_cast<IT *>(indices_out), static_cast<CT *>(sorted_coords_out), \
-                         stream)
+                         bounds_host_out, stream)
     if (coord_dtype == MNT_INT32 && index_dtype == MNT_INT32) {
       MNT_CASE(int32_t, int32_t);
     } else if (coord_dtype == MNT_INT32) {

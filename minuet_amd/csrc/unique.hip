@@ -250,12 +250,8 @@ static void target_count_typed(const CT *coords, int64_t n, int ndim, const int6
   memset(&spec, 0, sizeof(spec));
   {
     Scope scope(stream);
-    long long *d_bounds = scope.alloc<long long>(2 * MNT_MAX_NDIM);
-    enqueue_bounds(coords, n, ndim, sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64, d_bounds, true, stream);
-    long long *h_bounds = static_cast<long long *>(arena.pinned());
-    MNT_HIP(hipMemcpyAsync(h_bounds, d_bounds, sizeof(long long) * 2 * MNT_MAX_NDIM,
-                           hipMemcpyDeviceToHost, stream));
-    MNT_HIP(hipStreamSynchronize(stream));
+    long long h_bounds[16];
+    read_bounds(coords, n, nullptr, 0, ndim, sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64, h_bounds, scope, stream);
     int bits = 0;
     spec.ndim = ndim;
     for (int k = ndim - 1; k >= 0; --k) {

@@ -45,6 +45,7 @@ class KernelMapCache(object):
         self._disable_reordering = disable_reordering
         self._kernel_maps_cache = dict()
         self._coordinates_cache = dict()
+        self._bounds_cache = dict()
         self.num_map_builds = 0
         self.num_coordinate_builds = 0
 
@@ -58,6 +59,15 @@ class KernelMapCache(object):
     def reset(self):
         self._coordinates_cache.clear()
         self._kernel_maps_cache.clear()
+        self._bounds_cache.clear()
+
+    def _known_bounds(self, coordinates: torch.Tensor):
+        """Host copy of the per-dimension min / max of a coordinate tensor seen
+        before (keyed by its storage), or None."""
+        return self._bounds_cache.get((coordinates.data_ptr(), coordinates.shape[0]))
+
+    def _remember_bounds(self, coordinates: torch.Tensor, bounds: np.ndarray):
+        self._bounds_cache[(coordinates.data_ptr(), coordinates.shape[0])] = np.array(bounds, dtype=np.int64)
 
     def get_target_coordinates(self, source_coordinates: torch.Tensor,
                                source_batch_dims: Optional[torch.Tensor],
@@ -79,6 +89,14 @@ class KernelMapCache(object):
         coords, batch_dims = _C.target_coordinates(source_coordinates.contiguous(),
                                                    source_batch_dims, target_stride)
         self.num_coordinate_builds += 1
+        known = self._known_bounds(source_coordinates)
+        if known is not None and source_coordinates.shape[0] > 0:
+            # floor(c / s) * s is monotone, so the extremes map to the extremes
+            ts = np.asarray(target_stride, dtype=np.int64)
+            derived = known.copy()
+            derived[:ndim] = np.floor_divide(known[:ndim], ts) * ts
+            derived[4:4 + ndim] = np.floor_divide(known[4:4 + ndim], ts) * ts
+            self._remember_bounds(coords, derived)
         entry = (coords, target_stride, batch_dims)
         self._coordinates_cache[target_stride] = entry
         return entry
@@ -108,10 +126,16 @@ class KernelMapCache(object):
 
         offsets = self._kernel_offsets(source_stride, kernel_size, kernel_dilation)
         reorder = not self._disable_reordering and not disable_reordering
-        built = _C.kernel_map_build(source_coordinates.contiguous(),
-                                    target_coordinates.contiguous(), offsets,
-                                    source_batch_dims, target_batch_dims, reorder=reorder)
+        source_coordinates = source_coordinates.contiguous()
+        target_coordinates = target_coordinates.contiguous()
+        built = _C.kernel_map_build(source_coordinates, target_coordinates, offsets,
+                                    source_batch_dims, target_batch_dims, reorder=reorder,
+                                    source_bounds=self._known_bounds(source_coordinates),
+                                    target_bounds=self._known_bounds(target_coordinates))
         self.num_map_builds += 1
+        if source_coordinates.shape[0] > 0 and target_coordinates.shape[0] > 0:
+            self._remember_bounds(source_coordinates, built["bounds"][:8])
+            self._remember_bounds(target_coordinates, built["bounds"][8:])
         index_dtype = (source_coordinates.dtype if source_batch_dims is None
                        else source_batch_dims.dtype)
         cast = (lambda t: t) if index_dtype == torch.int32 else (lambda t: t.to(index_dtype))

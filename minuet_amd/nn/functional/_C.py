@@ -41,7 +41,7 @@ SIGNATURES = {
     "mnt_buffer_total_size": (_sz, [_vp]),
     "mnt_buffer_used_size": (_sz, [_vp]),
     "mnt_reset_error": (_int, []),
-    "mnt_arg_sort_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _vp, _vp]),
+    "mnt_arg_sort_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _vp, _pi64, _vp]),
     "mnt_unique_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _pi64, _vp]),
     "mnt_fill_unique_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _int, _vp, _vp]),
     "mnt_target_coordinates_count": (_int, [_vp, _i64, _int, _int, _pi64, _vp, _i64, _int, _pi64, _vp]),
@@ -51,7 +51,7 @@ SIGNATURES = {
     "mnt_compute_kernel_map_sizes": (_int, [_vp, _i64, _i64, _int, _vp, _vp]),
     "mnt_compute_kernel_map_masks": (_int, [_vp, _i64, _i64, _i64, _int, _vp, _vp, _vp]),
     "mnt_kernel_map_query": (_int, [_vp, _i64, _vp, _i64, _pi64, _i64, _int, _int, _vp, _vp, _i64,
-                                    _int, _int, _vp, _pi64, _pi64, _vp]),
+                                    _int, _int, _pi64, _pi64, _pi64, _vp, _pi64, _pi64, _vp]),
     "mnt_kernel_map_emit": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "mnt_kernel_map_pair_lists": (_int, [_vp, _i64, _i64, _pi64, _vp, _vp, _vp]),
     "mnt_generate_padding_buckets": (_int, [_pi64, _i64, _int, _dbl, _pi64, _pi64]),
@@ -172,7 +172,7 @@ def cuda_arg_sort_coordinates(coordinates: torch.Tensor, enable_flattening: bool
     indices = torch.empty((n,), dtype=itype, device=device)
     with torch.cuda.device(device):
         _check(load_library().mnt_arg_sort_coordinates(
-            _ptr(coordinates), n, ndim, ccode, None, 1, _INT[itype], _ptr(indices), None,
+            _ptr(coordinates), n, ndim, ccode, None, 1, _INT[itype], _ptr(indices), None, None,
             _stream(device)))
     return indices
 
@@ -191,13 +191,16 @@ def cuda_multi_arg_sort_coordinates(coordinates: torch.Tensor, batch_dims: torch
     with torch.cuda.device(device):
         _check(load_library().mnt_arg_sort_coordinates(
             _ptr(coordinates), n, ndim, ccode, _ptr(batch_dims), batch_dims.numel() - 1, icode,
-            _ptr(indices), None, _stream(device)))
+            _ptr(indices), None, None, _stream(device)))
     return indices
 
 
-def sort_coordinates(coordinates: torch.Tensor, batch_dims: Optional[torch.Tensor] = None
-                     ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Arg-sort and the sorted rows in one library call (int32 indices)."""
+def sort_coordinates(coordinates: torch.Tensor, batch_dims: Optional[torch.Tensor] = None,
+                     return_bounds: bool = False):
+    """Arg-sort and the sorted rows in one library call (int32 indices unless
+    ``batch_dims`` says otherwise).  With ``return_bounds`` a third result holds
+    the per-dimension coordinate minima [0..3] and maxima [4..7] (numpy int64),
+    which ``kernel_map_build`` accepts to skip its own reduction."""
     _ensure_ndim("coordinates", coordinates, 2)
     device = _common_device([coordinates] + ([batch_dims] if batch_dims is not None else []))
     n, ndim = coordinates.shape
@@ -205,11 +208,14 @@ def sort_coordinates(coordinates: torch.Tensor, batch_dims: Optional[torch.Tenso
     itype = batch_dims.dtype if batch_dims is not None else torch.int32
     indices = torch.empty((n,), dtype=itype, device=device)
     out = torch.empty_like(coordinates)
+    bounds = np.zeros(8, dtype=np.int64)
     with torch.cuda.device(device):
         _check(load_library().mnt_arg_sort_coordinates(
             _ptr(coordinates), n, ndim, ccode, _ptr(batch_dims),
             batch_dims.numel() - 1 if batch_dims is not None else 1, _INT[itype], _ptr(indices),
-            _ptr(out), _stream(device)))
+            _ptr(out), bounds.ctypes.data_as(_pi64), _stream(device)))
+    if return_bounds:
+        return indices, out, bounds
     return indices, out
 
 
@@ -371,12 +377,14 @@ def kernel_map_build(sources: torch.Tensor, targets: torch.Tensor, offsets_host:
                      source_batch_dims: Optional[torch.Tensor],
                      target_batch_dims: Optional[torch.Tensor], reorder: bool,
                      want_masks: bool = True, want_lists: bool = False,
-                     want_dense: bool = False):
+                     want_dense: bool = False, source_bounds=None, target_bounds=None):
     """Fused kernel-map build: query + sizes + stable size order + rank tables
     and/or per-offset pair lists.  Returns a dict with ``sizes_host``,
-    ``order_host`` (numpy int64), ``sizes``/``order`` (int32 device) and the
-    requested tensors (``source_masks``, ``target_masks``, ``in_idx``,
-    ``out_idx``, ``kernel_map``)."""
+    ``order_host`` (numpy int64), ``sizes``/``order`` (int32 device), ``bounds``
+    (numpy int64 [16]: coordinate minima / maxima of sources then targets) and
+    the requested tensors (``source_masks``, ``target_masks``, ``in_idx``,
+    ``out_idx``, ``kernel_map``).  ``source_bounds`` / ``target_bounds`` (8
+    int64 each) skip the device-side bounds reduction when already known."""
     _ensure_ndim("sources", sources, 2)
     _ensure_ndim("targets", targets, 2)
     ndim = sources.size(1)
@@ -399,6 +407,9 @@ def kernel_map_build(sources: torch.Tensor, targets: torch.Tensor, offsets_host:
     dense = torch.empty((num_offsets, num_targets), dtype=torch.int32, device=device)
     sizes_host = np.zeros(num_offsets, dtype=np.int64)
     order_host = np.zeros(num_offsets, dtype=np.int64)
+    bounds = np.zeros(16, dtype=np.int64)
+    sb = None if source_bounds is None else np.ascontiguousarray(source_bounds, dtype=np.int64)
+    tb = None if target_bounds is None else np.ascontiguousarray(target_bounds, dtype=np.int64)
     lib = load_library()
     result = {}
     with torch.cuda.device(device):
@@ -408,8 +419,11 @@ def kernel_map_build(sources: torch.Tensor, targets: torch.Tensor, offsets_host:
             offs.ctypes.data_as(_pi64), num_offsets, ndim, ccode, _ptr(source_batch_dims),
             _ptr(target_batch_dims),
             source_batch_dims.numel() - 1 if source_batch_dims is not None else 1, bcode,
-            1 if reorder else 0, _ptr(dense), sizes_host.ctypes.data_as(_pi64),
-            order_host.ctypes.data_as(_pi64), stream))
+            1 if reorder else 0,
+            None if sb is None else sb.ctypes.data_as(_pi64),
+            None if tb is None else tb.ctypes.data_as(_pi64), bounds.ctypes.data_as(_pi64),
+            _ptr(dense), sizes_host.ctypes.data_as(_pi64), order_host.ctypes.data_as(_pi64),
+            stream))
         smask = tmask = in_idx = out_idx = None
         if want_masks:
             smask = torch.empty((num_offsets, num_sources), dtype=torch.int32, device=device)
@@ -423,6 +437,7 @@ def kernel_map_build(sources: torch.Tensor, targets: torch.Tensor, offsets_host:
         _check(lib.mnt_kernel_map_emit(_ptr(smask), _ptr(tmask), _ptr(in_idx), _ptr(out_idx),
                                        _ptr(sizes_dev), _ptr(order_dev), stream))
     result.update(sizes_host=sizes_host, order_host=order_host, sizes=sizes_dev, order=order_dev,
+                  bounds=bounds,
                   source_masks=smask, target_masks=tmask, in_idx=in_idx, out_idx=out_idx)
     if want_dense:
         result["kernel_map"] = dense
