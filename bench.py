@@ -48,8 +48,8 @@ def cpu_baseline(coords, offsets, budget_s=12.0):
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=200)
-    parser.add_argument("--warmup", type=int, default=20)
+    parser.add_argument("--steps", type=int, default=1000)
+    parser.add_argument("--warmup", type=int, default=100)
     parser.add_argument("--scale", type=float, default=1.0, help="voxel-count scale of the workload")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = parser.parse_args()
@@ -74,7 +74,11 @@ def main():
     coords_dev = torch.from_numpy(coords).to(device)
     n = coords.shape[0]
 
-    for _ in range(args.warmup):
+    # bring the GPU out of its idle power state before anything is measured
+    spin_until = time.perf_counter() + 1.5
+    while time.perf_counter() < spin_until:
+        map_step(_C, coords_dev, offsets)
+    for _ in range(max(1, args.warmup)):
         sorted_dev, built = map_step(_C, coords_dev, offsets)
     torch.cuda.synchronize()
     nnz = int(built["sizes_host"].sum())

@@ -94,6 +94,18 @@ class Arena {
   // 16 zero-initialised device counters for "last workgroup" tickets; every
   // kernel that uses one leaves it at zero again.
   unsigned *tickets();
+
+  // Completion handshake through the pinned block: a kernel ends by storing a
+  // fresh sequence number into flag word `slot` (after its results, with a
+  // system-scope release); wait_flag spins on that word on the host, which
+  // is several times quicker than a stream synchronisation.  After two
+  // seconds it falls back to hipStreamSynchronize so that a failed kernel
+  // surfaces as an error instead of a hang.
+  static constexpr size_t kFlagOffset = 512;      // 8 words of 64 bytes each
+  static constexpr size_t kPlanOffset = 1024;     // mirrored sizes / order
+  unsigned long long next_sequence() { return ++sequence_; }
+  unsigned long long *flag_device(int slot);
+  void wait_flag(int slot, unsigned long long sequence);
   // Long-lived device blocks that survive scopes (state of the two-phase entry
   // points; slot 0: target coordinates, slot 1: kernel-map build).  Grows to
   // at least `bytes`; 0 returns the current block.
@@ -131,6 +143,7 @@ class Arena {
   void *pinned_ = nullptr;
   void *pinned_device_ = nullptr;
   unsigned *tickets_ = nullptr;
+  unsigned long long sequence_ = 0;
   void *persistent_[2] = {nullptr, nullptr};
   size_t persistent_size_[2] = {0, 0};
 };

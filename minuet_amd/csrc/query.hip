@@ -204,7 +204,8 @@ __global__ __launch_bounds__(256) void tile_scan_kernel(unsigned *__restrict__ t
                                                         int num_tiles, unsigned *row_sizes,
                                                         int reorder, unsigned *__restrict__ plan,
                                                         unsigned *__restrict__ plan_host,
-                                                        unsigned *ticket) {
+                                                        unsigned *ticket, unsigned long long *flag,
+                                                        unsigned long long sequence) {
   __shared__ unsigned partial[256];
   __shared__ bool s_last;
   unsigned *row = tile_counts + static_cast<long long>(blockIdx.x) * num_tiles;
@@ -270,6 +271,10 @@ __global__ __launch_bounds__(256) void tile_scan_kernel(unsigned *__restrict__ t
       total += sorted_sizes[j];
     }
     prefix[num_offsets] = total;
+    if (flag != nullptr) {
+      __threadfence_system();
+      __hip_atomic_store(flag, sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
   }
 }
 
@@ -623,7 +628,7 @@ extern "C" int mnt_compute_kernel_map_sizes(const void *kernel_map, int64_t num_
     unsigned *tile_counts = scope.alloc<unsigned>(static_cast<size_t>(num_offsets) * num_tiles);
     unsigned *row_sizes = scope.alloc<unsigned>(num_offsets);
     enqueue_count_tiles(kernel_map, index_dtype, num_offsets, num_targets, tile_counts, num_tiles, stream);
-    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes, 0, nullptr, nullptr, nullptr);
+    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes, 0, nullptr, nullptr, nullptr, nullptr, 0);
     check_launch("tile_scan_kernel");
     const unsigned grid = grid_for(num_offsets, 256);
     if (index_dtype == MNT_INT32) {
@@ -652,7 +657,7 @@ extern "C" int mnt_compute_kernel_map_masks(const void *kernel_map, int64_t num_
     unsigned *row_sizes = scope.alloc<unsigned>(num_offsets);
     if (num_targets > 0) {
       enqueue_count_tiles(kernel_map, index_dtype, num_offsets, num_targets, tile_counts, num_tiles, stream);
-      tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes, 0, nullptr, nullptr, nullptr);
+      tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes, 0, nullptr, nullptr, nullptr, nullptr, 0);
       check_launch("tile_scan_kernel");
     }
     if (index_dtype == MNT_INT32) {
@@ -687,7 +692,7 @@ extern "C" int mnt_kernel_map_pair_lists(const int32_t *kernel_map, int64_t num_
     for (int64_t o = 0; o <= num_offsets; ++o) base[o] = static_cast<unsigned>(cumsum_host[o]);
     MNT_HIP(hipMemcpyAsync(row_base, base.data(), sizeof(unsigned) * (num_offsets + 1), hipMemcpyHostToDevice, stream));
     enqueue_count_tiles(kernel_map, MNT_INT32, num_offsets, num_targets, tile_counts, num_tiles, stream);
-    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes, 0, nullptr, nullptr, nullptr);
+    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes, 0, nullptr, nullptr, nullptr, nullptr, 0);
     check_launch("tile_scan_kernel");
     enqueue_emit<int32_t>(kernel_map, 0, num_targets, static_cast<int>(num_offsets), tile_counts,
                           num_tiles, nullptr, row_base, nullptr, nullptr, in_idx_out, out_idx_out, stream);
@@ -743,12 +748,14 @@ extern "C" int mnt_kernel_map_query(const void *sources, int64_t num_sources, co
                 kernel_map_out, MNT_INT32, tile_counts, scope, stream);
     }
     // sizes + order, mirrored into pinned host memory (past the bounds slots)
-    unsigned *h_plan = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned()) + 1024);
-    unsigned *d_plan_host = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned_device()) + 1024);
+    unsigned *h_plan = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned()) + Arena::kPlanOffset);
+    unsigned *d_plan_host = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned_device()) + Arena::kPlanOffset);
+    const unsigned long long sequence = arena.next_sequence();
     tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(
-        tile_counts, num_tiles, row_sizes, reorder, plan, d_plan_host, arena.tickets() + 1);
+        tile_counts, num_tiles, row_sizes, reorder, plan, d_plan_host, arena.tickets() + 1,
+        arena.flag_device(1), sequence);
     check_launch("tile_scan_kernel");
-    MNT_HIP(hipStreamSynchronize(stream));
+    arena.wait_flag(1, sequence);
     profile_mark("map_sizes_order+sync", stream);
     for (int64_t j = 0; j < num_offsets; ++j) {
       order_host_out[j] = h_plan[j];

@@ -1,4 +1,6 @@
 // Library plumbing: last-error slot, per-stream scratch arena, buffer knobs.
+#include <atomic>
+#include <chrono>
 #include <map>
 #include <mutex>
 
@@ -101,7 +103,8 @@ size_t Arena::used() const {
 
 void *Arena::pinned() {
   if (!pinned_) {
-    MNT_HIP(hipHostMalloc(&pinned_, kPinnedBytes, hipHostMallocDefault));
+    MNT_HIP(hipHostMalloc(&pinned_, kPinnedBytes, hipHostMallocMapped | hipHostMallocCoherent));
+    memset(pinned_, 0, kPinnedBytes);
     MNT_HIP(hipHostGetDevicePointer(&pinned_device_, pinned_, 0));
   }
   return pinned_;
@@ -110,6 +113,30 @@ void *Arena::pinned() {
 void *Arena::pinned_device() {
   pinned();
   return pinned_device_;
+}
+
+unsigned long long *Arena::flag_device(int slot) {
+  return reinterpret_cast<unsigned long long *>(static_cast<char *>(pinned_device()) + kFlagOffset +
+                                                static_cast<size_t>(slot) * 64);
+}
+
+void Arena::wait_flag(int slot, unsigned long long sequence) {
+  volatile unsigned long long *flag = reinterpret_cast<volatile unsigned long long *>(
+      static_cast<char *>(pinned()) + kFlagOffset + static_cast<size_t>(slot) * 64);
+  const auto start = std::chrono::steady_clock::now();
+  unsigned spins = 0;
+  while (*flag != sequence) {
+    if ((++spins & 0x3FFFu) == 0) {
+      const auto waited = std::chrono::steady_clock::now() - start;
+      if (waited > std::chrono::seconds(2)) {
+        MNT_HIP(hipStreamSynchronize(stream_));
+        MNT_CHECK(*flag == sequence, "a kernel finished without signalling its completion flag");
+        break;
+      }
+    }
+    __builtin_ia32_pause();
+  }
+  std::atomic_thread_fence(std::memory_order_acquire);
 }
 
 unsigned *Arena::tickets() {

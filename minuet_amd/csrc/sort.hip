@@ -26,7 +26,8 @@ constexpr int kBoundsMaxBlocks = 256;
 template <typename CT>
 __global__ __launch_bounds__(kBoundsBlock) void bounds_kernel(
     const CT *__restrict__ a, long long na, int blocks_a, const CT *__restrict__ b, long long nb,
-    int ndim, long long *partial, unsigned *ticket, long long *out) {
+    int ndim, long long *partial, unsigned *ticket, long long *out, unsigned long long *flag,
+    unsigned long long sequence) {
   const bool second = static_cast<int>(blockIdx.x) >= blocks_a;
   const CT *coords = second ? b : a;
   const long long n = second ? nb : na;
@@ -135,6 +136,11 @@ __global__ __launch_bounds__(kBoundsBlock) void bounds_kernel(
     }
     out[threadIdx.x] = v;
   }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __threadfence_system();
+    __hip_atomic_store(flag, sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
 }
 
 void read_bounds(const void *a, int64_t na, const void *b, int64_t nb, int ndim, int coord_dtype,
@@ -148,17 +154,19 @@ void read_bounds(const void *a, int64_t na, const void *b, int64_t nb, int ndim,
   unsigned *ticket = scope.arena().tickets();
   long long *h_out = static_cast<long long *>(scope.arena().pinned());
   long long *d_out = static_cast<long long *>(scope.arena().pinned_device());
+  const unsigned long long sequence = scope.arena().next_sequence();
+  unsigned long long *flag = scope.arena().flag_device(0);
   if (coord_dtype == MNT_INT32) {
     bounds_kernel<int32_t><<<grid, kBoundsBlock, 0, stream>>>(
         static_cast<const int32_t *>(a), na, blocks_a, static_cast<const int32_t *>(b), nb, ndim,
-        partial, ticket, d_out);
+        partial, ticket, d_out, flag, sequence);
   } else {
     bounds_kernel<int64_t><<<grid, kBoundsBlock, 0, stream>>>(
         static_cast<const int64_t *>(a), na, blocks_a, static_cast<const int64_t *>(b), nb, ndim,
-        partial, ticket, d_out);
+        partial, ticket, d_out, flag, sequence);
   }
   check_launch("bounds_kernel");
-  MNT_HIP(hipStreamSynchronize(stream));
+  scope.arena().wait_flag(0, sequence);
   if (na > 0) memcpy(out, h_out, sizeof(long long) * 8);
   if (nb > 0) memcpy(out + 8, h_out + 8, sizeof(long long) * 8);
 }
@@ -186,7 +194,7 @@ void upload_ints(const std::vector<int> &host, int *dst, hipStream_t stream) {
   }
 }
 
-// ------------------------------------------------------------------ pack ----
+// ------------------------------------------------------------------ keys ----
 
 // One sort round packs a subset of the fields (dimensions, batch id) into a
 // 64-bit key.  Field ndim.. is unused; index MNT_MAX_NDIM is the batch id.
@@ -198,60 +206,110 @@ struct SortSpec {
   int num_batches;
 };
 
+// Pass input taken from key / value arrays of an earlier pass (vals may be
+// null for a keys-only sort).
+struct PlainSource {
+  const unsigned long long *keys;
+  const unsigned *vals;
+  __device__ __forceinline__ void load(long long i, unsigned long long &key, unsigned &val) const {
+    key = keys[i];
+    val = vals ? vals[i] : 0u;
+  }
+};
+
+// Pass input computed on the fly from the coordinate rows: the first pass of a
+// round never materialises its keys.  perm (nullable) is the order left by
+// the previous round.
 template <typename CT, typename IT>
-__global__ __launch_bounds__(256) void pack_keys_kernel(const CT *__restrict__ coords,
-                                                        long long n, SortSpec spec,
-                                                        const IT *__restrict__ batch_dims,
-                                                        const unsigned *__restrict__ perm_in,
-                                                        unsigned long long *__restrict__ keys,
-                                                        unsigned *__restrict__ vals) {
-  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
-  for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
-       i += stride) {
-    const long long row = perm_in ? static_cast<long long>(perm_in[i]) : i;
-    unsigned long long key = 0;
+struct CoordSource {
+  const CT *coords;
+  const IT *batch_dims;
+  const unsigned *perm;
+  SortSpec spec;
+  __device__ __forceinline__ void load(long long i, unsigned long long &key, unsigned &val) const {
+    const long long row = perm ? static_cast<long long>(perm[i]) : i;
+    unsigned long long k64 = 0;
 #pragma unroll
     for (int k = 0; k < MNT_MAX_NDIM; ++k) {
       if (k < spec.ndim && spec.mask[k]) {
         unsigned long long v =
             static_cast<unsigned long long>(static_cast<long long>(coords[row * spec.ndim + k])) -
             spec.lo[k];
-        key |= (v & spec.mask[k]) << spec.shift[k];
+        k64 |= (v & spec.mask[k]) << spec.shift[k];
       }
     }
     if (spec.mask[MNT_MAX_NDIM]) {
       unsigned long long b = batch_of<IT>(row, batch_dims, spec.num_batches);
-      key |= (b & spec.mask[MNT_MAX_NDIM]) << spec.shift[MNT_MAX_NDIM];
+      k64 |= (b & spec.mask[MNT_MAX_NDIM]) << spec.shift[MNT_MAX_NDIM];
     }
-    keys[i] = key;
-    vals[i] = static_cast<unsigned>(row);
+    key = k64;
+    val = static_cast<unsigned>(row);
   }
-}
+};
+
+// Pass output into key / value arrays for the next pass.
+struct PlainSink {
+  unsigned long long *keys;
+  unsigned *vals;
+  __device__ __forceinline__ void store(unsigned pos, unsigned long long key, unsigned val) const {
+    keys[pos] = key;
+    if (vals) vals[pos] = val;
+  }
+};
+
+// Output of the very last pass: the permutation and (optionally) the sorted
+// coordinate rows, so no separate gather pass is needed.
+template <typename CT, typename IT>
+struct FinalSink {
+  const CT *coords;
+  int ndim;
+  IT *indices;
+  CT *sorted;
+  __device__ __forceinline__ void store(unsigned pos, unsigned long long, unsigned val) const {
+    if (indices) indices[pos] = static_cast<IT>(val);
+    if (sorted) {
+      for (int k = 0; k < ndim; ++k) {
+        sorted[static_cast<long long>(pos) * ndim + k] = coords[static_cast<long long>(val) * ndim + k];
+      }
+    }
+  }
+};
 
 // ------------------------------------------------------------ radix sort ----
 
-constexpr int kRadixBits = 8;
-constexpr int kRadix = 1 << kRadixBits;
+constexpr int kMaxRadixBits = 11;
+constexpr int kMaxRadix = 1 << kMaxRadixBits;
 constexpr int kSortBlock = 256;
+constexpr int kSortWaves = kSortBlock / kWave;
 
-template <int ITEMS>
-__global__ __launch_bounds__(kSortBlock) void radix_hist_kernel(
-    const unsigned long long *__restrict__ keys, long long n, int shift,
-    unsigned *__restrict__ counts, int num_tiles) {
-  __shared__ unsigned hist[kRadix];
-  hist[threadIdx.x] = 0;
+// Digit histogram of one tile; counts are digit-major: counts[d * num_tiles + tile].
+template <int ITEMS, typename Source>
+__global__ __launch_bounds__(kSortBlock) void radix_hist_kernel(Source src, long long n, int shift,
+                                                                int radix_bits,
+                                                                unsigned *__restrict__ counts,
+                                                                int num_tiles) {
+  __shared__ unsigned hist[kMaxRadix];
+  const int radix = 1 << radix_bits;
+  for (int d = threadIdx.x; d < radix; d += kSortBlock) hist[d] = 0;
   __syncthreads();
   const long long base = static_cast<long long>(blockIdx.x) * (kSortBlock * ITEMS);
 #pragma unroll
   for (int r = 0; r < ITEMS; ++r) {
-    long long i = base + r * kSortBlock + threadIdx.x;
-    if (i < n) atomicAdd(&hist[(keys[i] >> shift) & (kRadix - 1)], 1u);
+    const long long i = base + r * kSortBlock + threadIdx.x;
+    if (i < n) {
+      unsigned long long key;
+      unsigned val;
+      src.load(i, key, val);
+      atomicAdd(&hist[static_cast<unsigned>(key >> shift) & (radix - 1)], 1u);
+    }
   }
   __syncthreads();
-  counts[static_cast<long long>(threadIdx.x) * num_tiles + blockIdx.x] = hist[threadIdx.x];
+  for (int d = threadIdx.x; d < radix; d += kSortBlock) {
+    counts[static_cast<long long>(d) * num_tiles + blockIdx.x] = hist[d];
+  }
 }
 
-// Exclusive scan of a flat array by one workgroup (digit-major tile counts).
+// Exclusive scan of a flat array by one workgroup (small arrays only).
 __global__ __launch_bounds__(1024) void scan_counts_kernel(unsigned *__restrict__ data,
                                                            long long total) {
   __shared__ unsigned partial[1024];
@@ -289,7 +347,7 @@ void enqueue_exclusive_scan(unsigned *data, int64_t total, hipStream_t stream) {
 __global__ __launch_bounds__(kSortBlock) void digit_scan_kernel(unsigned *__restrict__ counts,
                                                                 int num_tiles,
                                                                 unsigned *__restrict__ totals) {
-  __shared__ unsigned wave_sums[kSortBlock / kWave];
+  __shared__ unsigned wave_sums[kSortWaves];
   __shared__ unsigned carry_s;
   unsigned *row = counts + static_cast<long long>(blockIdx.x) * num_tiles;
   const int tid = threadIdx.x;
@@ -309,7 +367,7 @@ __global__ __launch_bounds__(kSortBlock) void digit_scan_kernel(unsigned *__rest
     __syncthreads();
     unsigned before = carry_s;
     unsigned all = 0;
-    for (int ww = 0; ww < kSortBlock / kWave; ++ww) {
+    for (int ww = 0; ww < kSortWaves; ++ww) {
       if (ww < w) before += wave_sums[ww];
       all += wave_sums[ww];
     }
@@ -323,20 +381,22 @@ __global__ __launch_bounds__(kSortBlock) void digit_scan_kernel(unsigned *__rest
 
 // Stable scatter of one tile.  Wave w owns the contiguous slice
 // [w*64*ITEMS, (w+1)*64*ITEMS) of the tile and walks it 64 items at a time, so
-// (wave, round, lane) order equals input order; ranks within a digit follow it.
-template <int ITEMS>
+// (wave, round, lane) order equals input order.  Lanes with the same digit
+// find each other with one ballot per digit bit; the rank of an item is its
+// wave's running counter for the digit plus the number of equal lanes below.
+template <int ITEMS, typename Source, typename Sink>
 __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
-    const unsigned long long *__restrict__ keys_in, const unsigned *__restrict__ vals_in,
-    unsigned long long *__restrict__ keys_out, unsigned *__restrict__ vals_out, long long n,
-    int shift, const unsigned *__restrict__ offsets, const unsigned *__restrict__ totals,
-    int num_tiles) {
-  constexpr int kWaves = kSortBlock / kWave;
-  __shared__ volatile unsigned cnt[kWaves][kRadix];
-  __shared__ unsigned digit_wave_sums[kWaves];
+    Source src, Sink dst, long long n, int shift, int radix_bits,
+    const unsigned *__restrict__ offsets, const unsigned *__restrict__ totals, int num_tiles) {
+  __shared__ volatile unsigned cnt[kSortWaves][kMaxRadix];
+  __shared__ unsigned scan_sums[kSortWaves];
+  const int radix = 1 << radix_bits;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int w = tid >> 6;
-  for (int i = tid; i < kWaves * kRadix; i += kSortBlock) (&cnt[0][0])[i] = 0;
+  for (int ww = 0; ww < kSortWaves; ++ww) {
+    for (int d = tid; d < radix; d += kSortBlock) cnt[ww][d] = 0;
+  }
   __syncthreads();
 
   const long long base =
@@ -349,15 +409,18 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
   for (int r = 0; r < ITEMS; ++r) {
     const long long i = base + r * kWave + lane;
     const bool valid = i < n;
-    key[r] = valid ? keys_in[i] : ~0ull;
-    val[r] = valid ? vals_in[i] : 0u;
-    const unsigned d = static_cast<unsigned>(key[r] >> shift) & (kRadix - 1);
+    key[r] = ~0ull;
+    val[r] = 0u;
+    if (valid) src.load(i, key[r], val[r]);
+    const unsigned d = static_cast<unsigned>(key[r] >> shift) & (radix - 1);
     unsigned long long peers = __ballot(valid);
 #pragma unroll
-    for (int b = 0; b < kRadixBits; ++b) {
-      const bool bit = (d >> b) & 1u;
-      const unsigned long long vote = __ballot(valid && bit);
-      peers &= bit ? vote : ~vote;
+    for (int b = 0; b < kMaxRadixBits; ++b) {
+      if (b < radix_bits) {
+        const bool bit = (d >> b) & 1u;
+        const unsigned long long vote = __ballot(valid && bit);
+        peers &= bit ? vote : ~vote;
+      }
     }
     const unsigned below = __popcll(peers & below_mask);
     const unsigned prev = cnt[w][d];
@@ -366,24 +429,37 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     if (valid && below == 0) cnt[w][d] = prev + __popcll(peers);
     __builtin_amdgcn_wave_barrier();
   }
-  // digit bases: exclusive scan of the 256 digit totals (thread d <-> digit d)
-  const unsigned total_d = totals[tid];
-  unsigned inc_d = total_d;
-  for (int off = 1; off < kWave; off <<= 1) {
-    unsigned u = __shfl_up(inc_d, off);
-    if (lane >= off) inc_d += u;
+  // digit bases: exclusive scan of the digit totals; thread t owns the
+  // contiguous digits [t*per, (t+1)*per)
+  const int per = (radix + kSortBlock - 1) / kSortBlock;
+  unsigned local_total = 0;
+  for (int j = 0; j < per; ++j) {
+    const int d = tid * per + j;
+    if (d < radix) local_total += totals[d];
   }
-  if (lane == kWave - 1) digit_wave_sums[w] = inc_d;
+  unsigned inc = local_total;
+  for (int off = 1; off < kWave; off <<= 1) {
+    unsigned u = __shfl_up(inc, off);
+    if (lane >= off) inc += u;
+  }
+  if (lane == kWave - 1) scan_sums[w] = inc;
   __syncthreads();
   {
-    unsigned run = inc_d - total_d;
-    for (int ww = 0; ww < w; ++ww) run += digit_wave_sums[ww];
-    run += offsets[static_cast<long long>(tid) * num_tiles + blockIdx.x];
+    unsigned run = inc - local_total;
+    for (int ww = 0; ww < w; ++ww) run += scan_sums[ww];
+    for (int j = 0; j < per; ++j) {
+      const int d = tid * per + j;
+      if (d < radix) {
+        const unsigned total_d = totals[d];
+        unsigned at = run + offsets[static_cast<long long>(d) * num_tiles + blockIdx.x];
 #pragma unroll
-    for (int ww = 0; ww < kWaves; ++ww) {
-      unsigned c = cnt[ww][tid];
-      cnt[ww][tid] = run;
-      run += c;
+        for (int ww = 0; ww < kSortWaves; ++ww) {
+          const unsigned c = cnt[ww][d];
+          cnt[ww][d] = at;
+          at += c;
+        }
+        run += total_d;
+      }
     }
   }
   __syncthreads();
@@ -391,53 +467,68 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
   for (int r = 0; r < ITEMS; ++r) {
     const long long i = base + r * kWave + lane;
     if (i < n) {
-      const unsigned d = static_cast<unsigned>(key[r] >> shift) & (kRadix - 1);
-      const unsigned pos = cnt[w][d] + rank[r];
-      keys_out[pos] = key[r];
-      vals_out[pos] = val[r];
+      const unsigned d = static_cast<unsigned>(key[r] >> shift) & (radix - 1);
+      dst.store(cnt[w][d] + rank[r], key[r], val[r]);
     }
   }
 }
 
-template <int ITEMS>
-static void radix_sort_impl(unsigned long long *&keys, unsigned *&vals, unsigned long long *&keys_alt,
-                            unsigned *&vals_alt, int64_t n, int bits, unsigned *counts,
-                            hipStream_t stream) {
-  const int num_tiles = static_cast<int>(div_ceil(n, kSortBlock * ITEMS));
-  const int passes = static_cast<int>(div_ceil(bits, kRadixBits));
-  for (int p = 0; p < passes; ++p) {
-    const int shift = p * kRadixBits;
-    radix_hist_kernel<ITEMS><<<num_tiles, kSortBlock, 0, stream>>>(keys, n, shift, counts, num_tiles);
-    check_launch("radix_hist_kernel");
-    unsigned *totals = counts + static_cast<long long>(kRadix) * num_tiles;
-    digit_scan_kernel<<<kRadix, kSortBlock, 0, stream>>>(counts, num_tiles, totals);
-    check_launch("digit_scan_kernel");
-    radix_scatter_kernel<ITEMS><<<num_tiles, kSortBlock, 0, stream>>>(
-        keys, vals, keys_alt, vals_alt, n, shift, counts, totals, num_tiles);
-    check_launch("radix_scatter_kernel");
-    std::swap(keys, keys_alt);
-    std::swap(vals, vals_alt);
-  }
-}
+static int items_for(int64_t n) { return n <= (int64_t(1) << 20) ? 4 : 16; }
 
 size_t radix_counts_len(int64_t n) {
-  int items = n <= (int64_t(1) << 20) ? 4 : 16;
-  return static_cast<size_t>(kRadix) * static_cast<size_t>(div_ceil(n, kSortBlock * items)) + kRadix;
+  return static_cast<size_t>(kMaxRadix) * static_cast<size_t>(div_ceil(n, kSortBlock * items_for(n))) +
+         kMaxRadix;
+}
+
+// Number of passes and digit width for `bits` key bits: as few passes as 11-bit
+// digits allow, digits then split evenly.
+static void pass_plan(int bits, int &passes, int &radix_bits) {
+  passes = static_cast<int>(div_ceil(bits, kMaxRadixBits));
+  radix_bits = static_cast<int>(div_ceil(bits, passes));
+}
+
+template <int ITEMS, typename Source, typename Sink>
+static void radix_pass(const Source &src, const Sink &dst, int64_t n, int shift, int radix_bits,
+                       unsigned *counts, hipStream_t stream) {
+  const int num_tiles = static_cast<int>(div_ceil(n, kSortBlock * ITEMS));
+  const int radix = 1 << radix_bits;
+  unsigned *totals = counts + static_cast<size_t>(radix) * num_tiles;
+  radix_hist_kernel<ITEMS, Source><<<num_tiles, kSortBlock, 0, stream>>>(src, n, shift, radix_bits, counts, num_tiles);
+  check_launch("radix_hist_kernel");
+  digit_scan_kernel<<<radix, kSortBlock, 0, stream>>>(counts, num_tiles, totals);
+  check_launch("digit_scan_kernel");
+  radix_scatter_kernel<ITEMS, Source, Sink><<<num_tiles, kSortBlock, 0, stream>>>(
+      src, dst, n, shift, radix_bits, counts, totals, num_tiles);
+  check_launch("radix_scatter_kernel");
+}
+
+template <typename Source, typename Sink>
+static void radix_pass_any(const Source &src, const Sink &dst, int64_t n, int shift, int radix_bits,
+                           unsigned *counts, hipStream_t stream) {
+  if (items_for(n) == 4) {
+    radix_pass<4>(src, dst, n, shift, radix_bits, counts, stream);
+  } else {
+    radix_pass<16>(src, dst, n, shift, radix_bits, counts, stream);
+  }
 }
 
 void radix_sort_pairs(unsigned long long *&keys, unsigned *&vals, unsigned long long *&keys_alt,
                       unsigned *&vals_alt, int64_t n, int bits, unsigned *counts,
                       hipStream_t stream) {
   if (n <= 1 || bits <= 0) return;
-  if (n <= (int64_t(1) << 20)) {
-    radix_sort_impl<4>(keys, vals, keys_alt, vals_alt, n, bits, counts, stream);
-  } else {
-    radix_sort_impl<16>(keys, vals, keys_alt, vals_alt, n, bits, counts, stream);
+  int passes, radix_bits;
+  pass_plan(bits, passes, radix_bits);
+  for (int p = 0; p < passes; ++p) {
+    radix_pass_any(PlainSource{keys, vals}, PlainSink{keys_alt, vals ? vals_alt : nullptr}, n,
+                   p * radix_bits, radix_bits, counts, stream);
+    std::swap(keys, keys_alt);
+    if (vals) std::swap(vals, vals_alt);
   }
 }
 
 // --------------------------------------------------------------- outputs ----
 
+// Identity / gather emit for the cases without any radix pass.
 template <typename CT, typename IT>
 __global__ __launch_bounds__(256) void emit_sorted_kernel(const CT *__restrict__ coords, long long n,
                                                           int ndim,
@@ -447,10 +538,10 @@ __global__ __launch_bounds__(256) void emit_sorted_kernel(const CT *__restrict__
   const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
   for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
        i += stride) {
-    const unsigned row = perm[i];
+    const long long row = perm ? static_cast<long long>(perm[i]) : i;
     if (indices_out) indices_out[i] = static_cast<IT>(row);
     if (sorted_out) {
-      for (int k = 0; k < ndim; ++k) sorted_out[i * ndim + k] = coords[static_cast<long long>(row) * ndim + k];
+      for (int k = 0; k < ndim; ++k) sorted_out[i * ndim + k] = coords[row * ndim + k];
     }
   }
 }
@@ -484,48 +575,98 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
   widths[MNT_MAX_NDIM] = batched ? bit_width(static_cast<unsigned long long>(num_batches - 1)) : 0;
   lows[MNT_MAX_NDIM] = 0;
 
-  unsigned long long *keys = scope.alloc<unsigned long long>(n);
-  unsigned long long *keys_alt = scope.alloc<unsigned long long>(n);
-  unsigned *vals = scope.alloc<unsigned>(n);
-  unsigned *vals_alt = scope.alloc<unsigned>(n);
-  unsigned *counts = scope.alloc<unsigned>(radix_counts_len(n));
-
   int order[MNT_MAX_NDIM + 1];
   int num_fields = 0;
   for (int k = ndim - 1; k >= 0; --k) order[num_fields++] = k;
   if (batched) order[num_fields++] = MNT_MAX_NDIM;
 
-  const unsigned grid = grid_for(n, 256, 4096);
-  bool first = true;
+  // rounds: greedy groups of fields that fit one 64-bit key
+  struct Round {
+    SortSpec spec;
+    int bits;
+  };
+  std::vector<Round> rounds;
   int f = 0;
   while (f < num_fields) {
-    SortSpec spec;
-    memset(&spec, 0, sizeof(spec));
-    spec.ndim = ndim;
-    spec.num_batches = static_cast<int>(num_batches);
+    Round round;
+    memset(&round.spec, 0, sizeof(SortSpec));
+    round.spec.ndim = ndim;
+    round.spec.num_batches = static_cast<int>(num_batches);
     int bits = 0;
     while (f < num_fields && bits + widths[order[f]] <= 64) {
-      int k = order[f];
+      const int k = order[f];
       if (widths[k] > 0) {
-        spec.lo[k] = lows[k];
-        spec.mask[k] = widths[k] >= 64 ? ~0ull : ((1ull << widths[k]) - 1ull);
-        spec.shift[k] = bits;
+        round.spec.lo[k] = lows[k];
+        round.spec.mask[k] = widths[k] >= 64 ? ~0ull : ((1ull << widths[k]) - 1ull);
+        round.spec.shift[k] = bits;
         bits += widths[k];
       }
       ++f;
     }
-    if (bits == 0 && !first) continue;   // nothing to order by in this group
-    pack_keys_kernel<CT, IT><<<grid, 256, 0, stream>>>(coords, n, spec, batch_dims,
-                                                       first ? nullptr : vals, keys, vals);
-    check_launch("pack_keys_kernel");
-    first = false;
-    profile_mark("sort_pack", stream);
-    radix_sort_pairs(keys, vals, keys_alt, vals_alt, n, bits, counts, stream);
-    profile_mark("sort_radix", stream);
+    round.bits = bits;
+    if (bits > 0) rounds.push_back(round);
   }
-  emit_sorted_kernel<CT, IT><<<grid, 256, 0, stream>>>(coords, n, ndim, vals, indices_out, sorted_out);
-  check_launch("emit_sorted_kernel");
-  profile_mark("sort_emit", stream);
+
+  const unsigned grid = grid_for(n, 256, 4096);
+  if (rounds.empty()) {   // all rows equal: the stable order is the identity
+    emit_sorted_kernel<CT, IT><<<grid, 256, 0, stream>>>(coords, n, ndim, nullptr, indices_out, sorted_out);
+    check_launch("emit_sorted_kernel");
+    profile_mark("sort_emit", stream);
+    return;
+  }
+
+  int total_passes = 0;
+  for (const Round &round : rounds) {
+    int passes, rb;
+    pass_plan(round.bits, passes, rb);
+    total_passes += passes;
+  }
+  unsigned long long *keys = nullptr, *keys_alt = nullptr;
+  unsigned *vals = nullptr, *vals_alt = nullptr;
+  if (total_passes > 1) {
+    keys = scope.alloc<unsigned long long>(n);
+    vals = scope.alloc<unsigned>(n);
+    if (total_passes > 2) {
+      keys_alt = scope.alloc<unsigned long long>(n);
+      vals_alt = scope.alloc<unsigned>(n);
+    }
+  }
+  unsigned *counts = scope.alloc<unsigned>(radix_counts_len(n));
+  const FinalSink<CT, IT> final_sink{coords, ndim, indices_out, sorted_out};
+
+  int done = 0;
+  const unsigned *perm = nullptr;     // order left by the previous round
+  for (size_t r = 0; r < rounds.size(); ++r) {
+    int passes, rb;
+    pass_plan(rounds[r].bits, passes, rb);
+    const CoordSource<CT, IT> coord_src{coords, batch_dims, perm, rounds[r].spec};
+    for (int p = 0; p < passes; ++p) {
+      const bool first = p == 0;
+      const bool last = done + 1 == total_passes;
+      const int shift = p * rb;
+      if (first && last) {
+        radix_pass_any(coord_src, final_sink, n, shift, rb, counts, stream);
+      } else if (first) {
+        // the previous round's order lives in `vals`; write into the other pair
+        unsigned long long *k_out = perm == vals ? keys_alt : keys;
+        unsigned *v_out = perm == vals ? vals_alt : vals;
+        radix_pass_any(coord_src, PlainSink{k_out, v_out}, n, shift, rb, counts, stream);
+        if (perm == vals) {
+          std::swap(keys, keys_alt);
+          std::swap(vals, vals_alt);
+        }
+      } else if (last) {
+        radix_pass_any(PlainSource{keys, vals}, final_sink, n, shift, rb, counts, stream);
+      } else {
+        radix_pass_any(PlainSource{keys, vals}, PlainSink{keys_alt, vals_alt}, n, shift, rb, counts, stream);
+        std::swap(keys, keys_alt);
+        std::swap(vals, vals_alt);
+      }
+      ++done;
+    }
+    perm = vals;
+  }
+  profile_mark("sort_radix", stream);
 }
 
 }  // namespace mnt

@@ -163,7 +163,7 @@ __global__ __launch_bounds__(256) void pack_target_keys_kernel(
              << spec.batch_shift;
     }
     keys[i] = key;
-    vals[i] = static_cast<unsigned>(i);
+    if (vals) vals[i] = static_cast<unsigned>(i);
   }
 }
 
@@ -283,8 +283,7 @@ static void target_count_typed(const CT *coords, int64_t n, int ndim, const int6
     char *keep = static_cast<char *>(arena.persistent(0, key_bytes + (static_cast<size_t>(n) + 1) * 4));
     unsigned long long *keys = scope.alloc<unsigned long long>(n);
     unsigned long long *keys_alt = scope.alloc<unsigned long long>(n);
-    unsigned *vals = scope.alloc<unsigned>(n);
-    unsigned *vals_alt = scope.alloc<unsigned>(n);
+    unsigned *vals = nullptr, *vals_alt = nullptr;      // keys-only sort
     unsigned *counts = scope.alloc<unsigned>(radix_counts_len(n));
     const unsigned grid = grid_for(n, 256, 4096);
     pack_target_keys_kernel<CT, IT><<<grid, 256, 0, stream>>>(coords, n, spec, batch_dims, keys, vals);
