@@ -28,10 +28,12 @@ namespace mnt {
 constexpr int kQueryBlock = 256;          // emit / count kernels
 constexpr int kQueryThreads = 512;        // query kernel: one target per lane
 constexpr int kTargetsPerTile = 512;
-constexpr int kWindowChunk = 2048;
+constexpr int kWindowChunk = 4096;
 constexpr int kWindowPad = 64;            // sentinel keys behind a full chunk
-constexpr long long kMaxWalkGap = 4;      // largest key gap bridged by walking
+constexpr int kGroupSpan = 4;             // key span of one offset group
 constexpr int kGroupsInFlight = 3;
+constexpr int kMaxSamples = 2048;         // sampled source keys for the window search
+constexpr int kDirectStride = 256;        // sample stride up to which no refinement is needed
 
 template <typename CT, typename BT>
 struct KeyReader {
@@ -46,12 +48,13 @@ struct KeyReader {
   }
 };
 
-// First index in [0, count) whose key is >= q, found by one wavefront probing
-// 64 equally spaced rows per step.  All lanes must call with the same q.
+// First index in [lo, hi) whose key is >= q (hi if none), found by one
+// wavefront probing 64 equally spaced rows per step.  All lanes must call
+// with the same arguments.
 template <typename CT, typename BT>
 __device__ __forceinline__ long long wave_lower_bound(const KeyReader<CT, BT> &src, const Frame &f,
-                                                      unsigned long long q) {
-  long long lo = 0, hi = src.count;
+                                                      unsigned long long q, long long lo,
+                                                      long long hi) {
   const int lane = lane_id();
   while (hi > lo) {
     const long long len = hi - lo;
@@ -72,7 +75,12 @@ __device__ __forceinline__ long long wave_lower_bound(const KeyReader<CT, BT> &s
 
 // sorted_delta[i] / sorted_offset[i]: packed delta and original row of the i-th
 // offset in ascending key order; group_start[g] .. group_start[g+1] are the
-// offsets of walk group g.
+// offsets of group g, whose deltas lie within kGroupSpan of the first one.
+//
+// Because source keys are unique and ascending, the key at window position
+// p + j is at least win[p] + j; so once p = lower_bound(first query of the
+// group) is known, every query of the group can only sit in win[p .. p+span]:
+// one search plus span+1 independent LDS reads resolve the whole group.
 template <typename CT, typename BT, typename OT>
 __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     KeyReader<CT, BT> src, KeyReader<CT, BT> tgt, Frame frame,
@@ -85,24 +93,54 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
   __shared__ unsigned long long s_next_first;
 
   const int tid = threadIdx.x;
+  const int w = tid >> 6;
+  const long long num_sources = src.count;
   const long long num_targets = tgt.count;
   const long long t0 = static_cast<long long>(blockIdx.x) * kTargetsPerTile;
   const long long t_end = t0 + kTargetsPerTile < num_targets ? t0 + kTargetsPerTile : num_targets;
 
   for (int o = tid; o < num_offsets; o += kQueryThreads) s_counts[o] = 0;
 
-  // window of sources that can match any (offset, target) pair of this tile
-  const int w = tid >> 6;
-  if (w < 2) {
-    const unsigned long long edge =
-        w == 0 ? tgt(t0, frame) + static_cast<unsigned long long>(sorted_delta[0])
-               : tgt(t_end - 1, frame) + static_cast<unsigned long long>(sorted_delta[num_offsets - 1]) + 1ull;
-    const long long pos = wave_lower_bound<CT, BT>(src, frame, edge);
-    if (lane_id() == 0) s_bounds[w] = pos;
+  // ---- window of sources that can match any (offset, target) pair of the tile.
+  // Level 1: up to 2048 evenly spaced source keys are staged in LDS (one round
+  // of loads) and searched there; level 2 (long arrays only) narrows the
+  // remaining interval with a wave-cooperative search in global memory.
+  const long long stride = (num_sources + kMaxSamples - 1) / kMaxSamples;
+  const int num_samples = static_cast<int>((num_sources + stride - 1) / stride);
+  for (int i = tid; i < kMaxSamples; i += kQueryThreads) {
+    win[i] = i < num_samples ? src(static_cast<long long>(i) * stride, frame) : ~0ull;
   }
   const long long t = t0 + tid;
   const bool valid = t < t_end;
   const unsigned long long key = valid ? tgt(t, frame) : 0ull;
+  unsigned long long edge = 0;
+  if (w < 2) {
+    edge = w == 0 ? tgt(t0, frame) + static_cast<unsigned long long>(sorted_delta[0])
+                  : tgt(t_end - 1, frame) + static_cast<unsigned long long>(sorted_delta[num_offsets - 1]) + 1ull;
+  }
+  __syncthreads();
+  if (w < 2) {
+    // number of samples below the edge
+    int below = 0;
+    for (int step = kMaxSamples / 2; step >= 1; step >>= 1) {
+      if (win[below + step - 1] < edge) below += step;
+    }
+    below += win[below] < edge ? 1 : 0;       // win[kMaxSamples - 1 .. ] may all be below
+    if (below > num_samples) below = num_samples;
+    long long pos;
+    if (w == 0) {
+      // keys before sample (below-1) are smaller than it, hence below the edge
+      long long lo = below > 0 ? static_cast<long long>(below - 1) * stride : 0;
+      long long hi = static_cast<long long>(below) * stride < num_sources ? static_cast<long long>(below) * stride : num_sources;
+      pos = stride <= kDirectStride ? lo : wave_lower_bound<CT, BT>(src, frame, edge, lo, hi);
+    } else {
+      // keys from sample `below` on are at least the edge
+      long long hi = static_cast<long long>(below) * stride < num_sources ? static_cast<long long>(below) * stride : num_sources;
+      long long lo = below > 0 ? static_cast<long long>(below - 1) * stride : 0;
+      pos = stride <= kDirectStride ? hi : wave_lower_bound<CT, BT>(src, frame, edge, lo, hi);
+    }
+    if (lane_id() == 0) s_bounds[w] = pos;
+  }
   __syncthreads();
   const long long w_lo = s_bounds[0];
   const long long w_hi = s_bounds[1] > w_lo ? s_bounds[1] : w_lo;
@@ -113,8 +151,11 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     const long long c0 = w_lo + static_cast<long long>(c) * kWindowChunk;
     const long long c1 = c0 + kWindowChunk < w_hi ? c0 + kWindowChunk : w_hi;
     const int len = static_cast<int>(c1 - c0);
-    if (c > 0) __syncthreads();
-    for (int i = tid; i < kWindowChunk + kWindowPad; i += kQueryThreads) {
+    __syncthreads();                          // everyone is done with the previous content
+    int top = 1;
+    while (top * 2 < len) top *= 2;           // highest power of two below len (>= 1)
+    const int fill = 2 * top + kWindowPad < kWindowChunk + kWindowPad ? 2 * top + kWindowPad : kWindowChunk + kWindowPad;
+    for (int i = tid; i < fill; i += kQueryThreads) {
       win[i] = i < len ? src(c0 + i, frame) : ~0ull;
     }
     if (tid == 0) s_next_first = c1 < w_hi ? src(c1, frame) : ~0ull;
@@ -123,8 +164,6 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     const unsigned long long next_first = s_next_first;
     const bool is_first = c == 0;
     const bool is_last = c == num_chunks - 1;
-    int top = 1;
-    while (top * 2 < len) top *= 2;      // highest power of two below len (>= 1)
 
     for (int g0 = 0; g0 < num_groups; g0 += kGroupsInFlight) {
       // lower bound of the first query of up to three groups, in lockstep
@@ -147,16 +186,21 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
         if (g0 + j >= num_groups) continue;       // uniform across the workgroup
         int p = pos[j];
         p += win[p] < q0[j] ? 1 : 0;
+        unsigned long long cand[kGroupSpan + 1];
+#pragma unroll
+        for (int x = 0; x <= kGroupSpan; ++x) cand[x] = win[p + x];
         const int i_end = group_start[g0 + j + 1];
         for (int i = group_start[g0 + j]; i < i_end; ++i) {
           const unsigned long long q = key + static_cast<unsigned long long>(sorted_delta[i]);
           const bool mine = valid && (is_first || q >= first_key) && (is_last || q < next_first);
-          while (mine && win[p] < q) ++p;
-          const bool hit = mine && win[p] == q;
+          int at = -1;
+#pragma unroll
+          for (int x = 0; x <= kGroupSpan; ++x) at = cand[x] == q ? x : at;
+          const bool hit = mine && at >= 0;
           const int o = sorted_offset[i];
           if (mine) {
             kernel_map[static_cast<long long>(o) * num_targets + t] =
-                hit ? static_cast<OT>(c0 + p) : static_cast<OT>(-1);
+                hit ? static_cast<OT>(c0 + p + at) : static_cast<OT>(-1);
           }
           const unsigned hits = __popcll(__ballot(hit));
           if (tile_counts != nullptr && hits != 0 && lane_id() == 0) atomicAdd(&s_counts[o], hits);
@@ -408,7 +452,9 @@ static QueryPlan make_plan(const long long *src_bounds, const long long *tgt_bou
   for (int64_t i = 0; i < num_offsets; ++i) {
     plan.sorted_delta[i] = keyed[i].first;
     plan.sorted_offset[i] = keyed[i].second;
-    if (i == 0 || keyed[i].first - keyed[i - 1].first > kMaxWalkGap) plan.group_start.push_back(static_cast<int>(i));
+    if (i == 0 || keyed[i].first - keyed[plan.group_start.back()].first > kGroupSpan) {
+      plan.group_start.push_back(static_cast<int>(i));
+    }
   }
   plan.group_start.push_back(static_cast<int>(num_offsets));
   return plan;

@@ -17,8 +17,9 @@ from typing import Optional, Sequence, Tuple
 import numpy as np
 import torch
 
-_LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))),
-                         "lib", "libminuet_hip.so")
+_LIB_PATH = os.environ.get("MINUET_AMD_LIBRARY") or os.path.join(
+    os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))), "lib",
+    "libminuet_hip.so")
 _lib = None
 
 _INT = {torch.int32: 0, torch.int64: 1}
