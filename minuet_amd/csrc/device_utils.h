@@ -50,19 +50,32 @@ __device__ __forceinline__ bool is_batch_end(long long end, const IT *__restrict
   return lo <= num_batches && static_cast<long long>(dims[lo]) == end;
 }
 
+// Loads the (up to four) coordinates of one row without branching on the
+// number of dimensions: slots past ndim re-read coordinate 0, so all loads
+// are issued together instead of one after another.
+template <typename CT>
+__device__ __forceinline__ void load_row(const CT *__restrict__ row, int ndim,
+                                         long long (&c)[MNT_MAX_NDIM]) {
+  CT raw[MNT_MAX_NDIM];
+#pragma unroll
+  for (int k = 0; k < MNT_MAX_NDIM; ++k) raw[k] = row[k < ndim ? k : 0];
+#pragma unroll
+  for (int k = 0; k < MNT_MAX_NDIM; ++k) c[k] = static_cast<long long>(raw[k]);
+}
+
 // Key of one row under a Frame (see common.h).  `batch` is ignored when the
 // frame has no batch field.
 template <typename CT>
 __device__ __forceinline__ unsigned long long pack_row(const CT *__restrict__ row,
                                                        const Frame &f, int batch) {
+  long long c[MNT_MAX_NDIM];
+  load_row<CT>(row, f.ndim, c);
   unsigned long long key = 0;
 #pragma unroll
   for (int k = 0; k < MNT_MAX_NDIM; ++k) {
-    if (k < f.ndim) {
-      unsigned long long v = static_cast<unsigned long long>(static_cast<long long>(row[k])) -
-                             static_cast<unsigned long long>(f.lo[k]);
-      key |= v << f.shift[k];
-    }
+    const unsigned long long v =
+        static_cast<unsigned long long>(c[k]) - static_cast<unsigned long long>(f.lo[k]);
+    key |= k < f.ndim ? (v << f.shift[k]) : 0ull;
   }
   if (f.batch_width > 0) key |= static_cast<unsigned long long>(batch) << f.batch_shift;
   return key;

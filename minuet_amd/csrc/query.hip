@@ -32,8 +32,7 @@ constexpr int kWindowChunk = 4096;
 constexpr int kWindowPad = 64;            // sentinel keys behind a full chunk
 constexpr int kGroupSpan = 4;             // key span of one offset group
 constexpr int kGroupsInFlight = 3;
-constexpr int kMaxSamples = 2048;         // sampled source keys for the window search
-constexpr int kDirectStride = 256;        // sample stride up to which no refinement is needed
+
 
 template <typename CT, typename BT>
 struct KeyReader {
@@ -73,9 +72,78 @@ __device__ __forceinline__ long long wave_lower_bound(const KeyReader<CT, BT> &s
   return lo;
 }
 
-// sorted_delta[i] / sorted_offset[i]: packed delta and original row of the i-th
-// offset in ascending key order; group_start[g] .. group_start[g+1] are the
-// offsets of group g, whose deltas lie within kGroupSpan of the first one.
+// Resolves every (offset, target) pair of the tile against the window chunk
+// staged in LDS as keys of type K relative to `base` (K = 32 bits when the
+// chunk's key range allows, which halves the LDS traffic of the searches).
+// A query outside [base, base + max K) cannot match and is forced to miss.
+template <typename K, typename OT>
+__device__ __forceinline__ void resolve_chunk(
+    const K *__restrict__ win, int top, unsigned long long base, long long c0,
+    unsigned long long key, bool valid, bool is_first, bool is_last,
+    unsigned long long first_key, unsigned long long next_first, const int4 *s_groups,
+    const int2 *s_members, int num_groups, unsigned *s_counts, bool count_hits, long long t,
+    long long num_targets, OT *__restrict__ kernel_map) {
+  constexpr unsigned long long kLimit = static_cast<unsigned long long>(static_cast<K>(~static_cast<K>(0)));
+  for (int g0 = 0; g0 < num_groups; g0 += kGroupsInFlight) {
+    // lower bound of the first query of up to three groups, in lockstep
+    int4 group[kGroupsInFlight];
+    unsigned long long q0[kGroupsInFlight];
+    K q0_rel[kGroupsInFlight];
+    int pos[kGroupsInFlight];
+#pragma unroll
+    for (int j = 0; j < kGroupsInFlight; ++j) {
+      group[j] = s_groups[g0 + j < num_groups ? g0 + j : num_groups - 1];
+      const unsigned long long first_delta =
+          static_cast<unsigned long long>(static_cast<unsigned>(group[j].x)) |
+          (static_cast<unsigned long long>(static_cast<unsigned>(group[j].y)) << 32);
+      q0[j] = key + first_delta;
+      const unsigned long long d = q0[j] - base;
+      q0_rel[j] = q0[j] < base ? static_cast<K>(0)
+                               : (d < kLimit ? static_cast<K>(d) : static_cast<K>(kLimit - 1));
+      pos[j] = 0;
+    }
+    for (int step = top; step >= 1; step >>= 1) {
+#pragma unroll
+      for (int j = 0; j < kGroupsInFlight; ++j) {
+        if (win[pos[j] + step - 1] < q0_rel[j]) pos[j] += step;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kGroupsInFlight; ++j) {
+      if (g0 + j >= num_groups) continue;       // uniform across the workgroup
+      int p = pos[j];
+      p += win[p] < q0_rel[j] ? 1 : 0;
+      K cand[kGroupSpan + 1];
+#pragma unroll
+      for (int x = 0; x <= kGroupSpan; ++x) cand[x] = win[p + x];
+      for (int m = 0; m < group[j].w; ++m) {
+        const int2 member = s_members[group[j].z + m];
+        const unsigned long long q = q0[j] + static_cast<unsigned long long>(member.x);
+        const bool mine = valid && (is_first || q >= first_key) && (is_last || q < next_first);
+        const unsigned long long d = q - base;
+        const bool in_range = q >= base && d < kLimit;
+        const K q_rel = static_cast<K>(d);
+        int at = -1;
+#pragma unroll
+        for (int x = 0; x <= kGroupSpan; ++x) at = cand[x] == q_rel ? x : at;
+        const bool hit = mine && in_range && at >= 0;
+        const int o = member.y;
+        if (mine) {
+          kernel_map[static_cast<long long>(o) * num_targets + t] =
+              hit ? static_cast<OT>(c0 + p + at) : static_cast<OT>(-1);
+        }
+        const unsigned hits = __popcll(__ballot(hit));
+        if (count_hits && hits != 0 && lane_id() == 0) atomicAdd(&s_counts[o], hits);
+      }
+    }
+  }
+}
+
+// Offsets are visited in ascending key order, in groups whose deltas lie within
+// kGroupSpan of the group's first one.  `tables` holds, as 32-bit words,
+//   group g : first delta (low, high), index of its first member, member count
+//   member i: delta minus the group's first delta, original offset row
+// (groups first, then members); the kernel copies it into LDS once.
 //
 // Because source keys are unique and ascending, the key at window position
 // p + j is at least win[p] + j; so once p = lower_bound(first query of the
@@ -83,14 +151,16 @@ __device__ __forceinline__ long long wave_lower_bound(const KeyReader<CT, BT> &s
 // one search plus span+1 independent LDS reads resolve the whole group.
 template <typename CT, typename BT, typename OT>
 __global__ __launch_bounds__(kQueryThreads) void query_kernel(
-    KeyReader<CT, BT> src, KeyReader<CT, BT> tgt, Frame frame,
-    const long long *__restrict__ sorted_delta, const int *__restrict__ sorted_offset,
-    const int *__restrict__ group_start, int num_groups, int num_offsets,
+    KeyReader<CT, BT> src, KeyReader<CT, BT> tgt, Frame frame, const int *__restrict__ tables,
+    int num_groups, int num_offsets, long long delta_min, long long delta_max,
     OT *__restrict__ kernel_map, unsigned *__restrict__ tile_counts, int num_tiles) {
-  extern __shared__ unsigned s_counts[];                 // [num_offsets]
+  extern __shared__ __align__(16) unsigned s_dynamic[];
   __shared__ unsigned long long win[kWindowChunk + kWindowPad];
   __shared__ long long s_bounds[2];
-  __shared__ unsigned long long s_next_first;
+  // dynamic LDS: [group table: 4 words each][member table: 2 words each][hit counts]
+  const int4 *s_groups = reinterpret_cast<const int4 *>(s_dynamic);
+  const int2 *s_members = reinterpret_cast<const int2 *>(s_dynamic + 4 * num_groups);
+  unsigned *s_counts = s_dynamic + 4 * num_groups + 2 * num_offsets;
 
   const int tid = threadIdx.x;
   const int w = tid >> 6;
@@ -99,46 +169,19 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
   const long long t0 = static_cast<long long>(blockIdx.x) * kTargetsPerTile;
   const long long t_end = t0 + kTargetsPerTile < num_targets ? t0 + kTargetsPerTile : num_targets;
 
+  for (int i = tid; i < 4 * num_groups + 2 * num_offsets; i += kQueryThreads) s_dynamic[i] = tables[i];
   for (int o = tid; o < num_offsets; o += kQueryThreads) s_counts[o] = 0;
 
-  // ---- window of sources that can match any (offset, target) pair of the tile.
-  // Level 1: up to 2048 evenly spaced source keys are staged in LDS (one round
-  // of loads) and searched there; level 2 (long arrays only) narrows the
-  // remaining interval with a wave-cooperative search in global memory.
-  const long long stride = (num_sources + kMaxSamples - 1) / kMaxSamples;
-  const int num_samples = static_cast<int>((num_sources + stride - 1) / stride);
-  for (int i = tid; i < kMaxSamples; i += kQueryThreads) {
-    win[i] = i < num_samples ? src(static_cast<long long>(i) * stride, frame) : ~0ull;
-  }
+  // ---- window of sources that can match any (offset, target) pair of the tile:
+  // wavefront 0 finds its lower end, wavefront 1 its upper end
   const long long t = t0 + tid;
   const bool valid = t < t_end;
   const unsigned long long key = valid ? tgt(t, frame) : 0ull;
-  unsigned long long edge = 0;
   if (w < 2) {
-    edge = w == 0 ? tgt(t0, frame) + static_cast<unsigned long long>(sorted_delta[0])
-                  : tgt(t_end - 1, frame) + static_cast<unsigned long long>(sorted_delta[num_offsets - 1]) + 1ull;
-  }
-  __syncthreads();
-  if (w < 2) {
-    // number of samples below the edge
-    int below = 0;
-    for (int step = kMaxSamples / 2; step >= 1; step >>= 1) {
-      if (win[below + step - 1] < edge) below += step;
-    }
-    below += win[below] < edge ? 1 : 0;       // win[kMaxSamples - 1 .. ] may all be below
-    if (below > num_samples) below = num_samples;
-    long long pos;
-    if (w == 0) {
-      // keys before sample (below-1) are smaller than it, hence below the edge
-      long long lo = below > 0 ? static_cast<long long>(below - 1) * stride : 0;
-      long long hi = static_cast<long long>(below) * stride < num_sources ? static_cast<long long>(below) * stride : num_sources;
-      pos = stride <= kDirectStride ? lo : wave_lower_bound<CT, BT>(src, frame, edge, lo, hi);
-    } else {
-      // keys from sample `below` on are at least the edge
-      long long hi = static_cast<long long>(below) * stride < num_sources ? static_cast<long long>(below) * stride : num_sources;
-      long long lo = below > 0 ? static_cast<long long>(below - 1) * stride : 0;
-      pos = stride <= kDirectStride ? hi : wave_lower_bound<CT, BT>(src, frame, edge, lo, hi);
-    }
+    const unsigned long long edge =
+        w == 0 ? tgt(t0, frame) + static_cast<unsigned long long>(delta_min)
+               : tgt(t_end - 1, frame) + static_cast<unsigned long long>(delta_max) + 1ull;
+    const long long pos = wave_lower_bound<CT, BT>(src, frame, edge, 0, num_sources);
     if (lane_id() == 0) s_bounds[w] = pos;
   }
   __syncthreads();
@@ -151,61 +194,38 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     const long long c0 = w_lo + static_cast<long long>(c) * kWindowChunk;
     const long long c1 = c0 + kWindowChunk < w_hi ? c0 + kWindowChunk : w_hi;
     const int len = static_cast<int>(c1 - c0);
-    __syncthreads();                          // everyone is done with the previous content
+    if (c > 0) __syncthreads();               // everyone is done with the previous chunk
     int top = 1;
     while (top * 2 < len) top *= 2;           // highest power of two below len (>= 1)
     const int fill = 2 * top + kWindowPad < kWindowChunk + kWindowPad ? 2 * top + kWindowPad : kWindowChunk + kWindowPad;
-    for (int i = tid; i < fill; i += kQueryThreads) {
-      win[i] = i < len ? src(c0 + i, frame) : ~0ull;
+    // first and last key of the chunk and the first key behind it: the same
+    // addresses for every lane, issued together with the staging loads
+    const unsigned long long first_key = len > 0 ? src(c0, frame) : ~0ull;
+    const unsigned long long last_key = len > 0 ? src(c1 - 1, frame) : 0ull;
+    const unsigned long long next_first = c1 < w_hi ? src(c1, frame) : ~0ull;
+    const bool narrow = len > 0 && last_key - first_key < 0xffffffffull;
+    if (narrow) {
+      unsigned *win32 = reinterpret_cast<unsigned *>(win);
+      for (int i = tid; i < fill; i += kQueryThreads) {
+        win32[i] = i < len ? static_cast<unsigned>(src(c0 + i, frame) - first_key) : 0xffffffffu;
+      }
+    } else {
+      for (int i = tid; i < fill; i += kQueryThreads) {
+        win[i] = i < len ? src(c0 + i, frame) : ~0ull;
+      }
     }
-    if (tid == 0) s_next_first = c1 < w_hi ? src(c1, frame) : ~0ull;
     __syncthreads();
-    const unsigned long long first_key = win[0];
-    const unsigned long long next_first = s_next_first;
     const bool is_first = c == 0;
     const bool is_last = c == num_chunks - 1;
-
-    for (int g0 = 0; g0 < num_groups; g0 += kGroupsInFlight) {
-      // lower bound of the first query of up to three groups, in lockstep
-      unsigned long long q0[kGroupsInFlight];
-      int pos[kGroupsInFlight];
-#pragma unroll
-      for (int j = 0; j < kGroupsInFlight; ++j) {
-        const int g = g0 + j < num_groups ? g0 + j : num_groups - 1;
-        q0[j] = key + static_cast<unsigned long long>(sorted_delta[group_start[g]]);
-        pos[j] = 0;
-      }
-      for (int step = top; step >= 1; step >>= 1) {
-#pragma unroll
-        for (int j = 0; j < kGroupsInFlight; ++j) {
-          if (win[pos[j] + step - 1] < q0[j]) pos[j] += step;
-        }
-      }
-#pragma unroll
-      for (int j = 0; j < kGroupsInFlight; ++j) {
-        if (g0 + j >= num_groups) continue;       // uniform across the workgroup
-        int p = pos[j];
-        p += win[p] < q0[j] ? 1 : 0;
-        unsigned long long cand[kGroupSpan + 1];
-#pragma unroll
-        for (int x = 0; x <= kGroupSpan; ++x) cand[x] = win[p + x];
-        const int i_end = group_start[g0 + j + 1];
-        for (int i = group_start[g0 + j]; i < i_end; ++i) {
-          const unsigned long long q = key + static_cast<unsigned long long>(sorted_delta[i]);
-          const bool mine = valid && (is_first || q >= first_key) && (is_last || q < next_first);
-          int at = -1;
-#pragma unroll
-          for (int x = 0; x <= kGroupSpan; ++x) at = cand[x] == q ? x : at;
-          const bool hit = mine && at >= 0;
-          const int o = sorted_offset[i];
-          if (mine) {
-            kernel_map[static_cast<long long>(o) * num_targets + t] =
-                hit ? static_cast<OT>(c0 + p + at) : static_cast<OT>(-1);
-          }
-          const unsigned hits = __popcll(__ballot(hit));
-          if (tile_counts != nullptr && hits != 0 && lane_id() == 0) atomicAdd(&s_counts[o], hits);
-        }
-      }
+    if (narrow) {
+      resolve_chunk<unsigned, OT>(reinterpret_cast<const unsigned *>(win), top, first_key, c0, key, valid,
+                                  is_first, is_last, first_key, next_first, s_groups, s_members,
+                                  num_groups, s_counts, tile_counts != nullptr, t, num_targets,
+                                  kernel_map);
+    } else {
+      resolve_chunk<unsigned long long, OT>(win, top, 0ull, c0, key, valid, is_first, is_last, first_key,
+                                            next_first, s_groups, s_members, num_groups, s_counts,
+                                            tile_counts != nullptr, t, num_targets, kernel_map);
     }
   }
   if (tile_counts != nullptr) {
@@ -392,9 +412,9 @@ static int width_of(unsigned long long range) {
 
 struct QueryPlan {
   Frame frame;
-  std::vector<long long> sorted_delta;   // packed offsets in ascending order
-  std::vector<int> sorted_offset;        // original row of each
-  std::vector<int> group_start;          // walk groups over the sorted order
+  std::vector<int> tables;               // group and member tables of query_kernel
+  int num_groups;
+  long long delta_min, delta_max;
 };
 
 // Builds the packing frame from the coordinate bounds of sources and targets
@@ -447,16 +467,28 @@ static QueryPlan make_plan(const long long *src_bounds, const long long *tgt_bou
                    [](const std::pair<long long, int> &x, const std::pair<long long, int> &y) {
                      return x.first < y.first;
                    });
-  plan.sorted_delta.resize(num_offsets);
-  plan.sorted_offset.resize(num_offsets);
+  std::vector<int> group_start;
   for (int64_t i = 0; i < num_offsets; ++i) {
-    plan.sorted_delta[i] = keyed[i].first;
-    plan.sorted_offset[i] = keyed[i].second;
-    if (i == 0 || keyed[i].first - keyed[plan.group_start.back()].first > kGroupSpan) {
-      plan.group_start.push_back(static_cast<int>(i));
+    if (i == 0 || keyed[i].first - keyed[group_start.back()].first > kGroupSpan) {
+      group_start.push_back(static_cast<int>(i));
     }
   }
-  plan.group_start.push_back(static_cast<int>(num_offsets));
+  plan.num_groups = static_cast<int>(group_start.size());
+  group_start.push_back(static_cast<int>(num_offsets));
+  plan.tables.assign(4 * plan.num_groups + 2 * num_offsets, 0);
+  for (int g = 0; g < plan.num_groups; ++g) {
+    const unsigned long long first = static_cast<unsigned long long>(keyed[group_start[g]].first);
+    plan.tables[4 * g + 0] = static_cast<int>(static_cast<unsigned>(first & 0xffffffffull));
+    plan.tables[4 * g + 1] = static_cast<int>(static_cast<unsigned>(first >> 32));
+    plan.tables[4 * g + 2] = group_start[g];
+    plan.tables[4 * g + 3] = group_start[g + 1] - group_start[g];
+    for (int i = group_start[g]; i < group_start[g + 1]; ++i) {
+      plan.tables[4 * plan.num_groups + 2 * i + 0] = static_cast<int>(keyed[i].first - keyed[group_start[g]].first);
+      plan.tables[4 * plan.num_groups + 2 * i + 1] = keyed[i].second;
+    }
+  }
+  plan.delta_min = num_offsets > 0 ? keyed.front().first : 0;
+  plan.delta_max = num_offsets > 0 ? keyed.back().first : 0;
   return plan;
 }
 
@@ -491,17 +523,17 @@ static void check_query_args(const QueryArgs &a, int64_t num_offsets) {
 }
 
 template <typename CT, typename BT, typename OT>
-static void launch_query(const QueryArgs &a, const QueryPlan &plan, const long long *d_delta,
-                         const int *d_offset, const int *d_group, int num_offsets, OT *kernel_map,
-                         unsigned *tile_counts, int num_tiles, hipStream_t stream) {
+static void launch_query(const QueryArgs &a, const QueryPlan &plan, const int *d_tables,
+                         int num_offsets, OT *kernel_map, unsigned *tile_counts, int num_tiles,
+                         hipStream_t stream) {
   KeyReader<CT, BT> src{static_cast<const CT *>(a.sources), static_cast<const BT *>(a.source_batch_dims),
                         static_cast<int>(a.num_batches), a.num_sources};
   KeyReader<CT, BT> tgt{static_cast<const CT *>(a.targets), static_cast<const BT *>(a.target_batch_dims),
                         static_cast<int>(a.num_batches), a.num_targets};
-  const size_t dyn = sizeof(unsigned) * static_cast<size_t>(num_offsets > 0 ? num_offsets : 1);
+  const size_t dyn = sizeof(unsigned) * (plan.tables.size() + static_cast<size_t>(num_offsets) + 4);
   query_kernel<CT, BT, OT><<<num_tiles, kQueryThreads, dyn, stream>>>(
-      src, tgt, plan.frame, d_delta, d_offset, d_group, static_cast<int>(plan.group_start.size()) - 1,
-      num_offsets, kernel_map, tile_counts, num_tiles);
+      src, tgt, plan.frame, d_tables, plan.num_groups, num_offsets, plan.delta_min, plan.delta_max,
+      kernel_map, tile_counts, num_tiles);
   check_launch("query_kernel");
 }
 
@@ -538,19 +570,14 @@ static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t n
   profile_mark("query_bounds+sync", stream);
   QueryPlan plan = make_plan(bounds, bounds + 8, offsets_host, num_offsets, a.ndim,
                              batched ? a.num_batches : 1);
-  // Upload the plan as kernel arguments of a tiny copy kernel: nothing to
+  // Upload the tables as kernel arguments of a tiny copy kernel: nothing to
   // keep alive on the host and no staging buffer another call could overwrite.
   const int no = static_cast<int>(num_offsets);
-  const int ng = static_cast<int>(plan.group_start.size());
-  std::vector<int> words(2 * no + no + ng);
-  memcpy(words.data(), plan.sorted_delta.data(), sizeof(long long) * no);
-  memcpy(words.data() + 2 * no, plan.sorted_offset.data(), sizeof(int) * no);
-  memcpy(words.data() + 3 * no, plan.group_start.data(), sizeof(int) * ng);
-  int *d_words = scope.alloc<int>(words.size() + 2);
-  upload_ints(words, d_words, stream);
-  const long long *d_delta = reinterpret_cast<const long long *>(d_words);
-  const int *d_offset = d_words + 2 * no;
-  const int *d_group = d_words + 3 * no;
+  MNT_CHECK(plan.tables.size() * sizeof(int) + sizeof(unsigned) * (num_offsets + 4) <= 24 * 1024,
+            "too many kernel offsets (%lld) for the query kernel's table space",
+            static_cast<long long>(num_offsets));
+  int *d_tables = scope.alloc<int>(plan.tables.size());
+  upload_ints(plan.tables, d_tables, stream);
   QueryArgs b = a;
   if (!batched) {
     b.source_batch_dims = nullptr;
@@ -560,9 +587,9 @@ static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t n
   const bool c32 = a.coord_dtype == MNT_INT32;
   const bool b32 = !batched || a.batch_dtype == MNT_INT32;
   const bool o32 = out_dtype == MNT_INT32;
-#define MNT_Q(CT, BT, OT)                                                                        \
-  launch_query<CT, BT, OT>(b, plan, d_delta, d_offset, d_group, no, static_cast<OT *>(kernel_map), \
-                           tile_counts, num_tiles, stream)
+#define MNT_Q(CT, BT, OT)                                                                 \
+  launch_query<CT, BT, OT>(b, plan, d_tables, no, static_cast<OT *>(kernel_map), tile_counts, \
+                           num_tiles, stream)
   if (c32 && b32 && o32) MNT_Q(int32_t, int32_t, int32_t);
   else if (c32 && b32) MNT_Q(int32_t, int32_t, int64_t);
   else if (c32 && o32) MNT_Q(int32_t, int64_t, int32_t);

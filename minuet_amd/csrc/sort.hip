@@ -41,13 +41,12 @@ __global__ __launch_bounds__(kBoundsBlock) void bounds_kernel(
   }
   const long long stride = static_cast<long long>(my_blocks) * kBoundsBlock;
   for (long long i = static_cast<long long>(my_block) * kBoundsBlock + threadIdx.x; i < n; i += stride) {
+    long long c[MNT_MAX_NDIM];
+    load_row<CT>(coords + i * ndim, ndim, c);     // slots past ndim repeat coordinate 0
 #pragma unroll
     for (int k = 0; k < MNT_MAX_NDIM; ++k) {
-      if (k < ndim) {
-        long long v = static_cast<long long>(coords[i * ndim + k]);
-        lo[k] = v < lo[k] ? v : lo[k];
-        hi[k] = v > hi[k] ? v : hi[k];
-      }
+      lo[k] = c[k] < lo[k] ? c[k] : lo[k];
+      hi[k] = c[k] > hi[k] ? c[k] : hi[k];
     }
   }
   __shared__ long long s_lo[kBoundsBlock / kWave][MNT_MAX_NDIM], s_hi[kBoundsBlock / kWave][MNT_MAX_NDIM];
@@ -228,15 +227,14 @@ struct CoordSource {
   SortSpec spec;
   __device__ __forceinline__ void load(long long i, unsigned long long &key, unsigned &val) const {
     const long long row = perm ? static_cast<long long>(perm[i]) : i;
+    long long c[MNT_MAX_NDIM];
+    load_row<CT>(coords + row * spec.ndim, spec.ndim, c);
     unsigned long long k64 = 0;
 #pragma unroll
     for (int k = 0; k < MNT_MAX_NDIM; ++k) {
-      if (k < spec.ndim && spec.mask[k]) {
-        unsigned long long v =
-            static_cast<unsigned long long>(static_cast<long long>(coords[row * spec.ndim + k])) -
-            spec.lo[k];
-        k64 |= (v & spec.mask[k]) << spec.shift[k];
-      }
+      // fields that are not part of this round (or past ndim) have mask 0
+      const unsigned long long v = static_cast<unsigned long long>(c[k]) - spec.lo[k];
+      k64 |= (v & spec.mask[k]) << spec.shift[k];
     }
     if (spec.mask[MNT_MAX_NDIM]) {
       unsigned long long b = batch_of<IT>(row, batch_dims, spec.num_batches);
