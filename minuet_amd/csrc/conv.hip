@@ -134,9 +134,9 @@ __device__ __forceinline__ float to_float(T v) { return static_cast<float>(v); }
 // One lane group per target row: sums its buffer rows in offset order in fp32
 // and writes the row once.  The buffer holds elements of type TB (the output
 // type, or fp32 when the output type is too coarse to round partial products
-// to), the output elements of type T.  With `accumulate` the previous content
-// of the row (the centre-offset product written by the direct GEMM) is the
-// initial value.
+// to), the output elements of type T.  `direct` (nullable) holds one more
+// buffer row per target, indexed by the target itself: the centre-offset
+// product of the shortcut, which needs no rank table.
 template <typename TB, typename T, int VB, int NV, typename IT>
 __global__ __launch_bounds__(256) void scatter_kernel(const TB *__restrict__ buffer,
                                                       unsigned char *__restrict__ targets,
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(256) void scatter_kernel(const TB *__restrict__ buf
                                                       const int *__restrict__ row_start,
                                                       long long num_targets, int num_offsets,
                                                       int channels, int lanes_per_row,
-                                                      int accumulate) {
+                                                      const TB *__restrict__ direct) {
   typedef typename VecOf<VB>::type V;
   constexpr int E = VB / static_cast<int>(sizeof(T));
   constexpr int BB = E * static_cast<int>(sizeof(TB));          // buffer bytes per vector
@@ -158,9 +158,12 @@ __global__ __launch_bounds__(256) void scatter_kernel(const TB *__restrict__ buf
   unsigned char *dst = targets + t * channels * static_cast<long long>(sizeof(T));
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
-    if (accumulate) {
-      V raw = *reinterpret_cast<const V *>(dst + (lr + i * lanes_per_row) * VB);
-      const T *e = reinterpret_cast<const T *>(&raw);
+    if (direct != nullptr) {
+      const TB *piece = direct + t * channels + (lr + i * lanes_per_row) * E;
+      BV raw[NBV];
+#pragma unroll
+      for (int v = 0; v < NBV; ++v) raw[v] = reinterpret_cast<const BV *>(piece)[v];
+      const TB *e = reinterpret_cast<const TB *>(raw);
 #pragma unroll
       for (int k = 0; k < E; ++k) acc[i][k] = to_float(e[k]);
     } else {
@@ -438,14 +441,14 @@ static void launch_gather(const LaneShape &sh, const void *sources, void *buffer
 template <typename TB, typename T, typename IT>
 static void launch_scatter(const LaneShape &sh, const TB *buffer, void *targets, const IT *masks,
                            const int *row_start, int64_t num_targets, int num_offsets, int channels,
-                           int accumulate, hipStream_t stream) {
+                           const TB *direct, hipStream_t stream) {
   if (num_targets == 0) return;
   const unsigned grid = static_cast<unsigned>(div_ceil(num_targets * sh.lanes_per_row, 256));
 #define MNT_S(VB, NV)                                                                              \
   scatter_kernel<TB, T, VB, NV, IT><<<grid, 256, 0, stream>>>(buffer,                              \
                                                           static_cast<unsigned char *>(targets), masks, \
                                                           row_start, num_targets, num_offsets,        \
-                                                          channels, sh.lanes_per_row, accumulate)
+                                                          channels, sh.lanes_per_row, direct)
 #define MNT_SV(VB)                 \
   switch (sh.nv) {                 \
     case 1: MNT_S(VB, 1); break;   \
@@ -601,7 +604,9 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
   const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
   typedef typename BufferOf<T>::type TB;
   T *abuf = scope.alloc<T>(rows * K);
-  TB *cbuf = scope.alloc<TB>(rows * N);
+  // with the shortcut the centre offset's product takes one extra buffer row per target
+  TB *cbuf = scope.alloc<TB>((rows + (plan.shortcut ? static_cast<size_t>(Tn) : 0)) * N);
+  TB *direct = plan.shortcut ? cbuf + rows * N : nullptr;
 
   const LaneShape gsh = lane_shape(gather_tile, K, sizeof(T), sources, abuf, "num_source_features");
   launch_gather<IT>(gsh, sources, abuf, source_masks, d_row_start, S, active,
@@ -613,13 +618,13 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
     std::vector<int> meta = direct_meta(S, static_cast<int>(O - 1));
     int *d_direct = scope.alloc<int>(meta.size());
     upload_ints(meta, d_direct, stream);
-    launch_gemm<T, T>(sources, out, wt, d_direct, meta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
+    launch_gemm<T, TB>(sources, direct, wt, d_direct, meta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
   }
   profile_mark("gemm", stream);
 
   const LaneShape ssh = lane_shape(scatter_tile, N, sizeof(T), cbuf, out, "num_target_features");
   launch_scatter<TB, T, IT>(ssh, cbuf, out, target_masks, d_row_start, Tn, active,
-                            static_cast<int>(N), plan.shortcut ? 1 : 0, stream);
+                            static_cast<int>(N), direct, stream);
   profile_mark("scatter", stream);
 }
 
@@ -751,7 +756,7 @@ static float time_scatter_typed(int64_t tile, const ForwardPlan &plan, const IT 
   Scope scope(stream);
   const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
   typedef typename BufferOf<T>::type TB;
-  TB *cbuf = scope.alloc<TB>(rows * N);
+  TB *cbuf = scope.alloc<TB>((rows + (plan.shortcut ? static_cast<size_t>(Tn) : 0)) * N);
   T *out = scope.alloc<T>(static_cast<size_t>(Tn > 0 ? Tn : 1) * N);
   int *d_row_start = scope.alloc<int>(plan.row_start.size());
   upload_ints(plan.row_start, d_row_start, stream);
@@ -759,7 +764,8 @@ static float time_scatter_typed(int64_t tile, const ForwardPlan &plan, const IT 
   TimerScope timer(stream);
   timer.begin();
   launch_scatter<TB, T, IT>(sh, cbuf, out, target_masks, d_row_start, Tn,
-                            static_cast<int>(plan.active_offsets), static_cast<int>(N), 0, stream);
+                            static_cast<int>(plan.active_offsets), static_cast<int>(N),
+                            plan.shortcut ? cbuf + rows * N : nullptr, stream);
   return timer.end();
 }
 
@@ -775,12 +781,13 @@ static float time_gemm_typed(const ForwardPlan &plan, const T *weights, int64_t 
   T *wt = scope.alloc<T>(static_cast<size_t>(O) * Np * Kp);
   T *abuf = scope.alloc<T>(rows * K);
   TB *cbuf = scope.alloc<TB>(rows * N);
-  T *direct_a = nullptr, *direct_c = nullptr;
+  T *direct_a = nullptr;
+  TB *direct_c = nullptr;
   int *d_direct = nullptr;
   std::vector<int> dmeta;
   if (plan.shortcut) {
     direct_a = scope.alloc<T>(static_cast<size_t>(S) * K);
-    direct_c = scope.alloc<T>(static_cast<size_t>(S) * N);
+    direct_c = scope.alloc<TB>(static_cast<size_t>(S) * N);
     dmeta = direct_meta(S, static_cast<int>(O - 1));
     d_direct = scope.alloc<int>(dmeta.size());
     upload_ints(dmeta, d_direct, stream);
@@ -798,7 +805,7 @@ static float time_gemm_typed(const ForwardPlan &plan, const T *weights, int64_t 
   timer.begin();
   launch_gemm<T, TB>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
   if (plan.shortcut) {
-    launch_gemm<T, T>(direct_a, direct_c, wt, d_direct, dmeta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
+    launch_gemm<T, TB>(direct_a, direct_c, wt, d_direct, dmeta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
   }
   return timer.end();
 }

@@ -1,0 +1,146 @@
+"""Sparse UNet (BASELINE configuration 4 shape, reduced voxel count) against an
+oracle that replays the same network layer by layer on the CPU in float64."""
+import numpy as np
+import pytest
+import torch
+
+import minuet_oracle as orc
+import minuet_amd as minuet
+from helpers import dev, host
+from minuet_amd.nn.functional import _C
+from minuet_amd.synthetic import make_cloud
+from minuet_amd.unet import ResidualBlock, SparseUNet
+
+pytestmark = pytest.mark.gpu
+
+
+class Ref:
+    """float64 activations with coordinates, mirroring SparseTensor."""
+
+    def __init__(self, f, c, bd, stride):
+        self.f, self.c, self.bd, self.stride = f, c, bd, stride
+
+
+def _w(t):
+    return host(t.detach().double())
+
+
+def ref_forward(module, x, levels):
+    """Replays `module` on Ref `x`; `levels` maps a stride to (coords, batch_dims)
+    of the tensors seen at that stride (what the kernel-map cache remembers)."""
+    if isinstance(module, minuet.nn.SparseConv):
+        bias = None if module.bias is None else _w(module.bias)
+        if module.transposed:
+            fine_stride = tuple(a // b for a, b in zip(x.stride, module.stride))
+            fc, fbd = levels[fine_stride]
+            f, c, bd, s = orc.conv_layer(x.c, x.bd, x.f, _w(module.kernel), module.kernel_size,
+                                         stride=module.stride, source_stride=x.stride,
+                                         transposed_from=(fc, fbd, fine_stride), bias=bias)
+        else:
+            f, c, bd, s = orc.conv_layer(x.c, x.bd, x.f, _w(module.kernel), module.kernel_size,
+                                         stride=module.stride, dilation=module.dilation,
+                                         source_stride=x.stride, bias=bias)
+        levels.setdefault(tuple(s), (c, bd))
+        return Ref(f, c, bd, tuple(s))
+    if isinstance(module, minuet.nn.BatchNorm):
+        scale = _w(module.weight) / np.sqrt(_w(module.running_var) + module.eps)
+        return Ref((x.f - _w(module.running_mean)) * scale + _w(module.bias), x.c, x.bd, x.stride)
+    if isinstance(module, minuet.nn.ReLU):
+        return Ref(np.maximum(x.f, 0.0), x.c, x.bd, x.stride)
+    if isinstance(module, torch.nn.Sequential):
+        for child in module:
+            x = ref_forward(child, x, levels)
+        return x
+    if isinstance(module, ResidualBlock):
+        y = ref_forward(module.norm2, ref_forward(module.conv2, ref_forward(
+            module.relu, ref_forward(module.norm1, ref_forward(module.conv1, x, levels), levels), levels),
+            levels), levels)
+        skip = x if module.project is None else ref_forward(module.project, x, levels)
+        return Ref(np.maximum(y.f + skip.f, 0.0), y.c, y.bd, y.stride)
+    if isinstance(module, SparseUNet):
+        levels[x.stride] = (x.c, x.bd)
+        x = ref_forward(module.stem, x, levels)
+        skips = [x]
+        for down, encode in zip(module.down, module.encode):
+            x = ref_forward(encode, ref_forward(down, x, levels), levels)
+            skips.append(x)
+        skips.pop()
+        for up, decode in zip(module.up, module.decode):
+            u = ref_forward(up, x, levels)
+            s = skips.pop()
+            assert np.array_equal(u.c, s.c)
+            x = ref_forward(decode, Ref(np.concatenate([u.f, s.f], axis=1), u.c, u.bd, u.stride), levels)
+        return ref_forward(module.head, x, levels)
+    raise TypeError(type(module))
+
+
+def build_input(scale, seed_shift=0):
+    cloud = make_cloud(4, scale)
+    coords, bd = cloud["coords"], cloud["batch_dims"]
+    order = orc.arg_sort_coordinates(coords, bd)
+    return coords[order], bd
+
+
+def test_unet_fp32_matches_layerwise_oracle():
+    torch.manual_seed(0)
+    coords, bd = build_input(0.02)
+    rng = np.random.default_rng(0)
+    feats = rng.normal(size=(coords.shape[0], 4))
+    net = SparseUNet(4, 16, dtype=torch.float32, device="cuda").eval()
+    for m in net.modules():                      # non-trivial BatchNorm statistics
+        if isinstance(m, minuet.nn.BatchNorm):
+            m.running_mean.uniform_(-0.2, 0.2)
+            m.running_var.uniform_(0.5, 1.5)
+            m.weight.data.uniform_(0.8, 1.2)
+            m.bias.data.uniform_(-0.1, 0.1)
+    cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+    minuet.set_kernel_map_cache(net, cache)
+    idx, sorted_dev = _C.sort_coordinates(dev(coords), dev(bd))
+    assert np.array_equal(host(sorted_dev), coords)          # input was sorted by the oracle
+    x = minuet.SparseTensor(dev(feats).float(), sorted_dev, batch_dims=dev(bd))
+    with torch.no_grad():
+        y = net(x)
+    ref = ref_forward(net, Ref(feats.astype(np.float32).astype(np.float64), coords, bd, (1, 1, 1)), {})
+    np.testing.assert_array_equal(host(y.C), ref.c)
+    np.testing.assert_array_equal(host(y.batch_dims), ref.bd)
+    assert y.stride == (1, 1, 1)
+    err = np.abs(host(y.F.double()) - ref.f).max()
+    assert err <= 2e-4 * np.abs(ref.f).max(), f"end-to-end fp32 error {err:.3e}"
+    # 4 strided levels + 5 submanifold maps, every transposed layer reuses a forward map
+    assert cache.num_coordinate_builds == 4 and cache.num_map_builds == 9
+
+    half = SparseUNet(4, 16, dtype=torch.float16, device="cuda").eval()
+    half.load_state_dict({k: v.half() for k, v in net.state_dict().items()})
+    cache16 = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+    minuet.set_kernel_map_cache(half, cache16)
+    with torch.no_grad():
+        y16 = half(minuet.SparseTensor(x.F.half(), x.C, batch_dims=x.batch_dims))
+    diff = (y16.F.float() - y.F).abs().max().item()
+    assert diff <= 5e-2 * y.F.pow(2).mean().sqrt().item() + 5e-2 * y.F.abs().max().item()
+
+
+def test_unet_full_size_properties():
+    """Configuration-4 size (2 x ~100k voxels, fp16): structural checks that do not
+    need the oracle at this size."""
+    coords, bd = build_input(1.0)
+    net = SparseUNet(4, 32, dtype=torch.float16, device="cuda").eval()
+    cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+    minuet.set_kernel_map_cache(net, cache)
+    feats = torch.randn(coords.shape[0], 4, device="cuda").half()
+    x = minuet.SparseTensor(feats, dev(coords), batch_dims=dev(bd))
+    with torch.no_grad():
+        y = net(x)
+        cache.reset()
+        y2 = net(x)
+    assert torch.equal(y.C, x.C) and y.F.shape == (coords.shape[0], 32)
+    assert torch.isfinite(y.F).all()
+    assert torch.equal(y.F, y2.F)                     # deterministic: no atomics anywhere
+    # linearity of one conv layer in its input (same kernel map, fp32 accumulate)
+    conv = net.encode[0][0].conv1
+    t = minuet.SparseTensor(torch.randn(y.C.shape[0] // 1, 32, device="cuda").half(), x.C, batch_dims=x.batch_dims)
+    a = minuet.SparseTensor(t.F, t.C, stride=1, batch_dims=t.batch_dims)
+    with torch.no_grad():
+        cache.reset()
+        fa = conv(a).F.float()
+        f2a = conv(minuet.SparseTensor(a.F * 2, a.C, batch_dims=a.batch_dims)).F.float()
+    assert (f2a - 2 * fa).abs().max().item() <= 2e-2 * fa.pow(2).mean().sqrt().item()
