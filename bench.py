@@ -45,6 +45,82 @@ def cpu_baseline(coords, offsets, budget_s=12.0):
                       f"{coords.shape[0]}-voxel cloud; median"}
 
 
+def _time_ms(fn, warmup, reps):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    return 1e3 * (time.perf_counter() - t0) / reps
+
+
+def extras(device):
+    """The other two parts of the metric, measured briefly: layer throughput
+    (configurations 1 and 3) and sparse UNet forward latency (configuration 4,
+    kernel-map cache reset before every forward)."""
+    import torch
+    import minuet_amd as minuet
+    from minuet_amd.nn.functional import _C
+    from minuet_amd.synthetic import make_cloud
+    from minuet_amd.unet import SparseUNet
+
+    out = {}
+    with torch.no_grad():
+        # configuration 1: submanifold 3x3x3, 32 -> 32, fp32
+        c1 = torch.from_numpy(make_cloud(1)["coords"]).to(device)
+        _, s1 = _C.sort_coordinates(c1)
+        conv = minuet.nn.SparseConv3d(32, 32, 3, dtype=torch.float32, device=device)
+        cache = minuet.nn.KernelMapCache(3, torch.int32, device)
+        conv.set_kernel_map_cache(cache)
+        conv.tunable_config.update(gather_tile_size=0, scatter_tile_size=0)
+        x = minuet.SparseTensor(torch.randn(s1.shape[0], 32, device=device), s1)
+        warm = _time_ms(lambda: conv(x), 20, 200)
+
+        def cold1():
+            cache.reset()
+            conv(x)
+        cold = _time_ms(cold1, 20, 200)
+        out["config1_layer_fp32"] = {"voxels": int(s1.shape[0]), "ms_map_cached": round(warm, 4),
+                                     "ms_map_included": round(cold, 4),
+                                     "mvoxels_per_s_map_cached": round(s1.shape[0] / warm / 1e3, 1)}
+        # configuration 3: stride-2 down conv 64 -> 128 then transposed 128 -> 64, fp16
+        c3 = torch.from_numpy(make_cloud(3)["coords"]).to(device)
+        _, s3 = _C.sort_coordinates(c3)
+        down = minuet.nn.SparseConv3d(64, 128, 2, stride=2, dtype=torch.float16, device=device)
+        up = minuet.nn.SparseConv(3, 128, 64, 2, stride=2, transposed=True, dtype=torch.float16, device=device)
+        cache3 = minuet.nn.KernelMapCache(3, torch.int32, device)
+        for m in (down, up):
+            m.set_kernel_map_cache(cache3)
+            m.tunable_config.update(gather_tile_size=0, scatter_tile_size=0)
+        x3 = minuet.SparseTensor(torch.randn(s3.shape[0], 64, device=device).half(), s3)
+        pair = _time_ms(lambda: up(down(x3)), 20, 200)
+        out["config3_down_up_fp16"] = {"voxels": int(s3.shape[0]), "ms_map_cached": round(pair, 4),
+                                       "mvoxels_per_s_map_cached": round(s3.shape[0] / pair / 1e3, 1)}
+        # configuration 4: sparse UNet forward, fp16, batch of two scans
+        cloud = make_cloud(4)
+        c4 = torch.from_numpy(cloud["coords"]).to(device)
+        bd = torch.from_numpy(cloud["batch_dims"]).to(device)
+        _, s4 = _C.sort_coordinates(c4, bd)
+        net = SparseUNet(4, 32, dtype=torch.float16, device=device).eval()
+        cache4 = minuet.nn.KernelMapCache(3, torch.int32, device)
+        minuet.set_kernel_map_cache(net, cache4)
+        for m in net.modules():
+            if isinstance(m, minuet.nn.SparseConv):
+                m.tunable_config.update(gather_tile_size=0, scatter_tile_size=0)
+        x4 = minuet.SparseTensor(torch.randn(s4.shape[0], 4, device=device).half(), s4, batch_dims=bd)
+
+        def forward():
+            cache4.reset()
+            net(x4)
+        lat = _time_ms(forward, 5, 30)
+        out["config4_unet_fp16"] = {"voxels": int(s4.shape[0]), "batch": 2,
+                                    "forward_ms_cold_cache": round(lat, 3)}
+    return out
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -52,6 +128,11 @@ def main():
     parser.add_argument("--warmup", type=int, default=100)
     parser.add_argument("--scale", type=float, default=1.0, help="voxel-count scale of the workload")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    parser.add_argument("--no-extras", action="store_true",
+                        help="skip the layer-throughput and UNet-latency side measurements")
+    parser.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
+                        help="also run one plain device copy of this many MiB (a known-size "
+                             "reference for scaling profiler byte counters)")
     args = parser.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every box of this run has a single MI355X and the "
@@ -73,6 +154,14 @@ def main():
     offsets32 = offsets.astype(np.int32)
     coords_dev = torch.from_numpy(coords).to(device)
     n = coords.shape[0]
+
+    if args.copy_calibration > 0:
+        src = torch.empty(args.copy_calibration << 20, dtype=torch.uint8, device=device).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # bring the GPU out of its idle power state before anything is measured
     spin_until = time.perf_counter() + 1.5
@@ -147,6 +236,8 @@ def main():
                                   "frac": round(bytes_map / (wall_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 5),
                                   "stage_ms": {k: round(v, 5) for k, v in stage_ms.items()}}},
     }
+    if not args.no_extras:
+        result["extra"] = extras(device)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(coords, offsets32)
     else:
