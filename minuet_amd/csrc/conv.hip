@@ -100,7 +100,10 @@ template <>
 struct VecOf<2> { typedef unsigned short type; };
 
 // One lane group per source row: the row is read once, then copied to the
-// buffer row of every offset that uses it.
+// buffer row of every offset that uses it.  Rank-table entries are fetched
+// eight offsets at a time so that their latencies overlap.
+constexpr int kMaskBatch = 8;
+
 template <int VB, int NV, typename IT>
 __global__ __launch_bounds__(256) void gather_kernel(const unsigned char *__restrict__ sources,
                                                      unsigned char *__restrict__ buffer,
@@ -117,12 +120,21 @@ __global__ __launch_bounds__(256) void gather_kernel(const unsigned char *__rest
   const unsigned char *src = sources + s * row_bytes;
 #pragma unroll
   for (int i = 0; i < NV; ++i) value[i] = *reinterpret_cast<const V *>(src + (lr + i * lanes_per_row) * VB);
-  for (int o = 0; o < num_offsets; ++o) {
-    const long long d = static_cast<long long>(source_masks[static_cast<long long>(o) * num_sources + s]);
-    if (d < 0) continue;
-    unsigned char *dst = buffer + (static_cast<long long>(row_start[o]) + d) * row_bytes;
+  for (int o0 = 0; o0 < num_offsets; o0 += kMaskBatch) {
+    long long d[kMaskBatch];
 #pragma unroll
-    for (int i = 0; i < NV; ++i) *reinterpret_cast<V *>(dst + (lr + i * lanes_per_row) * VB) = value[i];
+    for (int j = 0; j < kMaskBatch; ++j) {
+      const int o = o0 + j < num_offsets ? o0 + j : num_offsets - 1;
+      d[j] = static_cast<long long>(source_masks[static_cast<long long>(o) * num_sources + s]);
+    }
+#pragma unroll
+    for (int j = 0; j < kMaskBatch; ++j) {
+      if (o0 + j < num_offsets && d[j] >= 0) {
+        unsigned char *dst = buffer + (static_cast<long long>(row_start[o0 + j]) + d[j]) * row_bytes;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) *reinterpret_cast<V *>(dst + (lr + i * lanes_per_row) * VB) = value[i];
+      }
+    }
   }
 }
 
@@ -171,19 +183,46 @@ __global__ __launch_bounds__(256) void scatter_kernel(const TB *__restrict__ buf
       for (int k = 0; k < E; ++k) acc[i][k] = 0.0f;
     }
   }
-  for (int o = 0; o < num_offsets; ++o) {
-    const long long d = static_cast<long long>(target_masks[static_cast<long long>(o) * num_targets + t]);
-    if (d < 0) continue;
-    const TB *src = buffer + (static_cast<long long>(row_start[o]) + d) * channels;
+  // rank-table entries are fetched 32 offsets at a time and buffer rows a
+  // sub-batch at a time (all loads of a batch in flight together), then
+  // summed in offset order
+  constexpr int kMasks = 32;
+  constexpr int kRows = NV * NBV <= 2 ? 8 : 4;
+  for (int o0 = 0; o0 < num_offsets; o0 += kMasks) {
+    int d[kMasks];
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const TB *piece = src + (lr + i * lanes_per_row) * E;
-      BV raw[NBV];
+    for (int j = 0; j < kMasks; ++j) {
+      const int o = o0 + j < num_offsets ? o0 + j : num_offsets - 1;
+      const int v = static_cast<int>(target_masks[static_cast<long long>(o) * num_targets + t]);
+      d[j] = o0 + j < num_offsets ? v : -1;
+    }
 #pragma unroll
-      for (int v = 0; v < NBV; ++v) raw[v] = reinterpret_cast<const BV *>(piece)[v];
-      const TB *e = reinterpret_cast<const TB *>(raw);
+    for (int j0 = 0; j0 < kMasks; j0 += kRows) {
+      if (o0 + j0 >= num_offsets) break;
+      BV raw[kRows][NV][NBV];
 #pragma unroll
-      for (int k = 0; k < E; ++k) acc[i][k] += to_float(e[k]);
+      for (int j = 0; j < kRows; ++j) {
+        if (d[j0 + j] >= 0) {
+          const TB *src = buffer + (static_cast<long long>(row_start[o0 + j0 + j]) + d[j0 + j]) * channels;
+#pragma unroll
+          for (int i = 0; i < NV; ++i) {
+            const TB *piece = src + (lr + i * lanes_per_row) * E;
+#pragma unroll
+            for (int v = 0; v < NBV; ++v) raw[j][i][v] = reinterpret_cast<const BV *>(piece)[v];
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kRows; ++j) {
+        if (d[j0 + j] >= 0) {
+#pragma unroll
+          for (int i = 0; i < NV; ++i) {
+            const TB *e = reinterpret_cast<const TB *>(raw[j][i]);
+#pragma unroll
+            for (int k = 0; k < E; ++k) acc[i][k] += to_float(e[k]);
+          }
+        }
+      }
     }
   }
 #pragma unroll
@@ -235,25 +274,31 @@ struct Mfma<float> {
 
 constexpr int kGemmBlock = 256;
 constexpr int kGemmRows = 128;          // rows of A per workgroup (32 per wavefront)
-constexpr int kChunkBytes = 128;        // bytes of K staged per row and step
+constexpr int kChunkBytes = 128;        // bytes of K per row and step
 constexpr int kLdsRowBytes = kChunkBytes + 16;
+constexpr int kMaxChannelBlocks = 8;    // 32-channel blocks per workgroup (256 channels)
 
 // meta: [G | tile_prefix (G+1) | row_start (G+1) | rows (G) | weight (G)]
 //
-// out^T = W^T x A^T per tile: the first MFMA operand holds 32 output channels,
-// the second 32 data rows, so every lane ends up with 4 consecutive channels
-// of ONE data row per accumulator group and stores them as one vector.
-// The K order inside a 128-byte chunk is permuted identically for both
-// operands (lane half h of step kk reads bytes [32*kk + 16*h, +16) of the
-// row), which leaves the dot products unchanged.
-template <typename T, typename TC, int TN, bool VEC>
+// One workgroup multiplies 128 buffer rows of one offset by that offset's
+// weights: out^T = W^T x A^T.  The first MFMA operand holds 32 output
+// channels, the second 32 data rows, so every lane ends up with 4 consecutive
+// channels of ONE data row per accumulator group and stores them as one vector.
+//
+// A never passes through LDS: lane (r, h) of a wavefront loads, for step kk of
+// a 128-byte chunk of row r, the 16 bytes at offset 32*kk + 16*h — exactly its
+// MFMA operand.  The same K permutation is applied to the weights (lane half
+// h of step kk reads the same bytes of its channel row), which leaves the
+// dot products unchanged.  Only the weights (W^T, K-contiguous, padded) are
+// staged in LDS, shared by the four wavefronts; all NB channel blocks are
+// accumulated in registers, so A is read exactly once.
+template <typename T, typename TC, int NB, bool VEC>
 __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
     const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt,
     const int *__restrict__ meta, int K, int N, int Kp, int Np) {
   constexpr int EPC = 16 / static_cast<int>(sizeof(T));        // elements per 16-byte piece
   constexpr int KC = kChunkBytes / static_cast<int>(sizeof(T));
-  constexpr int NB = TN / 32;
-  __shared__ __align__(16) unsigned char a_lds[kGemmRows * kLdsRowBytes];
+  constexpr int TN = NB * 32;
   __shared__ __align__(16) unsigned char b_lds[TN * kLdsRowBytes];
 
   const int G = meta[0];
@@ -284,6 +329,9 @@ __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
   const int wv = tid >> 6;
   const int r = lane & 31;
   const int h = lane >> 5;
+  const int row = wv * 32 + r;
+  const bool row_ok = row < valid;
+  const T *a_row = a + (row_base + row) * K;
 
   floatx16 acc[NB];
 #pragma unroll
@@ -292,57 +340,79 @@ __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
     for (int j = 0; j < 16; ++j) acc[b][j] = 0.0f;
   }
 
-  for (int k0 = 0; k0 < Kp; k0 += KC) {
-    // stage A: 128 rows x 8 pieces
+  // Software pipeline over the K chunks: the A pieces and the W^T pieces of
+  // chunk i+1 are loaded into registers while chunk i is multiplied.
+  constexpr int kSteps = kChunkBytes / 32;
+  constexpr int kWPieces = (TN * 8 + kGemmBlock - 1) / kGemmBlock;
+  uint4 frag[kSteps], frag_next[kSteps];
+  uint4 wpiece[kWPieces];
+
+  auto load_a = [&](int k0, uint4 (&dst)[kSteps]) {
 #pragma unroll
-    for (int i = 0; i < (kGemmRows * 8) / kGemmBlock; ++i) {
-      const int piece = tid + i * kGemmBlock;
-      const int row = piece >> 3;
-      const int q = piece & 7;
-      const int k = k0 + q * EPC;
+    for (int kk = 0; kk < kSteps; ++kk) {
+      const int k = k0 + kk * 2 * EPC + h * EPC;
       uint4 v = make_uint4(0u, 0u, 0u, 0u);
-      if (row < valid) {
-        const T *src = a + (row_base + row) * K + k;
+      if (row_ok) {
         if (VEC && k + EPC <= K) {
-          v = *reinterpret_cast<const uint4 *>(src);
+          v = *reinterpret_cast<const uint4 *>(a_row + k);
         } else {
           T *e = reinterpret_cast<T *>(&v);
 #pragma unroll
           for (int x = 0; x < EPC; ++x) {
-            if (k + x < K) e[x] = src[x];
+            if (k + x < K) e[x] = a_row[k + x];
           }
         }
       }
-      *reinterpret_cast<uint4 *>(a_lds + row * kLdsRowBytes + q * 16) = v;
+      dst[kk] = v;
     }
-    // stage W^T: TN channels x 8 pieces (always in bounds: padded to [Np][Kp])
+  };
+  auto load_w = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < (TN * 8 + kGemmBlock - 1) / kGemmBlock; ++i) {
+    for (int i = 0; i < kWPieces; ++i) {
+      const int piece = tid + i * kGemmBlock;
+      const int n = piece >> 3;
+      const int q = piece & 7;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (piece < TN * 8 && n0 + n < Np) {
+        v = *reinterpret_cast<const uint4 *>(w_base + static_cast<long long>(n) * Kp + k0 + q * EPC);
+      }
+      wpiece[i] = v;
+    }
+  };
+
+  load_a(0, frag);
+  load_w(0);
+  for (int k0 = 0; k0 < Kp; k0 += KC) {
+    if (k0 > 0) __syncthreads();                   // previous chunk of W^T fully consumed
+#pragma unroll
+    for (int i = 0; i < kWPieces; ++i) {
       const int piece = tid + i * kGemmBlock;
       if (piece < TN * 8) {
-        const int n = piece >> 3;
-        const int q = piece & 7;
-        uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (n0 + n < Np) v = *reinterpret_cast<const uint4 *>(w_base + static_cast<long long>(n) * Kp + k0 + q * EPC);
-        *reinterpret_cast<uint4 *>(b_lds + n * kLdsRowBytes + q * 16) = v;
+        *reinterpret_cast<uint4 *>(b_lds + (piece >> 3) * kLdsRowBytes + (piece & 7) * 16) = wpiece[i];
       }
     }
     __syncthreads();
+    const bool more = k0 + KC < Kp;
+    if (more) {
+      load_a(k0 + KC, frag_next);
+      load_w(k0 + KC);
+    }
 #pragma unroll
-    for (int kk = 0; kk < kChunkBytes / 32; ++kk) {
+    for (int kk = 0; kk < kSteps; ++kk) {
       const int off = kk * 32 + h * 16;
-      const uint4 rows_frag = *reinterpret_cast<const uint4 *>(a_lds + (wv * 32 + r) * kLdsRowBytes + off);
 #pragma unroll
       for (int b = 0; b < NB; ++b) {
         const uint4 chan_frag = *reinterpret_cast<const uint4 *>(b_lds + (b * 32 + r) * kLdsRowBytes + off);
-        acc[b] = Mfma<T>::run(chan_frag, rows_frag, acc[b]);
+        acc[b] = Mfma<T>::run(chan_frag, frag[kk], acc[b]);
       }
     }
-    __syncthreads();
+    if (more) {
+#pragma unroll
+      for (int kk = 0; kk < kSteps; ++kk) frag[kk] = frag_next[kk];
+    }
   }
 
-  const int row = wv * 32 + r;
-  if (row < valid) {
+  if (row_ok) {
     TC *dst = c + (row_base + row) * N;
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
@@ -474,6 +544,17 @@ static void launch_scatter(const LaneShape &sh, const TB *buffer, void *targets,
   check_launch("scatter_kernel");
 }
 
+template <typename T, typename TC, int NB>
+static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int num_tiles, int K, int N,
+                           int Kp, int Np, bool vec, hipStream_t stream) {
+  dim3 grid(num_tiles, static_cast<unsigned>(div_ceil(Np, NB * 32)));
+  if (vec) {
+    grouped_gemm_kernel<T, TC, NB, true><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np);
+  } else {
+    grouped_gemm_kernel<T, TC, NB, false><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np);
+  }
+}
+
 template <typename T, typename TC>
 static void launch_gemm(const T *a, TC *c, const T *wt, const int *meta, int num_tiles, int K, int N,
                         int Kp, int Np, hipStream_t stream) {
@@ -481,24 +562,19 @@ static void launch_gemm(const T *a, TC *c, const T *wt, const int *meta, int num
   const bool vec = (static_cast<int64_t>(K) * sizeof(T)) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(a) % 16 == 0 && N % 4 == 0 &&
                    reinterpret_cast<uintptr_t>(c) % 16 == 0;
-  const int tn = Np >= 128 ? 128 : (Np >= 64 ? 64 : 32);
-  dim3 grid(num_tiles, static_cast<unsigned>(div_ceil(Np, tn)));
-#define MNT_MM(TN)                                                                              \
-  do {                                                                                          \
-    if (vec) {                                                                                  \
-      grouped_gemm_kernel<T, TC, TN, true><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np);  \
-    } else {                                                                                    \
-      grouped_gemm_kernel<T, TC, TN, false><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np); \
-    }                                                                                           \
-  } while (0)
-  if (tn == 128) {
-    MNT_MM(128);
-  } else if (tn == 64) {
-    MNT_MM(64);
-  } else {
-    MNT_MM(32);
+  // all channels in one workgroup up to 256; wider outputs are cut into
+  // 256-channel slices (A is then read once per slice)
+  const int blocks = Np / 32;
+  switch (blocks >= kMaxChannelBlocks ? kMaxChannelBlocks : blocks) {
+    case 1: launch_gemm_nb<T, TC, 1>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
+    case 2: launch_gemm_nb<T, TC, 2>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
+    case 3: launch_gemm_nb<T, TC, 3>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
+    case 4: launch_gemm_nb<T, TC, 4>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
+    case 5: launch_gemm_nb<T, TC, 5>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
+    case 6: launch_gemm_nb<T, TC, 6>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
+    case 7: launch_gemm_nb<T, TC, 7>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
+    default: launch_gemm_nb<T, TC, 8>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
   }
-#undef MNT_MM
   check_launch("grouped_gemm_kernel");
 }
 
