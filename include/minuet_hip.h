@@ -206,6 +206,11 @@ int mnt_cumsum_kernel_padded_sizes(const int64_t *sizes_host, int64_t num_offset
  * the call synchronises once.  gather_tile / scatter_tile are elements per
  * lane (0 = pick automatically).  parallel is accepted for signature
  * compatibility (all offsets run in one grouped launch).
+ * gather_index (nullable, int32[nnz]): the in_idx list of mnt_kernel_map_emit
+ * for the same kernel map, i.e. per offset, in the order of `order`, the
+ * source row of each buffer row.  With it the Gather step is folded into the
+ * GEMM's operand load (no gather buffer, source_masks unused); without it
+ * the three steps run as separate kernels.  Both forms give identical output.
  * Replaces cuda_sparse_convolution_forward,
  * csrc/minuet/torch/cuda_sparse_convolution_forward.cu:136-213 and
  * SparseConvolutionForward::operator(),
@@ -221,6 +226,7 @@ int mnt_sparse_convolution_forward(int64_t gather_tile, int64_t scatter_tile,
                                    int64_t num_offsets, int64_t num_source_features,
                                    int64_t num_target_features,
                                    int index_dtype, int float_dtype,
+                                   const int32_t *gather_index,
                                    void *out, void *stream);
 
 /* Timers used by the autotuner: run the named stage once on scratch buffers and

@@ -11,6 +11,7 @@
 // are multiplied in ONE grouped launch whose tiles never cross an offset, so
 // padded rows are never computed.
 #include <algorithm>
+#include <cstring>
 
 #include "device_utils.h"
 #include "sort.h"
@@ -65,12 +66,24 @@ static void cumsum_padded(const int64_t *sizes, int64_t n, const std::vector<int
 
 // wt[j][n][k] = w[order[j]][k][n], zero-padded to [Np][Kp]: the K-contiguous,
 // transposed form the GEMM stages into LDS.  Takes the place of PermuteWeights
-// (csrc/minuet/cuda/kernels/permute_weights.cuh:8-36).
+// (csrc/minuet/cuda/kernels/permute_weights.cuh:8-36).  The same launch also
+// carries the forward plan's small integer tables (row starts, GEMM group
+// descriptors) to the device as a by-value argument, so that a forward pass
+// needs no separate upload.
+constexpr int kPlanInts = 512;
+struct PlanChunk {
+  int v[kPlanInts];
+};
+
 template <typename T, typename IT>
 __global__ __launch_bounds__(256) void pack_weights_kernel(const T *__restrict__ w,
                                                            const IT *__restrict__ order,
                                                            int num_offsets, int K, int N, int Kp,
-                                                           int Np, T *__restrict__ wt) {
+                                                           int Np, T *__restrict__ wt, PlanChunk plan,
+                                                           int plan_count, int *__restrict__ plan_out) {
+  if (blockIdx.x == 0) {
+    for (int i = threadIdx.x; i < plan_count; i += blockDim.x) plan_out[i] = plan.v[i];
+  }
   const long long total = static_cast<long long>(num_offsets) * Np * Kp;
   const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
   for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride) {
@@ -143,14 +156,15 @@ __global__ __launch_bounds__(256) void gather_kernel(const unsigned char *__rest
 template <typename T>
 __device__ __forceinline__ float to_float(T v) { return static_cast<float>(v); }
 
-// One lane group per target row: sums its buffer rows in offset order in fp32
+// Fallback for kernels with more offsets than the listed form below stages:
+// one lane group per target row sums its buffer rows in offset order in fp32
 // and writes the row once.  The buffer holds elements of type TB (the output
 // type, or fp32 when the output type is too coarse to round partial products
 // to), the output elements of type T.  `direct` (nullable) holds one more
 // buffer row per target, indexed by the target itself: the centre-offset
 // product of the shortcut, which needs no rank table.
 template <typename TB, typename T, int VB, int NV, typename IT>
-__global__ __launch_bounds__(256) void scatter_kernel(const TB *__restrict__ buffer,
+__global__ __launch_bounds__(256) void scatter_wide_kernel(const TB *__restrict__ buffer,
                                                       unsigned char *__restrict__ targets,
                                                       const IT *__restrict__ target_masks,
                                                       const int *__restrict__ row_start,
@@ -235,6 +249,167 @@ __global__ __launch_bounds__(256) void scatter_kernel(const TB *__restrict__ buf
   }
 }
 
+// Scatter in two phases per workgroup of `tile_targets` (a power of two)
+// consecutive targets.
+//   1. Listing: thread (part, target) reads its share of the target's rank
+//      table column (consecutive lanes read consecutive addresses), and the
+//      valid entries are compacted, in offset order, into a per-target list of
+//      buffer rows in LDS.
+//   2. Summation: one lane group per target walks that list, a batch of rows in
+//      flight at a time, sums in fp32 in offset order and writes the row once.
+// The buffer holds elements of type TB (the output type, or fp32 when the
+// output type is too coarse to round partial products to), the output elements
+// of type T.  `direct` (nullable) holds one more buffer row per target, indexed
+// by the target itself: the centre-offset product of the shortcut, which needs
+// no rank table.  Dynamic LDS: (num_offsets + 256 / tile_targets) * tile_targets
+// ints.
+constexpr int kScatterBlock = 256;
+
+template <typename TB, typename T, int VB, int NV, typename IT>
+__global__ __launch_bounds__(kScatterBlock) void scatter_kernel(
+    const TB *__restrict__ buffer, unsigned char *__restrict__ targets,
+    const IT *__restrict__ target_masks, const int *__restrict__ row_start, long long num_targets,
+    int num_offsets, int channels, int lanes_per_row, const TB *__restrict__ direct,
+    int tile_shift) {
+  typedef typename VecOf<VB>::type V;
+  constexpr int E = VB / static_cast<int>(sizeof(T));
+  constexpr int BB = E * static_cast<int>(sizeof(TB));          // buffer bytes per vector
+  typedef typename VecOf<(BB > 16 ? 16 : BB)>::type BV;
+  constexpr int NBV = BB > 16 ? BB / 16 : 1;
+  constexpr int kBatch = 8;
+  extern __shared__ int scatter_lds[];
+  const int tile = 1 << tile_shift;
+  const int parts = kScatterBlock >> tile_shift;
+  int *list = scatter_lds;                       // [num_offsets][tile]
+  int *counts = scatter_lds + num_offsets * tile;  // [parts][tile]
+  const int tid = static_cast<int>(threadIdx.x);
+  const long long t0 = static_cast<long long>(blockIdx.x) << tile_shift;
+
+  {
+    const int tt = tid & (tile - 1);
+    const int part = tid >> tile_shift;
+    const int share = (num_offsets + parts - 1) / parts;
+    const int o_lo = part * share;
+    const int o_hi = min(num_offsets, o_lo + share);
+    const long long t = min(t0 + tt, num_targets - 1);
+    const IT *column = target_masks + t;
+    // the first batch stays in registers across the barrier; later batches
+    // (kernels with more than 8 * parts offsets) are read again
+    int first[kBatch];
+    int count = 0;
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const int o = o_lo + j;
+      first[j] = o < o_hi ? static_cast<int>(column[static_cast<long long>(o) * num_targets]) : -1;
+    }
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) count += first[j] >= 0 ? 1 : 0;
+    for (int o0 = o_lo + kBatch; o0 < o_hi; o0 += kBatch) {
+      int more[kBatch];
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        const int o = o0 + j;
+        more[j] = o < o_hi ? static_cast<int>(column[static_cast<long long>(o) * num_targets]) : -1;
+      }
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) count += more[j] >= 0 ? 1 : 0;
+    }
+    counts[part * tile + tt] = count;
+    __syncthreads();
+    int at = 0;
+    for (int p = 0; p < part; ++p) at += counts[p * tile + tt];
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      if (first[j] >= 0) {
+        list[at * tile + tt] = row_start[o_lo + j] + first[j];
+        ++at;
+      }
+    }
+    for (int o0 = o_lo + kBatch; o0 < o_hi; o0 += kBatch) {
+      int more[kBatch];
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        const int o = o0 + j;
+        more[j] = o < o_hi ? static_cast<int>(column[static_cast<long long>(o) * num_targets]) : -1;
+      }
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        if (more[j] >= 0) {
+          list[at * tile + tt] = row_start[o0 + j] + more[j];
+          ++at;
+        }
+      }
+    }
+    __syncthreads();
+  }
+
+  constexpr int kRows = NV * NBV <= 2 ? 8 : 4;
+  const int groups = kScatterBlock / lanes_per_row;
+  const int group = tid / lanes_per_row;
+  const int lr = tid - group * lanes_per_row;
+  if (group >= groups) return;
+  for (int tt = group; tt < tile; tt += groups) {
+    const long long t = t0 + tt;
+    if (t >= num_targets) break;
+    int n = 0;
+    for (int p = 0; p < parts; ++p) n += counts[p * tile + tt];
+    float acc[NV][E];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      if (direct != nullptr) {
+        const TB *piece = direct + t * channels + (lr + i * lanes_per_row) * E;
+        BV raw[NBV];
+#pragma unroll
+        for (int v = 0; v < NBV; ++v) raw[v] = reinterpret_cast<const BV *>(piece)[v];
+        const TB *e = reinterpret_cast<const TB *>(raw);
+#pragma unroll
+        for (int k = 0; k < E; ++k) acc[i][k] = to_float(e[k]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < E; ++k) acc[i][k] = 0.0f;
+      }
+    }
+    for (int k0 = 0; k0 < n; k0 += kRows) {
+      int row[kRows];
+#pragma unroll
+      for (int j = 0; j < kRows; ++j) row[j] = k0 + j < n ? list[(k0 + j) * tile + tt] : -1;
+      BV raw[kRows][NV][NBV];
+#pragma unroll
+      for (int j = 0; j < kRows; ++j) {
+        if (row[j] >= 0) {
+          const TB *src = buffer + static_cast<long long>(row[j]) * channels;
+#pragma unroll
+          for (int i = 0; i < NV; ++i) {
+            const TB *piece = src + (lr + i * lanes_per_row) * E;
+#pragma unroll
+            for (int v = 0; v < NBV; ++v) raw[j][i][v] = reinterpret_cast<const BV *>(piece)[v];
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kRows; ++j) {
+        if (row[j] >= 0) {
+#pragma unroll
+          for (int i = 0; i < NV; ++i) {
+            const TB *e = reinterpret_cast<const TB *>(raw[j][i]);
+#pragma unroll
+            for (int k = 0; k < E; ++k) acc[i][k] += to_float(e[k]);
+          }
+        }
+      }
+    }
+    unsigned char *dst = targets + t * channels * static_cast<long long>(sizeof(T));
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      V raw;
+      T *e = reinterpret_cast<T *>(&raw);
+#pragma unroll
+      for (int k = 0; k < E; ++k) e[k] = static_cast<T>(acc[i][k]);
+      *reinterpret_cast<V *>(dst + (lr + i * lanes_per_row) * VB) = raw;
+    }
+  }
+}
+
 // Element type of the GEMM-output / scatter-input buffer for feature type T.
 // bfloat16 keeps only 8 significant bits, so rounding every partial product
 // to it would cost more accuracy than the output rounding itself.
@@ -278,7 +453,7 @@ constexpr int kChunkBytes = 128;        // bytes of K per row and step
 constexpr int kLdsRowBytes = kChunkBytes + 16;
 constexpr int kMaxChannelBlocks = 8;    // 32-channel blocks per workgroup (256 channels)
 
-// meta: [G | tile_prefix (G+1) | row_start (G+1) | rows (G) | weight (G)]
+// meta: [G | tile_prefix (G+1) | row_start (G+1) | rows (G) | weight (G) | list_start (G)]
 //
 // One workgroup multiplies 128 buffer rows of one offset by that offset's
 // weights: out^T = W^T x A^T.  The first MFMA operand holds 32 output
@@ -292,10 +467,16 @@ constexpr int kMaxChannelBlocks = 8;    // 32-channel blocks per workgroup (256 
 // dot products unchanged.  Only the weights (W^T, K-contiguous, padded) are
 // staged in LDS, shared by the four wavefronts; all NB channel blocks are
 // accumulated in registers, so A is read exactly once.
+//
+// With `gather_index` (nullable) the Gather step is folded into the A load:
+// data row i of group g is then row gather_index[list_start[g] + i] of `a`
+// (the source features) instead of buffer row row_start[g] + i, and no gather
+// buffer exists.  The output rows stay in buffer order either way.
 template <typename T, typename TC, int NB, bool VEC>
 __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
     const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt,
-    const int *__restrict__ meta, int K, int N, int Kp, int Np) {
+    const int *__restrict__ meta, int K, int N, int Kp, int Np,
+    const int *__restrict__ gather_index) {
   constexpr int EPC = 16 / static_cast<int>(sizeof(T));        // elements per 16-byte piece
   constexpr int KC = kChunkBytes / static_cast<int>(sizeof(T));
   constexpr int TN = NB * 32;
@@ -306,6 +487,7 @@ __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
   const int *row_start = tile_prefix + G + 1;
   const int *rows = row_start + G + 1;
   const int *weight = rows + G;
+  const int *list_start = weight + G;
 
   const int tile = blockIdx.x;
   int lo = 0, hi = G - 1;
@@ -331,7 +513,11 @@ __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
   const int h = lane >> 5;
   const int row = wv * 32 + r;
   const bool row_ok = row < valid;
-  const T *a_row = a + (row_base + row) * K;
+  long long a_index = row_base + row;
+  if (gather_index != nullptr) {
+    a_index = row_ok ? gather_index[static_cast<long long>(list_start[g]) + r0 + row] : 0;
+  }
+  const T *a_row = a + a_index * K;
 
   floatx16 acc[NB];
 #pragma unroll
@@ -508,17 +694,32 @@ static void launch_gather(const LaneShape &sh, const void *sources, void *buffer
   check_launch("gather_kernel");
 }
 
+// Largest kernel (offset count) the listed scatter stages in LDS; larger ones
+// take the direct form.
+constexpr int kScatterListedOffsets = 343;
+
 template <typename TB, typename T, typename IT>
 static void launch_scatter(const LaneShape &sh, const TB *buffer, void *targets, const IT *masks,
                            const int *row_start, int64_t num_targets, int num_offsets, int channels,
                            const TB *direct, hipStream_t stream) {
   if (num_targets == 0) return;
-  const unsigned grid = static_cast<unsigned>(div_ceil(num_targets * sh.lanes_per_row, 256));
-#define MNT_S(VB, NV)                                                                              \
-  scatter_kernel<TB, T, VB, NV, IT><<<grid, 256, 0, stream>>>(buffer,                              \
-                                                          static_cast<unsigned char *>(targets), masks, \
-                                                          row_start, num_targets, num_offsets,        \
-                                                          channels, sh.lanes_per_row, direct)
+  const bool listed = num_offsets <= kScatterListedOffsets && sh.lanes_per_row <= kScatterBlock;
+  const int tile_shift = num_offsets <= 128 ? 6 : 5;
+  const unsigned grid =
+      listed ? static_cast<unsigned>(div_ceil(num_targets, int64_t{1} << tile_shift))
+             : static_cast<unsigned>(div_ceil(num_targets * sh.lanes_per_row, 256));
+  const size_t lds =
+      static_cast<size_t>(num_offsets + (kScatterBlock >> tile_shift)) * sizeof(int) << tile_shift;
+#define MNT_S(VB, NV)                                                                               \
+  if (listed) {                                                                                     \
+    scatter_kernel<TB, T, VB, NV, IT><<<grid, kScatterBlock, lds, stream>>>(                        \
+        buffer, static_cast<unsigned char *>(targets), masks, row_start, num_targets, num_offsets,  \
+        channels, sh.lanes_per_row, direct, tile_shift);                                            \
+  } else {                                                                                          \
+    scatter_wide_kernel<TB, T, VB, NV, IT><<<grid, 256, 0, stream>>>(                               \
+        buffer, static_cast<unsigned char *>(targets), masks, row_start, num_targets, num_offsets,  \
+        channels, sh.lanes_per_row, direct);                                                        \
+  }
 #define MNT_SV(VB)                 \
   switch (sh.nv) {                 \
     case 1: MNT_S(VB, 1); break;   \
@@ -546,18 +747,20 @@ static void launch_scatter(const LaneShape &sh, const TB *buffer, void *targets,
 
 template <typename T, typename TC, int NB>
 static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int num_tiles, int K, int N,
-                           int Kp, int Np, bool vec, hipStream_t stream) {
+                           int Kp, int Np, bool vec, const int *gather_index, hipStream_t stream) {
   dim3 grid(num_tiles, static_cast<unsigned>(div_ceil(Np, NB * 32)));
   if (vec) {
-    grouped_gemm_kernel<T, TC, NB, true><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np);
+    grouped_gemm_kernel<T, TC, NB, true><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np,
+                                                                          gather_index);
   } else {
-    grouped_gemm_kernel<T, TC, NB, false><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np);
+    grouped_gemm_kernel<T, TC, NB, false><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np,
+                                                                          gather_index);
   }
 }
 
 template <typename T, typename TC>
 static void launch_gemm(const T *a, TC *c, const T *wt, const int *meta, int num_tiles, int K, int N,
-                        int Kp, int Np, hipStream_t stream) {
+                        int Kp, int Np, const int *gather_index, hipStream_t stream) {
   if (num_tiles == 0) return;
   const bool vec = (static_cast<int64_t>(K) * sizeof(T)) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(a) % 16 == 0 && N % 4 == 0 &&
@@ -566,14 +769,14 @@ static void launch_gemm(const T *a, TC *c, const T *wt, const int *meta, int num
   // 256-channel slices (A is then read once per slice)
   const int blocks = Np / 32;
   switch (blocks >= kMaxChannelBlocks ? kMaxChannelBlocks : blocks) {
-    case 1: launch_gemm_nb<T, TC, 1>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
-    case 2: launch_gemm_nb<T, TC, 2>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
-    case 3: launch_gemm_nb<T, TC, 3>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
-    case 4: launch_gemm_nb<T, TC, 4>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
-    case 5: launch_gemm_nb<T, TC, 5>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
-    case 6: launch_gemm_nb<T, TC, 6>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
-    case 7: launch_gemm_nb<T, TC, 7>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
-    default: launch_gemm_nb<T, TC, 8>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, stream); break;
+    case 1: launch_gemm_nb<T, TC, 1>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
+    case 2: launch_gemm_nb<T, TC, 2>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
+    case 3: launch_gemm_nb<T, TC, 3>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
+    case 4: launch_gemm_nb<T, TC, 4>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
+    case 5: launch_gemm_nb<T, TC, 5>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
+    case 6: launch_gemm_nb<T, TC, 6>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
+    case 7: launch_gemm_nb<T, TC, 7>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
+    default: launch_gemm_nb<T, TC, 8>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
   }
   check_launch("grouped_gemm_kernel");
 }
@@ -610,15 +813,20 @@ static ForwardPlan make_forward_plan(const int64_t *sizes, int64_t num_offsets, 
     if (sizes[j] > 0) groups.push_back(static_cast<int>(j));
   }
   const int G = static_cast<int>(groups.size());
-  plan.meta.assign(1 + (G + 1) + (G + 1) + G + G, 0);
+  plan.meta.assign(1 + (G + 1) + (G + 1) + G + G + G, 0);
   plan.meta[0] = G;
   int *tile_prefix = plan.meta.data() + 1;
   int *row_start = tile_prefix + G + 1;
   int *rows = row_start + G + 1;
   int *weight = rows + G;
+  int *list_start = weight + G;
   int tiles = 0;
+  int64_t listed = 0;
+  int next = 0;
   for (int i = 0; i < G; ++i) {
     const int j = groups[i];
+    for (; next < j; ++next) listed += sizes[next];
+    list_start[i] = static_cast<int>(listed);
     tile_prefix[i] = tiles;
     row_start[i] = static_cast<int>(plan.cum[j]);
     rows[i] = static_cast<int>(sizes[j]);
@@ -634,7 +842,7 @@ static ForwardPlan make_forward_plan(const int64_t *sizes, int64_t num_offsets, 
 static std::vector<int> direct_meta(int64_t rows, int weight_index) {
   // one group: all rows of the source tensor against one weight matrix
   std::vector<int> meta = {1, 0, static_cast<int>(div_ceil(rows, kGemmRows)), 0, static_cast<int>(rows),
-                           static_cast<int>(rows), weight_index};
+                           static_cast<int>(rows), weight_index, 0};
   return meta;
 }
 
@@ -655,8 +863,8 @@ static void read_sizes(const void *sizes_dev, int index_dtype, int64_t num_offse
 template <typename T, typename IT>
 static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const ForwardPlan &plan,
                           const T *sources, const T *weights, const IT *source_masks,
-                          const IT *target_masks, const IT *order, int64_t S, int64_t Tn, int64_t O,
-                          int64_t K, int64_t N, T *out, hipStream_t stream) {
+                          const IT *target_masks, const IT *order, const int *gather_index, int64_t S,
+                          int64_t Tn, int64_t O, int64_t K, int64_t N, T *out, hipStream_t stream) {
   Scope scope(stream);
   const int kc = kChunkBytes / static_cast<int>(sizeof(T));
   const int Kp = static_cast<int>(div_ceil(K, kc) * kc);
@@ -664,37 +872,61 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
   const int active = static_cast<int>(plan.active_offsets);
 
   profile_mark("enter:forward", stream);
+  // one integer table for the whole pass: row starts, GEMM groups, and the
+  // single-group descriptor of the centre-offset product
+  std::vector<int> ints(plan.row_start);
+  const size_t meta_at = ints.size();
+  ints.insert(ints.end(), plan.meta.begin(), plan.meta.end());
+  const size_t direct_at = ints.size();
+  std::vector<int> dmeta;
+  if (plan.shortcut) {
+    dmeta = direct_meta(S, static_cast<int>(O - 1));
+    ints.insert(ints.end(), dmeta.begin(), dmeta.end());
+  }
+  int *d_ints = scope.alloc<int>(ints.size());
+  int *d_row_start = d_ints;
+  int *d_meta = d_ints + meta_at;
+  int *d_direct = d_ints + direct_at;
   T *wt = scope.alloc<T>(static_cast<size_t>(O) * Np * Kp);
   {
+    PlanChunk chunk;
+    int count = 0;
+    if (ints.size() <= static_cast<size_t>(kPlanInts)) {
+      count = static_cast<int>(ints.size());
+      std::memcpy(chunk.v, ints.data(), ints.size() * sizeof(int));
+    } else {
+      upload_ints(ints, d_ints, stream);
+    }
     const long long total = static_cast<long long>(O) * Np * Kp;
     pack_weights_kernel<T, IT><<<grid_for(total, 256, 4096), 256, 0, stream>>>(
-        weights, order, static_cast<int>(O), static_cast<int>(K), static_cast<int>(N), Kp, Np, wt);
+        weights, order, static_cast<int>(O), static_cast<int>(K), static_cast<int>(N), Kp, Np, wt, chunk,
+        count, d_ints);
     check_launch("pack_weights_kernel");
   }
-  int *d_row_start = scope.alloc<int>(plan.row_start.size());
-  upload_ints(plan.row_start, d_row_start, stream);
-  int *d_meta = scope.alloc<int>(plan.meta.size());
-  upload_ints(plan.meta, d_meta, stream);
   profile_mark("pack_weights", stream);
 
   const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
   typedef typename BufferOf<T>::type TB;
-  T *abuf = scope.alloc<T>(rows * K);
   // with the shortcut the centre offset's product takes one extra buffer row per target
   TB *cbuf = scope.alloc<TB>((rows + (plan.shortcut ? static_cast<size_t>(Tn) : 0)) * N);
   TB *direct = plan.shortcut ? cbuf + rows * N : nullptr;
 
-  const LaneShape gsh = lane_shape(gather_tile, K, sizeof(T), sources, abuf, "num_source_features");
-  launch_gather<IT>(gsh, sources, abuf, source_masks, d_row_start, S, active,
-                    static_cast<int>(K * sizeof(T)), stream);
-  profile_mark("gather", stream);
-
-  launch_gemm<T, TB>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
+  if (gather_index != nullptr) {
+    // Gather folded into the GEMM's A load: no gather buffer
+    launch_gemm<T, TB>(sources, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp,
+                       Np, gather_index, stream);
+  } else {
+    T *abuf = scope.alloc<T>(rows * K);
+    const LaneShape gsh = lane_shape(gather_tile, K, sizeof(T), sources, abuf, "num_source_features");
+    launch_gather<IT>(gsh, sources, abuf, source_masks, d_row_start, S, active,
+                      static_cast<int>(K * sizeof(T)), stream);
+    profile_mark("gather", stream);
+    launch_gemm<T, TB>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np,
+                       nullptr, stream);
+  }
   if (plan.shortcut) {
-    std::vector<int> meta = direct_meta(S, static_cast<int>(O - 1));
-    int *d_direct = scope.alloc<int>(meta.size());
-    upload_ints(meta, d_direct, stream);
-    launch_gemm<T, TB>(sources, direct, wt, d_direct, meta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
+    launch_gemm<T, TB>(sources, direct, wt, d_direct, dmeta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np,
+                       nullptr, stream);
   }
   profile_mark("gemm", stream);
 
@@ -750,7 +982,8 @@ extern "C" int mnt_sparse_convolution_forward(
     int has_threshold, double threshold, const void *sources, const void *weights,
     const void *source_masks, const void *target_masks, const void *kernel_map_order,
     const void *kernel_map_sizes, const int64_t *sizes_host, int64_t S, int64_t T, int64_t O,
-    int64_t K, int64_t N, int index_dtype, int float_dtype, void *out, void *stream_) {
+    int64_t K, int64_t N, int index_dtype, int float_dtype, const int32_t *gather_index, void *out,
+    void *stream_) {
   (void)parallel;
   return guarded([&] {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -778,7 +1011,7 @@ extern "C" int mnt_sparse_convolution_forward(
   forward_typed<FT, IT>(gather_tile, scatter_tile, plan, static_cast<const FT *>(sources),          \
                         static_cast<const FT *>(weights), static_cast<const IT *>(source_masks),    \
                         static_cast<const IT *>(target_masks), static_cast<const IT *>(kernel_map_order), \
-                        S, T, O, K, N, static_cast<FT *>(out), stream)
+                        gather_index, S, T, O, K, N, static_cast<FT *>(out), stream)
     MNT_DISPATCH_FI(float_dtype, index_dtype, MNT_CALL);
 #undef MNT_CALL
   });
@@ -870,7 +1103,8 @@ static float time_gemm_typed(const ForwardPlan &plan, const T *weights, int64_t 
   }
   const long long total = static_cast<long long>(O) * Np * Kp;
   pack_weights_kernel<T, int32_t><<<grid_for(total, 256, 4096), 256, 0, stream>>>(
-      weights, nullptr, static_cast<int>(O), static_cast<int>(K), static_cast<int>(N), Kp, Np, wt);
+      weights, nullptr, static_cast<int>(O), static_cast<int>(K), static_cast<int>(N), Kp, Np, wt,
+      PlanChunk{}, 0, nullptr);
   check_launch("pack_weights_kernel");
   // operands of a timing run are scratch: clear them so no NaN patterns slow or trap anything
   MNT_HIP(hipMemsetAsync(abuf, 0, rows * K * sizeof(T), stream));
@@ -879,9 +1113,11 @@ static float time_gemm_typed(const ForwardPlan &plan, const T *weights, int64_t 
   upload_ints(plan.meta, d_meta, stream);
   TimerScope timer(stream);
   timer.begin();
-  launch_gemm<T, TB>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
+  launch_gemm<T, TB>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np,
+                     nullptr, stream);
   if (plan.shortcut) {
-    launch_gemm<T, TB>(direct_a, direct_c, wt, d_direct, dmeta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np, stream);
+    launch_gemm<T, TB>(direct_a, direct_c, wt, d_direct, dmeta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np,
+                       nullptr, stream);
   }
   return timer.end();
 }

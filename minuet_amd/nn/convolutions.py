@@ -130,7 +130,7 @@ class KernelMapCache(object):
         target_coordinates = target_coordinates.contiguous()
         built = _C.kernel_map_build(source_coordinates, target_coordinates, offsets,
                                     source_batch_dims, target_batch_dims, reorder=reorder,
-                                    source_bounds=self._known_bounds(source_coordinates),
+                                    want_lists=True, source_bounds=self._known_bounds(source_coordinates),
                                     target_bounds=self._known_bounds(target_coordinates))
         self.num_map_builds += 1
         if source_coordinates.shape[0] > 0 and target_coordinates.shape[0] > 0:
@@ -142,7 +142,12 @@ class KernelMapCache(object):
         sizes = cast(built["sizes"])
         sizes.host_sizes = tuple(int(v) for v in built["sizes_host"])
         order = cast(built["order"]) if reorder else None
-        entry = (cast(built["source_masks"]), cast(built["target_masks"]), order, sizes)
+        source_masks, target_masks = cast(built["source_masks"]), cast(built["target_masks"])
+        # buffer row -> feature row on either side of the map: what a layer
+        # (forward or transposed) gathers through
+        source_masks.gather_index = built["in_idx"]
+        target_masks.gather_index = built["out_idx"]
+        entry = (source_masks, target_masks, order, sizes)
         self._kernel_maps_cache[key] = entry
         return entry
 

@@ -59,7 +59,7 @@ SIGNATURES = {
     "mnt_cumsum_kernel_padded_sizes": (_int, [_pi64, _i64, _pi64, _i64, _pi64]),
     "mnt_sparse_convolution_forward": (_int, [_i64, _i64, _int, _i64, _int, _dbl, _vp, _vp, _vp, _vp,
                                               _vp, _vp, _pi64, _i64, _i64, _i64, _i64, _i64, _int,
-                                              _int, _vp, _vp]),
+                                              _int, _vp, _vp, _vp]),
     "mnt_time_gather": (_int, [_i64, _int, _int, _dbl, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
                                _int, _pf, _vp]),
     "mnt_time_scatter": (_int, [_i64, _int, _int, _dbl, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
@@ -518,9 +518,12 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
                                     target_masks: torch.Tensor,
                                     kernel_map_order: Optional[torch.Tensor],
                                     kernel_map_sizes: torch.Tensor,
-                                    kernel_map_sizes_host=None) -> torch.Tensor:
+                                    kernel_map_sizes_host=None,
+                                    gather_index: Optional[torch.Tensor] = None) -> torch.Tensor:
     """csrc/minuet/torch/cuda_sparse_convolution_forward.cu:136-213.  The extra
-    ``kernel_map_sizes_host`` spares the device read-back of the sizes."""
+    ``kernel_map_sizes_host`` spares the device read-back of the sizes;
+    ``gather_index`` (int32, the kernel map's source row per buffer row) folds
+    the Gather step into the GEMM."""
     fn = "CUDASparseConvolutionForward"
     _ensure_ndim("sources", sources, 2)
     S, T, O, K, N = _conv_shapes(weights, source_masks, target_masks, kernel_map_sizes)
@@ -540,14 +543,20 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
     icode = _int_code(itype, "index", fn)
     out = torch.empty((T, N), dtype=weights.dtype, device=device)
     keep, sizes_ptr = _host_sizes_arg(kernel_map_sizes_host, O)
+    if gather_index is not None:
+        if gather_index.dtype != torch.int32 or gather_index.device != device:
+            _fail("gather_index must be an int32 tensor on the device of the features")
+        if kernel_map_sizes_host is None or gather_index.numel() != int(sum(kernel_map_sizes_host)):
+            _fail("gather_index needs the host sizes and one entry per kernel map hit")
+        gather_index = gather_index.contiguous()
     with torch.cuda.device(device):
         _check(load_library().mnt_sparse_convolution_forward(
             int(gather_tile_size), int(scatter_tile_size), 1 if allow_shortcut_matmul else 0,
             int(parallel), 0 if threshold is None else 1,
             0.0 if threshold is None else float(threshold), _ptr(sources), _ptr(weights),
             _ptr(source_masks), _ptr(target_masks), _ptr(kernel_map_order),
-            _ptr(kernel_map_sizes), sizes_ptr, S, T, O, K, N, icode, fcode, _ptr(out),
-            _stream(device)))
+            _ptr(kernel_map_sizes), sizes_ptr, S, T, O, K, N, icode, fcode, _ptr(gather_index),
+            _ptr(out), _stream(device)))
     del keep
     return out
 

@@ -60,16 +60,20 @@ def sparse_convolution_forward(sources: torch.Tensor, weights: torch.Tensor,
     """Output features ``[N_out, C_out]`` of one sparse convolution given the rank
     tables of its kernel map (reference: convolution.py:110-155).  A host copy
     of the sizes attached to ``kernel_map_sizes`` as attribute ``host_sizes``
-    (``KernelMapCache`` does that) avoids a device read-back per call."""
+    (``KernelMapCache`` does that) avoids a device read-back per call; an int32
+    tensor attached to ``source_masks`` as attribute ``gather_index`` (the
+    source row of every buffer row, also from ``KernelMapCache``) lets the GEMM
+    read the source rows directly instead of going through a gather buffer."""
     if not sources.is_cuda:
         raise NotImplementedError
     if parallel is None:
         parallel = GEMM_PARALLEL_LEVEL
     host_sizes = getattr(kernel_map_sizes, "host_sizes", None)
+    gather_index = getattr(source_masks, "gather_index", None) if host_sizes is not None else None
     if kernel_map_order is not None:
         kernel_map_order = kernel_map_order.contiguous()
     return _C.cuda_sparse_convolution_forward(
         gather_tile_size, scatter_tile_size, allow_shortcut_matmul, parallel, threshold,
         sources.contiguous(), weights.contiguous(), source_masks.contiguous(),
         target_masks.contiguous(), kernel_map_order, kernel_map_sizes.contiguous(),
-        kernel_map_sizes_host=host_sizes)
+        kernel_map_sizes_host=host_sizes, gather_index=gather_index)

@@ -47,6 +47,26 @@ def make_layer_case(seed, n, extent, kernel, cin, cout, kind, stride=1, batched=
     return src, sbd, tgt, tbd, off, feats, weights
 
 
+def with_host_sizes(sizes):
+    tensor = dev(sizes)
+    tensor.host_sizes = tuple(int(v) for v in sizes)
+    return tensor
+
+
+def with_gather_index(source_masks, sizes):
+    """Rank table on the device carrying its inverse (buffer row -> source row),
+    derived here from the table itself."""
+    start = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+    index = np.full(int(start[-1]), -1, dtype=np.int32)
+    for j in range(source_masks.shape[0]):
+        hit = np.nonzero(source_masks[j] >= 0)[0]
+        index[start[j] + source_masks[j, hit]] = hit
+    assert (index >= 0).all()
+    tensor = dev(source_masks)
+    tensor.gather_index = dev(index)
+    return tensor
+
+
 @pytest.mark.parametrize("kind", ["fp32", "fp16", "bf16"])
 @pytest.mark.parametrize("kernel,stride,cin,cout,n,extent", [
     (3, 1, 32, 32, 20000, 60), (3, 1, 64, 64, 6000, 25), (2, 2, 64, 128, 20000, 50),
@@ -67,6 +87,14 @@ def test_forward_functional(kind, kernel, stride, cin, cout, n, extent):
                 allow_shortcut_matmul=shortcut and stride == 1, threshold=threshold)
             assert out.dtype == dtype and out.shape == (tgt.shape[0], cout)
             assert_features_close(out, ref, kind)
+            # Gather folded into the GEMM: same products, same summation order
+            fused = F.sparse_convolution_forward(
+                sources=dev(feats).to(dtype), weights=dev(weights).to(dtype),
+                source_masks=with_gather_index(esm, esizes), target_masks=dev(etm),
+                kernel_map_order=dev(eorder), kernel_map_sizes=with_host_sizes(esizes),
+                gather_tile_size=0, scatter_tile_size=0,
+                allow_shortcut_matmul=shortcut and stride == 1, threshold=threshold)
+            assert torch.equal(fused, out)
 
 
 @pytest.mark.parametrize("tile", [1, 2, 4, 8, 16, 32])
