@@ -33,6 +33,12 @@ extern "C" {
 #define MNT_FLOAT16 1
 #define MNT_BFLOAT16 2
 
+/* activation applied by the fused forward's epilogue */
+#define MNT_ACT_NONE 0
+#define MNT_ACT_RELU 1
+#define MNT_ACT_LEAKY_RELU 2
+#define MNT_ACT_RELU6 3
+
 #define MNT_MAX_NDIM 4
 
 /* ---- library ----------------------------------------------------------- */
@@ -228,6 +234,35 @@ int mnt_sparse_convolution_forward(int64_t gather_tile, int64_t scatter_tile,
                                    int index_dtype, int float_dtype,
                                    const int32_t *gather_index,
                                    void *out, void *stream);
+
+/* The same forward with an epilogue applied to every summed output row before
+ * it is rounded to float_dtype:
+ *   out[t][c] = act(sum[t][c] * channel_scale[c] + channel_shift[c] + residual[t][c])
+ * channel_scale / channel_shift: fp32[Cout] device vectors, residual: [T, Cout]
+ * of float_dtype (16-byte aligned); each is skipped when NULL.  activation is
+ * one of MNT_ACT_*; negative_slope is used by MNT_ACT_LEAKY_RELU only.  This is
+ * how the layers that follow a convolution in the reference's networks
+ * (the bias add of minuet/nn/convolutions.py:496-497, an inference-mode
+ * minuet/nn/normalizations.py BatchNorm, minuet/nn/activations.py ReLU /
+ * LeakyReLU / ReLU6 and a residual sum) are absorbed into Scatter's single
+ * write of the output row. */
+int mnt_sparse_convolution_forward_fused(int64_t gather_tile, int64_t scatter_tile,
+                                         int allow_shortcut_matmul, int64_t parallel,
+                                         int has_threshold, double threshold,
+                                         const void *sources, const void *weights,
+                                         const void *source_masks, const void *target_masks,
+                                         const void *kernel_map_order,
+                                         const void *kernel_map_sizes,
+                                         const int64_t *sizes_host,
+                                         int64_t num_sources, int64_t num_targets,
+                                         int64_t num_offsets, int64_t num_source_features,
+                                         int64_t num_target_features,
+                                         int index_dtype, int float_dtype,
+                                         const int32_t *gather_index,
+                                         const float *channel_scale, const float *channel_shift,
+                                         const void *residual, int activation,
+                                         float negative_slope,
+                                         void *out, void *stream);
 
 /* Timers used by the autotuner: run the named stage once on scratch buffers and
  * return the elapsed milliseconds through ms_out (synchronise).

@@ -156,6 +156,61 @@ __global__ __launch_bounds__(256) void gather_kernel(const unsigned char *__rest
 template <typename T>
 __device__ __forceinline__ float to_float(T v) { return static_cast<float>(v); }
 
+// What Scatter applies to a summed row before rounding it to the output type:
+//   v = act(sum * scale[c] + shift[c] + residual[t][c])
+// scale / shift are per-channel fp32 vectors, residual a [T, C] tensor of the
+// output type; each is skipped when null.  An inference-mode BatchNorm folds
+// into (scale, shift), a bias into shift, a skip connection into residual.
+struct Epilogue {
+  const float *scale;
+  const float *shift;
+  const void *residual;
+  int activation;      // MNT_ACT_*
+  float slope;         // LeakyReLU negative slope
+};
+
+template <typename T, typename V, int E, int NV>
+__device__ __forceinline__ void finish_row(float (&acc)[NV][E], const Epilogue &ep, long long t,
+                                           int channels, int lr, int lanes_per_row,
+                                           unsigned char *__restrict__ dst) {
+  constexpr int VB = E * static_cast<int>(sizeof(T));
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int piece = lr + i * lanes_per_row;
+    if (ep.scale != nullptr) {
+#pragma unroll
+      for (int k = 0; k < E; ++k) acc[i][k] *= ep.scale[piece * E + k];
+    }
+    if (ep.shift != nullptr) {
+#pragma unroll
+      for (int k = 0; k < E; ++k) acc[i][k] += ep.shift[piece * E + k];
+    }
+    if (ep.residual != nullptr) {
+      const V raw = *reinterpret_cast<const V *>(static_cast<const unsigned char *>(ep.residual) +
+                                                 t * channels * static_cast<long long>(sizeof(T)) +
+                                                 piece * VB);
+      const T *e = reinterpret_cast<const T *>(&raw);
+#pragma unroll
+      for (int k = 0; k < E; ++k) acc[i][k] += to_float(e[k]);
+    }
+    if (ep.activation == MNT_ACT_RELU) {
+#pragma unroll
+      for (int k = 0; k < E; ++k) acc[i][k] = fmaxf(acc[i][k], 0.0f);
+    } else if (ep.activation == MNT_ACT_LEAKY_RELU) {
+#pragma unroll
+      for (int k = 0; k < E; ++k) acc[i][k] = acc[i][k] > 0.0f ? acc[i][k] : acc[i][k] * ep.slope;
+    } else if (ep.activation == MNT_ACT_RELU6) {
+#pragma unroll
+      for (int k = 0; k < E; ++k) acc[i][k] = fminf(fmaxf(acc[i][k], 0.0f), 6.0f);
+    }
+    V raw;
+    T *e = reinterpret_cast<T *>(&raw);
+#pragma unroll
+    for (int k = 0; k < E; ++k) e[k] = static_cast<T>(acc[i][k]);
+    *reinterpret_cast<V *>(dst + piece * VB) = raw;
+  }
+}
+
 // Fallback for kernels with more offsets than the listed form below stages:
 // one lane group per target row sums its buffer rows in offset order in fp32
 // and writes the row once.  The buffer holds elements of type TB (the output
@@ -170,7 +225,7 @@ __global__ __launch_bounds__(256) void scatter_wide_kernel(const TB *__restrict_
                                                       const int *__restrict__ row_start,
                                                       long long num_targets, int num_offsets,
                                                       int channels, int lanes_per_row,
-                                                      const TB *__restrict__ direct) {
+                                                      const TB *__restrict__ direct, Epilogue ep) {
   typedef typename VecOf<VB>::type V;
   constexpr int E = VB / static_cast<int>(sizeof(T));
   constexpr int BB = E * static_cast<int>(sizeof(TB));          // buffer bytes per vector
@@ -239,14 +294,7 @@ __global__ __launch_bounds__(256) void scatter_wide_kernel(const TB *__restrict_
       }
     }
   }
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    V raw;
-    T *e = reinterpret_cast<T *>(&raw);
-#pragma unroll
-    for (int k = 0; k < E; ++k) e[k] = static_cast<T>(acc[i][k]);
-    *reinterpret_cast<V *>(dst + (lr + i * lanes_per_row) * VB) = raw;
-  }
+  finish_row<T, V, E, NV>(acc, ep, t, channels, lr, lanes_per_row, dst);
 }
 
 // Scatter in two phases per workgroup of `tile_targets` (a power of two)
@@ -270,7 +318,7 @@ __global__ __launch_bounds__(kScatterBlock) void scatter_kernel(
     const TB *__restrict__ buffer, unsigned char *__restrict__ targets,
     const IT *__restrict__ target_masks, const int *__restrict__ row_start, long long num_targets,
     int num_offsets, int channels, int lanes_per_row, const TB *__restrict__ direct,
-    int tile_shift) {
+    int tile_shift, Epilogue ep) {
   typedef typename VecOf<VB>::type V;
   constexpr int E = VB / static_cast<int>(sizeof(T));
   constexpr int BB = E * static_cast<int>(sizeof(TB));          // buffer bytes per vector
@@ -399,14 +447,7 @@ __global__ __launch_bounds__(kScatterBlock) void scatter_kernel(
       }
     }
     unsigned char *dst = targets + t * channels * static_cast<long long>(sizeof(T));
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      V raw;
-      T *e = reinterpret_cast<T *>(&raw);
-#pragma unroll
-      for (int k = 0; k < E; ++k) e[k] = static_cast<T>(acc[i][k]);
-      *reinterpret_cast<V *>(dst + (lr + i * lanes_per_row) * VB) = raw;
-    }
+    finish_row<T, V, E, NV>(acc, ep, t, channels, lr, lanes_per_row, dst);
   }
 }
 
@@ -701,7 +742,7 @@ constexpr int kScatterListedOffsets = 343;
 template <typename TB, typename T, typename IT>
 static void launch_scatter(const LaneShape &sh, const TB *buffer, void *targets, const IT *masks,
                            const int *row_start, int64_t num_targets, int num_offsets, int channels,
-                           const TB *direct, hipStream_t stream) {
+                           const TB *direct, const Epilogue &ep, hipStream_t stream) {
   if (num_targets == 0) return;
   const bool listed = num_offsets <= kScatterListedOffsets && sh.lanes_per_row <= kScatterBlock;
   const int tile_shift = num_offsets <= 128 ? 6 : 5;
@@ -714,11 +755,11 @@ static void launch_scatter(const LaneShape &sh, const TB *buffer, void *targets,
   if (listed) {                                                                                     \
     scatter_kernel<TB, T, VB, NV, IT><<<grid, kScatterBlock, lds, stream>>>(                        \
         buffer, static_cast<unsigned char *>(targets), masks, row_start, num_targets, num_offsets,  \
-        channels, sh.lanes_per_row, direct, tile_shift);                                            \
+        channels, sh.lanes_per_row, direct, tile_shift, ep);                                        \
   } else {                                                                                          \
     scatter_wide_kernel<TB, T, VB, NV, IT><<<grid, 256, 0, stream>>>(                               \
         buffer, static_cast<unsigned char *>(targets), masks, row_start, num_targets, num_offsets,  \
-        channels, sh.lanes_per_row, direct);                                                        \
+        channels, sh.lanes_per_row, direct, ep);                                                    \
   }
 #define MNT_SV(VB)                 \
   switch (sh.nv) {                 \
@@ -863,8 +904,9 @@ static void read_sizes(const void *sizes_dev, int index_dtype, int64_t num_offse
 template <typename T, typename IT>
 static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const ForwardPlan &plan,
                           const T *sources, const T *weights, const IT *source_masks,
-                          const IT *target_masks, const IT *order, const int *gather_index, int64_t S,
-                          int64_t Tn, int64_t O, int64_t K, int64_t N, T *out, hipStream_t stream) {
+                          const IT *target_masks, const IT *order, const int *gather_index,
+                          const Epilogue &epilogue, int64_t S, int64_t Tn, int64_t O, int64_t K,
+                          int64_t N, T *out, hipStream_t stream) {
   Scope scope(stream);
   const int kc = kChunkBytes / static_cast<int>(sizeof(T));
   const int Kp = static_cast<int>(div_ceil(K, kc) * kc);
@@ -932,7 +974,7 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
 
   const LaneShape ssh = lane_shape(scatter_tile, N, sizeof(T), cbuf, out, "num_target_features");
   launch_scatter<TB, T, IT>(ssh, cbuf, out, target_masks, d_row_start, Tn, active,
-                            static_cast<int>(N), direct, stream);
+                            static_cast<int>(N), direct, epilogue, stream);
   profile_mark("scatter", stream);
 }
 
@@ -977,13 +1019,14 @@ extern "C" int mnt_cumsum_kernel_padded_sizes(const int64_t *sizes_host, int64_t
     }                                                                 \
   } while (0)
 
-extern "C" int mnt_sparse_convolution_forward(
+extern "C" int mnt_sparse_convolution_forward_fused(
     int64_t gather_tile, int64_t scatter_tile, int allow_shortcut_matmul, int64_t parallel,
     int has_threshold, double threshold, const void *sources, const void *weights,
     const void *source_masks, const void *target_masks, const void *kernel_map_order,
     const void *kernel_map_sizes, const int64_t *sizes_host, int64_t S, int64_t T, int64_t O,
-    int64_t K, int64_t N, int index_dtype, int float_dtype, const int32_t *gather_index, void *out,
-    void *stream_) {
+    int64_t K, int64_t N, int index_dtype, int float_dtype, const int32_t *gather_index,
+    const float *channel_scale, const float *channel_shift, const void *residual, int activation,
+    float negative_slope, void *out, void *stream_) {
   (void)parallel;
   return guarded([&] {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -993,6 +1036,12 @@ extern "C" int mnt_sparse_convolution_forward(
                   O <= 65535 && K <= 65536 && N <= 65536,
               "bad shape S=%lld T=%lld O=%lld Cin=%lld Cout=%lld", (long long)S, (long long)T,
               (long long)O, (long long)K, (long long)N);
+    MNT_CHECK(activation >= MNT_ACT_NONE && activation <= MNT_ACT_RELU6, "unknown activation code %d",
+              activation);
+    MNT_CHECK(reinterpret_cast<uintptr_t>(residual) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(channel_scale) % 4 == 0 &&
+                  reinterpret_cast<uintptr_t>(channel_shift) % 4 == 0,
+              "epilogue operands are not aligned (residual: 16 bytes, scale / shift: 4 bytes)");
     if (T == 0) return;
     MNT_CHECK(out != nullptr, "out is null");
     std::vector<int64_t> sizes;
@@ -1007,14 +1056,29 @@ extern "C" int mnt_sparse_convolution_forward(
     }
     ForwardPlan plan = make_forward_plan(sizes.data(), O, S, T, allow_shortcut_matmul != 0,
                                          has_threshold != 0, threshold);
+    const Epilogue epilogue = {channel_scale, channel_shift, residual, activation, negative_slope};
 #define MNT_CALL(FT, IT)                                                                          \
   forward_typed<FT, IT>(gather_tile, scatter_tile, plan, static_cast<const FT *>(sources),          \
                         static_cast<const FT *>(weights), static_cast<const IT *>(source_masks),    \
                         static_cast<const IT *>(target_masks), static_cast<const IT *>(kernel_map_order), \
-                        gather_index, S, T, O, K, N, static_cast<FT *>(out), stream)
+                        gather_index, epilogue, S, T, O, K, N, static_cast<FT *>(out), stream)
     MNT_DISPATCH_FI(float_dtype, index_dtype, MNT_CALL);
 #undef MNT_CALL
   });
+}
+
+extern "C" int mnt_sparse_convolution_forward(
+    int64_t gather_tile, int64_t scatter_tile, int allow_shortcut_matmul, int64_t parallel,
+    int has_threshold, double threshold, const void *sources, const void *weights,
+    const void *source_masks, const void *target_masks, const void *kernel_map_order,
+    const void *kernel_map_sizes, const int64_t *sizes_host, int64_t S, int64_t T, int64_t O,
+    int64_t K, int64_t N, int index_dtype, int float_dtype, const int32_t *gather_index, void *out,
+    void *stream_) {
+  return mnt_sparse_convolution_forward_fused(
+      gather_tile, scatter_tile, allow_shortcut_matmul, parallel, has_threshold, threshold, sources,
+      weights, source_masks, target_masks, kernel_map_order, kernel_map_sizes, sizes_host, S, T, O, K,
+      N, index_dtype, float_dtype, gather_index, nullptr, nullptr, nullptr, MNT_ACT_NONE, 0.0f, out,
+      stream_);
 }
 
 // ---------------------------------------------------------- stage timers ----
@@ -1074,7 +1138,7 @@ static float time_scatter_typed(int64_t tile, const ForwardPlan &plan, const IT 
   timer.begin();
   launch_scatter<TB, T, IT>(sh, cbuf, out, target_masks, d_row_start, Tn,
                             static_cast<int>(plan.active_offsets), static_cast<int>(N),
-                            plan.shortcut ? cbuf + rows * N : nullptr, stream);
+                            plan.shortcut ? cbuf + rows * N : nullptr, Epilogue{}, stream);
   return timer.end();
 }
 

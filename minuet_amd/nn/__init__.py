@@ -3,3 +3,4 @@ from .convolutions import *
 from .activations import *
 from .normalizations import *
 from .pooling import *
+from .fused import *

@@ -300,9 +300,23 @@ class SparseConv(Module):
             self._tuning_data = None
 
     # ------------------------------------------------------------- forward ----
-    def forward(self, inputs: SparseTensor) -> SparseTensor:
+    def forward(self, inputs: SparseTensor,
+                epilogue: Optional[F.Epilogue] = None) -> SparseTensor:
+        """``epilogue`` (not in the reference, whose layers end at the bias add,
+        convolutions.py:446-499) is applied to the output rows in the same pass
+        that writes them: ``act(conv(x) * scale + shift + residual)``, with the
+        bias, if any, added before the scale."""
+        if epilogue is not None and self.bias is not None:
+            bias = self.bias.float()
+            shift = bias if epilogue.scale is None else bias * epilogue.scale.float()
+            if epilogue.shift is not None:
+                shift = shift + epilogue.shift.float()
+            epilogue = F.Epilogue(epilogue.scale, shift, epilogue.residual, epilogue.activation,
+                                  epilogue.negative_slope)
         if self.is_trivial:
             features = torch.mm(inputs.F, self.kernel.view(self.in_channels, self.out_channels))
+            if epilogue is not None:
+                features = epilogue.apply(features)
             coordinates, stride, batch_dims = inputs.C, inputs.stride, inputs.batch_dims
         else:
             cache = self._kernel_map_cache
@@ -326,8 +340,8 @@ class SparseConv(Module):
                 gather_tile_size=self._tunable_config["gather_tile_size"],
                 scatter_tile_size=self._tunable_config["scatter_tile_size"],
                 allow_shortcut_matmul=self._allow_shortcut_matmul,
-                threshold=self._tunable_config["threshold"])
-        if self.bias is not None:
+                threshold=self._tunable_config["threshold"], epilogue=epilogue)
+        if self.bias is not None and epilogue is None:
             features += self.bias
         return SparseTensor(features=features, coordinates=coordinates, stride=stride,
                             batch_dims=batch_dims)

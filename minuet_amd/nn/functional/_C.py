@@ -60,6 +60,10 @@ SIGNATURES = {
     "mnt_sparse_convolution_forward": (_int, [_i64, _i64, _int, _i64, _int, _dbl, _vp, _vp, _vp, _vp,
                                               _vp, _vp, _pi64, _i64, _i64, _i64, _i64, _i64, _int,
                                               _int, _vp, _vp, _vp]),
+    "mnt_sparse_convolution_forward_fused": (_int, [_i64, _i64, _int, _i64, _int, _dbl, _vp, _vp, _vp,
+                                                    _vp, _vp, _vp, _pi64, _i64, _i64, _i64, _i64,
+                                                    _i64, _int, _int, _vp, _vp, _vp, _vp, _int,
+                                                    _c.c_float, _vp, _vp]),
     "mnt_time_gather": (_int, [_i64, _int, _int, _dbl, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
                                _int, _pf, _vp]),
     "mnt_time_scatter": (_int, [_i64, _int, _int, _dbl, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
@@ -502,6 +506,64 @@ def _conv_shapes(weights, source_masks, target_masks, kernel_map_sizes):
             weights.size(2))
 
 
+ACTIVATION_CODES = {None: 0, "relu": 1, "leaky_relu": 2, "relu6": 3}
+
+
+class Epilogue:
+    """What the forward applies to each summed output row before rounding:
+    ``act(row * scale + shift + residual)``.  ``scale`` / ``shift``: fp32
+    ``[C_out]``; ``residual``: ``[N_out, C_out]`` of the feature dtype;
+    ``activation``: ``None``, ``"relu"``, ``"leaky_relu"`` or ``"relu6"``."""
+
+    __slots__ = ("scale", "shift", "residual", "activation", "negative_slope")
+
+    def __init__(self, scale: Optional[torch.Tensor] = None, shift: Optional[torch.Tensor] = None,
+                 residual: Optional[torch.Tensor] = None, activation: Optional[str] = None,
+                 negative_slope: float = 0.01):
+        if activation not in ACTIVATION_CODES:
+            raise ValueError(f"unknown activation {activation!r}")
+        self.scale, self.shift, self.residual = scale, shift, residual
+        self.activation, self.negative_slope = activation, negative_slope
+
+    def checked(self, num_targets: int, channels: int, dtype: torch.dtype, device) -> "Epilogue":
+        """Copy with operands validated and laid out the way the kernel reads them."""
+        def vector(name, t):
+            if t is None:
+                return None
+            if t.shape != (channels,) or t.device != device:
+                _fail(f"epilogue {name} must be a [{channels}] tensor on the device of the features")
+            return t.to(torch.float32).contiguous()
+        residual = self.residual
+        if residual is not None:
+            if residual.shape != (num_targets, channels) or residual.dtype != dtype or \
+                    residual.device != device:
+                _fail(f"epilogue residual must be a [{num_targets}, {channels}] {dtype} tensor on "
+                      "the device of the features")
+            residual = residual.contiguous()
+            if residual.data_ptr() % 16:
+                residual = residual.clone()
+        return Epilogue(vector("scale", self.scale), vector("shift", self.shift), residual,
+                        self.activation, self.negative_slope)
+
+    def apply(self, features: torch.Tensor) -> torch.Tensor:
+        """The same arithmetic with tensor expressions (fp32, one rounding), for
+        paths that do not go through Scatter."""
+        value = features.float()
+        if self.scale is not None:
+            value = value * self.scale.float()
+        if self.shift is not None:
+            value = value + self.shift.float()
+        if self.residual is not None:
+            value = value + self.residual.float()
+        if self.activation == "relu":
+            value = torch.relu(value)
+        elif self.activation == "leaky_relu":
+            value = torch.nn.functional.leaky_relu(value, self.negative_slope)
+        elif self.activation == "relu6":
+            value = torch.nn.functional.relu6(value)
+        return value.to(features.dtype)
+
+
 def _host_sizes_arg(sizes_host, num_offsets):
     if sizes_host is None:
         return None, None
@@ -519,11 +581,13 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
                                     kernel_map_order: Optional[torch.Tensor],
                                     kernel_map_sizes: torch.Tensor,
                                     kernel_map_sizes_host=None,
-                                    gather_index: Optional[torch.Tensor] = None) -> torch.Tensor:
+                                    gather_index: Optional[torch.Tensor] = None,
+                                    epilogue: Optional["Epilogue"] = None) -> torch.Tensor:
     """csrc/minuet/torch/cuda_sparse_convolution_forward.cu:136-213.  The extra
     ``kernel_map_sizes_host`` spares the device read-back of the sizes;
     ``gather_index`` (int32, the kernel map's source row per buffer row) folds
-    the Gather step into the GEMM."""
+    the Gather step into the GEMM; ``epilogue`` is applied to every output row
+    before it is rounded to the feature dtype."""
     fn = "CUDASparseConvolutionForward"
     _ensure_ndim("sources", sources, 2)
     S, T, O, K, N = _conv_shapes(weights, source_masks, target_masks, kernel_map_sizes)
@@ -549,14 +613,16 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
         if kernel_map_sizes_host is None or gather_index.numel() != int(sum(kernel_map_sizes_host)):
             _fail("gather_index needs the host sizes and one entry per kernel map hit")
         gather_index = gather_index.contiguous()
+    ep = Epilogue() if epilogue is None else epilogue.checked(T, N, weights.dtype, device)
     with torch.cuda.device(device):
-        _check(load_library().mnt_sparse_convolution_forward(
+        _check(load_library().mnt_sparse_convolution_forward_fused(
             int(gather_tile_size), int(scatter_tile_size), 1 if allow_shortcut_matmul else 0,
             int(parallel), 0 if threshold is None else 1,
             0.0 if threshold is None else float(threshold), _ptr(sources), _ptr(weights),
             _ptr(source_masks), _ptr(target_masks), _ptr(kernel_map_order),
             _ptr(kernel_map_sizes), sizes_ptr, S, T, O, K, N, icode, fcode, _ptr(gather_index),
-            _ptr(out), _stream(device)))
+            _ptr(ep.scale), _ptr(ep.shift), _ptr(ep.residual), ACTIVATION_CODES[ep.activation],
+            float(ep.negative_slope), _ptr(out), _stream(device)))
     del keep
     return out
 

@@ -7,7 +7,9 @@ import torch
 from . import _C
 
 __all__ = ["cuda_time_gather", "cuda_time_scatter", "sparse_convolution_forward",
-           "cuda_time_gemm", "set_gemm_parallel_level"]
+           "cuda_time_gemm", "set_gemm_parallel_level", "Epilogue"]
+
+Epilogue = _C.Epilogue
 
 GEMM_PARALLEL_LEVEL = 4
 
@@ -56,14 +58,17 @@ def sparse_convolution_forward(sources: torch.Tensor, weights: torch.Tensor,
                                kernel_map_sizes: torch.Tensor, gather_tile_size: int,
                                scatter_tile_size: int, allow_shortcut_matmul: bool = False,
                                parallel: Optional[int] = None,
-                               threshold: Optional[float] = 0) -> torch.Tensor:
+                               threshold: Optional[float] = 0,
+                               epilogue: Optional[_C.Epilogue] = None) -> torch.Tensor:
     """Output features ``[N_out, C_out]`` of one sparse convolution given the rank
     tables of its kernel map (reference: convolution.py:110-155).  A host copy
     of the sizes attached to ``kernel_map_sizes`` as attribute ``host_sizes``
     (``KernelMapCache`` does that) avoids a device read-back per call; an int32
     tensor attached to ``source_masks`` as attribute ``gather_index`` (the
     source row of every buffer row, also from ``KernelMapCache``) lets the GEMM
-    read the source rows directly instead of going through a gather buffer."""
+    read the source rows directly instead of going through a gather buffer.
+    ``epilogue`` (:class:`Epilogue`) is applied to each output row inside
+    Scatter, before the row is rounded to the feature dtype."""
     if not sources.is_cuda:
         raise NotImplementedError
     if parallel is None:
@@ -76,4 +81,4 @@ def sparse_convolution_forward(sources: torch.Tensor, weights: torch.Tensor,
         gather_tile_size, scatter_tile_size, allow_shortcut_matmul, parallel, threshold,
         sources.contiguous(), weights.contiguous(), source_masks.contiguous(),
         target_masks.contiguous(), kernel_map_order, kernel_map_sizes.contiguous(),
-        kernel_map_sizes_host=host_sizes, gather_index=gather_index)
+        kernel_map_sizes_host=host_sizes, gather_index=gather_index, epilogue=epilogue)

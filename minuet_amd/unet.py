@@ -2,11 +2,13 @@
 encoder stages (32/64/128/256 channels), four transposed-convolution decoder
 stages with skip concatenation, two residual 3x3x3 submanifold blocks per
 stage.  Everything is assembled from the public modules of this package, the
-way a user of the reference would write it."""
+way a user of the reference would write it; in evaluation mode the
+BatchNorm / ReLU / residual-sum layers ride the convolutions' output pass."""
 import torch
 from torch import nn
 
 from minuet_amd.nn import BatchNorm, ReLU, SparseConv, SparseConv3d
+from minuet_amd.nn.fused import FusedSequential, conv_norm_act
 from minuet_amd.nn import functional as F
 from minuet_amd.tensors import SparseTensor
 
@@ -30,13 +32,13 @@ class ResidualBlock(nn.Module):
         self.relu = ReLU(inplace=True)
         self.project = None
         if in_channels != out_channels:
-            self.project = nn.Sequential(SparseConv3d(in_channels, out_channels, 1, **factory),
-                                         BatchNorm(out_channels, **factory))
+            self.project = FusedSequential(SparseConv3d(in_channels, out_channels, 1, **factory),
+                                           BatchNorm(out_channels, **factory))
 
     def forward(self, x: SparseTensor) -> SparseTensor:
-        y = self.norm2(self.conv2(self.relu(self.norm1(self.conv1(x)))))
         skip = x if self.project is None else self.project(x)
-        return self.relu(_with_features(y, y.F + skip.F))
+        y = conv_norm_act(self.conv1, self.norm1, self.relu, x)
+        return conv_norm_act(self.conv2, self.norm2, self.relu, y, residual=skip.F)
 
 
 class SparseUNet(nn.Module):
@@ -48,13 +50,13 @@ class SparseUNet(nn.Module):
                  dtype=None, device=None):
         super().__init__()
         factory = {"dtype": dtype, "device": device}
-        self.stem = nn.Sequential(SparseConv3d(in_channels, stem, 3, **factory),
+        self.stem = FusedSequential(SparseConv3d(in_channels, stem, 3, **factory),
                                   BatchNorm(stem, **factory), ReLU(inplace=True))
         self.down = nn.ModuleList()
         self.encode = nn.ModuleList()
         widths = [stem]
         for width in encoder:
-            self.down.append(nn.Sequential(SparseConv3d(widths[-1], width, 2, stride=2, **factory),
+            self.down.append(FusedSequential(SparseConv3d(widths[-1], width, 2, stride=2, **factory),
                                            BatchNorm(width, **factory), ReLU(inplace=True)))
             self.encode.append(nn.Sequential(ResidualBlock(width, width, **factory),
                                              ResidualBlock(width, width, **factory)))
@@ -64,7 +66,7 @@ class SparseUNet(nn.Module):
         current = widths[-1]
         for level, width in enumerate(decoder):
             skip = widths[len(encoder) - 1 - level]
-            self.up.append(nn.Sequential(
+            self.up.append(FusedSequential(
                 SparseConv(3, current, width, 2, stride=2, transposed=True, **factory),
                 BatchNorm(width, **factory), ReLU(inplace=True)))
             self.decode.append(nn.Sequential(ResidualBlock(width + skip, width, **factory),

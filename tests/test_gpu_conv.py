@@ -97,6 +97,100 @@ def test_forward_functional(kind, kernel, stride, cin, cout, n, extent):
             assert torch.equal(fused, out)
 
 
+@pytest.mark.parametrize("kind", ["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("activation", [None, "relu", "leaky_relu", "relu6"])
+def test_forward_epilogue(kind, activation):
+    """act(conv * scale + shift + residual) applied inside Scatter equals the
+    same arithmetic on the float64 convolution output."""
+    src, sbd, tgt, tbd, off, feats, weights = make_layer_case(11, 6000, 24, 3, 32, 48, kind)
+    esm, etm, eorder, esizes, _ = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=True)
+    conv = orc.sparse_convolution_forward(feats, weights, esm, etm, eorder, esizes)
+    rng = np.random.default_rng(12)
+    scale = rng.uniform(0.5, 1.5, size=48).astype(np.float32)
+    shift = rng.uniform(-0.5, 0.5, size=48).astype(np.float32)
+    residual = quantise(rng.normal(size=conv.shape), kind)
+    dtype = TORCH[kind]
+    for use_scale, use_shift, use_residual in [(True, True, True), (False, True, False),
+                                               (True, False, False), (False, False, True)]:
+        ref = conv.copy()
+        if use_scale:
+            ref = ref * scale.astype(np.float64)
+        if use_shift:
+            ref = ref + shift.astype(np.float64)
+        if use_residual:
+            ref = ref + residual
+        if activation == "relu":
+            ref = np.maximum(ref, 0.0)
+        elif activation == "leaky_relu":
+            ref = np.where(ref > 0, ref, ref * 0.2)
+        elif activation == "relu6":
+            ref = np.clip(ref, 0.0, 6.0)
+        epilogue = F.Epilogue(dev(scale) if use_scale else None, dev(shift) if use_shift else None,
+                              dev(residual).to(dtype) if use_residual else None, activation, 0.2)
+        for shortcut in (False, True):
+            out = F.sparse_convolution_forward(
+                sources=dev(feats).to(dtype), weights=dev(weights).to(dtype),
+                source_masks=dev(esm), target_masks=dev(etm), kernel_map_order=dev(eorder),
+                kernel_map_sizes=dev(esizes), gather_tile_size=0, scatter_tile_size=0,
+                allow_shortcut_matmul=shortcut, threshold=0, epilogue=epilogue)
+            assert_features_close(out, ref, kind)
+
+
+def test_epilogue_rejects_bad_operands():
+    src, sbd, tgt, tbd, off, feats, weights = make_layer_case(5, 500, 8, 3, 32, 32, "fp32")
+    esm, etm, eorder, esizes, _ = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=True)
+    args = dict(sources=dev(feats).float(), weights=dev(weights).float(), source_masks=dev(esm),
+                target_masks=dev(etm), kernel_map_order=dev(eorder), kernel_map_sizes=dev(esizes),
+                gather_tile_size=0, scatter_tile_size=0)
+    with pytest.raises(RuntimeError, match="epilogue scale"):
+        F.sparse_convolution_forward(epilogue=F.Epilogue(scale=torch.ones(31, device="cuda")), **args)
+    with pytest.raises(RuntimeError, match="epilogue residual"):
+        F.sparse_convolution_forward(
+            epilogue=F.Epilogue(residual=torch.ones(tgt.shape[0], 32, device="cuda").half()), **args)
+    with pytest.raises(ValueError, match="unknown activation"):
+        F.Epilogue(activation="gelu")
+
+
+def test_fused_sequential_matches_modules():
+    """Sequential(conv, BatchNorm, LeakyReLU) folded into one pass: equal to the
+    module-by-module result within fp16 rounding in evaluation mode, and
+    exactly the module-by-module path in training mode."""
+    torch.manual_seed(3)
+    src, sbd, tgt, tbd, off, feats, weights = make_layer_case(21, 5000, 20, 3, 16, 32, "fp16")
+    plain = torch.nn.Sequential(
+        minuet.nn.SparseConv3d(16, 32, 3, bias=True, dtype=torch.float16, device="cuda"),
+        minuet.nn.BatchNorm(32, dtype=torch.float16, device="cuda"),
+        minuet.nn.LeakyReLU(0.1))
+    plain[1].running_mean.uniform_(-0.2, 0.2)
+    plain[1].running_var.uniform_(0.5, 1.5)
+    plain[0].bias.data.uniform_(-0.3, 0.3)
+    cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+    minuet.set_kernel_map_cache(plain, cache)
+    fused = minuet.nn.fuse_conv_norm_act(plain)
+    assert isinstance(fused, minuet.nn.FusedSequential)
+    assert list(fused.state_dict().keys()) == list(plain.state_dict().keys())
+    x = minuet.SparseTensor(dev(feats).half(), dev(src))
+    with torch.no_grad():
+        plain.eval(), fused.eval()
+        a, b = plain(x), fused(x)
+        assert torch.equal(a.C, b.C)
+        rms = a.F.float().pow(2).mean().sqrt().item()
+        assert (a.F.float() - b.F.float()).abs().max().item() <= 2e-2 * rms
+        # float64 replay of the three modules
+        w = host(plain[0].kernel.double())
+        esm, etm, eorder, esizes, _ = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=True)
+        ref = orc.sparse_convolution_forward(feats, w, esm, etm, eorder, esizes) + host(plain[0].bias.double())
+        bn = plain[1]
+        ref = (ref - host(bn.running_mean.double())) / np.sqrt(host(bn.running_var.double()) + bn.eps)
+        ref = ref * host(bn.weight.double()) + host(bn.bias.double())
+        ref = np.where(ref > 0, ref, 0.1 * ref)
+        assert_features_close(b.F, ref, "fp16")
+    plain.train(), fused.train()
+    torch.manual_seed(1)
+    a = plain(x)
+    assert torch.equal(fused(x).F, a.F)       # batch statistics: nothing is folded
+
+
 @pytest.mark.parametrize("tile", [1, 2, 4, 8, 16, 32])
 def test_forward_tile_sizes(tile):
     src, sbd, tgt, tbd, off, feats, weights = make_layer_case(5, 5000, 20, 3, 32, 64, "fp16")
