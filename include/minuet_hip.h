@@ -285,6 +285,38 @@ int mnt_time_gemm(int allow_shortcut_matmul, int64_t parallel, int has_threshold
                   int64_t num_source_features, int64_t num_target_features,
                   int index_dtype, int float_dtype, float *ms_out, void *stream);
 
+/* The same convolution computed output-stationary from the dense kernel map
+ * instead of the rank tables: kernel_map[O, T] (int32, source row per
+ * (offset, target) in the ORIGINAL offset order, -1 for none), i.e. the output
+ * of mnt_query_sorted_index_with_offsets / mnt_kernel_map_query; weights
+ * [O, Cin, Cout] in the same offset order.  No gather or GEMM-output buffer is
+ * written: each wavefront keeps 32 output rows in its matrix accumulators and
+ * walks the offsets.  Requires Cin * sizeof(element) to be a multiple of 16
+ * and at most 128, Cout % 4 == 0 and Cout <= 128; it pays for small channel counts, where the three-kernel
+ * form is bound by the buffer traffic.  The epilogue arguments are those of
+ * mnt_sparse_convolution_forward_fused.  Results agree with the other forms to
+ * rounding (sums are kept in fp32 over all offsets and rounded once).
+ * Covers the same reference code as mnt_sparse_convolution_forward
+ * (csrc/minuet/cuda/functions/sparse_convolution.cu:504-661); the reference
+ * has no single-kernel counterpart. */
+int mnt_sparse_convolution_forward_implicit(const void *sources, const void *weights,
+                                            const int32_t *kernel_map,
+                                            int64_t num_sources, int64_t num_targets,
+                                            int64_t num_offsets, int64_t num_source_features,
+                                            int64_t num_target_features, int float_dtype,
+                                            const float *channel_scale,
+                                            const float *channel_shift, const void *residual,
+                                            int activation, float negative_slope,
+                                            void *out, void *stream);
+
+/* The dense kernel map of the transposed layer that shares a forward layer's
+ * map (minuet/nn/convolutions.py:119-133 reuses the forward map with the rank
+ * tables swapped): inverse_out[O, S] with inverse_out[o][m] = t wherever
+ * kernel_map[o][t] = m, -1 elsewhere.  Feeds
+ * mnt_sparse_convolution_forward_implicit for transposed convolutions. */
+int mnt_kernel_map_invert(const int32_t *kernel_map, int64_t num_offsets, int64_t num_targets,
+                          int64_t num_sources, int32_t *inverse_out, void *stream);
+
 /* ---- stage timing -------------------------------------------------------- */
 
 /* mnt_profile_enable(1) makes the instrumented entry points (sort, query, emit,

@@ -1,0 +1,358 @@
+// Output-stationary forward of a sparse convolution ("implicit GEMM"): the
+// whole of Gather -> GEMM -> Scatter
+// (csrc/minuet/cuda/functions/sparse_convolution.cu:504-661) in one kernel
+// that never materialises the gather or GEMM-output buffers.
+//
+// It works from the dense kernel map M[O, T] (source row per (offset, target),
+// -1 for none; csrc/minuet/cuda/kernels/query_sorted_index_with_offsets.cuh)
+// instead of the rank tables.  One wavefront owns 32 consecutive targets and
+// keeps their output rows in MFMA accumulators; for every offset it loads the
+// source rows M[o, t] straight into its MFMA operand registers (zeros where
+// there is no source) and multiplies them by W_o, which the four wavefronts of
+// a workgroup share through LDS.  A wavefront skips an offset none of its 32
+// targets uses, so the wasted matrix work is bounded by how scattered the hits
+// are along the sorted target order.  Sums are kept in fp32 across all offsets
+// in ascending offset order and rounded once, after the epilogue.
+//
+// Compared with the three-kernel form this trades HBM traffic (no buffer rows
+// written and read back) for matrix work on empty rows, which pays while the
+// channel counts are small; the host entry point leaves the choice to the
+// caller.
+#include <algorithm>
+
+#include "conv_device.h"
+#include "device_utils.h"
+
+namespace mnt {
+
+constexpr int kImplicitBlock = 256;
+constexpr int kImplicitTargets = 128;     // per workgroup, 32 per wavefront
+constexpr int kImplicitMaxBlocks = 4;     // 32-channel output blocks (128 channels)
+
+// wt: packed weights [O][Np][KC] (W^T, K-contiguous, zero-padded to one
+// 128-byte chunk per row; see pack_weights_kernel).  Requires
+// K * sizeof(T) <= 128, K % (16 / sizeof(T)) == 0 and N % 4 == 0.
+// Register sets of the pipeline: 16-byte pieces of one thread's share of a
+// weight tile, and of one lane's source row.
+template <int N>
+struct Pieces {
+  uint4 v[N];
+};
+
+typedef unsigned uint4v __attribute__((ext_vector_type(4)));
+
+// Buffer offset that is out of range for every source tensor this kernel
+// accepts: such a load returns zeros without touching memory.
+constexpr unsigned kNoRow = 0xFFFFFFF0u;
+
+// KS: 32-byte steps of K that hold data (source rows are at most KS * 32 bytes).
+template <typename T, int NB, int KS>
+__global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
+    const T *__restrict__ sources, unsigned source_bytes, const T *__restrict__ wt,
+    const int *__restrict__ kernel_map, long long num_targets, int num_offsets, int K, int N,
+    unsigned char *__restrict__ out, Epilogue ep) {
+  constexpr int EPC = 16 / static_cast<int>(sizeof(T));
+  constexpr int KC = kChunkBytes / static_cast<int>(sizeof(T));
+  constexpr int kSteps = KS;
+  constexpr int Np = NB * 32;
+  constexpr int kRowPieces = 2 * KS;                     // 16-byte pieces of a weight row in use
+  constexpr int kWPieces = (Np * kRowPieces + kImplicitBlock - 1) / kImplicitBlock;
+  constexpr int kBufferBytes = Np * kLdsRowBytes;
+  __shared__ __align__(16) unsigned char w_lds[2 * kBufferBytes];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wv = tid >> 6;
+  const int r = lane & 31;
+  const int h = lane >> 5;
+  const long long t = static_cast<long long>(blockIdx.x) * kImplicitTargets + wv * 32 + r;
+  const bool t_ok = t < num_targets;
+
+  floatx16 acc[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[b][j] = 0.0f;
+  }
+
+  // Every global load below is unconditional (addresses are clamped, the
+  // values of lanes without a source are replaced when they are used), so
+  // that the loads of later stages never have to be waited for early.
+  const long long t_safe = t_ok ? t : num_targets - 1;
+  auto load_index = [&](int o) -> int {
+    return kernel_map[static_cast<long long>(o < num_offsets ? o : num_offsets - 1) * num_targets + t_safe];
+  };
+  auto entry = [&](int value, int o) -> int { return (t_ok && o < num_offsets) ? value : -1; };
+  // piece i of this thread: 16 bytes of weight row (piece / kRowPieces) at
+  // position (piece % kRowPieces); threads past the tile repeat its last piece
+  auto load_w = [&](int o) -> Pieces<kWPieces> {
+    const T *base = wt + static_cast<long long>(o < num_offsets ? o : num_offsets - 1) * Np * KC;
+    Pieces<kWPieces> set;
+#pragma unroll
+    for (int i = 0; i < kWPieces; ++i) {
+      const int piece = min(tid + i * kImplicitBlock, Np * kRowPieces - 1);
+      set.v[i] = *reinterpret_cast<const uint4 *>(base + (piece / kRowPieces) * KC +
+                                                  (piece % kRowPieces) * EPC);
+    }
+    return set;
+  };
+  auto store_w = [&](int buffer, const Pieces<kWPieces> &set) {
+#pragma unroll
+    for (int i = 0; i < kWPieces; ++i) {
+      const int piece = min(tid + i * kImplicitBlock, Np * kRowPieces - 1);
+      *reinterpret_cast<uint4 *>(w_lds + buffer * kBufferBytes + (piece / kRowPieces) * kLdsRowBytes +
+                                 (piece % kRowPieces) * 16) = set.v[i];
+    }
+  };
+  // Source rows come through a buffer resource: lanes without a source (and
+  // pieces past the end of a row) use an out-of-range offset, which yields the
+  // zeros the product needs and no memory access.
+  const __amdgpu_buffer_rsrc_t source_buffer = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<T *>(sources), 0, source_bytes, 0x00020000);
+  const unsigned row_bytes = static_cast<unsigned>(K) * sizeof(T);
+  auto load_a = [&](int index) -> Pieces<KS> {
+    Pieces<KS> set;
+#pragma unroll
+    for (int kk = 0; kk < kSteps; ++kk) {
+      const unsigned at = (kk * 2 + h) * 16u;
+      const unsigned offset =
+          (index >= 0 && at < row_bytes) ? static_cast<unsigned>(index) * row_bytes + at : kNoRow;
+      const uint4v v = __builtin_amdgcn_raw_buffer_load_b128(source_buffer, offset, 0, 0);
+      set.v[kk] = make_uint4(v.x, v.y, v.z, v.w);
+    }
+    return set;
+  };
+
+  // Software pipeline over the offsets: while offset o is multiplied, the
+  // source rows of offset o+2 and the weights of offset o+3 are already on
+  // their way, and kernel-map entries are read five offsets ahead.  The loop
+  // is unrolled by six so that the roles of the register sets (three sets of
+  // source rows, three of weights, six kernel-map entries) rotate without
+  // copies: a register is never touched while its load is in flight.
+  int m0 = load_index(0), m1 = load_index(1), m2 = load_index(2), m3 = load_index(3),
+      m4 = load_index(4), m5 = 0;
+  Pieces<KS> a0, a1, a2;
+  Pieces<kWPieces> w0, w1, w2;
+  w2 = load_w(0);
+  a0 = load_a(entry(m0, 0));
+  w0 = load_w(1);
+  a1 = load_a(entry(m1, 1));
+  w1 = load_w(2);
+  store_w(0, w2);
+  __syncthreads();
+
+  int o = 0;
+  // offset o: multiply A_CUR (rows of M_CUR) by the weights in LDS buffer o & 1;
+  // fetch rows of offset o+2 (entries M_A) into A_NEW, weights of offset o+3
+  // into W_NEW and the kernel-map entry of offset o+5 into M_NEW; put the
+  // weights of offset o+1 (W_STORE) into the other LDS buffer.
+#define MNT_STAGE(A_CUR, A_NEW, W_STORE, W_NEW, M_CUR, M_A, M_NEW)                                 \
+  {                                                                                                \
+    W_NEW = load_w(o + 3);                                                                         \
+    A_NEW = load_a(entry(M_A, o + 2));                                                             \
+    M_NEW = load_index(o + 5);                                                                     \
+    if (__ballot(entry(M_CUR, o) >= 0) != 0ull) {                                                  \
+      const unsigned char *w_buf = w_lds + (o & 1) * kBufferBytes;                                 \
+      _Pragma("unroll") for (int kk = 0; kk < kSteps; ++kk) {                                      \
+        const int off = kk * 32 + h * 16;                                                          \
+        _Pragma("unroll") for (int b = 0; b < NB; ++b) {                                           \
+          const uint4 chan =                                                                       \
+              *reinterpret_cast<const uint4 *>(w_buf + (b * 32 + r) * kLdsRowBytes + off);         \
+          acc[b] = Mfma<T>::run(chan, A_CUR.v[kk], acc[b]);                                        \
+        }                                                                                          \
+      }                                                                                            \
+    }                                                                                              \
+    store_w((o + 1) & 1, W_STORE);                                                                 \
+    __syncthreads();                                                                               \
+    if (++o == num_offsets) break;                                                                 \
+  }
+  while (true) {
+    MNT_STAGE(a0, a2, w0, w2, m0, m2, m5)
+    MNT_STAGE(a1, a0, w1, w0, m1, m3, m0)
+    MNT_STAGE(a2, a1, w2, w1, m2, m4, m1)
+    MNT_STAGE(a0, a2, w0, w2, m3, m5, m2)
+    MNT_STAGE(a1, a0, w1, w0, m4, m0, m3)
+    MNT_STAGE(a2, a1, w2, w1, m5, m1, m4)
+  }
+#undef MNT_STAGE
+
+  if (!t_ok) return;
+  typedef typename VecOf<4 * sizeof(T)>::type V;
+  unsigned char *dst = out + t * N * static_cast<long long>(sizeof(T));
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int ch = b * 32 + q * 8 + h * 4;
+      if (ch >= N) continue;                 // N % 4 == 0: a group of four is all in or all out
+      float v[4];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) v[x] = acc[b][q * 4 + x];
+      if (ep.scale != nullptr) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) v[x] *= ep.scale[ch + x];
+      }
+      if (ep.shift != nullptr) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) v[x] += ep.shift[ch + x];
+      }
+      if (ep.residual != nullptr) {
+        const V raw = *reinterpret_cast<const V *>(static_cast<const unsigned char *>(ep.residual) +
+                                                   (t * N + ch) * static_cast<long long>(sizeof(T)));
+        const T *e = reinterpret_cast<const T *>(&raw);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) v[x] += to_float(e[x]);
+      }
+      if (ep.activation == MNT_ACT_RELU) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) v[x] = fmaxf(v[x], 0.0f);
+      } else if (ep.activation == MNT_ACT_LEAKY_RELU) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) v[x] = v[x] > 0.0f ? v[x] : v[x] * ep.slope;
+      } else if (ep.activation == MNT_ACT_RELU6) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) v[x] = fminf(fmaxf(v[x], 0.0f), 6.0f);
+      }
+      V raw;
+      T *e = reinterpret_cast<T *>(&raw);
+#pragma unroll
+      for (int x = 0; x < 4; ++x) e[x] = static_cast<T>(v[x]);
+      *reinterpret_cast<V *>(dst + ch * sizeof(T)) = raw;
+    }
+  }
+}
+
+// inverse[o][m] = t for every hit kernel_map[o][t] = m (at most one t per
+// (o, m): the targets of one offset are distinct translates of their sources).
+__global__ __launch_bounds__(256) void invert_map_kernel(const int *__restrict__ kernel_map,
+                                                         long long num_targets,
+                                                         long long num_sources, long long total,
+                                                         int *__restrict__ inverse) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int m = kernel_map[i];
+    if (m >= 0) {
+      const long long o = i / num_targets;
+      inverse[o * num_sources + m] = static_cast<int>(i - o * num_targets);
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void fill_minus_one_kernel(int *__restrict__ data, long long n) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
+    data[i] = -1;
+  }
+}
+
+template <typename T>
+static void implicit_typed(const T *sources, const T *weights, const int *kernel_map, int64_t S,
+                           int64_t Tn, int64_t O, int64_t K, int64_t N, const Epilogue &ep, T *out,
+                           hipStream_t stream) {
+  Scope scope(stream);
+  const int kc = kChunkBytes / static_cast<int>(sizeof(T));
+  const int Kp = static_cast<int>(div_ceil(K, kc) * kc);
+  const int Np = static_cast<int>(div_ceil(N, 32) * 32);
+  profile_mark("enter:implicit", stream);
+  T *wt = scope.alloc<T>(static_cast<size_t>(O) * Np * Kp);
+  const long long total = static_cast<long long>(O) * Np * Kp;
+  pack_weights_kernel<T, int32_t><<<grid_for(total, 256, 4096), 256, 0, stream>>>(
+      weights, nullptr, static_cast<int>(O), static_cast<int>(K), static_cast<int>(N), Kp, Np, wt,
+      PlanChunk{}, 0, nullptr);
+  check_launch("pack_weights_kernel");
+  profile_mark("pack_weights", stream);
+  const unsigned grid = static_cast<unsigned>(div_ceil(Tn, kImplicitTargets));
+  const unsigned source_bytes = static_cast<unsigned>(S * K * sizeof(T));
+#define MNT_IMPLICIT(NB, KS)                                                                       \
+  implicit_forward_kernel<T, NB, KS><<<grid, kImplicitBlock, 0, stream>>>(                         \
+      sources, source_bytes, wt, kernel_map, Tn, static_cast<int>(O), static_cast<int>(K),         \
+      static_cast<int>(N), reinterpret_cast<unsigned char *>(out), ep)
+#define MNT_IMPLICIT_NB(NB)               \
+  if (K * sizeof(T) <= 64) {              \
+    MNT_IMPLICIT(NB, 2);                  \
+  } else {                                \
+    MNT_IMPLICIT(NB, 4);                  \
+  }
+  switch (Np / 32) {
+    case 1: MNT_IMPLICIT_NB(1); break;
+    case 2: MNT_IMPLICIT_NB(2); break;
+    case 3: MNT_IMPLICIT_NB(3); break;
+    default: MNT_IMPLICIT_NB(4); break;
+  }
+#undef MNT_IMPLICIT_NB
+#undef MNT_IMPLICIT
+  check_launch("implicit_forward_kernel");
+  profile_mark("implicit", stream);
+}
+
+}  // namespace mnt
+
+using namespace mnt;
+
+extern "C" int mnt_sparse_convolution_forward_implicit(
+    const void *sources, const void *weights, const int32_t *kernel_map, int64_t S, int64_t T,
+    int64_t O, int64_t K, int64_t N, int float_dtype, const float *channel_scale,
+    const float *channel_shift, const void *residual, int activation, float negative_slope,
+    void *out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int esize = float_size(float_dtype);
+    MNT_CHECK(S >= 0 && T >= 0 && O >= 1 && K >= 1 && N >= 1 && S <= INT32_MAX && T <= INT32_MAX &&
+                  O <= 65535,
+              "bad shape S=%lld T=%lld O=%lld Cin=%lld Cout=%lld", (long long)S, (long long)T,
+              (long long)O, (long long)K, (long long)N);
+    MNT_CHECK(S * K * esize < static_cast<int64_t>(kNoRow),
+              "source features of %lld bytes exceed the 4 GiB a buffer resource addresses",
+              (long long)(S * K * esize));
+    MNT_CHECK((K * esize) % 16 == 0 && K * esize <= kChunkBytes && N % 4 == 0 &&
+                  N <= 32 * kImplicitMaxBlocks,
+              "Unsupported channel counts for the implicit forward: Cin = %lld (rows must be a multiple "
+              "of 16 bytes, at most %d), Cout = %lld (a multiple of 4, at most %d)",
+              (long long)K, kChunkBytes, (long long)N, 32 * kImplicitMaxBlocks);
+    MNT_CHECK(activation >= MNT_ACT_NONE && activation <= MNT_ACT_RELU6, "unknown activation code %d",
+              activation);
+    MNT_CHECK(reinterpret_cast<uintptr_t>(sources) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(residual) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(channel_scale) % 4 == 0 &&
+                  reinterpret_cast<uintptr_t>(channel_shift) % 4 == 0,
+              "operands are not aligned (features, out, residual: 16 bytes, scale / shift: 4 bytes)");
+    if (T == 0) return;
+    MNT_CHECK(out != nullptr && kernel_map != nullptr && weights != nullptr, "null operand");
+    const Epilogue ep = {channel_scale, channel_shift, residual, activation, negative_slope};
+    if (float_dtype == MNT_FLOAT32) {
+      implicit_typed<float>(static_cast<const float *>(sources), static_cast<const float *>(weights),
+                            kernel_map, S, T, O, K, N, ep, static_cast<float *>(out), stream);
+    } else if (float_dtype == MNT_FLOAT16) {
+      implicit_typed<half_t>(static_cast<const half_t *>(sources), static_cast<const half_t *>(weights),
+                             kernel_map, S, T, O, K, N, ep, static_cast<half_t *>(out), stream);
+    } else {
+      implicit_typed<bf16_t>(static_cast<const bf16_t *>(sources), static_cast<const bf16_t *>(weights),
+                             kernel_map, S, T, O, K, N, ep, static_cast<bf16_t *>(out), stream);
+    }
+  });
+}
+
+extern "C" int mnt_kernel_map_invert(const int32_t *kernel_map, int64_t num_offsets,
+                                     int64_t num_targets, int64_t num_sources,
+                                     int32_t *inverse_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MNT_CHECK(num_offsets >= 0 && num_targets >= 0 && num_sources >= 0 && num_targets <= INT32_MAX &&
+                  num_sources <= INT32_MAX,
+              "bad shape O=%lld T=%lld S=%lld", (long long)num_offsets, (long long)num_targets,
+              (long long)num_sources);
+    const long long filled = num_offsets * num_sources;
+    const long long total = num_offsets * num_targets;
+    if (filled > 0) {
+      MNT_CHECK(inverse_out != nullptr, "inverse_out is null");
+      fill_minus_one_kernel<<<grid_for(filled, 256, 8192), 256, 0, stream>>>(inverse_out, filled);
+      check_launch("fill_minus_one_kernel");
+    }
+    if (total > 0 && filled > 0) {
+      MNT_CHECK(kernel_map != nullptr, "kernel_map is null");
+      invert_map_kernel<<<grid_for(total, 256, 8192), 256, 0, stream>>>(kernel_map, num_targets, num_sources,
+                                                                         total, inverse_out);
+      check_launch("invert_map_kernel");
+    }
+  });
+}

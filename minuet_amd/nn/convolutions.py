@@ -119,6 +119,10 @@ class KernelMapCache(object):
         if hit is not None:
             source_masks, target_masks, order, sizes = hit
             if transposed:
+                if getattr(source_masks, "kernel_map", None) is None:
+                    # dense map of the transposed layer, made on first use
+                    source_masks.kernel_map = _C.kernel_map_invert(target_masks.kernel_map,
+                                                                   source_masks.shape[1])
                 source_masks, target_masks = target_masks, source_masks
             return source_masks, target_masks, order, sizes
         if transposed:
@@ -130,7 +134,7 @@ class KernelMapCache(object):
         target_coordinates = target_coordinates.contiguous()
         built = _C.kernel_map_build(source_coordinates, target_coordinates, offsets,
                                     source_batch_dims, target_batch_dims, reorder=reorder,
-                                    want_lists=True, source_bounds=self._known_bounds(source_coordinates),
+                                    want_lists=True, want_dense=True, source_bounds=self._known_bounds(source_coordinates),
                                     target_bounds=self._known_bounds(target_coordinates))
         self.num_map_builds += 1
         if source_coordinates.shape[0] > 0 and target_coordinates.shape[0] > 0:
@@ -147,6 +151,9 @@ class KernelMapCache(object):
         # (forward or transposed) gathers through
         source_masks.gather_index = built["in_idx"]
         target_masks.gather_index = built["out_idx"]
+        # source row per (offset, target) in the original offset order: what
+        # the single-kernel dataflow walks
+        target_masks.kernel_map = built["kernel_map"]
         entry = (source_masks, target_masks, order, sizes)
         self._kernel_maps_cache[key] = entry
         return entry
@@ -193,9 +200,11 @@ class SparseConv(Module):
             self.register_parameter("bias", None)
         self.reset_parameters()
         self._kernel_map_cache: Optional[KernelMapCache] = None
-        self._tunable_config = {"threshold": -1,
-                                "gather_tile_size": min(in_channels, 1),
-                                "scatter_tile_size": min(out_channels, 1)}
+        # Tile size 0 lets the library pick 16 bytes per lane.  (The reference
+        # starts from one element per thread, convolutions.py:277-281, and
+        # relies on autotune to leave that setting.)
+        self._tunable_config = {"threshold": -1, "gather_tile_size": 0, "scatter_tile_size": 0,
+                                "dataflow": "auto"}
         self._tuning_data = None
 
     @property
@@ -296,8 +305,45 @@ class SparseConv(Module):
                         self._tunable_config[key] = tile
                 if free_buffers:
                     F.cuda_free_buffers()
+            self._tune_dataflow()
         finally:
             self._tuning_data = None
+
+    def _tune_dataflow(self):
+        """Times one whole layer per dataflow on the recorded kernel maps (random
+        features) and keeps the faster one."""
+        best = None
+        for dataflow in ("gather_gemm_scatter", "implicit"):
+            total = 0.0
+            try:
+                for source_masks, target_masks, sizes in self._tuning_data:
+                    if dataflow == "implicit" and getattr(target_masks, "kernel_map", None) is None:
+                        raise RuntimeError("no dense kernel map")
+                    sources = torch.randn(source_masks.shape[1], self.in_channels,
+                                          device=self.kernel.device).to(self.kernel.dtype)
+                    order = getattr(sizes, "kernel_map_order", None)
+                    call = lambda: F.sparse_convolution_forward(
+                        sources=sources, weights=self.kernel, source_masks=source_masks,
+                        target_masks=target_masks, kernel_map_order=order, kernel_map_sizes=sizes,
+                        gather_tile_size=self._tunable_config["gather_tile_size"],
+                        scatter_tile_size=self._tunable_config["scatter_tile_size"],
+                        allow_shortcut_matmul=self._allow_shortcut_matmul and order is not None,
+                        threshold=self._tunable_config["threshold"], dataflow=dataflow)
+                    call()
+                    start = torch.cuda.Event(enable_timing=True)
+                    stop = torch.cuda.Event(enable_timing=True)
+                    start.record()
+                    for _ in range(max(1, self.__NUM_TUNING_ROUNDS__)):
+                        call()
+                    stop.record()
+                    stop.synchronize()
+                    total += start.elapsed_time(stop)
+            except RuntimeError:
+                F.cuda_reset_error()              # shape this dataflow does not offer
+                continue
+            if best is None or total < best:
+                best = total
+                self._tunable_config["dataflow"] = dataflow
 
     # ------------------------------------------------------------- forward ----
     def forward(self, inputs: SparseTensor,
@@ -333,6 +379,7 @@ class SparseConv(Module):
                 target_batch_dims=batch_dims, kernel_size=self.kernel_size,
                 kernel_dilation=self.dilation)
             if self._tuning_data is not None:
+                sizes.kernel_map_order = order
                 self._tuning_data.append((source_masks, target_masks, sizes))
             features = F.sparse_convolution_forward(
                 sources=inputs.F, weights=self.kernel, source_masks=source_masks,
@@ -340,7 +387,8 @@ class SparseConv(Module):
                 gather_tile_size=self._tunable_config["gather_tile_size"],
                 scatter_tile_size=self._tunable_config["scatter_tile_size"],
                 allow_shortcut_matmul=self._allow_shortcut_matmul,
-                threshold=self._tunable_config["threshold"], epilogue=epilogue)
+                threshold=self._tunable_config["threshold"], epilogue=epilogue,
+                dataflow=self._tunable_config.get("dataflow", "auto"))
         if self.bias is not None and epilogue is None:
             features += self.bias
         return SparseTensor(features=features, coordinates=coordinates, stride=stride,

@@ -64,6 +64,10 @@ SIGNATURES = {
                                                     _vp, _vp, _vp, _pi64, _i64, _i64, _i64, _i64,
                                                     _i64, _int, _int, _vp, _vp, _vp, _vp, _int,
                                                     _c.c_float, _vp, _vp]),
+    "mnt_sparse_convolution_forward_implicit": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
+                                                       _int, _vp, _vp, _vp, _int, _c.c_float, _vp,
+                                                       _vp]),
+    "mnt_kernel_map_invert": (_int, [_vp, _i64, _i64, _i64, _vp, _vp]),
     "mnt_time_gather": (_int, [_i64, _int, _int, _dbl, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
                                _int, _pf, _vp]),
     "mnt_time_scatter": (_int, [_i64, _int, _int, _dbl, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
@@ -624,6 +628,65 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
             _ptr(ep.scale), _ptr(ep.shift), _ptr(ep.residual), ACTIVATION_CODES[ep.activation],
             float(ep.negative_slope), _ptr(out), _stream(device)))
     del keep
+    return out
+
+
+def kernel_map_invert(kernel_map: torch.Tensor, num_sources: int) -> torch.Tensor:
+    """``[O, num_sources]`` int32 map with ``inverse[o, m] = t`` wherever
+    ``kernel_map[o, t] = m`` and -1 elsewhere: the dense kernel map of the
+    transposed layer that shares this map."""
+    _ensure_ndim("kernel_map", kernel_map, 2)
+    if kernel_map.dtype != torch.int32:
+        _fail("kernel_map_invert expects an int32 kernel map")
+    device = _common_device([kernel_map])
+    kernel_map = kernel_map.contiguous()
+    num_offsets, num_targets = kernel_map.shape
+    inverse = torch.empty((num_offsets, num_sources), dtype=torch.int32, device=device)
+    with torch.cuda.device(device):
+        _check(load_library().mnt_kernel_map_invert(_ptr(kernel_map), num_offsets, num_targets,
+                                                    num_sources, _ptr(inverse), _stream(device)))
+    return inverse
+
+
+IMPLICIT_MAX_TARGET_FEATURES = 128
+
+
+def implicit_forward_supported(num_source_features: int, num_target_features: int,
+                               dtype: torch.dtype) -> bool:
+    """Shapes ``sparse_convolution_forward_implicit`` accepts."""
+    row_bytes = num_source_features * dtype.itemsize
+    return (row_bytes % 16 == 0 and row_bytes <= 128 and num_target_features % 4 == 0
+            and num_target_features <= IMPLICIT_MAX_TARGET_FEATURES)
+
+
+def sparse_convolution_forward_implicit(sources: torch.Tensor, weights: torch.Tensor,
+                                        kernel_map: torch.Tensor,
+                                        epilogue: Optional[Epilogue] = None) -> torch.Tensor:
+    """Output-stationary forward from the dense kernel map ``[O, N_out]`` (int32,
+    original offset order): one kernel, no gather / GEMM-output buffers."""
+    fn = "sparse_convolution_forward_implicit"
+    _ensure_ndim("sources", sources, 2)
+    _ensure_ndim("weights", weights, 3)
+    _ensure_ndim("kernel_map", kernel_map, 2)
+    O, K, N = weights.shape
+    _ensure_dim("kernel_map", kernel_map, 0, O)
+    _ensure_dim("sources", sources, 1, K)
+    device = _common_device([sources, weights, kernel_map])
+    if kernel_map.dtype != torch.int32:
+        _fail("the implicit forward expects an int32 kernel map")
+    if sources.dtype != weights.dtype:
+        _fail(f"Found tensors with two different scalar types ({sources.dtype} != {weights.dtype})")
+    fcode = _float_code(weights.dtype, fn)
+    S, T = sources.size(0), kernel_map.size(1)
+    sources, weights, kernel_map = sources.contiguous(), weights.contiguous(), kernel_map.contiguous()
+    sources = sources if sources.data_ptr() % 16 == 0 else sources.clone()
+    out = torch.empty((T, N), dtype=weights.dtype, device=device)
+    ep = Epilogue() if epilogue is None else epilogue.checked(T, N, weights.dtype, device)
+    with torch.cuda.device(device):
+        _check(load_library().mnt_sparse_convolution_forward_implicit(
+            _ptr(sources), _ptr(weights), _ptr(kernel_map), S, T, O, K, N, fcode, _ptr(ep.scale),
+            _ptr(ep.shift), _ptr(ep.residual), ACTIVATION_CODES[ep.activation],
+            float(ep.negative_slope), _ptr(out), _stream(device)))
     return out
 
 

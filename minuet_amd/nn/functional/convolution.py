@@ -12,6 +12,7 @@ __all__ = ["cuda_time_gather", "cuda_time_scatter", "sparse_convolution_forward"
 Epilogue = _C.Epilogue
 
 GEMM_PARALLEL_LEVEL = 4
+DATAFLOWS = ("auto", "gather_gemm_scatter", "implicit")
 
 
 def set_gemm_parallel_level(level: int):
@@ -59,7 +60,8 @@ def sparse_convolution_forward(sources: torch.Tensor, weights: torch.Tensor,
                                scatter_tile_size: int, allow_shortcut_matmul: bool = False,
                                parallel: Optional[int] = None,
                                threshold: Optional[float] = 0,
-                               epilogue: Optional[_C.Epilogue] = None) -> torch.Tensor:
+                               epilogue: Optional[_C.Epilogue] = None,
+                               dataflow: str = "auto") -> torch.Tensor:
     """Output features ``[N_out, C_out]`` of one sparse convolution given the rank
     tables of its kernel map (reference: convolution.py:110-155).  A host copy
     of the sizes attached to ``kernel_map_sizes`` as attribute ``host_sizes``
@@ -68,9 +70,29 @@ def sparse_convolution_forward(sources: torch.Tensor, weights: torch.Tensor,
     source row of every buffer row, also from ``KernelMapCache``) lets the GEMM
     read the source rows directly instead of going through a gather buffer.
     ``epilogue`` (:class:`Epilogue`) is applied to each output row inside
-    Scatter, before the row is rounded to the feature dtype."""
+    Scatter, before the row is rounded to the feature dtype.
+
+    ``dataflow`` chooses between the reference's Gather -> GEMM -> Scatter
+    (``"gather_gemm_scatter"``) and the single-kernel output-stationary form
+    (``"implicit"``), which needs the dense kernel map attached to
+    ``target_masks`` as attribute ``kernel_map`` (``KernelMapCache`` does that)
+    and ``weights`` in their original offset order, as a layer holds them.
+    ``"auto"`` takes the implicit form where it is the faster one: 16-bit
+    features whose rows it can stage, and small fp32 layers with 2^D kernels."""
     if not sources.is_cuda:
         raise NotImplementedError
+    if dataflow not in DATAFLOWS:
+        raise ValueError(f"dataflow must be one of {DATAFLOWS}")
+    dense = getattr(target_masks, "kernel_map", None)
+    if dataflow == "implicit" and dense is None:
+        raise ValueError("the implicit dataflow needs target_masks.kernel_map (the dense kernel map)")
+    if dense is not None and dataflow != "gather_gemm_scatter":
+        fits = _C.implicit_forward_supported(weights.shape[1], weights.shape[2], weights.dtype)
+        # fp32 matrix work is 16x dearer than fp16: there the implicit form only
+        # pays where most (offset, target) pairs are hits, i.e. strided 2^D kernels
+        dense_hits = weights.shape[0] <= 8 and weights.shape[1] * weights.shape[2] <= 1024
+        if dataflow == "implicit" or (fits and (weights.dtype != torch.float32 or dense_hits)):
+            return _C.sparse_convolution_forward_implicit(sources, weights, dense, epilogue=epilogue)
     if parallel is None:
         parallel = GEMM_PARALLEL_LEVEL
     host_sizes = getattr(kernel_map_sizes, "host_sizes", None)

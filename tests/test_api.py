@@ -73,7 +73,8 @@ def test_conv_module_construction():
     assert conv.kernel.shape == (27, 8, 16) and conv.bias.shape == (16,)
     bound = 1.0 / np.sqrt(8 * 27)
     assert conv.kernel.abs().max() <= bound and conv.bias.abs().max() <= bound
-    assert conv.tunable_config == {"threshold": -1, "gather_tile_size": 1, "scatter_tile_size": 1}
+    assert conv.tunable_config == {"threshold": -1, "gather_tile_size": 0, "scatter_tile_size": 0,
+                                   "dataflow": "auto"}
     assert repr(conv) == "SparseConv3d(8, 16, kernel_size=(3, 3, 3))"
     up = minuet.nn.SparseConv(3, 8, 4, 2, stride=2, transposed=True)
     assert "stride=(2, 2, 2)" in repr(up) and "transposed=True" in repr(up) and "bias=False" in repr(up)
