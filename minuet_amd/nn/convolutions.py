@@ -206,6 +206,7 @@ class SparseConv(Module):
         self._tunable_config = {"threshold": -1, "gather_tile_size": 0, "scatter_tile_size": 0,
                                 "dataflow": "auto"}
         self._tuning_data = None
+        self._identity_map = None
 
     @property
     def _allow_shortcut_matmul(self) -> bool:
@@ -346,6 +347,27 @@ class SparseConv(Module):
                 self._tunable_config["dataflow"] = dataflow
 
     # ------------------------------------------------------------- forward ----
+    def _pointwise(self, features: torch.Tensor, epilogue: Optional[F.Epilogue]) -> torch.Tensor:
+        """1x1x1 kernel, stride 1: a plain ``features @ W`` (reference:
+        convolutions.py:452-455).  Where the single-kernel forward takes the
+        shape it runs there, as one offset whose kernel map is the identity,
+        so that an epilogue costs no extra pass; otherwise ``torch.mm``."""
+        weights = self.kernel.view(1, self.in_channels, self.out_channels)
+        needs_grad = torch.is_grad_enabled() and (features.requires_grad or weights.requires_grad)
+        if (features.is_cuda and not needs_grad
+                and self._tunable_config.get("dataflow", "auto") != "gather_gemm_scatter"
+                and features.dtype == weights.dtype
+                and _C.implicit_forward_supported(self.in_channels, self.out_channels, weights.dtype)):
+            rows = features.shape[0]
+            identity = self._identity_map
+            if identity is None or identity.shape[1] < rows or identity.device != features.device:
+                identity = torch.arange(rows, dtype=torch.int32, device=features.device).view(1, rows)
+                self._identity_map = identity
+            return _C.sparse_convolution_forward_implicit(features, weights, identity[:, :rows],
+                                                          epilogue=epilogue)
+        out = torch.mm(features, weights[0])
+        return out if epilogue is None else epilogue.apply(out)
+
     def forward(self, inputs: SparseTensor,
                 epilogue: Optional[F.Epilogue] = None) -> SparseTensor:
         """``epilogue`` (not in the reference, whose layers end at the bias add,
@@ -360,9 +382,7 @@ class SparseConv(Module):
             epilogue = F.Epilogue(epilogue.scale, shift, epilogue.residual, epilogue.activation,
                                   epilogue.negative_slope)
         if self.is_trivial:
-            features = torch.mm(inputs.F, self.kernel.view(self.in_channels, self.out_channels))
-            if epilogue is not None:
-                features = epilogue.apply(features)
+            features = self._pointwise(inputs.F, epilogue)
             coordinates, stride, batch_dims = inputs.C, inputs.stride, inputs.batch_dims
         else:
             cache = self._kernel_map_cache
