@@ -2,7 +2,11 @@
 
 A step is one kernel-map build from UNSORTED unique voxels to finished
 per-offset (in_idx, out_idx) lists: coordinate sort -> 3x3x3 query -> sizes ->
-pair lists, all through the C ABI of libminuet_hip.so.  Prints one JSON line.
+pair lists, all through the C ABI of libminuet_hip.so.  Prints one JSON line:
+the Map step is `value`; `extra` holds the other parts of the metric (layer
+throughput of configurations 1, 3 and 5, sparse UNet forward latency of
+configuration 4) and the Gather / grouped GEMM / Scatter kernels one by one
+with their algorithmic bytes and flops.
 """
 import argparse
 import json
@@ -18,6 +22,11 @@ for _p in (ROOT, os.path.join(ROOT, "oracle")):
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per query_kernel launch on this workload at scale 1: FETCH_SIZE and
+# WRITE_SIZE of rocprofv3 --pmc, each scaled by what the counter reads for a
+# plain 256 MiB device copy (2.000 and 1.000); the dense kernel map the kernel
+# writes accounts for 21.6 MB of it.
+QUERY_TRAFFIC_BYTES = 30.68e6
 
 
 def map_step(_C, coords_dev, offsets):
@@ -57,10 +66,92 @@ def _time_ms(fn, warmup, reps):
     return 1e3 * (time.perf_counter() - t0) / reps
 
 
-def extras(device):
-    """The other two parts of the metric, measured briefly: layer throughput
-    (configurations 1 and 3) and sparse UNet forward latency (configuration 4,
-    kernel-map cache reset before every forward)."""
+def _time_stats(fn, warmup, reps):
+    """Wall mean over `reps` back-to-back calls plus the distribution of the
+    per-call time between stream events (the events sit on torch's current
+    stream, the one the library is given)."""
+    import torch
+    mean = _time_ms(fn, warmup, reps)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+    marks[0].record()
+    for i in range(reps):
+        fn()
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    each = np.array([marks[i].elapsed_time(marks[i + 1]) for i in range(reps)])
+    return {"ms_mean": round(mean, 4), "ms_median": round(float(np.median(each)), 4),
+            "ms_p10": round(float(np.percentile(each, 10)), 4),
+            "ms_p90": round(float(np.percentile(each, 90)), 4), "iterations": reps}
+
+
+MFMA_PEAK_TFLOPS = {"fp16": 2500.0, "bf16": 2500.0, "fp32": 157.3}
+
+
+def layer_stages(device, config, channels, kernel_size, dtype_name):
+    """Gather, grouped GEMM and Scatter timed one by one through the library's
+    stage timers (the reference's cuda_time_* interface), then the whole layer
+    through both dataflows, with the algorithmic bytes / flops of each."""
+    import torch
+    import minuet_amd as minuet
+    from minuet_amd.nn import functional as F
+    from minuet_amd.nn.functional import _C
+    from minuet_amd.synthetic import make_cloud
+
+    dtype = {"fp16": torch.float16, "bf16": torch.bfloat16, "fp32": torch.float32}[dtype_name]
+    esize = torch.empty(0, dtype=dtype).element_size()
+    coords = torch.from_numpy(make_cloud(config)["coords"]).to(device)
+    _, sorted_dev = _C.sort_coordinates(coords)
+    conv = minuet.nn.SparseConv3d(channels, channels, kernel_size, dtype=dtype, device=device)
+    cache = minuet.nn.KernelMapCache(3, torch.int32, device)
+    conv.set_kernel_map_cache(cache)
+    x = minuet.SparseTensor(torch.randn(sorted_dev.shape[0], channels, device=device).to(dtype), sorted_dev)
+    with torch.no_grad():
+        conv(x)
+        source_masks, target_masks, order, sizes = next(iter(cache._kernel_maps_cache.values()))
+        host_sizes = np.asarray(sizes.host_sizes, dtype=np.int64)
+        voxels = int(sorted_dev.shape[0])
+        nnz = int(host_sizes.sum())
+        moved = nnz - voxels                       # the centre offset takes the shortcut
+        args = dict(weights=conv.kernel, source_masks=source_masks, target_masks=target_masks,
+                    kernel_map_sizes=sizes, allow_shortcut_matmul=True, threshold=-1)
+        med = lambda timer, **kw: float(np.median([timer(**args, **kw) for _ in range(15)]))
+        gather_ms = med(F.cuda_time_gather, tile_size=0)
+        scatter_ms = med(F.cuda_time_scatter, tile_size=0)
+        gemm_ms = med(F.cuda_time_gemm)
+        bytes_gather = voxels * channels * esize + moved * channels * esize + 4 * moved
+        bytes_scatter = moved * channels * esize + voxels * channels * esize + 4 * moved
+        flops = 2.0 * nnz * channels * channels
+        out = {"voxels": voxels, "nnz": nnz, "channels": channels, "dtype": dtype_name,
+               "offsets": int(host_sizes.shape[0])}
+
+        def hbm(nbytes, ms):
+            gbs = nbytes / (ms * 1e-3) / 1e9
+            return {"ms": round(ms, 4), "algorithmic_bytes": int(nbytes), "achieved_GBs": round(gbs, 1),
+                    "frac_of_8TBs": round(gbs / HBM_PEAK_GBS, 4)}
+        out["gather_kernel"] = hbm(bytes_gather, gather_ms)
+        out["scatter_kernel"] = hbm(bytes_scatter, scatter_ms)
+        tflops = flops / (gemm_ms * 1e-3) / 1e12
+        out["grouped_gemm_kernel"] = {"ms": round(gemm_ms, 4), "flops": flops, "achieved_TFLOPs": round(tflops, 1),
+                                      "frac_of_mfma_peak": round(tflops / MFMA_PEAK_TFLOPS[dtype_name], 4),
+                                      # rows in and out of the buffers: what bounds it at small widths
+                                      **{"hbm_" + k: v for k, v in hbm(2 * nnz * channels * esize, gemm_ms).items()
+                                         if k != "ms"}}
+        for flow in ("gather_gemm_scatter", "implicit"):
+            if flow == "implicit" and not _C.implicit_forward_supported(channels, channels, dtype):
+                continue
+            conv.tunable_config["dataflow"] = flow
+            stats = _time_stats(lambda: conv(x), 10, 50)
+            stats["mvoxels_per_s"] = round(voxels / stats["ms_mean"] / 1e3, 1)
+            stats["achieved_TFLOPs"] = round(flops / (stats["ms_mean"] * 1e-3) / 1e12, 1)
+            out["layer_" + flow] = stats
+    return out
+
+
+def extras(device, with_config5, section="all"):
+    """The other two parts of the metric: layer throughput (configurations 1, 3
+    and 5, kernel map cached and included) and sparse UNet forward latency
+    (configuration 4, kernel-map cache reset before every forward); plus the
+    Gather / GEMM / Scatter kernels one by one on the configuration-2 cloud."""
     import torch
     import minuet_amd as minuet
     from minuet_amd.nn.functional import _C
@@ -68,6 +159,10 @@ def extras(device):
     from minuet_amd.unet import SparseUNet
 
     out = {}
+    if section == "layer-kernels":
+        return {"config2_layer_kernels_fp16_c64": layer_stages(device, 2, 64, 3, "fp16")}
+    if section == "config5":
+        return {"config5_layer_bf16_c64_k5": layer_stages(device, 5, 64, 5, "bf16")}
     with torch.no_grad():
         # configuration 1: submanifold 3x3x3, 32 -> 32, fp32
         c1 = torch.from_numpy(make_cloud(1)["coords"]).to(device)
@@ -75,17 +170,16 @@ def extras(device):
         conv = minuet.nn.SparseConv3d(32, 32, 3, dtype=torch.float32, device=device)
         cache = minuet.nn.KernelMapCache(3, torch.int32, device)
         conv.set_kernel_map_cache(cache)
-        conv.tunable_config.update(gather_tile_size=0, scatter_tile_size=0)
         x = minuet.SparseTensor(torch.randn(s1.shape[0], 32, device=device), s1)
-        warm = _time_ms(lambda: conv(x), 20, 200)
+        warm = _time_stats(lambda: conv(x), 20, 200)
 
         def cold1():
             cache.reset()
             conv(x)
-        cold = _time_ms(cold1, 20, 200)
-        out["config1_layer_fp32"] = {"voxels": int(s1.shape[0]), "ms_map_cached": round(warm, 4),
-                                     "ms_map_included": round(cold, 4),
-                                     "mvoxels_per_s_map_cached": round(s1.shape[0] / warm / 1e3, 1)}
+        cold = _time_stats(cold1, 20, 200)
+        out["config1_layer_fp32"] = {"voxels": int(s1.shape[0]), "map_cached": warm, "map_included": cold,
+                                     "mvoxels_per_s_map_cached": round(s1.shape[0] / warm["ms_mean"] / 1e3, 1),
+                                     "mvoxels_per_s_map_included": round(s1.shape[0] / cold["ms_mean"] / 1e3, 1)}
         # configuration 3: stride-2 down conv 64 -> 128 then transposed 128 -> 64, fp16
         c3 = torch.from_numpy(make_cloud(3)["coords"]).to(device)
         _, s3 = _C.sort_coordinates(c3)
@@ -94,11 +188,15 @@ def extras(device):
         cache3 = minuet.nn.KernelMapCache(3, torch.int32, device)
         for m in (down, up):
             m.set_kernel_map_cache(cache3)
-            m.tunable_config.update(gather_tile_size=0, scatter_tile_size=0)
         x3 = minuet.SparseTensor(torch.randn(s3.shape[0], 64, device=device).half(), s3)
-        pair = _time_ms(lambda: up(down(x3)), 20, 200)
-        out["config3_down_up_fp16"] = {"voxels": int(s3.shape[0]), "ms_map_cached": round(pair, 4),
-                                       "mvoxels_per_s_map_cached": round(s3.shape[0] / pair / 1e3, 1)}
+        pair = _time_stats(lambda: up(down(x3)), 20, 200)
+
+        def cold3():
+            cache3.reset()
+            up(down(x3))
+        pair_cold = _time_stats(cold3, 10, 100)
+        out["config3_down_up_fp16"] = {"voxels": int(s3.shape[0]), "map_cached": pair, "map_included": pair_cold,
+                                       "mvoxels_per_s_map_cached": round(s3.shape[0] / pair["ms_mean"] / 1e3, 1)}
         # configuration 4: sparse UNet forward, fp16, batch of two scans
         cloud = make_cloud(4)
         c4 = torch.from_numpy(cloud["coords"]).to(device)
@@ -107,17 +205,22 @@ def extras(device):
         net = SparseUNet(4, 32, dtype=torch.float16, device=device).eval()
         cache4 = minuet.nn.KernelMapCache(3, torch.int32, device)
         minuet.set_kernel_map_cache(net, cache4)
-        for m in net.modules():
-            if isinstance(m, minuet.nn.SparseConv):
-                m.tunable_config.update(gather_tile_size=0, scatter_tile_size=0)
         x4 = minuet.SparseTensor(torch.randn(s4.shape[0], 4, device=device).half(), s4, batch_dims=bd)
 
         def forward():
             cache4.reset()
             net(x4)
-        lat = _time_ms(forward, 5, 30)
-        out["config4_unet_fp16"] = {"voxels": int(s4.shape[0]), "batch": 2,
-                                    "forward_ms_cold_cache": round(lat, 3)}
+        lat = _time_stats(forward, 5, 50)
+        kept = _time_stats(lambda: net(x4), 5, 50)
+        out["config4_unet_fp16"] = {"voxels": int(s4.shape[0]), "batch": 2, "cold_cache": lat,
+                                    "kernel_maps_cached": kept,
+                                    "forward_ms_cold_cache": lat["ms_median"]}
+        del net, cache4, x4
+    if section == "unet":
+        return {"config4_unet_fp16": out["config4_unet_fp16"]}
+    out["config2_layer_kernels_fp16_c64"] = layer_stages(device, 2, 64, 3, "fp16")
+    if with_config5:
+        out["config5_layer_bf16_c64_k5"] = layer_stages(device, 5, 64, 5, "bf16")
     return out
 
 
@@ -130,6 +233,12 @@ def main():
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     parser.add_argument("--no-extras", action="store_true",
                         help="skip the layer-throughput and UNet-latency side measurements")
+    parser.add_argument("--no-config5", action="store_true",
+                        help="skip the 1M-voxel 5x5x5 layer of configuration 5 (half a minute of "
+                             "cloud generation)")
+    parser.add_argument("--section", default="all",
+                        choices=["all", "layer-kernels", "config5", "unet"],
+                        help="which of the side measurements to run (profiles isolate one)")
     parser.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                         help="also run one plain device copy of this many MiB (a known-size "
                              "reference for scaling profiler byte counters)")
@@ -227,7 +336,7 @@ def main():
                      "achieved": None if achieved is None else round(achieved, 2),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": None if achieved is None else round(achieved / HBM_PEAK_GBS, 5),
-                     "traffic": None,
+                     "traffic": QUERY_TRAFFIC_BYTES if args.scale == 1.0 else None,
                      "algorithmic_bytes": bytes_query,
                      "avg_launch_ms": None if achieved is None else round(query_ms, 5),
                      "map_step": {"algorithmic_bytes": bytes_map,
@@ -237,7 +346,7 @@ def main():
                                   "stage_ms": {k: round(v, 5) for k, v in stage_ms.items()}}},
     }
     if not args.no_extras:
-        result["extra"] = extras(device)
+        result["extra"] = extras(device, not args.no_config5, args.section)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(coords, offsets32)
     else:
