@@ -5,6 +5,7 @@ import torch
 
 import minuet_oracle as orc
 from helpers import dev, host, random_cloud, sorted_unique
+import minuet_amd as minuet
 from minuet_amd.nn import functional as F
 from minuet_amd.nn.functional import _C
 
@@ -179,3 +180,44 @@ def test_kernel_map_build(reorder, kernel, stride, batched):
     e2in, e2out, _ = orc.kernel_map_pair_lists(dense)
     np.testing.assert_array_equal(host(in2), e2in)
     np.testing.assert_array_equal(host(out2), e2out)
+
+
+def test_voxelize_matches_numpy_unique():
+    """floor(p / voxel) -> distinct voxels in lexicographic order, and the
+    reverse map sends every point to its voxel (checked with np.unique)."""
+    rng = np.random.default_rng(31)
+    points = rng.uniform(-3.0, 3.0, size=(20000, 3)).astype(np.float32)
+    size = (0.25, 0.5, 0.125)
+    expect, inverse = np.unique(np.floor(points / np.asarray(size, dtype=np.float32)).astype(np.int32),
+                                axis=0, return_inverse=True)
+    voxels, reverse = F.voxelize(dev(points), voxel_size=size, return_reverse_indices=True)
+    assert voxels.dtype == torch.int32
+    np.testing.assert_array_equal(host(voxels), expect)
+    np.testing.assert_array_equal(host(reverse), inverse.reshape(-1))
+    np.testing.assert_array_equal(host(F.voxelize(dev(points), voxel_size=size)), expect)
+    only = F.voxelize(dev(points), voxel_size=100.0, dtype=torch.int64)
+    assert only.dtype == torch.int64 and only.shape[0] <= 8
+    with pytest.raises(NotImplementedError):
+        F.voxelize(torch.zeros(4, 3))
+
+
+def test_collate_sorts_each_cloud_and_carries_features():
+    clouds = [sorted_unique(random_cloud(n, 12, seed=s, lo=-6))[0] for n, s in ((700, 1), (300, 2), (1, 3))]
+    rng = np.random.default_rng(5)
+    shuffled, feats = [], []
+    for c in clouds:
+        perm = rng.permutation(c.shape[0])
+        shuffled.append(dev(c[perm]))
+        # a feature row that names its coordinate, so that the pairing can be checked
+        feats.append(dev(c[perm].astype(np.float32) * 2.0))
+    coords, bd, f = F.collate(shuffled, feats)
+    sizes = [c.shape[0] for c in clouds]
+    np.testing.assert_array_equal(host(bd), np.concatenate([[0], np.cumsum(sizes)]))
+    np.testing.assert_array_equal(host(coords), np.concatenate(clouds))
+    np.testing.assert_array_equal(host(f), np.concatenate(clouds).astype(np.float32) * 2.0)
+    x = minuet.SparseTensor(f, coords, batch_dims=bd)
+    assert x.batch_dims is not None and x.C.shape[0] == sum(sizes)
+    coords_only, bd2 = F.collate(shuffled)
+    assert torch.equal(coords_only, coords) and torch.equal(bd2, bd)
+    with pytest.raises(ValueError):
+        F.collate([])
