@@ -245,7 +245,12 @@ int mnt_sparse_convolution_forward(int64_t gather_tile, int64_t scatter_tile,
  * (the bias add of minuet/nn/convolutions.py:496-497, an inference-mode
  * minuet/nn/normalizations.py BatchNorm, minuet/nn/activations.py ReLU /
  * LeakyReLU / ReLU6 and a residual sum) are absorbed into Scatter's single
- * write of the output row. */
+ * write of the output row.
+ * packed_weights (nullable): the output of mnt_pack_weights for `weights`,
+ * kept by the caller for as long as the weights do not change; the pass then
+ * skips its own packing.  Packed weights are in the layer's own offset order,
+ * so with a kernel_map_order the call also needs order_host (int64[O], the
+ * host copy of kernel_map_order; NULL otherwise). */
 int mnt_sparse_convolution_forward_fused(int64_t gather_tile, int64_t scatter_tile,
                                          int allow_shortcut_matmul, int64_t parallel,
                                          int has_threshold, double threshold,
@@ -262,7 +267,19 @@ int mnt_sparse_convolution_forward_fused(int64_t gather_tile, int64_t scatter_ti
                                          const float *channel_scale, const float *channel_shift,
                                          const void *residual, int activation,
                                          float negative_slope,
+                                         const void *packed_weights,
+                                         const int64_t *order_host,
                                          void *out, void *stream);
+
+/* Weights [O, Cin, Cout] -> the layout the matrix kernels stage:
+ * packed[O][Np][Kp] = W^T per offset, K-contiguous, zero-padded to
+ * Np = ceil(Cout / 32) * 32 rows of Kp = ceil(Cin * e / 128) * 128 / e elements
+ * (e = element size).  Offsets stay in the order given.  Takes the place of
+ * PermuteWeights (csrc/minuet/cuda/kernels/permute_weights.cuh:8-36), which the
+ * reference runs inside every forward. */
+int mnt_pack_weights(const void *weights, int64_t num_offsets, int64_t num_source_features,
+                     int64_t num_target_features, int float_dtype, void *packed_out,
+                     void *stream);
 
 /* Timers used by the autotuner: run the named stage once on scratch buffers and
  * return the elapsed milliseconds through ms_out (synchronise).
@@ -294,7 +311,8 @@ int mnt_time_gemm(int allow_shortcut_matmul, int64_t parallel, int has_threshold
  * walks the offsets.  Requires Cin * sizeof(element) to be a multiple of 16
  * and at most 128, Cout % 4 == 0 and Cout <= 128; it pays for small channel counts, where the three-kernel
  * form is bound by the buffer traffic.  The epilogue arguments are those of
- * mnt_sparse_convolution_forward_fused.  Results agree with the other forms to
+ * mnt_sparse_convolution_forward_fused; packed_weights (nullable) is the
+ * output of mnt_pack_weights for `weights`.  Results agree with the other forms to
  * rounding (sums are kept in fp32 over all offsets and rounded once).
  * Covers the same reference code as mnt_sparse_convolution_forward
  * (csrc/minuet/cuda/functions/sparse_convolution.cu:504-661); the reference
@@ -307,6 +325,7 @@ int mnt_sparse_convolution_forward_implicit(const void *sources, const void *wei
                                             const float *channel_scale,
                                             const float *channel_shift, const void *residual,
                                             int activation, float negative_slope,
+                                            const void *packed_weights,
                                             void *out, void *stream);
 
 /* The dense kernel map of the transposed layer that shares a forward layer's

@@ -393,7 +393,7 @@ struct BufferOf<bf16_t> { typedef float type; };
 
 constexpr int kGemmBlock = 256;
 constexpr int kGemmRows = 128;          // rows of A per workgroup (32 per wavefront)
-constexpr int kMaxChannelBlocks = 8;    // 32-channel blocks per workgroup (256 channels)
+constexpr int kMaxChannelBlocks = 4;    // 32-channel blocks per workgroup (128 channels)
 
 // meta: [G | tile_prefix (G+1) | row_start (G+1) | rows (G) | weight (G) | list_start (G)]
 //
@@ -407,46 +407,56 @@ constexpr int kMaxChannelBlocks = 8;    // 32-channel blocks per workgroup (256 
 // MFMA operand.  The same K permutation is applied to the weights (lane half
 // h of step kk reads the same bytes of its channel row), which leaves the
 // dot products unchanged.  Only the weights (W^T, K-contiguous, padded) are
-// staged in LDS, shared by the four wavefronts; all NB channel blocks are
-// accumulated in registers, so A is read exactly once.
+// staged in LDS, shared by the four wavefronts; the NB channel blocks of a
+// workgroup (up to 128 channels) are accumulated in registers, so A is read
+// once per 128-channel slice of the output.
 //
 // With `gather_index` (nullable) the Gather step is folded into the A load:
 // data row i of group g is then row gather_index[list_start[g] + i] of `a`
 // (the source features) instead of buffer row row_start[g] + i, and no gather
-// buffer exists.  The output rows stay in buffer order either way.
+// buffer exists; a group with list_start < 0 reads row i of `a` itself (the
+// centre offset of the shortcut).  The output rows stay in buffer order.
+//
+// The tables reach the kernel either in device memory (`meta`) or, when
+// table_count > 0, as the by-value argument `table` (meta starts at entry
+// meta_at); workgroup (0, 0) then also copies the whole table to `table_out`
+// for the kernels that follow in the stream, so that no separate upload runs.
 template <typename T, typename TC, int NB, bool VEC>
 __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
     const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt,
     const int *__restrict__ meta, int K, int N, int Kp, int Np,
-    const int *__restrict__ gather_index) {
+    const int *__restrict__ gather_index, PlanChunk table, int table_count, int meta_at,
+    int *__restrict__ table_out) {
   constexpr int EPC = 16 / static_cast<int>(sizeof(T));        // elements per 16-byte piece
   constexpr int KC = kChunkBytes / static_cast<int>(sizeof(T));
   constexpr int TN = NB * 32;
   __shared__ __align__(16) unsigned char b_lds[TN * kLdsRowBytes];
 
-  const int G = meta[0];
-  const int *tile_prefix = meta + 1;
-  const int *row_start = tile_prefix + G + 1;
-  const int *rows = row_start + G + 1;
-  const int *weight = rows + G;
-  const int *list_start = weight + G;
+  if (table_count > 0 && blockIdx.x == 0 && blockIdx.y == 0) {
+    for (int i = threadIdx.x; i < table_count; i += kGemmBlock) table_out[i] = table.v[i];
+  }
+  auto entry = [&](int i) -> int { return table_count > 0 ? table.v[meta_at + i] : meta[i]; };
+  const int G = entry(0);
+  const int at_prefix = 1, at_start = at_prefix + G + 1, at_rows = at_start + G + 1, at_weight = at_rows + G,
+            at_list = at_weight + G;
 
   const int tile = blockIdx.x;
   int lo = 0, hi = G - 1;
   while (lo < hi) {
     const int mid = (lo + hi + 1) >> 1;
-    if (tile_prefix[mid] <= tile) {
+    if (entry(at_prefix + mid) <= tile) {
       lo = mid;
     } else {
       hi = mid - 1;
     }
   }
   const int g = lo;
-  const int r0 = (tile - tile_prefix[g]) * kGemmRows;
-  const int valid = min(kGemmRows, rows[g] - r0);
-  const long long row_base = static_cast<long long>(row_start[g]) + r0;
+  const int r0 = (tile - entry(at_prefix + g)) * kGemmRows;
+  const int valid = min(kGemmRows, entry(at_rows + g) - r0);
+  const long long row_base = static_cast<long long>(entry(at_start + g)) + r0;
   const int n0 = blockIdx.y * TN;
-  const T *w_base = wt + (static_cast<long long>(weight[g]) * Np + n0) * Kp;
+  const T *w_base = wt + (static_cast<long long>(entry(at_weight + g)) * Np + n0) * Kp;
+  const int list_at = entry(at_list + g);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -457,7 +467,8 @@ __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
   const bool row_ok = row < valid;
   long long a_index = row_base + row;
   if (gather_index != nullptr) {
-    a_index = row_ok ? gather_index[static_cast<long long>(list_start[g]) + r0 + row] : 0;
+    a_index = list_at < 0 ? r0 + row
+                          : (row_ok ? gather_index[static_cast<long long>(list_at) + r0 + row] : 0);
   }
   const T *a_row = a + a_index * K;
 
@@ -646,7 +657,14 @@ static void launch_scatter(const LaneShape &sh, const TB *buffer, void *targets,
                            const TB *direct, const Epilogue &ep, hipStream_t stream) {
   if (num_targets == 0) return;
   const bool listed = num_offsets <= kScatterListedOffsets && sh.lanes_per_row <= kScatterBlock;
-  const int tile_shift = num_offsets <= 128 ? 6 : 5;
+  // 64 targets per workgroup (32 for large kernels, so that the row lists fit
+  // in LDS); fewer when that would leave most of the chip without a workgroup,
+  // but never fewer than the lane groups of a workgroup
+  int tile_shift = num_offsets <= 128 ? 6 : 5;
+  const int groups = std::max(1, kScatterBlock / sh.lanes_per_row);
+  while (tile_shift > 3 && (num_targets >> tile_shift) < 1024 && (1 << (tile_shift - 1)) >= groups) {
+    --tile_shift;
+  }
   const unsigned grid =
       listed ? static_cast<unsigned>(div_ceil(num_targets, int64_t{1} << tile_shift))
              : static_cast<unsigned>(div_ceil(num_targets * sh.lanes_per_row, 256));
@@ -687,38 +705,53 @@ static void launch_scatter(const LaneShape &sh, const TB *buffer, void *targets,
   check_launch("scatter_kernel");
 }
 
+// Integer tables that ride a GEMM launch as a kernel argument (count == 0:
+// none, the kernel reads `meta` from device memory).
+struct RidingTable {
+  const std::vector<int> *ints = nullptr;
+  int meta_at = 0;
+  int *out = nullptr;
+};
+
 template <typename T, typename TC, int NB>
 static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int num_tiles, int K, int N,
-                           int Kp, int Np, bool vec, const int *gather_index, hipStream_t stream) {
+                           int Kp, int Np, bool vec, const int *gather_index, const RidingTable &riding,
+                           hipStream_t stream) {
   dim3 grid(num_tiles, static_cast<unsigned>(div_ceil(Np, NB * 32)));
+  PlanChunk chunk;
+  int count = 0;
+  if (riding.ints != nullptr) {
+    count = static_cast<int>(riding.ints->size());
+    std::memcpy(chunk.v, riding.ints->data(), count * sizeof(int));
+  }
   if (vec) {
-    grouped_gemm_kernel<T, TC, NB, true><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np,
-                                                                          gather_index);
+    grouped_gemm_kernel<T, TC, NB, true><<<grid, kGemmBlock, 0, stream>>>(
+        a, c, wt, meta, K, N, Kp, Np, gather_index, chunk, count, riding.meta_at, riding.out);
   } else {
-    grouped_gemm_kernel<T, TC, NB, false><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np,
-                                                                          gather_index);
+    grouped_gemm_kernel<T, TC, NB, false><<<grid, kGemmBlock, 0, stream>>>(
+        a, c, wt, meta, K, N, Kp, Np, gather_index, chunk, count, riding.meta_at, riding.out);
   }
 }
 
 template <typename T, typename TC>
 static void launch_gemm(const T *a, TC *c, const T *wt, const int *meta, int num_tiles, int K, int N,
-                        int Kp, int Np, const int *gather_index, hipStream_t stream) {
+                        int Kp, int Np, const int *gather_index, hipStream_t stream,
+                        const RidingTable &riding = RidingTable()) {
   if (num_tiles == 0) return;
   const bool vec = (static_cast<int64_t>(K) * sizeof(T)) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(a) % 16 == 0 && N % 4 == 0 &&
                    reinterpret_cast<uintptr_t>(c) % 16 == 0;
-  // all channels in one workgroup up to 256; wider outputs are cut into
-  // 256-channel slices (A is then read once per slice)
+  // All channels in one workgroup up to 128; wider outputs are cut into equal
+  // slices of at most 128 channels (A is then read once per slice).  Eight
+  // blocks per workgroup would read A once at 256 channels, but their 128
+  // accumulator registers leave one workgroup per CU and measured slower.
   const int blocks = Np / 32;
-  switch (blocks >= kMaxChannelBlocks ? kMaxChannelBlocks : blocks) {
-    case 1: launch_gemm_nb<T, TC, 1>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
-    case 2: launch_gemm_nb<T, TC, 2>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
-    case 3: launch_gemm_nb<T, TC, 3>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
-    case 4: launch_gemm_nb<T, TC, 4>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
-    case 5: launch_gemm_nb<T, TC, 5>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
-    case 6: launch_gemm_nb<T, TC, 6>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
-    case 7: launch_gemm_nb<T, TC, 7>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
-    default: launch_gemm_nb<T, TC, 8>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, stream); break;
+  const int slices = static_cast<int>(div_ceil(blocks, kMaxChannelBlocks));
+  switch (static_cast<int>(div_ceil(blocks, slices))) {
+    case 1: launch_gemm_nb<T, TC, 1>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream); break;
+    case 2: launch_gemm_nb<T, TC, 2>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream); break;
+    case 3: launch_gemm_nb<T, TC, 3>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream); break;
+    default: launch_gemm_nb<T, TC, 4>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream); break;
   }
   check_launch("grouped_gemm_kernel");
 }
@@ -806,8 +839,9 @@ template <typename T, typename IT>
 static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const ForwardPlan &plan,
                           const T *sources, const T *weights, const IT *source_masks,
                           const IT *target_masks, const IT *order, const int *gather_index,
-                          const Epilogue &epilogue, int64_t S, int64_t Tn, int64_t O, int64_t K,
-                          int64_t N, T *out, hipStream_t stream) {
+                          const Epilogue &epilogue, const T *packed, const int64_t *order_host,
+                          int64_t S, int64_t Tn, int64_t O, int64_t K, int64_t N, T *out,
+                          hipStream_t stream) {
   Scope scope(stream);
   const int kc = kChunkBytes / static_cast<int>(sizeof(T));
   const int Kp = static_cast<int>(div_ceil(K, kc) * kc);
@@ -815,26 +849,79 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
   const int active = static_cast<int>(plan.active_offsets);
 
   profile_mark("enter:forward", stream);
-  // one integer table for the whole pass: row starts, GEMM groups, and the
-  // single-group descriptor of the centre-offset product
+  const bool folded = gather_index != nullptr;      // Gather folded into the GEMM's A load
+  const bool ahead = packed != nullptr;             // weights packed by the caller
+  const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
+  const int64_t centre = ahead && order_host != nullptr && O > 0 ? order_host[O - 1] : O - 1;
+
+  // One integer table for the whole pass: row starts, then the GEMM groups.
+  // With the folded gather both products read the source features, so the
+  // centre offset of the shortcut joins the grouped launch as one more group
+  // (rows taken as they are, output after the other buffer rows); otherwise
+  // its single-group descriptor follows for a launch of its own.
+  std::vector<int> meta(plan.meta);
+  int num_tiles = plan.num_tiles;
+  if (ahead && order_host != nullptr) {
+    // weights packed ahead of time are in the layer's own offset order: point
+    // every GEMM group at the matrix of the offset its row stands for
+    const int G = meta[0];
+    int *weight = meta.data() + 1 + (G + 1) + (G + 1) + G;
+    for (int i = 0; i < G; ++i) weight[i] = static_cast<int>(order_host[weight[i]]);
+  }
+  const bool merged = plan.shortcut && folded;
+  if (merged) {
+    const int G = meta[0];
+    const int *tile_prefix = meta.data() + 1, *row_start = tile_prefix + G + 1, *count = row_start + G + 1,
+              *weight = count + G, *list_start = weight + G;
+    const int extra = static_cast<int>(div_ceil(S, kGemmRows));
+    std::vector<int> grown;
+    grown.push_back(G + 1);
+    grown.insert(grown.end(), tile_prefix, tile_prefix + G + 1);
+    grown.push_back(tile_prefix[G] + extra);
+    grown.insert(grown.end(), row_start, row_start + G);
+    grown.push_back(static_cast<int>(rows));
+    grown.push_back(static_cast<int>(rows + S));
+    grown.insert(grown.end(), count, count + G);
+    grown.push_back(static_cast<int>(S));
+    grown.insert(grown.end(), weight, weight + G);
+    grown.push_back(static_cast<int>(centre));
+    grown.insert(grown.end(), list_start, list_start + G);
+    grown.push_back(-1);
+    meta.swap(grown);
+    num_tiles += extra;
+  }
   std::vector<int> ints(plan.row_start);
   const size_t meta_at = ints.size();
-  ints.insert(ints.end(), plan.meta.begin(), plan.meta.end());
+  ints.insert(ints.end(), meta.begin(), meta.end());
   const size_t direct_at = ints.size();
   std::vector<int> dmeta;
-  if (plan.shortcut) {
-    dmeta = direct_meta(S, static_cast<int>(O - 1));
+  if (plan.shortcut && !merged) {
+    dmeta = direct_meta(S, static_cast<int>(centre));
     ints.insert(ints.end(), dmeta.begin(), dmeta.end());
   }
   int *d_ints = scope.alloc<int>(ints.size());
   int *d_row_start = d_ints;
   int *d_meta = d_ints + meta_at;
   int *d_direct = d_ints + direct_at;
-  T *wt = scope.alloc<T>(static_cast<size_t>(O) * Np * Kp);
-  {
+  const bool fits = ints.size() <= static_cast<size_t>(kPlanInts);
+  // the table travels as an argument of the first kernel of the pass: the
+  // packing kernel, or with packed weights and the folded gather the GEMM
+  RidingTable riding;
+  const T *wt = packed;
+  if (ahead) {
+    if (fits && folded && num_tiles > 0) {
+      riding.ints = &ints;
+      riding.meta_at = static_cast<int>(meta_at);
+      riding.out = d_ints;
+    } else {
+      upload_ints(ints, d_ints, stream);
+    }
+  } else {
+    T *fresh = scope.alloc<T>(static_cast<size_t>(O) * Np * Kp);
+    wt = fresh;
     PlanChunk chunk;
     int count = 0;
-    if (ints.size() <= static_cast<size_t>(kPlanInts)) {
+    if (fits) {
       count = static_cast<int>(ints.size());
       std::memcpy(chunk.v, ints.data(), ints.size() * sizeof(int));
     } else {
@@ -842,32 +929,30 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
     }
     const long long total = static_cast<long long>(O) * Np * Kp;
     pack_weights_kernel<T, IT><<<grid_for(total, 256, 4096), 256, 0, stream>>>(
-        weights, order, static_cast<int>(O), static_cast<int>(K), static_cast<int>(N), Kp, Np, wt, chunk,
+        weights, order, static_cast<int>(O), static_cast<int>(K), static_cast<int>(N), Kp, Np, fresh, chunk,
         count, d_ints);
     check_launch("pack_weights_kernel");
   }
   profile_mark("pack_weights", stream);
 
-  const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
   typedef typename BufferOf<T>::type TB;
   // with the shortcut the centre offset's product takes one extra buffer row per target
   TB *cbuf = scope.alloc<TB>((rows + (plan.shortcut ? static_cast<size_t>(Tn) : 0)) * N);
   TB *direct = plan.shortcut ? cbuf + rows * N : nullptr;
 
-  if (gather_index != nullptr) {
-    // Gather folded into the GEMM's A load: no gather buffer
-    launch_gemm<T, TB>(sources, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp,
-                       Np, gather_index, stream);
+  if (folded) {
+    launch_gemm<T, TB>(sources, cbuf, wt, d_meta, num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np,
+                       gather_index, stream, riding);
   } else {
     T *abuf = scope.alloc<T>(rows * K);
     const LaneShape gsh = lane_shape(gather_tile, K, sizeof(T), sources, abuf, "num_source_features");
     launch_gather<IT>(gsh, sources, abuf, source_masks, d_row_start, S, active,
                       static_cast<int>(K * sizeof(T)), stream);
     profile_mark("gather", stream);
-    launch_gemm<T, TB>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np,
+    launch_gemm<T, TB>(abuf, cbuf, wt, d_meta, num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np,
                        nullptr, stream);
   }
-  if (plan.shortcut) {
+  if (plan.shortcut && !merged) {
     launch_gemm<T, TB>(sources, direct, wt, d_direct, dmeta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np,
                        nullptr, stream);
   }
@@ -927,7 +1012,8 @@ extern "C" int mnt_sparse_convolution_forward_fused(
     const void *kernel_map_sizes, const int64_t *sizes_host, int64_t S, int64_t T, int64_t O,
     int64_t K, int64_t N, int index_dtype, int float_dtype, const int32_t *gather_index,
     const float *channel_scale, const float *channel_shift, const void *residual, int activation,
-    float negative_slope, void *out, void *stream_) {
+    float negative_slope, const void *packed_weights, const int64_t *order_host, void *out,
+    void *stream_) {
   (void)parallel;
   return guarded([&] {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -943,6 +1029,15 @@ extern "C" int mnt_sparse_convolution_forward_fused(
                   reinterpret_cast<uintptr_t>(channel_scale) % 4 == 0 &&
                   reinterpret_cast<uintptr_t>(channel_shift) % 4 == 0,
               "epilogue operands are not aligned (residual: 16 bytes, scale / shift: 4 bytes)");
+    MNT_CHECK(packed_weights == nullptr || kernel_map_order == nullptr || order_host != nullptr,
+              "weights packed ahead of time need the host copy of kernel_map_order");
+    MNT_CHECK(reinterpret_cast<uintptr_t>(packed_weights) % 16 == 0, "packed weights are not 16-byte aligned");
+    if (order_host != nullptr) {
+      for (int64_t j = 0; j < O; ++j) {
+        MNT_CHECK(order_host[j] >= 0 && order_host[j] < O, "order_host[%lld] = %lld is out of range",
+                  (long long)j, (long long)order_host[j]);
+      }
+    }
     if (T == 0) return;
     MNT_CHECK(out != nullptr, "out is null");
     std::vector<int64_t> sizes;
@@ -962,7 +1057,9 @@ extern "C" int mnt_sparse_convolution_forward_fused(
   forward_typed<FT, IT>(gather_tile, scatter_tile, plan, static_cast<const FT *>(sources),          \
                         static_cast<const FT *>(weights), static_cast<const IT *>(source_masks),    \
                         static_cast<const IT *>(target_masks), static_cast<const IT *>(kernel_map_order), \
-                        gather_index, epilogue, S, T, O, K, N, static_cast<FT *>(out), stream)
+                        gather_index, epilogue, static_cast<const FT *>(packed_weights),             \
+                        kernel_map_order != nullptr ? order_host : nullptr, S, T, O, K, N,          \
+                        static_cast<FT *>(out), stream)
     MNT_DISPATCH_FI(float_dtype, index_dtype, MNT_CALL);
 #undef MNT_CALL
   });
@@ -978,8 +1075,37 @@ extern "C" int mnt_sparse_convolution_forward(
   return mnt_sparse_convolution_forward_fused(
       gather_tile, scatter_tile, allow_shortcut_matmul, parallel, has_threshold, threshold, sources,
       weights, source_masks, target_masks, kernel_map_order, kernel_map_sizes, sizes_host, S, T, O, K,
-      N, index_dtype, float_dtype, gather_index, nullptr, nullptr, nullptr, MNT_ACT_NONE, 0.0f, out,
-      stream_);
+      N, index_dtype, float_dtype, gather_index, nullptr, nullptr, nullptr, MNT_ACT_NONE, 0.0f, nullptr,
+      nullptr, out, stream_);
+}
+
+extern "C" int mnt_pack_weights(const void *weights, int64_t O, int64_t K, int64_t N, int float_dtype,
+                                void *packed_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int esize = float_size(float_dtype);
+    MNT_CHECK(O >= 0 && O <= 65535 && K >= 1 && N >= 1 && K <= 65536 && N <= 65536,
+              "bad shape O=%lld Cin=%lld Cout=%lld", (long long)O, (long long)K, (long long)N);
+    if (O == 0) return;
+    MNT_CHECK(weights != nullptr && packed_out != nullptr, "null operand");
+    const int kc = kChunkBytes / esize;
+    const int Kp = static_cast<int>(div_ceil(K, kc) * kc);
+    const int Np = static_cast<int>(div_ceil(N, 32) * 32);
+    const long long total = static_cast<long long>(O) * Np * Kp;
+#define MNT_PACK(FT)                                                                               \
+  pack_weights_kernel<FT, int32_t><<<grid_for(total, 256, 4096), 256, 0, stream>>>(                \
+      static_cast<const FT *>(weights), nullptr, static_cast<int>(O), static_cast<int>(K),         \
+      static_cast<int>(N), Kp, Np, static_cast<FT *>(packed_out), PlanChunk{}, 0, nullptr)
+    if (float_dtype == MNT_FLOAT32) {
+      MNT_PACK(float);
+    } else if (float_dtype == MNT_FLOAT16) {
+      MNT_PACK(half_t);
+    } else {
+      MNT_PACK(bf16_t);
+    }
+#undef MNT_PACK
+    check_launch("pack_weights_kernel");
+  });
 }
 
 // ---------------------------------------------------------- stage timers ----

@@ -246,21 +246,25 @@ __global__ __launch_bounds__(256) void fill_minus_one_kernel(int *__restrict__ d
 }
 
 template <typename T>
-static void implicit_typed(const T *sources, const T *weights, const int *kernel_map, int64_t S,
-                           int64_t Tn, int64_t O, int64_t K, int64_t N, const Epilogue &ep, T *out,
-                           hipStream_t stream) {
+static void implicit_typed(const T *sources, const T *weights, const T *packed, const int *kernel_map,
+                           int64_t S, int64_t Tn, int64_t O, int64_t K, int64_t N, const Epilogue &ep,
+                           T *out, hipStream_t stream) {
   Scope scope(stream);
   const int kc = kChunkBytes / static_cast<int>(sizeof(T));
   const int Kp = static_cast<int>(div_ceil(K, kc) * kc);
   const int Np = static_cast<int>(div_ceil(N, 32) * 32);
   profile_mark("enter:implicit", stream);
-  T *wt = scope.alloc<T>(static_cast<size_t>(O) * Np * Kp);
-  const long long total = static_cast<long long>(O) * Np * Kp;
-  pack_weights_kernel<T, int32_t><<<grid_for(total, 256, 4096), 256, 0, stream>>>(
-      weights, nullptr, static_cast<int>(O), static_cast<int>(K), static_cast<int>(N), Kp, Np, wt,
-      PlanChunk{}, 0, nullptr);
-  check_launch("pack_weights_kernel");
-  profile_mark("pack_weights", stream);
+  const T *wt = packed;
+  if (packed == nullptr) {
+    T *fresh = scope.alloc<T>(static_cast<size_t>(O) * Np * Kp);
+    wt = fresh;
+    const long long total = static_cast<long long>(O) * Np * Kp;
+    pack_weights_kernel<T, int32_t><<<grid_for(total, 256, 4096), 256, 0, stream>>>(
+        weights, nullptr, static_cast<int>(O), static_cast<int>(K), static_cast<int>(N), Kp, Np, fresh,
+        PlanChunk{}, 0, nullptr);
+    check_launch("pack_weights_kernel");
+    profile_mark("pack_weights", stream);
+  }
   const unsigned grid = static_cast<unsigned>(div_ceil(Tn, kImplicitTargets));
   const unsigned source_bytes = static_cast<unsigned>(S * K * sizeof(T));
 #define MNT_IMPLICIT(NB, KS)                                                                       \
@@ -293,7 +297,7 @@ extern "C" int mnt_sparse_convolution_forward_implicit(
     const void *sources, const void *weights, const int32_t *kernel_map, int64_t S, int64_t T,
     int64_t O, int64_t K, int64_t N, int float_dtype, const float *channel_scale,
     const float *channel_shift, const void *residual, int activation, float negative_slope,
-    void *out, void *stream_) {
+    const void *packed_weights, void *out, void *stream_) {
   return guarded([&] {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const int esize = float_size(float_dtype);
@@ -317,17 +321,19 @@ extern "C" int mnt_sparse_convolution_forward_implicit(
                   reinterpret_cast<uintptr_t>(channel_shift) % 4 == 0,
               "operands are not aligned (features, out, residual: 16 bytes, scale / shift: 4 bytes)");
     if (T == 0) return;
-    MNT_CHECK(out != nullptr && kernel_map != nullptr && weights != nullptr, "null operand");
+    MNT_CHECK(out != nullptr && kernel_map != nullptr && (weights != nullptr || packed_weights != nullptr),
+              "null operand");
+    MNT_CHECK(reinterpret_cast<uintptr_t>(packed_weights) % 16 == 0, "packed weights are not 16-byte aligned");
     const Epilogue ep = {channel_scale, channel_shift, residual, activation, negative_slope};
     if (float_dtype == MNT_FLOAT32) {
       implicit_typed<float>(static_cast<const float *>(sources), static_cast<const float *>(weights),
-                            kernel_map, S, T, O, K, N, ep, static_cast<float *>(out), stream);
+                            static_cast<const float *>(packed_weights), kernel_map, S, T, O, K, N, ep, static_cast<float *>(out), stream);
     } else if (float_dtype == MNT_FLOAT16) {
       implicit_typed<half_t>(static_cast<const half_t *>(sources), static_cast<const half_t *>(weights),
-                             kernel_map, S, T, O, K, N, ep, static_cast<half_t *>(out), stream);
+                             static_cast<const half_t *>(packed_weights), kernel_map, S, T, O, K, N, ep, static_cast<half_t *>(out), stream);
     } else {
       implicit_typed<bf16_t>(static_cast<const bf16_t *>(sources), static_cast<const bf16_t *>(weights),
-                             kernel_map, S, T, O, K, N, ep, static_cast<bf16_t *>(out), stream);
+                             static_cast<const bf16_t *>(packed_weights), kernel_map, S, T, O, K, N, ep, static_cast<bf16_t *>(out), stream);
     }
   });
 }

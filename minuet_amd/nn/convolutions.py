@@ -146,6 +146,8 @@ class KernelMapCache(object):
         sizes = cast(built["sizes"])
         sizes.host_sizes = tuple(int(v) for v in built["sizes_host"])
         order = cast(built["order"]) if reorder else None
+        if order is not None:
+            order.host_order = tuple(int(v) for v in built["order_host"])
         source_masks, target_masks = cast(built["source_masks"]), cast(built["target_masks"])
         # buffer row -> feature row on either side of the map: what a layer
         # (forward or transposed) gathers through
@@ -207,6 +209,7 @@ class SparseConv(Module):
                                 "dataflow": "auto"}
         self._tuning_data = None
         self._identity_map = None
+        self._packed = None
 
     @property
     def _allow_shortcut_matmul(self) -> bool:
@@ -347,6 +350,38 @@ class SparseConv(Module):
                 self._tunable_config["dataflow"] = dataflow
 
     # ------------------------------------------------------------- forward ----
+    def _packed_kernel(self, pad: int = 0):
+        """``(weights, packed)``: the layer's weights (with ``pad`` zero input
+        channels appended) and the same in the layout the matrix kernels stage,
+        remade only when the parameter has changed (in-place updates bump its
+        version counter).  ``packed`` is None while gradients are recorded."""
+        kernel = self.kernel
+        if torch.is_grad_enabled() and kernel.requires_grad:
+            padded = kernel if pad == 0 else torch.nn.functional.pad(kernel, (0, 0, 0, pad))
+            return padded, None
+        key = (kernel.data_ptr(), kernel._version, kernel.dtype, kernel.device, pad)
+        if self._packed is None or self._packed[0] != key:
+            with torch.no_grad():
+                weights = kernel.detach()
+                if pad:
+                    weights = torch.nn.functional.pad(weights, (0, 0, 0, pad))
+                self._packed = (key, weights, F.pack_weights(weights))
+        return self._packed[1], self._packed[2]
+
+    def _row_padding(self, features: torch.Tensor, target_masks) -> int:
+        """Zero input channels to append so that feature rows become a multiple
+        of 16 bytes, when that lets a 16-bit layer (a stem with 3 or 4 input
+        channels, say) take the single-kernel dataflow; else 0."""
+        per_piece = 16 // features.element_size()
+        pad = -self.in_channels % per_piece
+        if (pad == 0 or features.dtype == torch.float32 or not features.is_cuda
+                or self._tunable_config.get("dataflow", "auto") == "gather_gemm_scatter"
+                or getattr(target_masks, "kernel_map", None) is None
+                or not _C.implicit_forward_supported(self.in_channels + pad, self.out_channels,
+                                                     features.dtype)):
+            return 0
+        return pad
+
     def _pointwise(self, features: torch.Tensor, epilogue: Optional[F.Epilogue]) -> torch.Tensor:
         """1x1x1 kernel, stride 1: a plain ``features @ W`` (reference:
         convolutions.py:452-455).  Where the single-kernel forward takes the
@@ -364,7 +399,8 @@ class SparseConv(Module):
                 identity = torch.arange(rows, dtype=torch.int32, device=features.device).view(1, rows)
                 self._identity_map = identity
             return _C.sparse_convolution_forward_implicit(features, weights, identity[:, :rows],
-                                                          epilogue=epilogue)
+                                                          epilogue=epilogue,
+                                                          packed_weights=self._packed_kernel()[1])
         out = torch.mm(features, weights[0])
         return out if epilogue is None else epilogue.apply(out)
 
@@ -401,14 +437,19 @@ class SparseConv(Module):
             if self._tuning_data is not None:
                 sizes.kernel_map_order = order
                 self._tuning_data.append((source_masks, target_masks, sizes))
+            sources = inputs.F
+            pad = self._row_padding(sources, target_masks)
+            if pad:
+                sources = torch.nn.functional.pad(sources, (0, pad))
+            weights, packed = self._packed_kernel(pad) if sources.is_cuda else (self.kernel, None)
             features = F.sparse_convolution_forward(
-                sources=inputs.F, weights=self.kernel, source_masks=source_masks,
+                sources=sources, weights=weights, source_masks=source_masks,
                 target_masks=target_masks, kernel_map_order=order, kernel_map_sizes=sizes,
                 gather_tile_size=self._tunable_config["gather_tile_size"],
                 scatter_tile_size=self._tunable_config["scatter_tile_size"],
                 allow_shortcut_matmul=self._allow_shortcut_matmul,
                 threshold=self._tunable_config["threshold"], epilogue=epilogue,
-                dataflow=self._tunable_config.get("dataflow", "auto"))
+                dataflow=self._tunable_config.get("dataflow", "auto"), packed_weights=packed)
         if self.bias is not None and epilogue is None:
             features += self.bias
         return SparseTensor(features=features, coordinates=coordinates, stride=stride,

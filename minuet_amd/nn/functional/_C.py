@@ -63,10 +63,11 @@ SIGNATURES = {
     "mnt_sparse_convolution_forward_fused": (_int, [_i64, _i64, _int, _i64, _int, _dbl, _vp, _vp, _vp,
                                                     _vp, _vp, _vp, _pi64, _i64, _i64, _i64, _i64,
                                                     _i64, _int, _int, _vp, _vp, _vp, _vp, _int,
-                                                    _c.c_float, _vp, _vp]),
+                                                    _c.c_float, _vp, _pi64, _vp, _vp]),
+    "mnt_pack_weights": (_int, [_vp, _i64, _i64, _i64, _int, _vp, _vp]),
     "mnt_sparse_convolution_forward_implicit": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                                                        _int, _vp, _vp, _vp, _int, _c.c_float, _vp,
-                                                       _vp]),
+                                                       _vp, _vp]),
     "mnt_kernel_map_invert": (_int, [_vp, _i64, _i64, _i64, _vp, _vp]),
     "mnt_time_gather": (_int, [_i64, _int, _int, _dbl, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
                                _int, _pf, _vp]),
@@ -111,13 +112,40 @@ def _fail(message: str):
 
 
 def _ptr(tensor: Optional[torch.Tensor]):
-    if tensor is None or tensor.numel() == 0:
-        return None if tensor is None else ctypes.c_void_p(tensor.data_ptr())
-    return ctypes.c_void_p(tensor.data_ptr())
+    """Device address as a plain int (what a ``c_void_p`` parameter accepts),
+    None for a missing or empty tensor's null pointer."""
+    if tensor is None:
+        return None
+    return tensor.data_ptr() or None
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _stream(device: torch.device):
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    """Handle of torch's current stream on ``device`` (an int; 0 / None is the
+    default stream)."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index) or None
+    return torch.cuda.current_stream(device).cuda_stream or None
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on(device: torch.device):
+    """Context that makes ``device`` current; free when it already is."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(device)
 
 
 def _ensure_ndim(name: str, tensor: torch.Tensor, ndim: int):
@@ -179,7 +207,7 @@ def cuda_arg_sort_coordinates(coordinates: torch.Tensor, enable_flattening: bool
     _check_ndim_supported(ndim, "CUDAArgSortCoordinates", coordinates.dtype)
     itype = torch.int32 if n <= 2 ** 31 - 1 else torch.int64
     indices = torch.empty((n,), dtype=itype, device=device)
-    with torch.cuda.device(device):
+    with _on(device):
         _check(load_library().mnt_arg_sort_coordinates(
             _ptr(coordinates), n, ndim, ccode, None, 1, _INT[itype], _ptr(indices), None, None,
             _stream(device)))
@@ -197,7 +225,7 @@ def cuda_multi_arg_sort_coordinates(coordinates: torch.Tensor, batch_dims: torch
     icode = _int_code(batch_dims.dtype, "index", "CUDAMultiArgSortCoordinates")
     _check_ndim_supported(ndim, "CUDAMultiArgSortCoordinates", coordinates.dtype)
     indices = torch.empty((n,), dtype=batch_dims.dtype, device=device)
-    with torch.cuda.device(device):
+    with _on(device):
         _check(load_library().mnt_arg_sort_coordinates(
             _ptr(coordinates), n, ndim, ccode, _ptr(batch_dims), batch_dims.numel() - 1, icode,
             _ptr(indices), None, None, _stream(device)))
@@ -218,7 +246,7 @@ def sort_coordinates(coordinates: torch.Tensor, batch_dims: Optional[torch.Tenso
     indices = torch.empty((n,), dtype=itype, device=device)
     out = torch.empty_like(coordinates)
     bounds = np.zeros(8, dtype=np.int64)
-    with torch.cuda.device(device):
+    with _on(device):
         _check(load_library().mnt_arg_sort_coordinates(
             _ptr(coordinates), n, ndim, ccode, _ptr(batch_dims),
             batch_dims.numel() - 1 if batch_dims is not None else 1, _INT[itype], _ptr(indices),
@@ -243,7 +271,7 @@ def _unique(coordinates: torch.Tensor, batch_dims: Optional[torch.Tensor], fn: s
     indices = torch.empty((n + 1,), dtype=itype, device=device)
     count = ctypes.c_int64(0)
     lib = load_library()
-    with torch.cuda.device(device):
+    with _on(device):
         # the reference passes len(batch_dims) as the batch count
         # (cuda_unique_coordinates.cu:51); results are the same with B
         _check(lib.mnt_unique_coordinates(
@@ -280,7 +308,7 @@ def target_coordinates(coordinates: torch.Tensor, batch_dims: Optional[torch.Ten
     stride = (ctypes.c_int64 * ndim)(*[int(s) for s in target_stride])
     count = ctypes.c_int64(0)
     lib = load_library()
-    with torch.cuda.device(device):
+    with _on(device):
         _check(lib.mnt_target_coordinates_count(
             _ptr(coordinates), n, ndim, ccode, stride, _ptr(batch_dims),
             batch_dims.numel() - 1 if batch_dims is not None else 1, icode, ctypes.byref(count),
@@ -309,7 +337,7 @@ def cuda_query_sorted_index_with_offsets(sources: torch.Tensor, targets: torch.T
     ccode = _int_code(ctype, "coordinate", fn)
     _check_ndim_supported(ndim, fn, ctype)
     out = torch.empty((offsets.size(0), targets.size(0)), dtype=ctype, device=device)
-    with torch.cuda.device(device):
+    with _on(device):
         _check(load_library().mnt_query_sorted_index_with_offsets(
             _ptr(sources), sources.size(0), _ptr(targets), targets.size(0), _ptr(offsets),
             offsets.size(0), ndim, ccode, None, None, 1, 0, _ptr(out), ccode, _stream(device)))
@@ -344,7 +372,7 @@ def cuda_multi_query_sorted_index_with_offsets(source_batch_dims: torch.Tensor,
     icode = _int_code(itype, "index", fn)
     _check_ndim_supported(ndim, fn, ctype)
     out = torch.empty((offsets.size(0), targets.size(0)), dtype=itype, device=device)
-    with torch.cuda.device(device):
+    with _on(device):
         _check(load_library().mnt_query_sorted_index_with_offsets(
             _ptr(sources), sources.size(0), _ptr(targets), targets.size(0), _ptr(offsets),
             offsets.size(0), ndim, ccode, _ptr(source_batch_dims), _ptr(target_batch_dims),
@@ -358,7 +386,7 @@ def cuda_compute_kernel_map_sizes(kernel_map: torch.Tensor) -> torch.Tensor:
     device = _common_device([kernel_map])
     icode = _int_code(kernel_map.dtype, "tensor", "CUDAComputeKernelMapSizes")
     sizes = torch.empty((kernel_map.size(0),), dtype=kernel_map.dtype, device=device)
-    with torch.cuda.device(device):
+    with _on(device):
         _check(load_library().mnt_compute_kernel_map_sizes(
             _ptr(kernel_map), kernel_map.size(0), kernel_map.size(1), icode, _ptr(sizes),
             _stream(device)))
@@ -375,7 +403,7 @@ def cuda_compute_kernel_map_masks(num_sources: int, kernel_map: torch.Tensor,
     num_offsets, num_targets = kernel_map.shape
     source_masks = torch.empty((num_offsets, num_sources), dtype=kernel_map.dtype, device=device)
     target_masks = torch.empty((num_offsets, num_targets), dtype=kernel_map.dtype, device=device)
-    with torch.cuda.device(device):
+    with _on(device):
         _check(load_library().mnt_compute_kernel_map_masks(
             _ptr(kernel_map), num_offsets, int(num_sources), num_targets, icode,
             _ptr(source_masks), _ptr(target_masks), _stream(device)))
@@ -421,7 +449,7 @@ def kernel_map_build(sources: torch.Tensor, targets: torch.Tensor, offsets_host:
     tb = None if target_bounds is None else np.ascontiguousarray(target_bounds, dtype=np.int64)
     lib = load_library()
     result = {}
-    with torch.cuda.device(device):
+    with _on(device):
         stream = _stream(device)
         _check(lib.mnt_kernel_map_query(
             _ptr(sources), num_sources, _ptr(targets), num_targets,
@@ -464,7 +492,7 @@ def kernel_map_pair_lists(kernel_map: torch.Tensor, sizes_host: Sequence[int]):
     cum[1:] = np.cumsum(np.asarray(sizes_host, dtype=np.int64))
     in_idx = torch.empty((int(cum[-1]),), dtype=torch.int32, device=device)
     out_idx = torch.empty_like(in_idx)
-    with torch.cuda.device(device):
+    with _on(device):
         _check(load_library().mnt_kernel_map_pair_lists(
             _ptr(kernel_map), num_offsets, num_targets, cum.ctypes.data_as(_pi64), _ptr(in_idx),
             _ptr(out_idx), _stream(device)))
@@ -536,6 +564,8 @@ class Epilogue:
                 return None
             if t.shape != (channels,) or t.device != device:
                 _fail(f"epilogue {name} must be a [{channels}] tensor on the device of the features")
+            if t.dtype == torch.float32 and t.is_contiguous():
+                return t
             return t.to(torch.float32).contiguous()
         residual = self.residual
         if residual is not None:
@@ -586,12 +616,16 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
                                     kernel_map_sizes: torch.Tensor,
                                     kernel_map_sizes_host=None,
                                     gather_index: Optional[torch.Tensor] = None,
-                                    epilogue: Optional["Epilogue"] = None) -> torch.Tensor:
+                                    epilogue: Optional["Epilogue"] = None,
+                                    packed_weights: Optional[torch.Tensor] = None,
+                                    kernel_map_order_host=None) -> torch.Tensor:
     """csrc/minuet/torch/cuda_sparse_convolution_forward.cu:136-213.  The extra
     ``kernel_map_sizes_host`` spares the device read-back of the sizes;
     ``gather_index`` (int32, the kernel map's source row per buffer row) folds
     the Gather step into the GEMM; ``epilogue`` is applied to every output row
-    before it is rounded to the feature dtype."""
+    before it is rounded to the feature dtype; ``packed_weights``
+    (:func:`pack_weights` of ``weights``) spares the packing pass and needs
+    ``kernel_map_order_host`` whenever there is a ``kernel_map_order``."""
     fn = "CUDASparseConvolutionForward"
     _ensure_ndim("sources", sources, 2)
     S, T, O, K, N = _conv_shapes(weights, source_masks, target_masks, kernel_map_sizes)
@@ -618,7 +652,17 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
             _fail("gather_index needs the host sizes and one entry per kernel map hit")
         gather_index = gather_index.contiguous()
     ep = Epilogue() if epilogue is None else epilogue.checked(T, N, weights.dtype, device)
-    with torch.cuda.device(device):
+    keep_order = order_ptr = None
+    if packed_weights is not None:
+        _check_packed(packed_weights, weights)
+        if kernel_map_order is not None:
+            if kernel_map_order_host is None:
+                _fail("packed weights need the host copy of kernel_map_order")
+            keep_order = np.ascontiguousarray(np.asarray(kernel_map_order_host, dtype=np.int64))
+            if keep_order.shape[0] != O:
+                _fail("host copy of kernel_map_order has the wrong length")
+            order_ptr = keep_order.ctypes.data_as(_pi64)
+    with _on(device):
         _check(load_library().mnt_sparse_convolution_forward_fused(
             int(gather_tile_size), int(scatter_tile_size), 1 if allow_shortcut_matmul else 0,
             int(parallel), 0 if threshold is None else 1,
@@ -626,9 +670,38 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
             _ptr(source_masks), _ptr(target_masks), _ptr(kernel_map_order),
             _ptr(kernel_map_sizes), sizes_ptr, S, T, O, K, N, icode, fcode, _ptr(gather_index),
             _ptr(ep.scale), _ptr(ep.shift), _ptr(ep.residual), ACTIVATION_CODES[ep.activation],
-            float(ep.negative_slope), _ptr(out), _stream(device)))
-    del keep
+            float(ep.negative_slope), _ptr(packed_weights), order_ptr, _ptr(out), _stream(device)))
+    del keep, keep_order
     return out
+
+
+def packed_weights_shape(weights: torch.Tensor):
+    """Shape of :func:`pack_weights`'s result for ``weights [O, C_in, C_out]``."""
+    O, K, N = weights.shape
+    per_chunk = 128 // weights.dtype.itemsize
+    return (O, (N + 31) // 32 * 32, (K + per_chunk - 1) // per_chunk * per_chunk)
+
+
+def pack_weights(weights: torch.Tensor) -> torch.Tensor:
+    """``weights [O, C_in, C_out]`` in the transposed, padded layout the matrix
+    kernels stage (offset order unchanged).  A layer keeps the result for as
+    long as its weights do not change and hands it to the forward functions."""
+    _ensure_ndim("weights", weights, 3)
+    device = _common_device([weights])
+    fcode = _float_code(weights.dtype, "pack_weights")
+    weights = weights.contiguous()
+    packed = torch.empty(packed_weights_shape(weights), dtype=weights.dtype, device=device)
+    O, K, N = weights.shape
+    with _on(device):
+        _check(load_library().mnt_pack_weights(_ptr(weights), O, K, N, fcode, _ptr(packed),
+                                               _stream(device)))
+    return packed
+
+
+def _check_packed(packed: torch.Tensor, weights: torch.Tensor):
+    if (tuple(packed.shape) != packed_weights_shape(weights) or packed.dtype != weights.dtype
+            or packed.device != weights.device or not packed.is_contiguous()):
+        _fail("packed_weights does not belong to these weights (shape, dtype, device or layout)")
 
 
 def kernel_map_invert(kernel_map: torch.Tensor, num_sources: int) -> torch.Tensor:
@@ -642,7 +715,7 @@ def kernel_map_invert(kernel_map: torch.Tensor, num_sources: int) -> torch.Tenso
     kernel_map = kernel_map.contiguous()
     num_offsets, num_targets = kernel_map.shape
     inverse = torch.empty((num_offsets, num_sources), dtype=torch.int32, device=device)
-    with torch.cuda.device(device):
+    with _on(device):
         _check(load_library().mnt_kernel_map_invert(_ptr(kernel_map), num_offsets, num_targets,
                                                     num_sources, _ptr(inverse), _stream(device)))
     return inverse
@@ -661,7 +734,8 @@ def implicit_forward_supported(num_source_features: int, num_target_features: in
 
 def sparse_convolution_forward_implicit(sources: torch.Tensor, weights: torch.Tensor,
                                         kernel_map: torch.Tensor,
-                                        epilogue: Optional[Epilogue] = None) -> torch.Tensor:
+                                        epilogue: Optional[Epilogue] = None,
+                                        packed_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Output-stationary forward from the dense kernel map ``[O, N_out]`` (int32,
     original offset order): one kernel, no gather / GEMM-output buffers."""
     fn = "sparse_convolution_forward_implicit"
@@ -682,11 +756,13 @@ def sparse_convolution_forward_implicit(sources: torch.Tensor, weights: torch.Te
     sources = sources if sources.data_ptr() % 16 == 0 else sources.clone()
     out = torch.empty((T, N), dtype=weights.dtype, device=device)
     ep = Epilogue() if epilogue is None else epilogue.checked(T, N, weights.dtype, device)
-    with torch.cuda.device(device):
+    if packed_weights is not None:
+        _check_packed(packed_weights, weights)
+    with _on(device):
         _check(load_library().mnt_sparse_convolution_forward_implicit(
             _ptr(sources), _ptr(weights), _ptr(kernel_map), S, T, O, K, N, fcode, _ptr(ep.scale),
             _ptr(ep.shift), _ptr(ep.residual), ACTIVATION_CODES[ep.activation],
-            float(ep.negative_slope), _ptr(out), _stream(device)))
+            float(ep.negative_slope), _ptr(packed_weights), _ptr(out), _stream(device)))
     return out
 
 
@@ -699,7 +775,7 @@ def _time_stage(name, lead_args, threshold, mask, weights, source_masks, target_
     icode = _int_code(itype, "index", name)
     ms = ctypes.c_float(0.0)
     first = weights if pass_weights else mask
-    with torch.cuda.device(device):
+    with _on(device):
         _check(getattr(load_library(), name)(
             *lead_args, 0 if threshold is None else 1,
             0.0 if threshold is None else float(threshold), _ptr(first), _ptr(kernel_map_sizes),

@@ -7,7 +7,9 @@ import torch
 from . import _C
 
 __all__ = ["cuda_time_gather", "cuda_time_scatter", "sparse_convolution_forward",
-           "cuda_time_gemm", "set_gemm_parallel_level", "Epilogue"]
+           "cuda_time_gemm", "set_gemm_parallel_level", "Epilogue", "pack_weights"]
+
+pack_weights = _C.pack_weights
 
 Epilogue = _C.Epilogue
 
@@ -61,7 +63,8 @@ def sparse_convolution_forward(sources: torch.Tensor, weights: torch.Tensor,
                                parallel: Optional[int] = None,
                                threshold: Optional[float] = 0,
                                epilogue: Optional[_C.Epilogue] = None,
-                               dataflow: str = "auto") -> torch.Tensor:
+                               dataflow: str = "auto",
+                               packed_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Output features ``[N_out, C_out]`` of one sparse convolution given the rank
     tables of its kernel map (reference: convolution.py:110-155).  A host copy
     of the sizes attached to ``kernel_map_sizes`` as attribute ``host_sizes``
@@ -78,7 +81,12 @@ def sparse_convolution_forward(sources: torch.Tensor, weights: torch.Tensor,
     ``target_masks`` as attribute ``kernel_map`` (``KernelMapCache`` does that)
     and ``weights`` in their original offset order, as a layer holds them.
     ``"auto"`` takes the implicit form where it is the faster one: 16-bit
-    features whose rows it can stage, and small fp32 layers with 2^D kernels."""
+    features whose rows it can stage, and small fp32 layers with 2^D kernels.
+
+    ``packed_weights`` (``pack_weights(weights)``, kept by the caller while the
+    weights are unchanged) spares the packing pass that otherwise starts every
+    call; with a ``kernel_map_order`` it also needs that tensor's host copy as
+    attribute ``host_order`` (from ``KernelMapCache``) and is ignored without."""
     if not sources.is_cuda:
         raise NotImplementedError
     if dataflow not in DATAFLOWS:
@@ -92,15 +100,21 @@ def sparse_convolution_forward(sources: torch.Tensor, weights: torch.Tensor,
         # pays where most (offset, target) pairs are hits, i.e. strided 2^D kernels
         dense_hits = weights.shape[0] <= 8 and weights.shape[1] * weights.shape[2] <= 1024
         if dataflow == "implicit" or (fits and (weights.dtype != torch.float32 or dense_hits)):
-            return _C.sparse_convolution_forward_implicit(sources, weights, dense, epilogue=epilogue)
+            return _C.sparse_convolution_forward_implicit(sources, weights, dense, epilogue=epilogue,
+                                                          packed_weights=packed_weights)
     if parallel is None:
         parallel = GEMM_PARALLEL_LEVEL
     host_sizes = getattr(kernel_map_sizes, "host_sizes", None)
     gather_index = getattr(source_masks, "gather_index", None) if host_sizes is not None else None
+    host_order = None
     if kernel_map_order is not None:
+        host_order = getattr(kernel_map_order, "host_order", None)
+        if host_order is None:
+            packed_weights = None
         kernel_map_order = kernel_map_order.contiguous()
     return _C.cuda_sparse_convolution_forward(
         gather_tile_size, scatter_tile_size, allow_shortcut_matmul, parallel, threshold,
         sources.contiguous(), weights.contiguous(), source_masks.contiguous(),
         target_masks.contiguous(), kernel_map_order, kernel_map_sizes.contiguous(),
-        kernel_map_sizes_host=host_sizes, gather_index=gather_index, epilogue=epilogue)
+        kernel_map_sizes_host=host_sizes, gather_index=gather_index, epilogue=epilogue,
+        packed_weights=packed_weights, kernel_map_order_host=host_order)

@@ -15,7 +15,9 @@ __all__ = ["as_tuple", "generate_kernel_offsets", "set_kernel_map_cache",
 def as_tuple(value, *, size: int = 3, name: Optional[str] = None):
     """A scalar becomes a ``size``-tuple of itself; an iterable must already have
     ``size`` elements (reference: helpers.py:138-162)."""
-    if not isinstance(value, Iterable):
+    if type(value) is tuple and len(value) == size:
+        return value
+    if isinstance(value, (int, float)) or not isinstance(value, Iterable):
         return tuple(value for _ in range(size))
     value = tuple(value)
     if len(value) != size:

@@ -95,6 +95,18 @@ def test_forward_functional(kind, kernel, stride, cin, cout, n, extent):
                 gather_tile_size=0, scatter_tile_size=0,
                 allow_shortcut_matmul=shortcut and stride == 1, threshold=threshold)
             assert torch.equal(fused, out)
+            # weights packed ahead of time (in the layer's own offset order)
+            order_dev = dev(eorder)
+            order_dev.host_order = tuple(int(v) for v in eorder)
+            w_dev = dev(weights).to(dtype)
+            ahead = F.sparse_convolution_forward(
+                sources=dev(feats).to(dtype), weights=w_dev,
+                source_masks=with_gather_index(esm, esizes), target_masks=dev(etm),
+                kernel_map_order=order_dev, kernel_map_sizes=with_host_sizes(esizes),
+                gather_tile_size=0, scatter_tile_size=0,
+                allow_shortcut_matmul=shortcut and stride == 1, threshold=threshold,
+                packed_weights=F.pack_weights(w_dev))
+            assert torch.equal(ahead, out)
 
 
 @pytest.mark.parametrize("kind", ["fp32", "fp16", "bf16"])
@@ -157,6 +169,9 @@ def test_forward_implicit(kind, kernel, stride, cin, cout, n, extent):
     out = _C.sparse_convolution_forward_implicit(dev(feats).to(dtype), dev(weights).to(dtype), dev(kmap))
     assert out.dtype == dtype and out.shape == (tgt.shape[0], cout)
     assert_features_close(out, conv, kind)
+    w_dev = dev(weights).to(dtype)
+    assert torch.equal(out, _C.sparse_convolution_forward_implicit(
+        dev(feats).to(dtype), w_dev, dev(kmap), packed_weights=F.pack_weights(w_dev)))
     rng = np.random.default_rng(5)
     scale = rng.uniform(0.5, 1.5, size=cout).astype(np.float32)
     shift = rng.uniform(-0.5, 0.5, size=cout).astype(np.float32)
@@ -181,6 +196,51 @@ def test_forward_implicit_rejects_unsupported_shapes():
     out = _C.sparse_convolution_forward_implicit(torch.ones(10, 8, device="cuda").half(),
                                                  torch.ones(27, 8, 32, device="cuda").half(), kmap)
     assert torch.count_nonzero(out).item() == 0                        # no hits: all zero
+
+
+def test_packed_weights_follow_the_parameter():
+    """A layer repacks its weights when (and only when) the parameter changes."""
+    src, sbd, tgt, tbd, off, feats, weights = make_layer_case(2, 3000, 16, 3, 32, 32, "fp16")
+    conv = minuet.nn.SparseConv3d(32, 32, 3, dtype=torch.float16, device="cuda")
+    conv.set_kernel_map_cache(minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda"))
+    x = minuet.SparseTensor(dev(feats).half(), dev(src))
+    with torch.no_grad():
+        for flow in ("gather_gemm_scatter", "implicit"):
+            conv.tunable_config["dataflow"] = flow
+            a = conv(x).F.clone()
+            first = conv._packed[2]
+            assert conv(x).F.equal(a) and conv._packed[2] is first
+            conv.kernel.mul_(2.0)                      # in place: same storage, new version
+            b = conv(x).F
+            assert conv._packed[2] is not first
+            assert (b.float() - 2 * a.float()).abs().max().item() <= 2e-2 * a.float().pow(2).mean().sqrt().item()
+            conv.kernel.mul_(0.5)
+    with pytest.raises(RuntimeError, match="does not belong"):
+        F.sparse_convolution_forward(
+            sources=x.F, weights=conv.kernel, source_masks=None, target_masks=None, kernel_map_order=None,
+            kernel_map_sizes=None, gather_tile_size=0, scatter_tile_size=0, dataflow="gather_gemm_scatter",
+            packed_weights=torch.zeros(3, device="cuda").half()) if False else _C._check_packed(
+                torch.zeros(3, device="cuda").half(), conv.kernel)
+
+
+@pytest.mark.parametrize("cin", [3, 4, 12])
+def test_narrow_rows_are_padded_for_the_single_kernel_form(cin):
+    """16-bit layers whose rows are not a multiple of 16 bytes (stems) still
+    take the implicit dataflow, through zero channels appended on the fly."""
+    src, sbd, tgt, tbd, off, feats, weights = make_layer_case(13, 4000, 18, 3, cin, 32, "fp16")
+    esm, etm, eorder, esizes, _ = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=True)
+    ref = orc.sparse_convolution_forward(feats, weights, esm, etm, eorder, esizes)
+    conv = minuet.nn.SparseConv3d(cin, 32, 3, dtype=torch.float16, device="cuda")
+    conv.kernel.data.copy_(dev(weights).half())
+    conv.set_kernel_map_cache(minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda"))
+    x = minuet.SparseTensor(dev(feats).half(), dev(src))
+    with torch.no_grad():
+        _C.profile_enable(True)
+        y = conv(x)
+        stages = [name for name, _ in _C.profile_read()]
+        _C.profile_enable(False)
+    assert "implicit" in stages and "scatter" not in stages
+    assert_features_close(y.F, ref, "fp16")
 
 
 def test_epilogue_rejects_bad_operands():
