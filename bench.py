@@ -106,6 +106,7 @@ def layer_stages(device, config, channels, kernel_size, dtype_name):
     conv.set_kernel_map_cache(cache)
     x = minuet.SparseTensor(torch.randn(sorted_dev.shape[0], channels, device=device).to(dtype), sorted_dev)
     with torch.no_grad():
+        conv.tunable_config["dataflow"] = "gather_gemm_scatter"     # builds the rank tables
         conv(x)
         source_masks, target_masks, order, sizes = next(iter(cache._kernel_maps_cache.values()))
         host_sizes = np.asarray(sizes.host_sizes, dtype=np.int64)

@@ -98,11 +98,14 @@ int mnt_fill_unique_coordinates(const void *sorted_coords, int64_t n, int ndim, 
  * sorted keys in the arena slot of this stream; phase 2 writes the coordinates
  * and target_batch_dims_out[num_batches+1] (nullable, element type
  * index_dtype).  Phase 2 must follow phase 1 on the same stream with no other
- * library call in between.  Replaces the torch expression in
+ * library call in between.  source_bounds_host (nullable, 8 x int64: minima
+ * in [0..3], maxima in [4..7]) spares the reduction over the coordinates and
+ * its wait when the caller knows them.  Replaces the torch expression in
  * KernelMapCache.get_target_coordinates, minuet/nn/convolutions.py:84-99. */
 int mnt_target_coordinates_count(const void *source_coords, int64_t n, int ndim, int coord_dtype,
                                  const int64_t *target_stride, const void *batch_dims,
                                  int64_t num_batches, int index_dtype,
+                                 const int64_t *source_bounds_host,
                                  int64_t *num_targets_out, void *stream);
 int mnt_target_coordinates_fill(void *target_coords_out, void *target_batch_dims_out,
                                 void *stream);
@@ -183,6 +186,27 @@ int mnt_kernel_map_emit(int32_t *source_masks_out, int32_t *target_masks_out,
 int mnt_kernel_map_pair_lists(const int32_t *kernel_map, int64_t num_offsets,
                               int64_t num_targets, const int64_t *cumsum_host,
                               int32_t *in_idx_out, int32_t *out_idx_out, void *stream);
+
+/* The two halves of mnt_kernel_map_query for callers that may never need the
+ * rank tables (the single-kernel forward reads the dense map only):
+ * mnt_kernel_map_dense runs the query alone (same arguments and kernel_map_out
+ * as mnt_kernel_map_query) and does not wait for anything when both bounds are
+ * given; mnt_kernel_map_tables derives sizes and order from such a dense map
+ * later, after which mnt_kernel_map_emit writes the tables as usual.  Same
+ * reference code as mnt_kernel_map_query (minuet/nn/convolutions.py:147-170). */
+int mnt_kernel_map_dense(const void *sources, int64_t num_sources,
+                         const void *targets, int64_t num_targets,
+                         const int64_t *offsets_host, int64_t num_offsets,
+                         int ndim, int coord_dtype,
+                         const void *source_batch_dims, const void *target_batch_dims,
+                         int64_t num_batches, int batch_dtype,
+                         const int64_t *source_bounds_host,
+                         const int64_t *target_bounds_host,
+                         int64_t *bounds_host_out,
+                         int32_t *kernel_map_out, void *stream);
+int mnt_kernel_map_tables(const int32_t *kernel_map, int64_t num_sources,
+                          int64_t num_targets, int64_t num_offsets, int reorder,
+                          int64_t *sizes_host_out, int64_t *order_host_out, void *stream);
 
 /* ---- GMaS: padding plan (host only) -------------------------------------- */
 

@@ -648,6 +648,30 @@ struct MapState {
   const void *kernel_map;
 };
 
+// Second half of the first phase of a kernel-map build: per-offset sizes and
+// the stable size order from the per-tile hit counts, mirrored into pinned
+// host memory (past the bounds slots), then the state the emit call reads.
+static void finish_sizes(Arena &arena, const MapState &state, unsigned *tile_counts,
+                         unsigned *row_sizes, unsigned *plan, int64_t *sizes_host_out,
+                         int64_t *order_host_out, hipStream_t stream) {
+  const int64_t num_offsets = state.num_offsets;
+  unsigned *h_plan = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned()) + Arena::kPlanOffset);
+  unsigned *d_plan_host = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned_device()) + Arena::kPlanOffset);
+  const unsigned long long sequence = arena.next_sequence();
+  tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(
+      tile_counts, state.num_tiles, row_sizes, state.reorder, plan, d_plan_host, arena.tickets() + 1,
+      arena.flag_device(1), sequence);
+  check_launch("tile_scan_kernel");
+  arena.wait_flag(1, sequence);
+  profile_mark("map_sizes_order+sync", stream);
+  for (int64_t j = 0; j < num_offsets; ++j) {
+    order_host_out[j] = h_plan[j];
+    sizes_host_out[j] = h_plan[2 * num_offsets + j];
+  }
+  memcpy(arena.map_state, &state, sizeof(state));
+  arena.map_state_valid = true;
+}
+
 }  // namespace mnt
 
 using namespace mnt;
@@ -820,22 +844,73 @@ extern "C" int mnt_kernel_map_query(const void *sources, int64_t num_sources, co
       run_query(a, offsets_host, num_offsets, source_bounds_host, target_bounds_host, bounds_host_out,
                 kernel_map_out, MNT_INT32, tile_counts, scope, stream);
     }
-    // sizes + order, mirrored into pinned host memory (past the bounds slots)
-    unsigned *h_plan = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned()) + Arena::kPlanOffset);
-    unsigned *d_plan_host = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned_device()) + Arena::kPlanOffset);
-    const unsigned long long sequence = arena.next_sequence();
-    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(
-        tile_counts, num_tiles, row_sizes, reorder, plan, d_plan_host, arena.tickets() + 1,
-        arena.flag_device(1), sequence);
-    check_launch("tile_scan_kernel");
-    arena.wait_flag(1, sequence);
-    profile_mark("map_sizes_order+sync", stream);
-    for (int64_t j = 0; j < num_offsets; ++j) {
-      order_host_out[j] = h_plan[j];
-      sizes_host_out[j] = h_plan[2 * num_offsets + j];
+    finish_sizes(arena, state, tile_counts, row_sizes, plan, sizes_host_out, order_host_out, stream);
+  });
+}
+
+extern "C" int mnt_kernel_map_dense(const void *sources, int64_t num_sources, const void *targets,
+                                    int64_t num_targets, const int64_t *offsets_host,
+                                    int64_t num_offsets, int ndim, int coord_dtype,
+                                    const void *source_batch_dims, const void *target_batch_dims,
+                                    int64_t num_batches, int batch_dtype,
+                                    const int64_t *source_bounds_host,
+                                    const int64_t *target_bounds_host, int64_t *bounds_host_out,
+                                    int32_t *kernel_map_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    QueryArgs a{sources, num_sources, targets, num_targets, ndim, coord_dtype,
+                source_batch_dims, target_batch_dims, num_batches, batch_dtype};
+    check_query_args(a, num_offsets);
+    MNT_CHECK(offsets_host != nullptr, "null argument");
+    if (bounds_host_out != nullptr) {
+      for (int i = 0; i < 16; ++i) bounds_host_out[i] = (i & 4) ? INT64_MIN : INT64_MAX;
     }
-    memcpy(arena.map_state, &state, sizeof(state));
-    arena.map_state_valid = true;
+    if (num_offsets == 0 || num_targets == 0) return;
+    MNT_CHECK(kernel_map_out != nullptr, "kernel_map_out is null");
+    if (num_sources == 0) {
+      enqueue_fill<int32_t>(kernel_map_out, num_offsets * num_targets, -1, stream);
+      return;
+    }
+    Scope scope(stream);
+    run_query(a, offsets_host, num_offsets, source_bounds_host, target_bounds_host, bounds_host_out,
+              kernel_map_out, MNT_INT32, nullptr, scope, stream);
+  });
+}
+
+extern "C" int mnt_kernel_map_tables(const int32_t *kernel_map, int64_t num_sources,
+                                     int64_t num_targets, int64_t num_offsets, int reorder,
+                                     int64_t *sizes_host_out, int64_t *order_host_out,
+                                     void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MNT_CHECK(num_sources >= 0 && num_targets >= 0 && num_offsets >= 0 && num_sources <= INT32_MAX &&
+                  num_targets <= INT32_MAX && num_offsets <= 65535,
+              "bad shape S=%lld T=%lld O=%lld", (long long)num_sources, (long long)num_targets,
+              (long long)num_offsets);
+    MNT_CHECK(sizes_host_out != nullptr && order_host_out != nullptr, "null argument");
+    Arena &arena = Arena::of(stream);
+    const int num_tiles = static_cast<int>(div_ceil(num_targets > 0 ? num_targets : 1, kTargetsPerTile));
+    const size_t words = static_cast<size_t>(num_offsets) * num_tiles + num_offsets + 4 * num_offsets + 1;
+    char *keep = static_cast<char *>(arena.persistent(1, 256 + words * sizeof(unsigned)));
+    unsigned *tile_counts = reinterpret_cast<unsigned *>(keep + 256);
+    unsigned *row_sizes = tile_counts + static_cast<size_t>(num_offsets) * num_tiles;
+    unsigned *plan = row_sizes + num_offsets;
+    MapState state{num_sources, num_targets, num_offsets, num_tiles, reorder, kernel_map};
+    arena.map_state_valid = false;
+    if (num_offsets == 0) {
+      memcpy(arena.map_state, &state, sizeof(state));
+      arena.map_state_valid = true;
+      return;
+    }
+    MNT_CHECK(sizeof(unsigned) * 3 * num_offsets + 1024 <= Arena::kPinnedBytes,
+              "too many kernel offsets (%lld)", static_cast<long long>(num_offsets));
+    if (num_targets == 0) {
+      enqueue_fill<unsigned>(tile_counts, static_cast<int64_t>(words), 0u, stream);
+    } else {
+      MNT_CHECK(kernel_map != nullptr, "kernel_map is null");
+      enqueue_count_tiles(kernel_map, MNT_INT32, num_offsets, num_targets, tile_counts, num_tiles, stream);
+    }
+    finish_sizes(arena, state, tile_counts, row_sizes, plan, sizes_host_out, order_host_out, stream);
   });
 }
 

@@ -22,6 +22,11 @@ void enqueue_exclusive_scan(unsigned *data, int64_t total, hipStream_t stream);
 // Number of 32-bit counters radix_sort_pairs needs for n items.
 size_t radix_counts_len(int64_t n);
 
+// Number of passes radix_sort_pairs makes over n keys of `bits` significant
+// bits: the sorted keys end up in the first buffer when it is even, in the
+// alternate one when it is odd.
+int radix_sort_passes(int64_t n, int bits);
+
 // Stable LSD radix sort of (key, value) pairs over the low `bits` bits.  The
 // sorted data ends up in keys / vals (the pointers are swapped with the
 // *_alt scratch buffers as passes complete).

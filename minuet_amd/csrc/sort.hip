@@ -473,6 +473,15 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
 
 static int items_for(int64_t n) { return n <= (int64_t(1) << 20) ? 4 : 16; }
 
+static void pass_plan(int bits, int &passes, int &radix_bits);
+
+int radix_sort_passes(int64_t n, int bits) {
+  if (n <= 1 || bits <= 0) return 0;
+  int passes, radix_bits;
+  pass_plan(bits, passes, radix_bits);
+  return passes;
+}
+
 size_t radix_counts_len(int64_t n) {
   return static_cast<size_t>(kMaxRadix) * static_cast<size_t>(div_ceil(n, kSortBlock * items_for(n))) +
          kMaxRadix;

@@ -182,10 +182,13 @@ __global__ __launch_bounds__(kScanBlock) void key_tile_sums_kernel(
 }
 
 // Writes the exclusive run index of every sorted key: rank[i] = number of runs
-// that end before position i (rank[n] = number of runs).
+// that end before position i (rank[n] = number of runs).  The thread that owns
+// the last key also hands the number of runs to the host: value into pinned
+// memory, then the sequence flag the host is spinning on.
 __global__ __launch_bounds__(kScanBlock) void key_rank_kernel(
     const unsigned long long *__restrict__ keys, long long n,
-    const unsigned *__restrict__ tile_bases, unsigned *__restrict__ rank) {
+    const unsigned *__restrict__ tile_bases, unsigned *__restrict__ rank,
+    unsigned *host_count, unsigned long long *flag, unsigned long long sequence) {
   const long long base = static_cast<long long>(blockIdx.x) * kScanTile + threadIdx.x * kScanItems;
   bool flags[kScanItems];
   unsigned count = 0;
@@ -203,6 +206,11 @@ __global__ __launch_bounds__(kScanBlock) void key_rank_kernel(
     long long i = base + r;
     run += flags[r] ? 1u : 0u;
     if (i < n) rank[i + 1] = run;
+    if (i == n - 1 && host_count != nullptr) {
+      *host_count = run;
+      __threadfence_system();
+      __hip_atomic_store(flag, sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
   }
 }
 
@@ -241,8 +249,8 @@ static int bit_width64(unsigned long long range) {
 
 template <typename CT, typename IT>
 static void target_count_typed(const CT *coords, int64_t n, int ndim, const int64_t *target_stride,
-                               const IT *batch_dims, int64_t num_batches, int64_t *count_out,
-                               hipStream_t stream) {
+                               const IT *batch_dims, int64_t num_batches,
+                               const int64_t *source_bounds, int64_t *count_out, hipStream_t stream) {
   Arena &arena = Arena::of(stream);
   arena.pending.valid = false;
   const bool batched = batch_dims != nullptr && num_batches > 1;
@@ -251,7 +259,11 @@ static void target_count_typed(const CT *coords, int64_t n, int ndim, const int6
   {
     Scope scope(stream);
     long long h_bounds[16];
-    read_bounds(coords, n, nullptr, 0, ndim, sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64, h_bounds, scope, stream);
+    if (source_bounds != nullptr) {
+      for (int i = 0; i < 8; ++i) h_bounds[i] = source_bounds[i];
+    } else {
+      read_bounds(coords, n, nullptr, 0, ndim, sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64, h_bounds, scope, stream);
+    }
     int bits = 0;
     spec.ndim = ndim;
     for (int k = ndim - 1; k >= 0; --k) {
@@ -281,27 +293,34 @@ static void target_count_typed(const CT *coords, int64_t n, int ndim, const int6
     // persistent block: sorted keys [n] then ranks [n+1]
     size_t key_bytes = (static_cast<size_t>(n) * 8 + 255) / 256 * 256;
     char *keep = static_cast<char *>(arena.persistent(0, key_bytes + (static_cast<size_t>(n) + 1) * 4));
-    unsigned long long *keys = scope.alloc<unsigned long long>(n);
-    unsigned long long *keys_alt = scope.alloc<unsigned long long>(n);
+    // the sort ping-pongs between two buffers: start in the one that makes it
+    // end in the persistent block
+    unsigned long long *kept_keys = reinterpret_cast<unsigned long long *>(keep);
+    unsigned long long *spare = scope.alloc<unsigned long long>(n);
+    const bool even = radix_sort_passes(n, bits) % 2 == 0;
+    unsigned long long *keys = even ? kept_keys : spare;
+    unsigned long long *keys_alt = even ? spare : kept_keys;
     unsigned *vals = nullptr, *vals_alt = nullptr;      // keys-only sort
     unsigned *counts = scope.alloc<unsigned>(radix_counts_len(n));
     const unsigned grid = grid_for(n, 256, 4096);
     pack_target_keys_kernel<CT, IT><<<grid, 256, 0, stream>>>(coords, n, spec, batch_dims, keys, vals);
     check_launch("pack_target_keys_kernel");
     radix_sort_pairs(keys, vals, keys_alt, vals_alt, n, bits, counts, stream);
-    MNT_HIP(hipMemcpyAsync(keep, keys, static_cast<size_t>(n) * 8, hipMemcpyDeviceToDevice, stream));
-    unsigned long long *kept_keys = reinterpret_cast<unsigned long long *>(keep);
+    MNT_CHECK(keys == kept_keys, "sorted keys did not end in the persistent block");
     unsigned *rank = reinterpret_cast<unsigned *>(keep + key_bytes);
     const int tiles = static_cast<int>(div_ceil(n, kScanTile));
     unsigned *tile_sums = scope.alloc<unsigned>(tiles);
     key_tile_sums_kernel<<<tiles, kScanBlock, 0, stream>>>(kept_keys, n, tile_sums);
     check_launch("key_tile_sums_kernel");
     enqueue_exclusive_scan(tile_sums, tiles, stream);
-    key_rank_kernel<<<tiles, kScanBlock, 0, stream>>>(kept_keys, n, tile_sums, rank);
+    // the count goes to pinned memory (past the 16 bounds slots) with flag 2
+    volatile unsigned *h = reinterpret_cast<volatile unsigned *>(static_cast<char *>(arena.pinned()) + 256);
+    unsigned *d = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned_device()) + 256);
+    const unsigned long long sequence = arena.next_sequence();
+    key_rank_kernel<<<tiles, kScanBlock, 0, stream>>>(kept_keys, n, tile_sums, rank, d, arena.flag_device(2),
+                                                     sequence);
     check_launch("key_rank_kernel");
-    unsigned *h = static_cast<unsigned *>(arena.pinned());
-    MNT_HIP(hipMemcpyAsync(h, rank + n, sizeof(unsigned), hipMemcpyDeviceToHost, stream));
-    MNT_HIP(hipStreamSynchronize(stream));
+    arena.wait_flag(2, sequence);
     *count_out = static_cast<int64_t>(*h);
   }
   auto &p = arena.pending;
@@ -405,8 +424,8 @@ extern "C" int mnt_fill_unique_coordinates(const void *sorted_coords, int64_t n,
 extern "C" int mnt_target_coordinates_count(const void *source_coords, int64_t n, int ndim,
                                             int coord_dtype, const int64_t *target_stride,
                                             const void *batch_dims, int64_t num_batches,
-                                            int index_dtype, int64_t *num_targets_out,
-                                            void *stream_) {
+                                            int index_dtype, const int64_t *source_bounds_host,
+                                            int64_t *num_targets_out, void *stream_) {
   return guarded([&] {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MNT_CHECK(ndim >= 1 && ndim <= MNT_MAX_NDIM, "ndim must be in [1, %d] but found %d",
@@ -431,8 +450,8 @@ extern "C" int mnt_target_coordinates_count(const void *source_coords, int64_t n
     if (batch_dims == nullptr) num_batches = 1;
 #define MNT_CALL(CT, IT)                                                                        \
   target_count_typed<CT, IT>(static_cast<const CT *>(source_coords), n, ndim, target_stride,      \
-                             static_cast<const IT *>(batch_dims), num_batches, num_targets_out,   \
-                             stream)
+                             static_cast<const IT *>(batch_dims), num_batches, source_bounds_host, \
+                             num_targets_out, stream)
     MNT_DISPATCH_CI(coord_dtype, index_dtype, MNT_CALL);
 #undef MNT_CALL
   });

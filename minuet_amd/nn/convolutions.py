@@ -34,7 +34,12 @@ class KernelMapCache(object):
     per ``(source stride, target stride, kernel size, dilation)``; a transposed
     layer looks up the map of its forward twin and swaps the two rank tables.
     ``reset()`` must be called before every new input
-    (reference: convolutions.py:18-173)."""
+    (reference: convolutions.py:18-173).
+
+    A map exists in up to two forms: the dense map (``get_dense_kernel_map``,
+    the query alone, no wait on the device) and the rank tables with sizes and
+    order (``get_kernel_map``, the reference's tuple), made from the dense map
+    when a layer asks for them."""
 
     def __init__(self, ndim: int, dtype: torch.dtype, device: Union[str, torch.device],
                  layout: str = "minuet", disable_reordering: bool = False):
@@ -43,7 +48,10 @@ class KernelMapCache(object):
         self._device = device
         self._layout = layout
         self._disable_reordering = disable_reordering
-        self._kernel_maps_cache = dict()
+        self._kernel_maps_cache = dict()        # key -> rank tables, order, sizes
+        self._key_memo = dict()
+        self._dense_maps_cache = dict()         # key -> dense kernel map [O, T]
+        self._inverse_maps_cache = dict()       # key -> its inverse [O, S] (transposed layers)
         self._coordinates_cache = dict()
         self._bounds_cache = dict()
         self.num_map_builds = 0
@@ -59,6 +67,8 @@ class KernelMapCache(object):
     def reset(self):
         self._coordinates_cache.clear()
         self._kernel_maps_cache.clear()
+        self._dense_maps_cache.clear()
+        self._inverse_maps_cache.clear()
         self._bounds_cache.clear()
 
     def _known_bounds(self, coordinates: torch.Tensor):
@@ -86,10 +96,11 @@ class KernelMapCache(object):
             return hit
         if transposed:
             raise RuntimeError(_TRANSPOSED_FIRST)
-        coords, batch_dims = _C.target_coordinates(source_coordinates.contiguous(),
-                                                   source_batch_dims, target_stride)
-        self.num_coordinate_builds += 1
         known = self._known_bounds(source_coordinates)
+        coords, batch_dims = _C.target_coordinates(source_coordinates.contiguous(),
+                                                   source_batch_dims, target_stride,
+                                                   source_bounds=known)
+        self.num_coordinate_builds += 1
         if known is not None and source_coordinates.shape[0] > 0:
             # floor(c / s) * s is monotone, so the extremes map to the extremes
             ts = np.asarray(target_stride, dtype=np.int64)
@@ -101,6 +112,67 @@ class KernelMapCache(object):
         self._coordinates_cache[target_stride] = entry
         return entry
 
+    def _map_key(self, ndim, source_stride, target_stride, kernel_size, kernel_dilation, transposed):
+        raw = (ndim, source_stride, target_stride, kernel_size, kernel_dilation, transposed)
+        try:
+            return self._key_memo[raw]
+        except (KeyError, TypeError):          # first time, or an unhashable argument
+            pass
+        result = self._make_map_key(*raw)
+        try:
+            self._key_memo[raw] = result
+        except TypeError:
+            pass
+        return result
+
+    @staticmethod
+    def _make_map_key(ndim, source_stride, target_stride, kernel_size, kernel_dilation, transposed):
+        source_stride = as_tuple(source_stride, size=ndim, name="source_stride")
+        target_stride = as_tuple(target_stride, size=ndim, name="target_stride")
+        kernel_size = as_tuple(kernel_size, size=ndim, name="kernel_size")
+        kernel_dilation = as_tuple(kernel_dilation, size=ndim, name="kernel_dilation")
+        strides = (target_stride, source_stride) if transposed else (source_stride, target_stride)
+        return strides + (kernel_size, kernel_dilation), source_stride, kernel_size, kernel_dilation
+
+    def get_dense_kernel_map(self, source_coordinates: torch.Tensor, source_stride,
+                             source_batch_dims: Optional[torch.Tensor],
+                             target_coordinates: torch.Tensor, target_stride,
+                             target_batch_dims: Optional[torch.Tensor], kernel_size,
+                             kernel_dilation, transposed: bool = False) -> torch.Tensor:
+        """The dense kernel map of a layer alone: ``[O, N_out]`` int32, source row
+        per (offset, output row) in the layer's own offset order, -1 for none
+        (the output of ``query_sorted_index_with_offsets``,
+        reference: convolutions.py:147-153).  This is all the single-kernel
+        dataflow needs; building it waits for nothing on the device.  A
+        transposed layer gets the inverse of its forward layer's map."""
+        key, source_stride, kernel_size, kernel_dilation = self._map_key(
+            source_coordinates.shape[1], source_stride, target_stride, kernel_size, kernel_dilation,
+            transposed)
+        dense = self._dense_maps_cache.get(key)
+        if dense is None:
+            if transposed:
+                raise RuntimeError(_TRANSPOSED_FIRST)
+            offsets = self._kernel_offsets(source_stride, kernel_size, kernel_dilation)
+            source_coordinates = source_coordinates.contiguous()
+            target_coordinates = target_coordinates.contiguous()
+            dense, bounds = _C.kernel_map_dense(
+                source_coordinates, target_coordinates, offsets, source_batch_dims, target_batch_dims,
+                source_bounds=self._known_bounds(source_coordinates),
+                target_bounds=self._known_bounds(target_coordinates))
+            self.num_map_builds += 1
+            if source_coordinates.shape[0] > 0 and target_coordinates.shape[0] > 0:
+                self._remember_bounds(source_coordinates, bounds[:8])
+                self._remember_bounds(target_coordinates, bounds[8:])
+            dense.num_sources = source_coordinates.shape[0]
+            self._dense_maps_cache[key] = dense
+        if not transposed:
+            return dense
+        inverse = self._inverse_maps_cache.get(key)
+        if inverse is None:
+            inverse = _C.kernel_map_invert(dense, dense.num_sources)
+            self._inverse_maps_cache[key] = inverse
+        return inverse
+
     def get_kernel_map(self, source_coordinates: torch.Tensor, source_stride,
                        source_batch_dims: Optional[torch.Tensor],
                        target_coordinates: torch.Tensor, target_stride,
@@ -108,38 +180,55 @@ class KernelMapCache(object):
                        disable_reordering: bool = False, transposed: bool = False):
         """``(source_masks, target_masks, kernel_map_order, kernel_map_sizes)`` of
         a layer (reference: convolutions.py:102-173)."""
-        ndim = source_coordinates.shape[1]
-        source_stride = as_tuple(source_stride, size=ndim, name="source_stride")
-        target_stride = as_tuple(target_stride, size=ndim, name="target_stride")
-        kernel_size = as_tuple(kernel_size, size=ndim, name="kernel_size")
-        kernel_dilation = as_tuple(kernel_dilation, size=ndim, name="kernel_dilation")
-        strides = (target_stride, source_stride) if transposed else (source_stride, target_stride)
-        key = strides + (kernel_size, kernel_dilation)
+        key, source_stride, kernel_size, kernel_dilation = self._map_key(
+            source_coordinates.shape[1], source_stride, target_stride, kernel_size, kernel_dilation,
+            transposed)
         hit = self._kernel_maps_cache.get(key)
-        if hit is not None:
-            source_masks, target_masks, order, sizes = hit
-            if transposed:
-                if getattr(source_masks, "kernel_map", None) is None:
-                    # dense map of the transposed layer, made on first use
-                    source_masks.kernel_map = _C.kernel_map_invert(target_masks.kernel_map,
-                                                                   source_masks.shape[1])
-                source_masks, target_masks = target_masks, source_masks
-            return source_masks, target_masks, order, sizes
+        if hit is None:
+            if transposed and key not in self._dense_maps_cache:
+                raise RuntimeError(_TRANSPOSED_FIRST)
+            hit = self._build_tables(key, source_coordinates, source_batch_dims, target_coordinates,
+                                     target_batch_dims, source_stride, kernel_size, kernel_dilation,
+                                     disable_reordering)
+        source_masks, target_masks, order, sizes = hit
         if transposed:
-            raise RuntimeError(_TRANSPOSED_FIRST)
+            source_masks, target_masks = target_masks, source_masks
+            if getattr(target_masks, "kernel_map", None) is None:
+                # dense map of the transposed layer, made on first use
+                inverse = self._inverse_maps_cache.get(key)
+                if inverse is None:
+                    inverse = _C.kernel_map_invert(source_masks.kernel_map, target_masks.shape[1])
+                    self._inverse_maps_cache[key] = inverse
+                target_masks.kernel_map = inverse
+        return source_masks, target_masks, order, sizes
 
-        offsets = self._kernel_offsets(source_stride, kernel_size, kernel_dilation)
+    def _build_tables(self, key, source_coordinates, source_batch_dims, target_coordinates,
+                      target_batch_dims, source_stride, kernel_size, kernel_dilation,
+                      disable_reordering):
+        """Rank tables, order and sizes of the forward layer of ``key``: from the
+        dense map when a layer already asked for that, else everything at once.
+        (For a transposed caller the coordinate arguments are the other way
+        round, but then the dense map exists and they are not used.)"""
         reorder = not self._disable_reordering and not disable_reordering
-        source_coordinates = source_coordinates.contiguous()
-        target_coordinates = target_coordinates.contiguous()
-        built = _C.kernel_map_build(source_coordinates, target_coordinates, offsets,
-                                    source_batch_dims, target_batch_dims, reorder=reorder,
-                                    want_lists=True, want_dense=True, source_bounds=self._known_bounds(source_coordinates),
-                                    target_bounds=self._known_bounds(target_coordinates))
-        self.num_map_builds += 1
-        if source_coordinates.shape[0] > 0 and target_coordinates.shape[0] > 0:
-            self._remember_bounds(source_coordinates, built["bounds"][:8])
-            self._remember_bounds(target_coordinates, built["bounds"][8:])
+        dense = self._dense_maps_cache.get(key)
+        if dense is not None:
+            # the query ran earlier for a layer that needed the dense map only
+            built = _C.kernel_map_tables(dense, dense.num_sources, reorder=reorder, want_lists=True)
+        else:
+            offsets = self._kernel_offsets(source_stride, kernel_size, kernel_dilation)
+            source_coordinates = source_coordinates.contiguous()
+            target_coordinates = target_coordinates.contiguous()
+            built = _C.kernel_map_build(source_coordinates, target_coordinates, offsets,
+                                        source_batch_dims, target_batch_dims, reorder=reorder,
+                                        want_lists=True, want_dense=True,
+                                        source_bounds=self._known_bounds(source_coordinates),
+                                        target_bounds=self._known_bounds(target_coordinates))
+            self.num_map_builds += 1
+            if source_coordinates.shape[0] > 0 and target_coordinates.shape[0] > 0:
+                self._remember_bounds(source_coordinates, built["bounds"][:8])
+                self._remember_bounds(target_coordinates, built["bounds"][8:])
+            built["kernel_map"].num_sources = source_coordinates.shape[0]
+            self._dense_maps_cache[key] = built["kernel_map"]
         index_dtype = (source_coordinates.dtype if source_batch_dims is None
                        else source_batch_dims.dtype)
         cast = (lambda t: t) if index_dtype == torch.int32 else (lambda t: t.to(index_dtype))
@@ -210,6 +299,7 @@ class SparseConv(Module):
         self._tuning_data = None
         self._identity_map = None
         self._packed = None
+        self._routes = dict()
 
     @property
     def _allow_shortcut_matmul(self) -> bool:
@@ -368,7 +458,7 @@ class SparseConv(Module):
                 self._packed = (key, weights, F.pack_weights(weights))
         return self._packed[1], self._packed[2]
 
-    def _row_padding(self, features: torch.Tensor, target_masks) -> int:
+    def _row_padding(self, features: torch.Tensor) -> int:
         """Zero input channels to append so that feature rows become a multiple
         of 16 bytes, when that lets a 16-bit layer (a stem with 3 or 4 input
         channels, say) take the single-kernel dataflow; else 0."""
@@ -376,11 +466,23 @@ class SparseConv(Module):
         pad = -self.in_channels % per_piece
         if (pad == 0 or features.dtype == torch.float32 or not features.is_cuda
                 or self._tunable_config.get("dataflow", "auto") == "gather_gemm_scatter"
-                or getattr(target_masks, "kernel_map", None) is None
                 or not _C.implicit_forward_supported(self.in_channels + pad, self.out_channels,
                                                      features.dtype)):
             return 0
         return pad
+
+    def _takes_implicit(self, features: torch.Tensor, pad: int) -> bool:
+        """Whether this call runs the single-kernel dataflow: forced by the
+        tunable ``dataflow``, or chosen where it is the faster one."""
+        dataflow = self._tunable_config.get("dataflow", "auto")
+        if dataflow == "gather_gemm_scatter" or not features.is_cuda:
+            return False
+        if features.dtype != self.kernel.dtype:
+            return False
+        if dataflow == "implicit":
+            return True
+        return F.prefers_implicit(self.kernel.shape[0], self.in_channels + pad, self.out_channels,
+                                  features.dtype)
 
     def _pointwise(self, features: torch.Tensor, epilogue: Optional[F.Epilogue]) -> torch.Tensor:
         """1x1x1 kernel, stride 1: a plain ``features @ W`` (reference:
@@ -428,32 +530,53 @@ class SparseConv(Module):
                 transposed=self.transposed, source_coordinates=inputs.C,
                 source_batch_dims=inputs.batch_dims, source_stride=inputs.stride,
                 kernel_stride=self.stride)
-            source_masks, target_masks, order, sizes = cache.get_kernel_map(
-                transposed=self.transposed, source_coordinates=inputs.C,
-                source_stride=inputs.stride, source_batch_dims=inputs.batch_dims,
-                target_coordinates=coordinates, target_stride=stride,
-                target_batch_dims=batch_dims, kernel_size=self.kernel_size,
-                kernel_dilation=self.dilation)
-            if self._tuning_data is not None:
-                sizes.kernel_map_order = order
-                self._tuning_data.append((source_masks, target_masks, sizes))
+            map_args = dict(transposed=self.transposed, source_coordinates=inputs.C,
+                            source_stride=inputs.stride, source_batch_dims=inputs.batch_dims,
+                            target_coordinates=coordinates, target_stride=stride,
+                            target_batch_dims=batch_dims, kernel_size=self.kernel_size,
+                            kernel_dilation=self.dilation)
             sources = inputs.F
-            pad = self._row_padding(sources, target_masks)
-            if pad:
-                sources = torch.nn.functional.pad(sources, (0, pad))
-            weights, packed = self._packed_kernel(pad) if sources.is_cuda else (self.kernel, None)
-            features = F.sparse_convolution_forward(
-                sources=sources, weights=weights, source_masks=source_masks,
-                target_masks=target_masks, kernel_map_order=order, kernel_map_sizes=sizes,
-                gather_tile_size=self._tunable_config["gather_tile_size"],
-                scatter_tile_size=self._tunable_config["scatter_tile_size"],
-                allow_shortcut_matmul=self._allow_shortcut_matmul,
-                threshold=self._tunable_config["threshold"], epilogue=epilogue,
-                dataflow=self._tunable_config.get("dataflow", "auto"), packed_weights=packed)
+            # the route depends on the layer, the feature type and the tunable
+            # dataflow only: decided once, then looked up
+            route_key = (sources.dtype, sources.is_cuda, self._tunable_config.get("dataflow", "auto"))
+            route = self._routes.get(route_key)
+            if route is None:
+                pad = self._row_padding(sources)
+                route = (pad, self._takes_implicit(sources, pad))
+                self._routes[route_key] = route
+            pad, implicit = route
+            if implicit and self._tuning_data is None:
+                # single-kernel dataflow: the dense map is all it needs
+                dense = cache.get_dense_kernel_map(**map_args)
+                if pad:
+                    sources = torch.nn.functional.pad(sources, (0, pad))
+                weights, packed = self._packed_kernel(pad)
+                features = _C.sparse_convolution_forward_implicit(sources, weights, dense,
+                                                                  epilogue=epilogue,
+                                                                  packed_weights=packed)
+            else:
+                features = self._forward_tables(cache, map_args, sources, epilogue)
         if self.bias is not None and epilogue is None:
             features += self.bias
         return SparseTensor(features=features, coordinates=coordinates, stride=stride,
                             batch_dims=batch_dims)
+
+    def _forward_tables(self, cache, map_args, sources, epilogue):
+        """Gather -> GEMM -> Scatter through the rank tables (the reference's
+        dataflow, convolutions.py:470-494)."""
+        source_masks, target_masks, order, sizes = cache.get_kernel_map(**map_args)
+        if self._tuning_data is not None:
+            sizes.kernel_map_order = order
+            self._tuning_data.append((source_masks, target_masks, sizes))
+        weights, packed = self._packed_kernel() if sources.is_cuda else (self.kernel, None)
+        return F.sparse_convolution_forward(
+            sources=sources, weights=weights, source_masks=source_masks,
+            target_masks=target_masks, kernel_map_order=order, kernel_map_sizes=sizes,
+            gather_tile_size=self._tunable_config["gather_tile_size"],
+            scatter_tile_size=self._tunable_config["scatter_tile_size"],
+            allow_shortcut_matmul=self._allow_shortcut_matmul,
+            threshold=self._tunable_config["threshold"], epilogue=epilogue,
+            dataflow="gather_gemm_scatter", packed_weights=packed)
 
 
 class SparseConv3d(SparseConv):

@@ -45,7 +45,8 @@ SIGNATURES = {
     "mnt_arg_sort_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _vp, _pi64, _vp]),
     "mnt_unique_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _pi64, _vp]),
     "mnt_fill_unique_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _int, _vp, _vp]),
-    "mnt_target_coordinates_count": (_int, [_vp, _i64, _int, _int, _pi64, _vp, _i64, _int, _pi64, _vp]),
+    "mnt_target_coordinates_count": (_int, [_vp, _i64, _int, _int, _pi64, _vp, _i64, _int, _pi64, _pi64,
+                                            _vp]),
     "mnt_target_coordinates_fill": (_int, [_vp, _vp, _vp]),
     "mnt_query_sorted_index_with_offsets": (_int, [_vp, _i64, _vp, _i64, _vp, _i64, _int, _int,
                                                    _vp, _vp, _i64, _int, _vp, _int, _vp]),
@@ -54,6 +55,9 @@ SIGNATURES = {
     "mnt_kernel_map_query": (_int, [_vp, _i64, _vp, _i64, _pi64, _i64, _int, _int, _vp, _vp, _i64,
                                     _int, _int, _pi64, _pi64, _pi64, _vp, _pi64, _pi64, _vp]),
     "mnt_kernel_map_emit": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "mnt_kernel_map_dense": (_int, [_vp, _i64, _vp, _i64, _pi64, _i64, _int, _int, _vp, _vp, _i64, _int,
+                                    _pi64, _pi64, _pi64, _vp, _vp]),
+    "mnt_kernel_map_tables": (_int, [_vp, _i64, _i64, _i64, _int, _pi64, _pi64, _vp]),
     "mnt_kernel_map_pair_lists": (_int, [_vp, _i64, _i64, _pi64, _vp, _vp, _vp]),
     "mnt_generate_padding_buckets": (_int, [_pi64, _i64, _int, _dbl, _pi64, _pi64]),
     "mnt_cumsum_kernel_padded_sizes": (_int, [_pi64, _i64, _pi64, _i64, _pi64]),
@@ -295,11 +299,13 @@ def cuda_multi_unique_coordinates(coordinates: torch.Tensor, batch_dims: torch.T
 
 
 def target_coordinates(coordinates: torch.Tensor, batch_dims: Optional[torch.Tensor],
-                       target_stride: Sequence[int]):
+                       target_stride: Sequence[int], source_bounds=None):
     """floor(c / stride) * stride, sorted and unique, plus the new batch
     boundaries — the tensor expression of minuet/nn/convolutions.py:84-99 as two
-    library calls."""
+    library calls.  ``source_bounds`` (8 int64: per-dimension minima, then
+    maxima of ``coordinates``) spares their reduction on the device."""
     _ensure_ndim("coordinates", coordinates, 2)
+    known = None if source_bounds is None else np.ascontiguousarray(source_bounds, dtype=np.int64)
     device = _common_device([coordinates] + ([batch_dims] if batch_dims is not None else []))
     n, ndim = coordinates.shape
     ccode = _int_code(coordinates.dtype, "coordinate", "target_coordinates")
@@ -311,7 +317,8 @@ def target_coordinates(coordinates: torch.Tensor, batch_dims: Optional[torch.Ten
     with _on(device):
         _check(lib.mnt_target_coordinates_count(
             _ptr(coordinates), n, ndim, ccode, stride, _ptr(batch_dims),
-            batch_dims.numel() - 1 if batch_dims is not None else 1, icode, ctypes.byref(count),
+            batch_dims.numel() - 1 if batch_dims is not None else 1, icode,
+            None if known is None else known.ctypes.data_as(_pi64), ctypes.byref(count),
             _stream(device)))
         out = torch.empty((count.value, ndim), dtype=coordinates.dtype, device=device)
         out_dims = torch.empty_like(batch_dims) if batch_dims is not None else None
@@ -479,6 +486,82 @@ def kernel_map_build(sources: torch.Tensor, targets: torch.Tensor, offsets_host:
     if want_dense:
         result["kernel_map"] = dense
     return result
+
+
+def kernel_map_dense(sources: torch.Tensor, targets: torch.Tensor, offsets_host: np.ndarray,
+                     source_batch_dims: Optional[torch.Tensor],
+                     target_batch_dims: Optional[torch.Tensor], source_bounds=None,
+                     target_bounds=None):
+    """The query alone: ``(kernel_map [O, T] int32, bounds)``.  Nothing is read
+    back when both bounds are given, so the call returns without waiting for
+    the device."""
+    _ensure_ndim("sources", sources, 2)
+    _ensure_ndim("targets", targets, 2)
+    ndim = sources.size(1)
+    _ensure_dim("targets", targets, 1, ndim)
+    ctype = _common_dtype([sources, targets])
+    tensors = [sources, targets]
+    if (source_batch_dims is None) != (target_batch_dims is None):
+        raise ValueError("source_batch_dims and target_batch_dims must be both provided or "
+                         "neither provided")
+    bcode = 0
+    if source_batch_dims is not None:
+        tensors += [source_batch_dims, target_batch_dims]
+        bcode = _int_code(_common_dtype([source_batch_dims, target_batch_dims]), "index",
+                          "kernel_map_dense")
+    device = _common_device(tensors)
+    ccode = _int_code(ctype, "coordinate", "kernel_map_dense")
+    offs = np.ascontiguousarray(np.asarray(offsets_host, dtype=np.int64).reshape(-1, ndim))
+    num_offsets = offs.shape[0]
+    dense = torch.empty((num_offsets, targets.size(0)), dtype=torch.int32, device=device)
+    bounds = np.zeros(16, dtype=np.int64)
+    sb = None if source_bounds is None else np.ascontiguousarray(source_bounds, dtype=np.int64)
+    tb = None if target_bounds is None else np.ascontiguousarray(target_bounds, dtype=np.int64)
+    with _on(device):
+        _check(load_library().mnt_kernel_map_dense(
+            _ptr(sources), sources.size(0), _ptr(targets), targets.size(0),
+            offs.ctypes.data_as(_pi64), num_offsets, ndim, ccode, _ptr(source_batch_dims),
+            _ptr(target_batch_dims),
+            source_batch_dims.numel() - 1 if source_batch_dims is not None else 1, bcode,
+            None if sb is None else sb.ctypes.data_as(_pi64),
+            None if tb is None else tb.ctypes.data_as(_pi64), bounds.ctypes.data_as(_pi64),
+            _ptr(dense), _stream(device)))
+    return dense, bounds
+
+
+def kernel_map_tables(kernel_map: torch.Tensor, num_sources: int, reorder: bool,
+                      want_lists: bool = True):
+    """Sizes, stable size order, rank tables and (optionally) pair lists of a
+    dense int32 kernel map made earlier by :func:`kernel_map_dense`: the rest
+    of what :func:`kernel_map_build` returns."""
+    _ensure_ndim("kernel_map", kernel_map, 2)
+    if kernel_map.dtype != torch.int32:
+        _fail("kernel_map_tables expects an int32 kernel map")
+    device = _common_device([kernel_map])
+    kernel_map = kernel_map.contiguous()
+    num_offsets, num_targets = kernel_map.shape
+    sizes_host = np.zeros(num_offsets, dtype=np.int64)
+    order_host = np.zeros(num_offsets, dtype=np.int64)
+    lib = load_library()
+    with _on(device):
+        stream = _stream(device)
+        _check(lib.mnt_kernel_map_tables(_ptr(kernel_map), num_sources, num_targets, num_offsets,
+                                         1 if reorder else 0, sizes_host.ctypes.data_as(_pi64),
+                                         order_host.ctypes.data_as(_pi64), stream))
+        smask = torch.empty((num_offsets, num_sources), dtype=torch.int32, device=device)
+        tmask = torch.empty((num_offsets, num_targets), dtype=torch.int32, device=device)
+        in_idx = out_idx = None
+        if want_lists:
+            nnz = int(sizes_host.sum())
+            in_idx = torch.empty((nnz,), dtype=torch.int32, device=device)
+            out_idx = torch.empty((nnz,), dtype=torch.int32, device=device)
+        sizes_dev = torch.empty((num_offsets,), dtype=torch.int32, device=device)
+        order_dev = torch.empty((num_offsets,), dtype=torch.int32, device=device)
+        _check(lib.mnt_kernel_map_emit(_ptr(smask), _ptr(tmask), _ptr(in_idx), _ptr(out_idx),
+                                       _ptr(sizes_dev), _ptr(order_dev), stream))
+    return dict(sizes_host=sizes_host, order_host=order_host, sizes=sizes_dev, order=order_dev,
+                source_masks=smask, target_masks=tmask, in_idx=in_idx, out_idx=out_idx,
+                kernel_map=kernel_map)
 
 
 def kernel_map_pair_lists(kernel_map: torch.Tensor, sizes_host: Sequence[int]):

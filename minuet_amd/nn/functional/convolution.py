@@ -7,7 +7,8 @@ import torch
 from . import _C
 
 __all__ = ["cuda_time_gather", "cuda_time_scatter", "sparse_convolution_forward",
-           "cuda_time_gemm", "set_gemm_parallel_level", "Epilogue", "pack_weights"]
+           "cuda_time_gemm", "set_gemm_parallel_level", "Epilogue", "pack_weights",
+           "prefers_implicit"]
 
 pack_weights = _C.pack_weights
 
@@ -23,6 +24,20 @@ def set_gemm_parallel_level(level: int):
     one grouped launch, so the value has no effect."""
     global GEMM_PARALLEL_LEVEL
     GEMM_PARALLEL_LEVEL = level
+
+
+def prefers_implicit(num_offsets: int, num_source_features: int, num_target_features: int,
+                     dtype: torch.dtype) -> bool:
+    """Whether ``dataflow="auto"`` takes the single-kernel form for a layer of
+    this shape: it must fit that kernel, and it must be the faster one, which
+    measurements say it is for 16-bit features.  fp32 matrix work is 16x dearer,
+    so there it only pays where most (offset, target) pairs are hits, i.e. for
+    small layers with strided 2^D kernels."""
+    if not _C.implicit_forward_supported(num_source_features, num_target_features, dtype):
+        return False
+    if dtype != torch.float32:
+        return True
+    return num_offsets <= 8 and num_source_features * num_target_features <= 1024
 
 
 def cuda_time_gather(weights: torch.Tensor, source_masks: torch.Tensor,
@@ -95,11 +110,8 @@ def sparse_convolution_forward(sources: torch.Tensor, weights: torch.Tensor,
     if dataflow == "implicit" and dense is None:
         raise ValueError("the implicit dataflow needs target_masks.kernel_map (the dense kernel map)")
     if dense is not None and dataflow != "gather_gemm_scatter":
-        fits = _C.implicit_forward_supported(weights.shape[1], weights.shape[2], weights.dtype)
-        # fp32 matrix work is 16x dearer than fp16: there the implicit form only
-        # pays where most (offset, target) pairs are hits, i.e. strided 2^D kernels
-        dense_hits = weights.shape[0] <= 8 and weights.shape[1] * weights.shape[2] <= 1024
-        if dataflow == "implicit" or (fits and (weights.dtype != torch.float32 or dense_hits)):
+        if dataflow == "implicit" or prefers_implicit(weights.shape[0], weights.shape[1],
+                                                      weights.shape[2], weights.dtype):
             return _C.sparse_convolution_forward_implicit(sources, weights, dense, epilogue=epilogue,
                                                           packed_weights=packed_weights)
     if parallel is None:
