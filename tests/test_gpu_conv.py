@@ -243,6 +243,37 @@ def test_narrow_rows_are_padded_for_the_single_kernel_form(cin):
     assert_features_close(y.F, ref, "fp16")
 
 
+def test_layers_on_empty_and_tiny_clouds():
+    """No voxels, one voxel, and a batch with an empty cloud, through both
+    dataflows of the module."""
+    for flow in ("gather_gemm_scatter", "implicit"):
+        conv = minuet.nn.SparseConv3d(16, 32, 3, dtype=torch.float16, device="cuda")
+        down = minuet.nn.SparseConv3d(16, 16, 2, stride=2, dtype=torch.float16, device="cuda")
+        for m in (conv, down):
+            m.tunable_config["dataflow"] = flow
+        with torch.no_grad():
+            for coords, bd in ((np.zeros((0, 3), dtype=np.int32), None),
+                               (np.array([[3, -2, 7]], dtype=np.int32), None),
+                               (np.array([[0, 0, 0], [0, 0, 1], [5, 5, 5]], dtype=np.int32),
+                                np.array([0, 0, 2, 3], dtype=np.int32))):
+                cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+                conv.set_kernel_map_cache(cache)
+                down.set_kernel_map_cache(cache)
+                n = coords.shape[0]
+                feats = torch.ones(n, 16, device="cuda").half()
+                x = minuet.SparseTensor(feats, dev(coords), batch_dims=dev(bd))
+                y = conv(x)
+                assert y.F.shape == (n, 32) and torch.equal(y.C, x.C)
+                if n:
+                    w = host(conv.kernel.detach().float()).astype(np.float64)
+                    ref, _, _, _ = orc.conv_layer(coords, bd, np.ones((n, 16)), w, 3)
+                    assert_features_close(y.F, ref, "fp16")
+                z = down(x)
+                expect, ebd = orc.target_coordinates(coords, bd, 2) if n else (coords, bd)
+                np.testing.assert_array_equal(host(z.C), expect)
+                assert z.F.shape == (expect.shape[0], 16)
+
+
 def test_epilogue_rejects_bad_operands():
     src, sbd, tgt, tbd, off, feats, weights = make_layer_case(5, 500, 8, 3, 32, 32, "fp32")
     esm, etm, eorder, esizes, _ = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=True)

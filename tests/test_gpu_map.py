@@ -221,3 +221,48 @@ def test_collate_sorts_each_cloud_and_carries_features():
     assert torch.equal(coords_only, coords) and torch.equal(bd2, bd)
     with pytest.raises(ValueError):
         F.collate([])
+
+
+@pytest.mark.parametrize("reorder", [True, False])
+@pytest.mark.parametrize("kernel,stride,batched", [(3, 1, True), (2, 2, False)])
+def test_dense_then_tables_equals_full_build(reorder, kernel, stride, batched):
+    """The query alone, and the rank tables made from its dense map later, give
+    exactly what the one-call build gives (and what the oracle gives)."""
+    src, sbd, tgt, tbd, off = _query_case(17, 20000, 40, -5, kernel, stride, batched=batched)
+    dense, bounds = _C.kernel_map_dense(dev(src), dev(tgt), off.astype(np.int64), dev(sbd), dev(tbd))
+    expect = orc.query_sorted_index_with_offsets(src, tgt, off, sbd, tbd, dtype=np.int32)
+    np.testing.assert_array_equal(host(dense), expect)
+    np.testing.assert_array_equal(bounds[:3], src.min(0))
+    np.testing.assert_array_equal(bounds[4:7], src.max(0))
+    np.testing.assert_array_equal(bounds[8:11], tgt.min(0))
+    np.testing.assert_array_equal(bounds[12:15], tgt.max(0))
+    # second call with the bounds known: same map, no reduction on the device
+    again, _ = _C.kernel_map_dense(dev(src), dev(tgt), off.astype(np.int64), dev(sbd), dev(tbd),
+                                   source_bounds=bounds[:8], target_bounds=bounds[8:])
+    assert torch.equal(again, dense)
+    tables = _C.kernel_map_tables(dense, src.shape[0], reorder=reorder, want_lists=True)
+    esm, etm, eorder, esizes, em = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=reorder)
+    np.testing.assert_array_equal(tables["sizes_host"], esizes.astype(np.int64))
+    if reorder:
+        np.testing.assert_array_equal(tables["order_host"], eorder.astype(np.int64))
+    np.testing.assert_array_equal(host(tables["source_masks"]), esm)
+    np.testing.assert_array_equal(host(tables["target_masks"]), etm)
+    ein, eout, _ = orc.kernel_map_pair_lists(em)
+    np.testing.assert_array_equal(host(tables["in_idx"]), ein)
+    np.testing.assert_array_equal(host(tables["out_idx"]), eout)
+
+
+def test_dense_and_tables_empty_inputs():
+    off = orc.generate_kernel_offsets(3, 3, 1, 1).astype(np.int64)
+    cloud = random_cloud(40, 4, seed=2)
+    none = np.zeros((0, 3), dtype=np.int32)
+    dense, _ = _C.kernel_map_dense(dev(none), dev(cloud), off, None, None)
+    assert dense.shape == (27, 40) and (host(dense) == -1).all()
+    tables = _C.kernel_map_tables(dense, 0, reorder=True)
+    assert tables["sizes_host"].sum() == 0 and tables["source_masks"].shape == (27, 0)
+    assert (host(tables["target_masks"]) == -1).all() and tables["in_idx"].numel() == 0
+    dense, _ = _C.kernel_map_dense(dev(cloud), dev(none), off, None, None)
+    assert dense.shape == (27, 0)
+    tables = _C.kernel_map_tables(dense, 40, reorder=False)
+    assert tables["sizes_host"].sum() == 0 and (host(tables["source_masks"]) == -1).all()
+    assert _C.kernel_map_invert(dense, 40).eq(-1).all()
