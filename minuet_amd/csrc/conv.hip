@@ -417,25 +417,32 @@ constexpr int kMaxChannelBlocks = 4;    // 32-channel blocks per workgroup (128 
 // buffer exists; a group with list_start < 0 reads row i of `a` itself (the
 // centre offset of the shortcut).  The output rows stay in buffer order.
 //
-// The tables reach the kernel either in device memory (`meta`) or, when
-// table_count > 0, as the by-value argument `table` (meta starts at entry
-// meta_at); workgroup (0, 0) then also copies the whole table to `table_out`
-// for the kernels that follow in the stream, so that no separate upload runs.
-template <typename T, typename TC, int NB, bool VEC>
-__global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
-    const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt,
-    const int *__restrict__ meta, int K, int N, int Kp, int Np,
-    const int *__restrict__ gather_index, PlanChunk table, int table_count, int meta_at,
-    int *__restrict__ table_out) {
+// The tables reach the kernel either in device memory (grouped_gemm_kernel) or
+// as a by-value argument (grouped_gemm_riding_kernel: meta starts at entry
+// meta_at of `table`); workgroup (0, 0) of the latter also copies the whole
+// table to `table_out` for the kernels that follow in the stream, so that no
+// separate upload runs.  Reading the tables from the argument segment costs
+// every workgroup a little, so large passes use the first form.
+struct MetaInMemory {
+  const int *meta;
+  __device__ __forceinline__ int operator()(int i) const { return meta[i]; }
+};
+struct MetaInArguments {
+  const PlanChunk *table;
+  int meta_at;
+  __device__ __forceinline__ int operator()(int i) const { return table->v[meta_at + i]; }
+};
+
+template <typename T, typename TC, int NB, bool VEC, typename Meta>
+__device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *__restrict__ c,
+                                                  const T *__restrict__ wt, const Meta &entry, int K,
+                                                  int N, int Kp, int Np,
+                                                  const int *__restrict__ gather_index) {
   constexpr int EPC = 16 / static_cast<int>(sizeof(T));        // elements per 16-byte piece
   constexpr int KC = kChunkBytes / static_cast<int>(sizeof(T));
   constexpr int TN = NB * 32;
   __shared__ __align__(16) unsigned char b_lds[TN * kLdsRowBytes];
 
-  if (table_count > 0 && blockIdx.x == 0 && blockIdx.y == 0) {
-    for (int i = threadIdx.x; i < table_count; i += kGemmBlock) table_out[i] = table.v[i];
-  }
-  auto entry = [&](int i) -> int { return table_count > 0 ? table.v[meta_at + i] : meta[i]; };
   const int G = entry(0);
   const int at_prefix = 1, at_start = at_prefix + G + 1, at_rows = at_start + G + 1, at_weight = at_rows + G,
             at_list = at_weight + G;
@@ -578,6 +585,27 @@ __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
   }
 }
 
+template <typename T, typename TC, int NB, bool VEC>
+__global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
+    const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt,
+    const int *__restrict__ meta, int K, int N, int Kp, int Np,
+    const int *__restrict__ gather_index) {
+  grouped_gemm_body<T, TC, NB, VEC>(a, c, wt, MetaInMemory{meta}, K, N, Kp, Np, gather_index);
+}
+
+// The same with the tables as a by-value argument.
+template <typename T, typename TC, int NB, bool VEC>
+__global__ __launch_bounds__(kGemmBlock) void grouped_gemm_riding_kernel(
+    const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt, int K, int N, int Kp, int Np,
+    const int *__restrict__ gather_index, PlanChunk table, int table_count, int meta_at,
+    int *__restrict__ table_out) {
+  if (blockIdx.x == 0 && blockIdx.y == 0) {
+    for (int i = threadIdx.x; i < table_count; i += kGemmBlock) table_out[i] = table.v[i];
+  }
+  grouped_gemm_body<T, TC, NB, VEC>(a, c, wt, MetaInArguments{&table, meta_at}, K, N, Kp, Np,
+                                    gather_index);
+}
+
 // ---------------------------------------------------------- host launchers ----
 
 static int pow2_vec(int64_t bytes_per_lane, int64_t row_bytes, const void *p0, const void *p1) {
@@ -707,6 +735,11 @@ static void launch_scatter(const LaneShape &sh, const TB *buffer, void *targets,
 
 // Integer tables that ride a GEMM launch as a kernel argument (count == 0:
 // none, the kernel reads `meta` from device memory).
+// Passes of at most this many GEMM tiles take their tables as an argument of
+// the GEMM (one launch less); larger ones upload them first, which costs a
+// launch but keeps the tables in device memory for thousands of workgroups.
+constexpr int kRidingMaxTiles = 4096;
+
 struct RidingTable {
   const std::vector<int> *ints = nullptr;
   int meta_at = 0;
@@ -718,18 +751,23 @@ static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int 
                            int Kp, int Np, bool vec, const int *gather_index, const RidingTable &riding,
                            hipStream_t stream) {
   dim3 grid(num_tiles, static_cast<unsigned>(div_ceil(Np, NB * 32)));
-  PlanChunk chunk;
-  int count = 0;
   if (riding.ints != nullptr) {
-    count = static_cast<int>(riding.ints->size());
+    PlanChunk chunk;
+    const int count = static_cast<int>(riding.ints->size());
     std::memcpy(chunk.v, riding.ints->data(), count * sizeof(int));
-  }
-  if (vec) {
-    grouped_gemm_kernel<T, TC, NB, true><<<grid, kGemmBlock, 0, stream>>>(
-        a, c, wt, meta, K, N, Kp, Np, gather_index, chunk, count, riding.meta_at, riding.out);
+    if (vec) {
+      grouped_gemm_riding_kernel<T, TC, NB, true><<<grid, kGemmBlock, 0, stream>>>(
+          a, c, wt, K, N, Kp, Np, gather_index, chunk, count, riding.meta_at, riding.out);
+    } else {
+      grouped_gemm_riding_kernel<T, TC, NB, false><<<grid, kGemmBlock, 0, stream>>>(
+          a, c, wt, K, N, Kp, Np, gather_index, chunk, count, riding.meta_at, riding.out);
+    }
+  } else if (vec) {
+    grouped_gemm_kernel<T, TC, NB, true><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np,
+                                                                          gather_index);
   } else {
-    grouped_gemm_kernel<T, TC, NB, false><<<grid, kGemmBlock, 0, stream>>>(
-        a, c, wt, meta, K, N, Kp, Np, gather_index, chunk, count, riding.meta_at, riding.out);
+    grouped_gemm_kernel<T, TC, NB, false><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np,
+                                                                           gather_index);
   }
 }
 
@@ -909,7 +947,7 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
   RidingTable riding;
   const T *wt = packed;
   if (ahead) {
-    if (fits && folded && num_tiles > 0) {
+    if (fits && folded && num_tiles > 0 && num_tiles <= kRidingMaxTiles) {
       riding.ints = &ints;
       riding.meta_at = static_cast<int>(meta_at);
       riding.out = d_ints;
