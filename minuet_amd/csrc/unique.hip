@@ -247,6 +247,151 @@ static int bit_width64(unsigned long long range) {
   return range == 0 ? 0 : 64 - __builtin_clzll(range);
 }
 
+// ---- bitmap form: when the packed keys span at most 2^28 values, the set of
+// distinct keys is a bitmap.  Marking it and walking it in key order yields
+// the sorted, duplicate-free targets without any sort.
+
+constexpr int kBitmapMaxBits = 28;                   // 32 MiB of bits
+constexpr int kBitmapWords = 8;                      // 32-bit words per thread
+constexpr int kBitmapTile = kScanBlock * kBitmapWords;
+
+template <typename CT, typename IT>
+__device__ __forceinline__ unsigned long long target_key(const CT *__restrict__ coords, long long i,
+                                                         const TargetSpec &spec,
+                                                         const IT *__restrict__ batch_dims) {
+  unsigned long long key = 0;
+#pragma unroll
+  for (int k = 0; k < MNT_MAX_NDIM; ++k) {
+    if (k < spec.ndim) {
+      long long cell = floor_div(static_cast<long long>(coords[i * spec.ndim + k]), spec.stride[k]);
+      key |= (static_cast<unsigned long long>(cell - spec.base[k]) & spec.mask[k]) << spec.shift[k];
+    }
+  }
+  if (spec.num_batches > 0) {
+    key |= static_cast<unsigned long long>(batch_of<IT>(i, batch_dims, spec.num_batches))
+           << spec.batch_shift;
+  }
+  return key;
+}
+
+template <typename CT, typename IT>
+__global__ __launch_bounds__(256) void mark_targets_kernel(const CT *__restrict__ coords, long long n,
+                                                           TargetSpec spec,
+                                                           const IT *__restrict__ batch_dims,
+                                                           unsigned *__restrict__ bitmap) {
+  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+  for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += stride) {
+    const unsigned long long key = target_key<CT, IT>(coords, i, spec, batch_dims);
+    atomicOr(&bitmap[key >> 5], 1u << (key & 31u));
+  }
+}
+
+__global__ __launch_bounds__(kScanBlock) void bitmap_tile_sums_kernel(const unsigned *__restrict__ bitmap,
+                                                                      long long words,
+                                                                      unsigned *__restrict__ tile_sums) {
+  const long long base = static_cast<long long>(blockIdx.x) * kBitmapTile + threadIdx.x * kBitmapWords;
+  unsigned count = 0;
+#pragma unroll
+  for (int r = 0; r < kBitmapWords; ++r) {
+    if (base + r < words) count += __popc(bitmap[base + r]);
+  }
+  unsigned total;
+  block_exclusive_scan(count, &total);
+  if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+}
+
+// Exclusive scan of the tile sums in place (tiles + 1 entries, the last one
+// receives the total) by one workgroup; the total also goes to the host.
+__global__ __launch_bounds__(1024) void bitmap_scan_kernel(unsigned *__restrict__ tile_sums, int tiles,
+                                                           unsigned *host_count,
+                                                           unsigned long long *flag,
+                                                           unsigned long long sequence) {
+  __shared__ unsigned partial[1024];
+  const int t = threadIdx.x;
+  const int chunk = (tiles + 1023) / 1024;
+  const int lo = t * chunk;
+  const int hi = min(tiles, lo + chunk);
+  unsigned sum = 0;
+  for (int i = lo; i < hi; ++i) sum += tile_sums[i];
+  partial[t] = sum;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {
+    const unsigned v = t >= off ? partial[t - off] : 0;
+    __syncthreads();
+    partial[t] += v;
+    __syncthreads();
+  }
+  unsigned run = partial[t] - sum;
+  for (int i = lo; i < hi; ++i) {
+    const unsigned v = tile_sums[i];
+    tile_sums[i] = run;
+    run += v;
+  }
+  if (t == 1023) {
+    const unsigned total = partial[1023];
+    tile_sums[tiles] = total;
+    *host_count = total;
+    __threadfence_system();
+    __hip_atomic_store(flag, sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+}
+
+template <typename CT, typename IT>
+__global__ __launch_bounds__(kScanBlock) void bitmap_emit_kernel(
+    const unsigned *__restrict__ bitmap, long long words, const unsigned *__restrict__ tile_bases,
+    int tiles, TargetSpec spec, CT *__restrict__ out, IT *__restrict__ batch_dims_out) {
+  const long long base = static_cast<long long>(blockIdx.x) * kBitmapTile + threadIdx.x * kBitmapWords;
+  unsigned word[kBitmapWords];
+  unsigned count = 0;
+#pragma unroll
+  for (int r = 0; r < kBitmapWords; ++r) {
+    word[r] = base + r < words ? bitmap[base + r] : 0u;
+    count += __popc(word[r]);
+  }
+  unsigned total;
+  unsigned run = block_exclusive_scan(count, &total) + tile_bases[blockIdx.x];
+#pragma unroll
+  for (int r = 0; r < kBitmapWords; ++r) {
+    const unsigned long long first_key = static_cast<unsigned long long>(base + r) << 5;
+    if (batch_dims_out != nullptr && base + r < words) {
+      // batch boundaries g << batch_shift that fall into this word
+      const unsigned long long step = 1ull << spec.batch_shift;
+      for (unsigned long long g = (first_key + step - 1) >> spec.batch_shift;
+           g < static_cast<unsigned long long>(spec.num_batches) && (g << spec.batch_shift) < first_key + 32;
+           ++g) {
+        const unsigned bit = static_cast<unsigned>((g << spec.batch_shift) - first_key);
+        batch_dims_out[g] = static_cast<IT>(run + __popc(word[r] & ((1u << bit) - 1u)));
+      }
+    }
+    unsigned bits = word[r];
+    while (bits != 0u) {
+      const unsigned bit = __ffs(bits) - 1;
+      bits &= bits - 1u;
+      const unsigned long long key = first_key | bit;
+#pragma unroll
+      for (int k = 0; k < MNT_MAX_NDIM; ++k) {
+        if (k < spec.ndim) {
+          const long long cell = static_cast<long long>((key >> spec.shift[k]) & spec.mask[k]) + spec.base[k];
+          out[static_cast<long long>(run) * spec.ndim + k] = static_cast<CT>(cell * spec.stride[k]);
+        }
+      }
+      ++run;
+    }
+  }
+  if (batch_dims_out != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
+    batch_dims_out[spec.num_batches] = static_cast<IT>(tile_bases[tiles]);
+  }
+}
+
+// What phase 2 needs to know about phase 1 (kept in the arena's pending blob).
+struct TargetState {
+  TargetSpec spec;
+  int bitmap;            // 1: bitmap form, 0: sorted keys + ranks
+  long long words;
+  int tiles;
+};
+
 template <typename CT, typename IT>
 static void target_count_typed(const CT *coords, int64_t n, int ndim, const int64_t *target_stride,
                                const IT *batch_dims, int64_t num_batches,
@@ -289,6 +434,45 @@ static void target_count_typed(const CT *coords, int64_t n, int ndim, const int6
     MNT_CHECK(bits <= 64,
               "coordinate range needs %d key bits; strided target generation supports at most 64",
               bits);
+    if (bits <= kBitmapMaxBits) {
+      const long long words = bits <= 5 ? 1 : (1ll << (bits - 5));
+      const int tiles = static_cast<int>(div_ceil(words, kBitmapTile));
+      // persistent block: bitmap [words] then tile bases [tiles + 1]
+      const size_t map_bytes = (static_cast<size_t>(words) * 4 + 255) / 256 * 256;
+      char *keep = static_cast<char *>(arena.persistent(0, map_bytes + (static_cast<size_t>(tiles) + 1) * 4));
+      unsigned *bitmap = reinterpret_cast<unsigned *>(keep);
+      unsigned *tile_bases = reinterpret_cast<unsigned *>(keep + map_bytes);
+      MNT_HIP(hipMemsetAsync(bitmap, 0, static_cast<size_t>(words) * 4, stream));
+      mark_targets_kernel<CT, IT><<<grid_for(n, 256, 4096), 256, 0, stream>>>(coords, n, spec, batch_dims, bitmap);
+      check_launch("mark_targets_kernel");
+      bitmap_tile_sums_kernel<<<tiles, kScanBlock, 0, stream>>>(bitmap, words, tile_bases);
+      check_launch("bitmap_tile_sums_kernel");
+      volatile unsigned *h = reinterpret_cast<volatile unsigned *>(static_cast<char *>(arena.pinned()) + 256);
+      unsigned *d = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned_device()) + 256);
+      const unsigned long long sequence = arena.next_sequence();
+      bitmap_scan_kernel<<<1, 1024, 0, stream>>>(tile_bases, tiles, d, arena.flag_device(2), sequence);
+      check_launch("bitmap_scan_kernel");
+      arena.wait_flag(2, sequence);
+      *count_out = static_cast<int64_t>(*h);
+      TargetState state;
+      memset(&state, 0, sizeof(state));
+      state.spec = spec;
+      state.bitmap = 1;
+      state.words = words;
+      state.tiles = tiles;
+      auto &p = arena.pending;
+      p.valid = true;
+      p.count = *count_out;
+      p.n = n;
+      p.num_batches = batched ? num_batches : 0;
+      p.ndim = ndim;
+      p.coord_dtype = sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64;
+      p.index_dtype = sizeof(IT) == 4 ? MNT_INT32 : MNT_INT64;
+      static_assert(sizeof(TargetState) <= sizeof(p.blob), "pending blob too small");
+      memcpy(p.blob, &state, sizeof(state));
+      p.batch_dims = batch_dims;
+      return;
+    }
 
     // persistent block: sorted keys [n] then ranks [n+1]
     size_t key_bytes = (static_cast<size_t>(n) * 8 + 255) / 256 * 256;
@@ -331,8 +515,10 @@ static void target_count_typed(const CT *coords, int64_t n, int ndim, const int6
   p.ndim = ndim;
   p.coord_dtype = sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64;
   p.index_dtype = sizeof(IT) == 4 ? MNT_INT32 : MNT_INT64;
-  static_assert(sizeof(TargetSpec) <= sizeof(p.blob), "pending blob too small");
-  memcpy(p.blob, &spec, sizeof(spec));
+  TargetState state;
+  memset(&state, 0, sizeof(state));
+  state.spec = spec;
+  memcpy(p.blob, &state, sizeof(state));
   p.batch_dims = batch_dims;
 }
 
@@ -340,9 +526,22 @@ template <typename CT, typename IT>
 static void target_fill_typed(CT *out, IT *batch_dims_out, hipStream_t stream) {
   Arena &arena = Arena::of(stream);
   auto &p = arena.pending;
-  TargetSpec spec;
-  memcpy(&spec, p.blob, sizeof(spec));
+  TargetState state;
+  memcpy(&state, p.blob, sizeof(state));
+  const TargetSpec spec = state.spec;
   const int64_t n = p.n;
+  if (state.bitmap) {
+    const size_t map_bytes = (static_cast<size_t>(state.words) * 4 + 255) / 256 * 256;
+    char *keep = static_cast<char *>(arena.persistent(0, 0));
+    const unsigned *bitmap = reinterpret_cast<const unsigned *>(keep);
+    const unsigned *tile_bases = reinterpret_cast<const unsigned *>(keep + map_bytes);
+    bitmap_emit_kernel<CT, IT><<<state.tiles, kScanBlock, 0, stream>>>(
+        bitmap, state.words, tile_bases, state.tiles, spec, out,
+        p.num_batches > 0 ? batch_dims_out : nullptr);
+    check_launch("bitmap_emit_kernel");
+    p.valid = false;
+    return;
+  }
   size_t key_bytes = (static_cast<size_t>(n) * 8 + 255) / 256 * 256;
   char *keep = static_cast<char *>(arena.persistent(0, 0));
   const unsigned long long *keys = reinterpret_cast<const unsigned long long *>(keep);

@@ -87,6 +87,27 @@ def test_target_coordinates(stride, batched):
         assert got_bd is None
 
 
+@pytest.mark.parametrize("extent,batches", [(3, 1), (40, 5), (1 << 11, 1), (1 << 13, 3), (1 << 20, 2)])
+def test_target_coordinates_bitmap_and_sorted_forms(extent, batches):
+    """Key ranges up to 2^28 take the bitmap form, wider ones the sorted one;
+    both must equal the oracle, with empty batches and known bounds alike."""
+    rng = np.random.default_rng(extent)
+    n = 6000
+    c = rng.integers(-extent, extent, size=(n, 3)).astype(np.int32)
+    cuts = np.sort(rng.integers(0, n, size=batches - 1)) if batches > 1 else np.zeros(0, dtype=np.int64)
+    bd = np.concatenate([[0], cuts, [n]]).astype(np.int32) if batches > 1 else None
+    if batches > 2:
+        bd[2] = bd[1]                                  # an empty cloud in the middle
+    c, bd = sorted_unique(c, bd)
+    for stride in ((2, 2, 2), (4, 4, 8)):
+        exp, exp_bd = orc.target_coordinates(c, bd, stride)
+        for known in (None, np.concatenate([c.min(0), [0], c.max(0), [0]]).astype(np.int64)):
+            got, got_bd = _C.target_coordinates(dev(c), dev(bd), stride, source_bounds=known)
+            np.testing.assert_array_equal(host(got), exp)
+            if bd is not None:
+                np.testing.assert_array_equal(host(got_bd), exp_bd)
+
+
 def _query_case(seed, n, extent, lo, kernel, stride=1, batched=False, cdtype=np.int32, idtype=np.int32):
     bd = None
     if batched:
