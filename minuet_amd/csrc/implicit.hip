@@ -28,6 +28,7 @@ namespace mnt {
 constexpr int kImplicitBlock = 256;
 constexpr int kImplicitTargets = 128;     // per workgroup, 32 per wavefront
 constexpr int kImplicitMaxBlocks = 4;     // 32-channel output blocks (128 channels)
+constexpr int64_t kImplicitWideTargets = 1 << 16;   // from here on: two target blocks per wavefront
 
 // wt: packed weights [O][Np][KC] (W^T, K-contiguous, zero-padded to one
 // 128-byte chunk per row; see pack_weights_kernel).  Requires
@@ -39,14 +40,61 @@ struct Pieces {
   uint4 v[N];
 };
 
+template <int N>
+struct Pieces2 {
+  int v[N];
+};
+
 typedef unsigned uint4v __attribute__((ext_vector_type(4)));
 
 // Buffer offset that is out of range for every source tensor this kernel
 // accepts: such a load returns zeros without touching memory.
 constexpr unsigned kNoRow = 0xFFFFFFF0u;
 
+// One output row's worth of epilogue and store: four consecutive channels of
+// target t held by this lane.
+template <typename T>
+__device__ __forceinline__ void finish_four(float (&v)[4], const Epilogue &ep, long long t, int ch, int N,
+                                            unsigned char *__restrict__ out) {
+  typedef typename VecOf<4 * sizeof(T)>::type V;
+  if (ep.scale != nullptr) {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) v[x] *= ep.scale[ch + x];
+  }
+  if (ep.shift != nullptr) {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) v[x] += ep.shift[ch + x];
+  }
+  if (ep.residual != nullptr) {
+    const V raw = *reinterpret_cast<const V *>(static_cast<const unsigned char *>(ep.residual) +
+                                               (t * N + ch) * static_cast<long long>(sizeof(T)));
+    const T *e = reinterpret_cast<const T *>(&raw);
+#pragma unroll
+    for (int x = 0; x < 4; ++x) v[x] += to_float(e[x]);
+  }
+  if (ep.activation == MNT_ACT_RELU) {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) v[x] = fmaxf(v[x], 0.0f);
+  } else if (ep.activation == MNT_ACT_LEAKY_RELU) {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) v[x] = v[x] > 0.0f ? v[x] : v[x] * ep.slope;
+  } else if (ep.activation == MNT_ACT_RELU6) {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) v[x] = fminf(fmaxf(v[x], 0.0f), 6.0f);
+  }
+  V raw;
+  T *e = reinterpret_cast<T *>(&raw);
+#pragma unroll
+  for (int x = 0; x < 4; ++x) e[x] = static_cast<T>(v[x]);
+  *reinterpret_cast<V *>(out + (t * N + ch) * static_cast<long long>(sizeof(T))) = raw;
+}
+
 // KS: 32-byte steps of K that hold data (source rows are at most KS * 32 bytes).
-template <typename T, int NB, int KS>
+// MW: 32-target blocks per wavefront.  With MW = 2 a wavefront owns 64 targets
+// and a workgroup 256: every weight fragment read from LDS feeds two matrix
+// operations and the weight tiles are staged half as often per target, at the
+// price of twice the accumulators and source-row registers.
+template <typename T, int NB, int KS, int MW>
 __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
     const T *__restrict__ sources, unsigned source_bytes, const T *__restrict__ wt,
     const int *__restrict__ kernel_map, long long num_targets, int num_offsets, int K, int N,
@@ -65,24 +113,38 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
   const int wv = tid >> 6;
   const int r = lane & 31;
   const int h = lane >> 5;
-  const long long t = static_cast<long long>(blockIdx.x) * kImplicitTargets + wv * 32 + r;
-  const bool t_ok = t < num_targets;
-
-  floatx16 acc[NB];
+  long long t[MW], t_safe[MW];
+  bool t_ok[MW];
 #pragma unroll
-  for (int b = 0; b < NB; ++b) {
-#pragma unroll
-    for (int j = 0; j < 16; ++j) acc[b][j] = 0.0f;
+  for (int m = 0; m < MW; ++m) {
+    t[m] = static_cast<long long>(blockIdx.x) * (kImplicitTargets * MW) + (wv * MW + m) * 32 + r;
+    t_ok[m] = t[m] < num_targets;
+    t_safe[m] = t_ok[m] ? t[m] : num_targets - 1;
   }
 
-  // Every global load below is unconditional (addresses are clamped, the
-  // values of lanes without a source are replaced when they are used), so
-  // that the loads of later stages never have to be waited for early.
-  const long long t_safe = t_ok ? t : num_targets - 1;
-  auto load_index = [&](int o) -> int {
-    return kernel_map[static_cast<long long>(o < num_offsets ? o : num_offsets - 1) * num_targets + t_safe];
+  floatx16 acc[MW][NB];
+#pragma unroll
+  for (int m = 0; m < MW; ++m) {
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[m][b][j] = 0.0f;
+    }
+  }
+
+  // Every global load below is unconditional (addresses are clamped, lanes
+  // without a source use an out-of-range buffer offset), so that the loads of
+  // later stages never have to be waited for early.
+  auto load_index = [&](int o) -> Pieces2<MW> {
+    Pieces2<MW> set;
+    const long long row = static_cast<long long>(o < num_offsets ? o : num_offsets - 1) * num_targets;
+#pragma unroll
+    for (int m = 0; m < MW; ++m) set.v[m] = kernel_map[row + t_safe[m]];
+    return set;
   };
-  auto entry = [&](int value, int o) -> int { return (t_ok && o < num_offsets) ? value : -1; };
+  auto entry = [&](const Pieces2<MW> &set, int m, int o) -> int {
+    return (t_ok[m] && o < num_offsets) ? set.v[m] : -1;
+  };
   // piece i of this thread: 16 bytes of weight row (piece / kRowPieces) at
   // position (piece % kRowPieces); threads past the tile repeat its last piece
   auto load_w = [&](int o) -> Pieces<kWPieces> {
@@ -110,15 +172,19 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
   const __amdgpu_buffer_rsrc_t source_buffer = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<T *>(sources), 0, source_bytes, 0x00020000);
   const unsigned row_bytes = static_cast<unsigned>(K) * sizeof(T);
-  auto load_a = [&](int index) -> Pieces<KS> {
-    Pieces<KS> set;
+  auto load_a = [&](const Pieces2<MW> &indices, int o) -> Pieces<KS * MW> {
+    Pieces<KS * MW> set;
 #pragma unroll
-    for (int kk = 0; kk < kSteps; ++kk) {
-      const unsigned at = (kk * 2 + h) * 16u;
-      const unsigned offset =
-          (index >= 0 && at < row_bytes) ? static_cast<unsigned>(index) * row_bytes + at : kNoRow;
-      const uint4v v = __builtin_amdgcn_raw_buffer_load_b128(source_buffer, offset, 0, 0);
-      set.v[kk] = make_uint4(v.x, v.y, v.z, v.w);
+    for (int m = 0; m < MW; ++m) {
+      const int index = entry(indices, m, o);
+#pragma unroll
+      for (int kk = 0; kk < kSteps; ++kk) {
+        const unsigned at = (kk * 2 + h) * 16u;
+        const unsigned offset =
+            (index >= 0 && at < row_bytes) ? static_cast<unsigned>(index) * row_bytes + at : kNoRow;
+        const uint4v v = __builtin_amdgcn_raw_buffer_load_b128(source_buffer, offset, 0, 0);
+        set.v[m * KS + kk] = make_uint4(v.x, v.y, v.z, v.w);
+      }
     }
     return set;
   };
@@ -129,14 +195,14 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
   // is unrolled by six so that the roles of the register sets (three sets of
   // source rows, three of weights, six kernel-map entries) rotate without
   // copies: a register is never touched while its load is in flight.
-  int m0 = load_index(0), m1 = load_index(1), m2 = load_index(2), m3 = load_index(3),
-      m4 = load_index(4), m5 = 0;
-  Pieces<KS> a0, a1, a2;
+  Pieces2<MW> m0 = load_index(0), m1 = load_index(1), m2 = load_index(2), m3 = load_index(3),
+              m4 = load_index(4), m5 = m4;
+  Pieces<KS * MW> a0, a1, a2;
   Pieces<kWPieces> w0, w1, w2;
   w2 = load_w(0);
-  a0 = load_a(entry(m0, 0));
+  a0 = load_a(m0, 0);
   w0 = load_w(1);
-  a1 = load_a(entry(m1, 1));
+  a1 = load_a(m1, 1);
   w1 = load_w(2);
   store_w(0, w2);
   __syncthreads();
@@ -144,21 +210,29 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
   int o = 0;
   // offset o: multiply A_CUR (rows of M_CUR) by the weights in LDS buffer o & 1;
   // fetch rows of offset o+2 (entries M_A) into A_NEW, weights of offset o+3
-  // into W_NEW and the kernel-map entry of offset o+5 into M_NEW; put the
+  // into W_NEW and the kernel-map entries of offset o+5 into M_NEW; put the
   // weights of offset o+1 (W_STORE) into the other LDS buffer.
 #define MNT_STAGE(A_CUR, A_NEW, W_STORE, W_NEW, M_CUR, M_A, M_NEW)                                 \
   {                                                                                                \
     W_NEW = load_w(o + 3);                                                                         \
-    A_NEW = load_a(entry(M_A, o + 2));                                                             \
+    A_NEW = load_a(M_A, o + 2);                                                                    \
     M_NEW = load_index(o + 5);                                                                     \
-    if (__ballot(entry(M_CUR, o) >= 0) != 0ull) {                                                  \
+    bool live[MW];                                                                                 \
+    bool any = false;                                                                              \
+    _Pragma("unroll") for (int m = 0; m < MW; ++m) {                                               \
+      live[m] = __ballot(entry(M_CUR, m, o) >= 0) != 0ull;                                         \
+      any = any || live[m];                                                                        \
+    }                                                                                              \
+    if (any) {                                                                                     \
       const unsigned char *w_buf = w_lds + (o & 1) * kBufferBytes;                                 \
       _Pragma("unroll") for (int kk = 0; kk < kSteps; ++kk) {                                      \
         const int off = kk * 32 + h * 16;                                                          \
         _Pragma("unroll") for (int b = 0; b < NB; ++b) {                                           \
           const uint4 chan =                                                                       \
               *reinterpret_cast<const uint4 *>(w_buf + (b * 32 + r) * kLdsRowBytes + off);         \
-          acc[b] = Mfma<T>::run(chan, A_CUR.v[kk], acc[b]);                                        \
+          _Pragma("unroll") for (int m = 0; m < MW; ++m) {                                         \
+            if (MW == 1 || live[m]) acc[m][b] = Mfma<T>::run(chan, A_CUR.v[m * KS + kk], acc[m][b]); \
+          }                                                                                        \
         }                                                                                          \
       }                                                                                            \
     }                                                                                              \
@@ -176,48 +250,20 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
   }
 #undef MNT_STAGE
 
-  if (!t_ok) return;
-  typedef typename VecOf<4 * sizeof(T)>::type V;
-  unsigned char *dst = out + t * N * static_cast<long long>(sizeof(T));
 #pragma unroll
-  for (int b = 0; b < NB; ++b) {
+  for (int m = 0; m < MW; ++m) {
+    if (!t_ok[m]) continue;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int ch = b * 32 + q * 8 + h * 4;
-      if (ch >= N) continue;                 // N % 4 == 0: a group of four is all in or all out
-      float v[4];
+    for (int b = 0; b < NB; ++b) {
 #pragma unroll
-      for (int x = 0; x < 4; ++x) v[x] = acc[b][q * 4 + x];
-      if (ep.scale != nullptr) {
+      for (int q = 0; q < 4; ++q) {
+        const int ch = b * 32 + q * 8 + h * 4;
+        if (ch >= N) continue;               // N % 4 == 0: a group of four is all in or all out
+        float v[4];
 #pragma unroll
-        for (int x = 0; x < 4; ++x) v[x] *= ep.scale[ch + x];
+        for (int x = 0; x < 4; ++x) v[x] = acc[m][b][q * 4 + x];
+        finish_four<T>(v, ep, t[m], ch, N, out);
       }
-      if (ep.shift != nullptr) {
-#pragma unroll
-        for (int x = 0; x < 4; ++x) v[x] += ep.shift[ch + x];
-      }
-      if (ep.residual != nullptr) {
-        const V raw = *reinterpret_cast<const V *>(static_cast<const unsigned char *>(ep.residual) +
-                                                   (t * N + ch) * static_cast<long long>(sizeof(T)));
-        const T *e = reinterpret_cast<const T *>(&raw);
-#pragma unroll
-        for (int x = 0; x < 4; ++x) v[x] += to_float(e[x]);
-      }
-      if (ep.activation == MNT_ACT_RELU) {
-#pragma unroll
-        for (int x = 0; x < 4; ++x) v[x] = fmaxf(v[x], 0.0f);
-      } else if (ep.activation == MNT_ACT_LEAKY_RELU) {
-#pragma unroll
-        for (int x = 0; x < 4; ++x) v[x] = v[x] > 0.0f ? v[x] : v[x] * ep.slope;
-      } else if (ep.activation == MNT_ACT_RELU6) {
-#pragma unroll
-        for (int x = 0; x < 4; ++x) v[x] = fminf(fmaxf(v[x], 0.0f), 6.0f);
-      }
-      V raw;
-      T *e = reinterpret_cast<T *>(&raw);
-#pragma unroll
-      for (int x = 0; x < 4; ++x) e[x] = static_cast<T>(v[x]);
-      *reinterpret_cast<V *>(dst + ch * sizeof(T)) = raw;
     }
   }
 }
@@ -267,23 +313,35 @@ static void implicit_typed(const T *sources, const T *weights, const T *packed, 
   }
   const unsigned grid = static_cast<unsigned>(div_ceil(Tn, kImplicitTargets));
   const unsigned source_bytes = static_cast<unsigned>(S * K * sizeof(T));
-#define MNT_IMPLICIT(NB, KS)                                                                       \
-  implicit_forward_kernel<T, NB, KS><<<grid, kImplicitBlock, 0, stream>>>(                         \
+  // Two target blocks per wavefront where that measured faster: 16-bit
+  // features, 33..64 output channels, and enough targets to fill the chip that
+  // way.  (With one channel block the compiler's register allocation leaves
+  // too few wavefronts per SIMD; in fp32 the matrix work dominates anyway.)
+  const bool wide = sizeof(T) == 2 && Np == 64 && Tn >= kImplicitWideTargets;
+  const unsigned grid_wide = static_cast<unsigned>(div_ceil(Tn, kImplicitTargets * 2));
+#define MNT_IMPLICIT(NB, KS, MW, GRID)                                                             \
+  implicit_forward_kernel<T, NB, KS, MW><<<GRID, kImplicitBlock, 0, stream>>>(                     \
       sources, source_bytes, wt, kernel_map, Tn, static_cast<int>(O), static_cast<int>(K),         \
       static_cast<int>(N), reinterpret_cast<unsigned char *>(out), ep)
-#define MNT_IMPLICIT_NB(NB)               \
+#define MNT_IMPLICIT_KS(NB, MW, GRID)     \
   if (K * sizeof(T) <= 64) {              \
-    MNT_IMPLICIT(NB, 2);                  \
+    MNT_IMPLICIT(NB, 2, MW, GRID);        \
   } else {                                \
-    MNT_IMPLICIT(NB, 4);                  \
+    MNT_IMPLICIT(NB, 4, MW, GRID);        \
   }
   switch (Np / 32) {
-    case 1: MNT_IMPLICIT_NB(1); break;
-    case 2: MNT_IMPLICIT_NB(2); break;
-    case 3: MNT_IMPLICIT_NB(3); break;
-    default: MNT_IMPLICIT_NB(4); break;
+    case 1: MNT_IMPLICIT_KS(1, 1, grid); break;
+    case 2:
+      if (wide) {
+        MNT_IMPLICIT_KS(2, 2, grid_wide);
+      } else {
+        MNT_IMPLICIT_KS(2, 1, grid);
+      }
+      break;
+    case 3: MNT_IMPLICIT_KS(3, 1, grid); break;
+    default: MNT_IMPLICIT_KS(4, 1, grid); break;
   }
-#undef MNT_IMPLICIT_NB
+#undef MNT_IMPLICIT_KS
 #undef MNT_IMPLICIT
   check_launch("implicit_forward_kernel");
   profile_mark("implicit", stream);
