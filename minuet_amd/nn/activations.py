@@ -9,8 +9,7 @@ __all__ = ["ReLU", "ReLU6", "LeakyReLU"]
 
 def _on_features(base):
     def forward(self, x: SparseTensor) -> SparseTensor:
-        return SparseTensor(features=base.forward(self, x.F), coordinates=x.C, stride=x.stride,
-                            batch_dims=x.batch_dims)
+        return SparseTensor.like(x, base.forward(self, x.F))
     return forward
 
 

@@ -558,8 +558,9 @@ class SparseConv(Module):
                 features = self._forward_tables(cache, map_args, sources, epilogue)
         if self.bias is not None and epilogue is None:
             features += self.bias
-        return SparseTensor(features=features, coordinates=coordinates, stride=stride,
-                            batch_dims=batch_dims)
+        if batch_dims is not None and len(batch_dims) <= 2:
+            batch_dims = None
+        return SparseTensor.like(inputs, features, coordinates, stride, batch_dims)
 
     def _forward_tables(self, cache, map_args, sources, epilogue):
         """Gather -> GEMM -> Scatter through the rank tables (the reference's

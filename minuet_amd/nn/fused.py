@@ -78,8 +78,7 @@ def conv_norm_act(conv: SparseConv, norm: Optional[torch.nn.BatchNorm1d], act: O
 
 
 def _like(x: SparseTensor, features: torch.Tensor) -> SparseTensor:
-    return SparseTensor(features=features, coordinates=x.C, stride=x.stride,
-                        batch_dims=x.batch_dims)
+    return SparseTensor.like(x, features)
 
 
 class FusedSequential(nn.Sequential):

@@ -11,5 +11,4 @@ class BatchNorm(torch.nn.BatchNorm1d):
     """:class:`torch.nn.BatchNorm1d` over the ``[N, C]`` feature tensor."""
 
     def forward(self, x: SparseTensor) -> SparseTensor:
-        return SparseTensor(features=super().forward(x.F), coordinates=x.C, stride=x.stride,
-                            batch_dims=x.batch_dims)
+        return SparseTensor.like(x, super().forward(x.F))

@@ -42,6 +42,19 @@ class SparseTensor(object):
         self._stride = as_tuple(stride, size=self.ndim, name="strides")
         self._batch_dims = batch_dims if batch_dims is not None and len(batch_dims) > 2 else None
 
+    @classmethod
+    def like(cls, other: "SparseTensor", features: torch.Tensor, coordinates=None, stride=None,
+             batch_dims=None) -> "SparseTensor":
+        """New tensor that takes from ``other`` whatever is not given.  For the
+        layers of this package, whose outputs are consistent by construction:
+        nothing is validated again."""
+        new = cls.__new__(cls)
+        new._features = features
+        new._coordinates = other._coordinates if coordinates is None else coordinates
+        new._stride = other._stride if stride is None else stride
+        new._batch_dims = other._batch_dims if coordinates is None else batch_dims
+        return new
+
     # ---- shape-like properties -------------------------------------------
     @property
     def F(self) -> torch.Tensor:

@@ -16,7 +16,7 @@ __all__ = ["ResidualBlock", "SparseUNet"]
 
 
 def _with_features(x: SparseTensor, features: torch.Tensor) -> SparseTensor:
-    return SparseTensor(features=features, coordinates=x.C, stride=x.stride, batch_dims=x.batch_dims)
+    return SparseTensor.like(x, features)
 
 
 class ResidualBlock(nn.Module):
