@@ -259,19 +259,11 @@ __global__ __launch_bounds__(kQueryBlock) void count_tiles_kernel(
 }
 
 // One workgroup per row: exclusive scan of its tile counts in place and the
-// row total.  With `plan` the last workgroup to finish (self-resetting
-// ticket) also derives the row order: stable ascending by size (reorder) or
-// identity, its inverse, the sizes in row order and their exclusive prefix.
-// plan layout (unsigned): order[O] | position_of[O] | sorted_sizes[O] | prefix[O+1];
-// the first three blocks are mirrored into plan_host (pinned host memory).
+// row total.
 __global__ __launch_bounds__(256) void tile_scan_kernel(unsigned *__restrict__ tile_counts,
-                                                        int num_tiles, unsigned *row_sizes,
-                                                        int reorder, unsigned *__restrict__ plan,
-                                                        unsigned *__restrict__ plan_host,
-                                                        unsigned *ticket, unsigned long long *flag,
-                                                        unsigned long long sequence) {
+                                                        int num_tiles,
+                                                        unsigned *__restrict__ row_sizes) {
   __shared__ unsigned partial[256];
-  __shared__ bool s_last;
   unsigned *row = tile_counts + static_cast<long long>(blockIdx.x) * num_tiles;
   const int t = threadIdx.x;
   const int chunk = (num_tiles + 255) / 256;
@@ -293,28 +285,35 @@ __global__ __launch_bounds__(256) void tile_scan_kernel(unsigned *__restrict__ t
     row[i] = run;
     run += v;
   }
-  if (t == 255) {
-    __hip_atomic_store(&row_sizes[blockIdx.x], partial[255], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  if (plan == nullptr) return;
-  const int num_offsets = gridDim.x;
-  __threadfence();
-  __syncthreads();
-  if (t == 0) s_last = atomicInc(ticket, gridDim.x - 1) == gridDim.x - 1;
-  __syncthreads();
-  if (!s_last) return;
-  __threadfence();
+  if (t == 255) row_sizes[blockIdx.x] = partial[255];
+}
+
+// One workgroup, launched after tile_scan_kernel: the row order from the row
+// totals, stable ascending by size (reorder) or identity, its inverse, the
+// sizes in row order and their exclusive prefix.
+// plan layout (unsigned): order[O] | position_of[O] | sorted_sizes[O] | prefix[O+1];
+// the first three blocks are mirrored into plan_host (pinned host memory) and
+// the sequence flag tells the host that they are there.  (A separate launch
+// instead of a "last workgroup" ticket inside tile_scan_kernel: the
+// device-wide fence every workgroup would need costs more than the launch.)
+__global__ __launch_bounds__(256) void map_plan_kernel(const unsigned *__restrict__ row_sizes,
+                                                       int num_offsets, int reorder,
+                                                       unsigned *__restrict__ plan,
+                                                       unsigned *__restrict__ plan_host,
+                                                       unsigned long long *flag,
+                                                       unsigned long long sequence) {
+  const int t = threadIdx.x;
   unsigned *order = plan;
   unsigned *position_of = plan + num_offsets;
   unsigned *sorted_sizes = plan + 2 * num_offsets;
   unsigned *prefix = plan + 3 * num_offsets;
   for (int o = t; o < num_offsets; o += 256) {
-    const unsigned mine = __hip_atomic_load(&row_sizes[o], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned mine = row_sizes[o];
     int pos = o;
     if (reorder) {
       pos = 0;
       for (int p = 0; p < num_offsets; ++p) {
-        const unsigned other = __hip_atomic_load(&row_sizes[p], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned other = row_sizes[p];
         pos += (other < mine || (other == mine && p < o)) ? 1 : 0;
       }
     }
@@ -658,10 +657,12 @@ static void finish_sizes(Arena &arena, const MapState &state, unsigned *tile_cou
   unsigned *h_plan = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned()) + Arena::kPlanOffset);
   unsigned *d_plan_host = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned_device()) + Arena::kPlanOffset);
   const unsigned long long sequence = arena.next_sequence();
-  tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(
-      tile_counts, state.num_tiles, row_sizes, state.reorder, plan, d_plan_host, arena.tickets() + 1,
-      arena.flag_device(1), sequence);
+  tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, state.num_tiles,
+                                                                           row_sizes);
   check_launch("tile_scan_kernel");
+  map_plan_kernel<<<1, 256, 0, stream>>>(row_sizes, static_cast<int>(num_offsets), state.reorder, plan,
+                                         d_plan_host, arena.flag_device(1), sequence);
+  check_launch("map_plan_kernel");
   arena.wait_flag(1, sequence);
   profile_mark("map_sizes_order+sync", stream);
   for (int64_t j = 0; j < num_offsets; ++j) {
@@ -725,7 +726,7 @@ extern "C" int mnt_compute_kernel_map_sizes(const void *kernel_map, int64_t num_
     unsigned *tile_counts = scope.alloc<unsigned>(static_cast<size_t>(num_offsets) * num_tiles);
     unsigned *row_sizes = scope.alloc<unsigned>(num_offsets);
     enqueue_count_tiles(kernel_map, index_dtype, num_offsets, num_targets, tile_counts, num_tiles, stream);
-    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes, 0, nullptr, nullptr, nullptr, nullptr, 0);
+    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes);
     check_launch("tile_scan_kernel");
     const unsigned grid = grid_for(num_offsets, 256);
     if (index_dtype == MNT_INT32) {
@@ -754,7 +755,7 @@ extern "C" int mnt_compute_kernel_map_masks(const void *kernel_map, int64_t num_
     unsigned *row_sizes = scope.alloc<unsigned>(num_offsets);
     if (num_targets > 0) {
       enqueue_count_tiles(kernel_map, index_dtype, num_offsets, num_targets, tile_counts, num_tiles, stream);
-      tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes, 0, nullptr, nullptr, nullptr, nullptr, 0);
+      tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes);
       check_launch("tile_scan_kernel");
     }
     if (index_dtype == MNT_INT32) {
@@ -789,7 +790,7 @@ extern "C" int mnt_kernel_map_pair_lists(const int32_t *kernel_map, int64_t num_
     for (int64_t o = 0; o <= num_offsets; ++o) base[o] = static_cast<unsigned>(cumsum_host[o]);
     MNT_HIP(hipMemcpyAsync(row_base, base.data(), sizeof(unsigned) * (num_offsets + 1), hipMemcpyHostToDevice, stream));
     enqueue_count_tiles(kernel_map, MNT_INT32, num_offsets, num_targets, tile_counts, num_tiles, stream);
-    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes, 0, nullptr, nullptr, nullptr, nullptr, 0);
+    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes);
     check_launch("tile_scan_kernel");
     enqueue_emit<int32_t>(kernel_map, 0, num_targets, static_cast<int>(num_offsets), tile_counts,
                           num_tiles, nullptr, row_base, nullptr, nullptr, in_idx_out, out_idx_out, stream);

@@ -18,16 +18,18 @@ namespace mnt {
 constexpr int kBoundsBlock = 256;
 constexpr int kBoundsMaxBlocks = 256;
 
-// Per-dimension min / max of up to two coordinate arrays in ONE launch with no
-// pre-initialised memory: every workgroup publishes its partial result, the
-// last one to finish (self-resetting ticket) folds all partials and writes
-// the 16 results straight into pinned host memory:
+// Per-dimension min / max of up to two coordinate arrays with no pre-initialised
+// memory, in two launches: every workgroup of bounds_kernel writes its partial
+// result, bounds_fold_kernel (one workgroup) folds the partials and writes the
+// 16 results straight into pinned host memory:
 //   out[0..3] = min of a, out[4..7] = max of a, out[8..11] / out[12..15] = b.
+// (One launch with a "last workgroup folds" ticket was measured slower: the
+// device-wide fence each workgroup needs before it takes its ticket costs more
+// than the second launch.)
 template <typename CT>
 __global__ __launch_bounds__(kBoundsBlock) void bounds_kernel(
     const CT *__restrict__ a, long long na, int blocks_a, const CT *__restrict__ b, long long nb,
-    int ndim, long long *partial, unsigned *ticket, long long *out, unsigned long long *flag,
-    unsigned long long sequence) {
+    int ndim, long long *__restrict__ partial) {
   const bool second = static_cast<int>(blockIdx.x) >= blocks_a;
   const CT *coords = second ? b : a;
   const long long n = second ? nb : na;
@@ -39,18 +41,27 @@ __global__ __launch_bounds__(kBoundsBlock) void bounds_kernel(
     lo[k] = INT64_MAX;
     hi[k] = INT64_MIN;
   }
+  // four rows per thread and trip, all loaded before any is compared (rows past
+  // the end re-read the last row, which changes no extreme)
   const long long stride = static_cast<long long>(my_blocks) * kBoundsBlock;
-  for (long long i = static_cast<long long>(my_block) * kBoundsBlock + threadIdx.x; i < n; i += stride) {
-    long long c[MNT_MAX_NDIM];
-    load_row<CT>(coords + i * ndim, ndim, c);     // slots past ndim repeat coordinate 0
+  for (long long i0 = static_cast<long long>(my_block) * kBoundsBlock + threadIdx.x; i0 < n;
+       i0 += 4 * stride) {
+    long long c[4][MNT_MAX_NDIM];
 #pragma unroll
-    for (int k = 0; k < MNT_MAX_NDIM; ++k) {
-      lo[k] = c[k] < lo[k] ? c[k] : lo[k];
-      hi[k] = c[k] > hi[k] ? c[k] : hi[k];
+    for (int r = 0; r < 4; ++r) {
+      const long long i = i0 + r * stride;
+      load_row<CT>(coords + (i < n ? i : n - 1) * ndim, ndim, c[r]);   // slots past ndim repeat coordinate 0
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+#pragma unroll
+      for (int k = 0; k < MNT_MAX_NDIM; ++k) {
+        lo[k] = c[r][k] < lo[k] ? c[r][k] : lo[k];
+        hi[k] = c[r][k] > hi[k] ? c[r][k] : hi[k];
+      }
     }
   }
   __shared__ long long s_lo[kBoundsBlock / kWave][MNT_MAX_NDIM], s_hi[kBoundsBlock / kWave][MNT_MAX_NDIM];
-  __shared__ bool s_last;
 #pragma unroll
   for (int k = 0; k < MNT_MAX_NDIM; ++k) {
     for (int off = 32; off > 0; off >>= 1) {
@@ -77,28 +88,26 @@ __global__ __launch_bounds__(kBoundsBlock) void bounds_kernel(
       long long u = is_max ? s_hi[ww][k] : s_lo[ww][k];
       v = is_max ? (u > v ? u : v) : (u < v ? u : v);
     }
-    __hip_atomic_store(&partial[static_cast<long long>(blockIdx.x) * 8 + threadIdx.x], v,
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    partial[static_cast<long long>(blockIdx.x) * 8 + threadIdx.x] = v;
   }
-  __threadfence();
-  __syncthreads();
-  if (threadIdx.x == 0) s_last = atomicInc(ticket, gridDim.x - 1) == gridDim.x - 1;
-  __syncthreads();
-  if (!s_last) return;
-  __threadfence();
-  // fold the partials: thread t takes workgroups t, t+256, ... of each array
+}
+
+__global__ __launch_bounds__(kBoundsBlock) void bounds_fold_kernel(
+    const long long *__restrict__ partial, int num_partials, int blocks_a, long long *out,
+    unsigned long long *flag, unsigned long long sequence) {
+  const int w = threadIdx.x >> 6;
+  // thread t takes the partials of workgroups t, t+256, ... of each array
   long long fa[8], fb[8];
 #pragma unroll
   for (int slot = 0; slot < 8; ++slot) {
     fa[slot] = slot >= MNT_MAX_NDIM ? INT64_MIN : INT64_MAX;
     fb[slot] = fa[slot];
   }
-  for (int blk = threadIdx.x; blk < static_cast<int>(gridDim.x); blk += kBoundsBlock) {
+  for (int blk = threadIdx.x; blk < num_partials; blk += kBoundsBlock) {
     const bool of_b = blk >= blocks_a;
 #pragma unroll
     for (int slot = 0; slot < 8; ++slot) {
-      const long long u = __hip_atomic_load(&partial[static_cast<long long>(blk) * 8 + slot],
-                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const long long u = partial[static_cast<long long>(blk) * 8 + slot];
       long long &dst = of_b ? fb[slot] : fa[slot];
       dst = slot >= MNT_MAX_NDIM ? (u > dst ? u : dst) : (u < dst ? u : dst);
     }
@@ -150,7 +159,6 @@ void read_bounds(const void *a, int64_t na, const void *b, int64_t nb, int ndim,
   const int blocks_b = nb > 0 ? static_cast<int>(std::min<int64_t>(div_ceil(nb, kBoundsBlock * 4), kBoundsMaxBlocks)) : 0;
   const int grid = blocks_a + blocks_b;
   long long *partial = scope.alloc<long long>(static_cast<size_t>(grid) * 8);
-  unsigned *ticket = scope.arena().tickets();
   long long *h_out = static_cast<long long *>(scope.arena().pinned());
   long long *d_out = static_cast<long long *>(scope.arena().pinned_device());
   const unsigned long long sequence = scope.arena().next_sequence();
@@ -158,13 +166,15 @@ void read_bounds(const void *a, int64_t na, const void *b, int64_t nb, int ndim,
   if (coord_dtype == MNT_INT32) {
     bounds_kernel<int32_t><<<grid, kBoundsBlock, 0, stream>>>(
         static_cast<const int32_t *>(a), na, blocks_a, static_cast<const int32_t *>(b), nb, ndim,
-        partial, ticket, d_out, flag, sequence);
+        partial);
   } else {
     bounds_kernel<int64_t><<<grid, kBoundsBlock, 0, stream>>>(
         static_cast<const int64_t *>(a), na, blocks_a, static_cast<const int64_t *>(b), nb, ndim,
-        partial, ticket, d_out, flag, sequence);
+        partial);
   }
   check_launch("bounds_kernel");
+  bounds_fold_kernel<<<1, kBoundsBlock, 0, stream>>>(partial, grid, blocks_a, d_out, flag, sequence);
+  check_launch("bounds_fold_kernel");
   scope.arena().wait_flag(0, sequence);
   if (na > 0) memcpy(out, h_out, sizeof(long long) * 8);
   if (nb > 0) memcpy(out + 8, h_out + 8, sizeof(long long) * 8);

@@ -342,6 +342,9 @@ __global__ __launch_bounds__(kScanBlock) void bitmap_emit_kernel(
     const unsigned *__restrict__ bitmap, long long words, const unsigned *__restrict__ tile_bases,
     int tiles, TargetSpec spec, CT *__restrict__ out, IT *__restrict__ batch_dims_out) {
   const long long base = static_cast<long long>(blockIdx.x) * kBitmapTile + threadIdx.x * kBitmapWords;
+  // a tile without a set bit has nothing to write, unless a batch boundary
+  // falls into it (then it is read like any other)
+  if (batch_dims_out == nullptr && tile_bases[blockIdx.x] == tile_bases[blockIdx.x + 1]) return;
   unsigned word[kBitmapWords];
   unsigned count = 0;
 #pragma unroll

@@ -456,6 +456,14 @@ def kernel_map_build(sources: torch.Tensor, targets: torch.Tensor, offsets_host:
     tb = None if target_bounds is None else np.ascontiguousarray(target_bounds, dtype=np.int64)
     lib = load_library()
     result = {}
+    # everything whose size is known goes before the query: the host then has
+    # less to do between the wait for the sizes and the second launch
+    smask = tmask = in_idx = out_idx = None
+    if want_masks:
+        smask = torch.empty((num_offsets, num_sources), dtype=torch.int32, device=device)
+        tmask = torch.empty((num_offsets, num_targets), dtype=torch.int32, device=device)
+    sizes_dev = torch.empty((num_offsets,), dtype=torch.int32, device=device)
+    order_dev = torch.empty((num_offsets,), dtype=torch.int32, device=device)
     with _on(device):
         stream = _stream(device)
         _check(lib.mnt_kernel_map_query(
@@ -468,16 +476,10 @@ def kernel_map_build(sources: torch.Tensor, targets: torch.Tensor, offsets_host:
             None if tb is None else tb.ctypes.data_as(_pi64), bounds.ctypes.data_as(_pi64),
             _ptr(dense), sizes_host.ctypes.data_as(_pi64), order_host.ctypes.data_as(_pi64),
             stream))
-        smask = tmask = in_idx = out_idx = None
-        if want_masks:
-            smask = torch.empty((num_offsets, num_sources), dtype=torch.int32, device=device)
-            tmask = torch.empty((num_offsets, num_targets), dtype=torch.int32, device=device)
         if want_lists:
             nnz = int(sizes_host.sum())
-            in_idx = torch.empty((nnz,), dtype=torch.int32, device=device)
-            out_idx = torch.empty((nnz,), dtype=torch.int32, device=device)
-        sizes_dev = torch.empty((num_offsets,), dtype=torch.int32, device=device)
-        order_dev = torch.empty((num_offsets,), dtype=torch.int32, device=device)
+            both = torch.empty((2, nnz), dtype=torch.int32, device=device)
+            in_idx, out_idx = both[0], both[1]
         _check(lib.mnt_kernel_map_emit(_ptr(smask), _ptr(tmask), _ptr(in_idx), _ptr(out_idx),
                                        _ptr(sizes_dev), _ptr(order_dev), stream))
     result.update(sizes_host=sizes_host, order_host=order_host, sizes=sizes_dev, order=order_dev,
