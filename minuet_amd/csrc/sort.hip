@@ -409,6 +409,19 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
 
   const long long base =
       static_cast<long long>(blockIdx.x) * (kSortBlock * ITEMS) + w * (kWave * ITEMS);
+  // thread t owns the contiguous digits [t*per, (t+1)*per) when the digit
+  // bases are formed below; their totals and this tile's offsets are fetched
+  // now, so that the loads overlap the ranking of the keys
+  constexpr int kMaxPer = kMaxRadix / kSortBlock;
+  const int per = (radix + kSortBlock - 1) / kSortBlock;
+  unsigned digit_total[kMaxPer], digit_offset[kMaxPer];
+#pragma unroll
+  for (int j = 0; j < kMaxPer; ++j) {
+    const int d = tid * per + j;
+    const bool mine = j < per && d < radix;
+    digit_total[j] = mine ? totals[d] : 0u;
+    digit_offset[j] = mine ? offsets[static_cast<long long>(d) * num_tiles + blockIdx.x] : 0u;
+  }
   unsigned long long key[ITEMS];
   unsigned val[ITEMS];
   unsigned rank[ITEMS];
@@ -420,6 +433,11 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     key[r] = ~0ull;
     val[r] = 0u;
     if (valid) src.load(i, key[r], val[r]);
+  }
+#pragma unroll
+  for (int r = 0; r < ITEMS; ++r) {
+    const long long i = base + r * kWave + lane;
+    const bool valid = i < n;
     const unsigned d = static_cast<unsigned>(key[r] >> shift) & (radix - 1);
     unsigned long long peers = __ballot(valid);
 #pragma unroll
@@ -437,14 +455,10 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
     if (valid && below == 0) cnt[w][d] = prev + __popcll(peers);
     __builtin_amdgcn_wave_barrier();
   }
-  // digit bases: exclusive scan of the digit totals; thread t owns the
-  // contiguous digits [t*per, (t+1)*per)
-  const int per = (radix + kSortBlock - 1) / kSortBlock;
+  // digit bases: exclusive scan of the digit totals
   unsigned local_total = 0;
-  for (int j = 0; j < per; ++j) {
-    const int d = tid * per + j;
-    if (d < radix) local_total += totals[d];
-  }
+#pragma unroll
+  for (int j = 0; j < kMaxPer; ++j) local_total += digit_total[j];
   unsigned inc = local_total;
   for (int off = 1; off < kWave; off <<= 1) {
     unsigned u = __shfl_up(inc, off);
@@ -455,18 +469,18 @@ __global__ __launch_bounds__(kSortBlock) void radix_scatter_kernel(
   {
     unsigned run = inc - local_total;
     for (int ww = 0; ww < w; ++ww) run += scan_sums[ww];
-    for (int j = 0; j < per; ++j) {
+#pragma unroll
+    for (int j = 0; j < kMaxPer; ++j) {
       const int d = tid * per + j;
-      if (d < radix) {
-        const unsigned total_d = totals[d];
-        unsigned at = run + offsets[static_cast<long long>(d) * num_tiles + blockIdx.x];
+      if (j < per && d < radix) {
+        unsigned at = run + digit_offset[j];
 #pragma unroll
         for (int ww = 0; ww < kSortWaves; ++ww) {
           const unsigned c = cnt[ww][d];
           cnt[ww][d] = at;
           at += c;
         }
-        run += total_d;
+        run += digit_total[j];
       }
     }
   }
