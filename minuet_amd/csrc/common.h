@@ -91,10 +91,6 @@ class Arena {
   void *pinned();
   // Device-side address of the same block (kernels may write results there).
   void *pinned_device();
-  // 16 zero-initialised device counters for "last workgroup" tickets; every
-  // kernel that uses one leaves it at zero again.
-  unsigned *tickets();
-
   // Completion handshake through the pinned block: a kernel ends by storing a
   // fresh sequence number into flag word `slot` (after its results, with a
   // system-scope release); wait_flag spins on that word on the host, which
@@ -142,7 +138,6 @@ class Arena {
   float growth_ = 1.0f;
   void *pinned_ = nullptr;
   void *pinned_device_ = nullptr;
-  unsigned *tickets_ = nullptr;
   unsigned long long sequence_ = 0;
   void *persistent_[2] = {nullptr, nullptr};
   size_t persistent_size_[2] = {0, 0};

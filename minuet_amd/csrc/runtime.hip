@@ -139,14 +139,6 @@ void Arena::wait_flag(int slot, unsigned long long sequence) {
   std::atomic_thread_fence(std::memory_order_acquire);
 }
 
-unsigned *Arena::tickets() {
-  if (!tickets_) {
-    MNT_HIP(hipMalloc(reinterpret_cast<void **>(&tickets_), 16 * sizeof(unsigned)));
-    MNT_HIP(hipMemset(tickets_, 0, 16 * sizeof(unsigned)));
-  }
-  return tickets_;
-}
-
 void *Arena::persistent(int slot, size_t bytes) {
   if (bytes > persistent_size_[slot]) {
     if (persistent_[slot]) {
