@@ -94,8 +94,10 @@ __global__ __launch_bounds__(kBoundsBlock) void bounds_kernel(
 
 __global__ __launch_bounds__(kBoundsBlock) void bounds_fold_kernel(
     const long long *__restrict__ partial, int num_partials, int blocks_a, long long *out,
+    long long *__restrict__ device_copy, unsigned *__restrict__ zero, int zero_count,
     unsigned long long *flag, unsigned long long sequence) {
   const int w = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < zero_count; i += kBoundsBlock) zero[i] = 0u;
   // thread t takes the partials of workgroups t, t+256, ... of each array
   long long fa[8], fb[8];
 #pragma unroll
@@ -143,6 +145,7 @@ __global__ __launch_bounds__(kBoundsBlock) void bounds_fold_kernel(
       v = is_max ? (u > v ? u : v) : (u < v ? u : v);
     }
     out[threadIdx.x] = v;
+    if (device_copy != nullptr) device_copy[threadIdx.x] = v;
   }
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -152,7 +155,7 @@ __global__ __launch_bounds__(kBoundsBlock) void bounds_fold_kernel(
 }
 
 void read_bounds(const void *a, int64_t na, const void *b, int64_t nb, int ndim, int coord_dtype,
-                 long long out[16], Scope &scope, hipStream_t stream) {
+                 long long out[16], Scope &scope, hipStream_t stream, const BoundsExtras *extras) {
   for (int i = 0; i < 16; ++i) out[i] = (i & 4) ? INT64_MIN : INT64_MAX;
   if (na <= 0 && nb <= 0) return;
   const int blocks_a = na > 0 ? static_cast<int>(std::min<int64_t>(div_ceil(na, kBoundsBlock * 4), kBoundsMaxBlocks)) : 0;
@@ -173,8 +176,11 @@ void read_bounds(const void *a, int64_t na, const void *b, int64_t nb, int ndim,
         partial);
   }
   check_launch("bounds_kernel");
-  bounds_fold_kernel<<<1, kBoundsBlock, 0, stream>>>(partial, grid, blocks_a, d_out, flag, sequence);
+  bounds_fold_kernel<<<1, kBoundsBlock, 0, stream>>>(
+      partial, grid, blocks_a, d_out, extras ? extras->device_copy : nullptr,
+      extras ? extras->zero : nullptr, extras ? extras->zero_count : 0, flag, sequence);
   check_launch("bounds_fold_kernel");
+  if (extras && extras->enqueue) extras->enqueue();
   scope.arena().wait_flag(0, sequence);
   if (na > 0) memcpy(out, h_out, sizeof(long long) * 8);
   if (nb > 0) memcpy(out + 8, h_out + 8, sizeof(long long) * 8);
@@ -557,6 +563,367 @@ void radix_sort_pairs(unsigned long long *&keys, unsigned *&vals, unsigned long 
   }
 }
 
+// ----------------------------------------------------------- bucket sort ----
+//
+// Sort of a cloud whose rows fit one 64-bit key: the rows are dealt into
+// buckets by the top bits of their key (about 128 rows per bucket), then every
+// bucket is ranked in LDS: a workgroup stages the whole bucket and its
+// threads count the words below their own; a large bucket is shared by
+// several workgroups.  A bucketed row is kept as
+// ((rest of the key) << idx_bits) | row, which is unique, so ranks are unique
+// and the order inside a bucket needs no stability from the dealing step:
+// cursors handed out by atomics will do.
+//
+// The bucket histogram, its scan and the dealing step are enqueued behind the
+// bounds kernels, before the host waits for the bounds; the kernels work out
+// the key layout from the bounds in device memory.  The host then learns the
+// bounds, the largest bucket and the number of ranking workgroups at once and
+// launches the ranking while the dealing step still runs.  A cloud with a
+// bucket beyond the LDS capacity (strong clustering) takes the radix passes
+// instead; the dealing step sees that for itself and does nothing.
+
+constexpr int kBucketMaxBits = 12;
+constexpr int kBucketMax = 1 << kBucketMaxBits;
+constexpr int kBucketCap = 8064;              // rows of the largest bucket: 64 KiB of LDS with padding
+constexpr int kBucketItems = 4;               // rows per thread when dealing
+constexpr int kBucketRows = 128;              // rows per bucket aimed at
+constexpr int64_t kBucketMinN = 2048;
+constexpr size_t kBucketHostOffset = 384;     // pinned block: largest bucket
+
+// Key layout of a sort that takes one round: fields from least to most
+// significant are dimensions ndim-1 .. 0, then the batch id.  bounds = lo[4],
+// hi[4].  Returns the key width; above 64 the spec is unusable.
+__host__ __device__ inline int single_round_spec(const long long *bounds, int ndim,
+                                                 int num_batches, SortSpec &spec) {
+  int bits = 0;
+#pragma unroll
+  for (int k = MNT_MAX_NDIM - 1; k >= 0; --k) {
+    spec.lo[k] = 0;
+    spec.mask[k] = 0;
+    spec.shift[k] = 0;
+    if (k < ndim) {
+      const unsigned long long range = static_cast<unsigned long long>(bounds[MNT_MAX_NDIM + k]) -
+                                       static_cast<unsigned long long>(bounds[k]);
+      const int w = range == 0 ? 0 : 64 - __builtin_clzll(range);
+      if (w > 0) {
+        spec.lo[k] = static_cast<unsigned long long>(bounds[k]);
+        spec.mask[k] = w >= 64 ? ~0ull : ((1ull << w) - 1ull);
+        spec.shift[k] = bits & 63;
+        bits += w;
+      }
+    }
+  }
+  spec.lo[MNT_MAX_NDIM] = 0;
+  spec.mask[MNT_MAX_NDIM] = 0;
+  spec.shift[MNT_MAX_NDIM] = 0;
+  if (num_batches > 1) {
+    const int w = 64 - __builtin_clzll(static_cast<unsigned long long>(num_batches - 1));
+    spec.mask[MNT_MAX_NDIM] = (1ull << w) - 1ull;
+    spec.shift[MNT_MAX_NDIM] = bits & 63;
+    bits += w;
+  }
+  spec.ndim = ndim;
+  spec.num_batches = num_batches;
+  return bits;
+}
+
+struct BucketLayout {
+  int msd_bits;     // key bits that select the bucket
+  int shift;        // key >> shift = bucket
+  int idx_bits;     // width of a row index
+  bool ok;          // one key holds a row and one word holds (rest, row)
+};
+
+__host__ __device__ inline BucketLayout bucket_layout(int bits, int msd_cap, int idx_bits) {
+  BucketLayout l;
+  l.msd_bits = bits < msd_cap ? bits : msd_cap;
+  l.shift = bits - l.msd_bits;
+  l.idx_bits = idx_bits;
+  l.ok = bits >= 1 && bits <= 64 && l.shift + idx_bits <= 64;
+  return l;
+}
+
+// Key layout from the bounds in device memory.
+template <typename CT, typename IT>
+__device__ __forceinline__ BucketLayout layout_on_device(
+    const CT *__restrict__ coords, const IT *__restrict__ batch_dims, int num_batches, int ndim,
+    const long long *__restrict__ bounds, int msd_cap, int idx_bits, CoordSource<CT, IT> &src) {
+  long long b[2 * MNT_MAX_NDIM];
+#pragma unroll
+  for (int i = 0; i < 2 * MNT_MAX_NDIM; ++i) b[i] = bounds[i];
+  src.coords = coords;
+  src.batch_dims = batch_dims;
+  src.perm = nullptr;
+  const int bits = single_round_spec(b, ndim, num_batches, src.spec);
+  return bucket_layout(bits, msd_cap, idx_bits);
+}
+
+// Rows per bucket; info[0] tells the scan kernel whether the layout holds.
+template <typename CT, typename IT>
+__global__ __launch_bounds__(kSortBlock) void bucket_hist_kernel(
+    const CT *__restrict__ coords, const IT *__restrict__ batch_dims, int num_batches, int ndim,
+    long long n, const long long *__restrict__ bounds, int msd_cap, int idx_bits,
+    unsigned *__restrict__ totals, unsigned *__restrict__ info) {
+  __shared__ unsigned hist[kBucketMax];
+  CoordSource<CT, IT> src;
+  const BucketLayout lay =
+      layout_on_device<CT, IT>(coords, batch_dims, num_batches, ndim, bounds, msd_cap, idx_bits, src);
+  if (blockIdx.x == 0 && threadIdx.x == 0) info[0] = lay.ok ? 1u : 0u;
+  if (!lay.ok) return;
+  const int buckets = 1 << lay.msd_bits;
+  for (int d = threadIdx.x; d < buckets; d += kSortBlock) hist[d] = 0;
+  __syncthreads();
+  const long long base = static_cast<long long>(blockIdx.x) * (kSortBlock * kBucketItems);
+  unsigned long long key[kBucketItems];
+#pragma unroll
+  for (int r = 0; r < kBucketItems; ++r) {
+    const long long i = base + r * kSortBlock + threadIdx.x;
+    unsigned val;
+    key[r] = 0;
+    if (i < n) src.load(i, key[r], val);
+  }
+#pragma unroll
+  for (int r = 0; r < kBucketItems; ++r) {
+    const long long i = base + r * kSortBlock + threadIdx.x;
+    if (i < n) atomicAdd(&hist[static_cast<unsigned>(key[r] >> lay.shift)], 1u);
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < buckets; d += kSortBlock) {
+    const unsigned c = hist[d];
+    if (c != 0) atomicAdd(&totals[d], c);
+  }
+}
+
+// How many threads share the ranking of one row of a bucket of m rows (as a
+// power of two): small buckets spread a row over 2 or 4 threads so that no
+// lane idles, large ones over 4 to 32 so that no thread scans more than about
+// 256 words.  A workgroup then takes 256 >> split rows.
+__device__ __forceinline__ unsigned bucket_split_log2(unsigned m) {
+  return m <= 64 ? 2u : m <= 128 ? 1u : m <= 256 ? 0u : m <= 1024 ? 2u : m <= 4096 ? 4u : 5u;
+}
+
+__device__ __forceinline__ uint2 bucket_chunk_entry(unsigned first_row, unsigned rows, unsigned chunk) {
+  return make_uint2(first_row, rows | (bucket_split_log2(rows) << 13) | (chunk << 16));
+}
+
+// One workgroup: bucket starts (exclusive scan of the totals, starts[buckets]
+// = n), cleared cursors, the list of (bucket, chunk of rows) pairs the
+// ranking kernel runs over, info[1] = whether the bucket sort goes ahead, and
+// for the host the largest bucket (all ones when the layout does not hold)
+// and the number of pairs.
+// chunks[i] = {first row of the bucket, rows of the bucket | split << 13 |
+// chunk << 16}.
+__global__ __launch_bounds__(1024) void bucket_scan_kernel(
+    const unsigned *__restrict__ totals, int buckets, unsigned *__restrict__ info,
+    unsigned *__restrict__ starts, unsigned *__restrict__ cursors, uint2 *__restrict__ chunks,
+    unsigned *host_out, unsigned long long *flag, unsigned long long sequence) {
+  constexpr int kPer = kBucketMax / 1024;
+  constexpr unsigned kShared = 1024;          // buckets of several chunks listed by whole wavefronts
+  __shared__ unsigned long long wave_both[1024 / kWave];
+  __shared__ unsigned s_max, s_shared;
+  __shared__ unsigned shared_first[kShared], shared_rows[kShared], shared_at[kShared];
+  const int t = threadIdx.x;
+  if (t == 0) {
+    s_max = 0;
+    s_shared = 0;
+  }
+  unsigned v[kPer];
+  unsigned sum = 0, biggest = 0, pieces = 0;
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int d = t * kPer + j;
+    v[j] = d < buckets ? totals[d] : 0u;
+    sum += v[j];
+    biggest = v[j] > biggest ? v[j] : biggest;
+    const unsigned rows = kSortBlock >> bucket_split_log2(v[j]);
+    pieces += v[j] <= kBucketCap ? (v[j] + rows - 1) / rows : 0u;
+  }
+  // both scans in one sweep: rows in the low half, chunks in the high half
+  // (fewer than 2^31 rows, so the low half never carries into the high one)
+  const unsigned long long mine_both =
+      static_cast<unsigned long long>(sum) | (static_cast<unsigned long long>(pieces) << 32);
+  unsigned long long inclusive = mine_both;
+  for (int off = 1; off < kWave; off <<= 1) {
+    const unsigned long long u = __shfl_up(inclusive, off);
+    if (static_cast<int>(lane_id()) >= off) inclusive += u;
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned u = __shfl_down(biggest, off);
+    biggest = u > biggest ? u : biggest;
+  }
+  if (lane_id() == kWave - 1) wave_both[t >> 6] = inclusive;
+  __syncthreads();                            // also orders the clearing of s_max and s_shared
+  if (lane_id() == 0 && biggest != 0) atomicMax(&s_max, biggest);
+  unsigned long long before = 0, all_both = 0;
+#pragma unroll
+  for (int w = 0; w < 1024 / kWave; ++w) {
+    const unsigned long long x = wave_both[w];
+    before += w < (t >> 6) ? x : 0ull;
+    all_both += x;
+  }
+  const unsigned long long exclusive = before + inclusive - mine_both;
+  unsigned run = static_cast<unsigned>(exclusive);
+  unsigned piece = static_cast<unsigned>(exclusive >> 32);
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int d = t * kPer + j;
+    if (d < buckets) {
+      starts[d] = run;
+      cursors[d] = 0u;
+      if (v[j] != 0 && v[j] <= kBucketCap) {
+        const unsigned rows = kSortBlock >> bucket_split_log2(v[j]);
+        const unsigned mine = (v[j] + rows - 1) / rows;
+        const unsigned slot = mine == 1 ? kShared : atomicAdd(&s_shared, 1u);
+        if (mine == 1) {
+          chunks[piece] = bucket_chunk_entry(run, v[j], 0);
+        } else if (slot < kShared) {
+          shared_first[slot] = run;
+          shared_rows[slot] = v[j];
+          shared_at[slot] = piece;
+        } else {
+          for (unsigned c = 0; c < mine; ++c) chunks[piece + c] = bucket_chunk_entry(run, v[j], c);
+        }
+        piece += mine;
+      }
+    }
+    run += v[j];
+  }
+  if (t == 1023) starts[buckets] = static_cast<unsigned>(all_both);
+  __syncthreads();
+  const unsigned listed = s_shared < kShared ? s_shared : kShared;
+  for (unsigned h = t >> 6; h < listed; h += 1024 / kWave) {
+    const unsigned rows = kSortBlock >> bucket_split_log2(shared_rows[h]);
+    const unsigned mine = (shared_rows[h] + rows - 1) / rows;
+    for (unsigned c = t & (kWave - 1); c < mine; c += kWave) {
+      chunks[shared_at[h] + c] = bucket_chunk_entry(shared_first[h], shared_rows[h], c);
+    }
+  }
+  if (t == 0) {
+    const bool go = info[0] != 0 && s_max <= kBucketCap;
+    info[1] = go ? 1u : 0u;
+    host_out[0] = info[0] != 0 ? s_max : 0xffffffffu;
+    host_out[1] = static_cast<unsigned>(all_both >> 32);
+    __threadfence_system();
+    __hip_atomic_store(flag, sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+}
+
+// Deals the rows of one tile into their buckets as (rest of key, row) words;
+// nothing to do when the scan kernel called the bucket sort off (info[1]).
+template <typename CT, typename IT>
+__global__ __launch_bounds__(kSortBlock) void bucket_deal_kernel(
+    const CT *__restrict__ coords, const IT *__restrict__ batch_dims, int num_batches, int ndim,
+    long long n, const long long *__restrict__ bounds, int msd_cap, int idx_bits_,
+    const unsigned *__restrict__ info, const unsigned *__restrict__ starts,
+    unsigned *__restrict__ cursors, unsigned long long *__restrict__ words) {
+  __shared__ unsigned hist[kBucketMax];
+  if (info[1] == 0) return;
+  CoordSource<CT, IT> src;
+  const BucketLayout lay =
+      layout_on_device<CT, IT>(coords, batch_dims, num_batches, ndim, bounds, msd_cap, idx_bits_, src);
+  const int shift = lay.shift, idx_bits = lay.idx_bits;
+  const int buckets = 1 << lay.msd_bits;
+  const int tid = threadIdx.x;
+  for (int d = tid; d < buckets; d += kSortBlock) hist[d] = 0;
+  __syncthreads();
+  const long long base = static_cast<long long>(blockIdx.x) * (kSortBlock * kBucketItems);
+  const unsigned long long rest_mask = (1ull << shift) - 1ull;
+  unsigned long long key[kBucketItems];
+  unsigned row[kBucketItems], place[kBucketItems];
+#pragma unroll
+  for (int r = 0; r < kBucketItems; ++r) {
+    const long long i = base + r * kSortBlock + tid;
+    key[r] = 0;
+    row[r] = 0;
+    if (i < n) src.load(i, key[r], row[r]);
+  }
+#pragma unroll
+  for (int r = 0; r < kBucketItems; ++r) {
+    const long long i = base + r * kSortBlock + tid;
+    place[r] = 0;
+    if (i < n) place[r] = atomicAdd(&hist[static_cast<unsigned>(key[r] >> shift)], 1u);
+  }
+  __syncthreads();
+  // a range of every bucket this tile has rows for: counts fetched first, then
+  // all cursor updates in flight together
+  constexpr int kPer = kBucketMax / kSortBlock;
+  unsigned count[kPer], first[kPer], got[kPer];
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int d = j * kSortBlock + tid;
+    count[j] = d < buckets ? hist[d] : 0u;
+  }
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int d = j * kSortBlock + tid;
+    first[j] = 0;
+    got[j] = 0;
+    if (count[j] != 0) {
+      first[j] = starts[d];
+      got[j] = atomicAdd(&cursors[d], count[j]);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int d = j * kSortBlock + tid;
+    if (count[j] != 0) hist[d] = first[j] + got[j];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < kBucketItems; ++r) {
+    const long long i = base + r * kSortBlock + tid;
+    if (i < n) {
+      const unsigned pos = hist[static_cast<unsigned>(key[r] >> shift)] + place[r];
+      words[pos] = ((key[r] & rest_mask) << idx_bits) | static_cast<unsigned long long>(row[r]);
+    }
+  }
+}
+
+// One workgroup per (bucket, chunk of rows): stages the whole bucket in LDS,
+// then 1 << split threads per row count the words below that row's word, each
+// over an interleaved share of the bucket; the sum is the row's place in the
+// bucket, and the row is written to its final place.
+template <typename CT, typename IT>
+__global__ __launch_bounds__(kSortBlock) void bucket_rank_kernel(
+    const unsigned long long *__restrict__ words, const uint2 *__restrict__ chunks, int idx_bits,
+    FinalSink<CT, IT> sink) {
+  extern __shared__ __align__(16) unsigned long long s_words[];
+  const unsigned tid = threadIdx.x;
+  const uint2 entry = chunks[blockIdx.x];
+  const unsigned start = entry.x;
+  const unsigned m = entry.y & 0x1fffu;
+  const unsigned split = (entry.y >> 13) & 7u;
+  const unsigned chunk = entry.y >> 16;
+  // words are read four at a time by each of the 1 << split sharers
+  const unsigned group = 4u << split;
+  const unsigned padded = (m + group - 1u) / group * group;
+  for (unsigned i = tid; i < padded; i += kSortBlock) s_words[i] = i < m ? words[start + i] : ~0ull;
+  __syncthreads();
+  const unsigned part = tid & ((1u << split) - 1u);
+  const unsigned e = chunk * (kSortBlock >> split) + (tid >> split);
+  const unsigned long long mine = e < m ? s_words[e] : 0ull;
+  unsigned rank = 0;
+  for (unsigned j = 4u * part; j < padded; j += group) {
+    const unsigned long long a = s_words[j], b = s_words[j + 1], c = s_words[j + 2], d = s_words[j + 3];
+    rank += (a < mine ? 1u : 0u) + (b < mine ? 1u : 0u) + (c < mine ? 1u : 0u) + (d < mine ? 1u : 0u);
+  }
+  // the sharers of a row sit in neighbouring lanes
+  for (unsigned off = 1; off < (1u << split); off <<= 1) rank += __shfl_xor(rank, off);
+  const unsigned long long idx_mask = (1ull << idx_bits) - 1ull;
+  if (e < m && part == 0) sink.store(start + rank, 0ull, static_cast<unsigned>(mine & idx_mask));
+}
+
+// Largest cloud the bucket sort takes (MINUET_BUCKET_SORT_MAX_ROWS overrides;
+// 0 switches it off).
+static int64_t bucket_sort_max_rows() {
+  static const int64_t value = [] {
+    const char *text = getenv("MINUET_BUCKET_SORT_MAX_ROWS");
+    if (text != nullptr && *text != 0) return static_cast<int64_t>(atoll(text));
+    return static_cast<int64_t>(1) << 19;
+  }();
+  return value;
+}
+
 // --------------------------------------------------------------- outputs ----
 
 // Identity / gather emit for the cases without any radix pass.
@@ -590,7 +957,50 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
 
   profile_mark("enter:arg_sort", stream);
   long long h_bounds[16];
-  read_bounds(coords, n, nullptr, 0, ndim, sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64, h_bounds, scope, stream);
+  // bucket sort, first half: histogram and scan enqueued behind the bounds
+  const int batches_in_key = batched ? static_cast<int>(num_batches) : 1;
+  const bool try_buckets = n >= kBucketMinN && n <= bucket_sort_max_rows();
+  const int idx_bits = bit_width(static_cast<unsigned long long>(n - 1));
+  const int msd_cap = std::max(1, std::min(kBucketMaxBits, bit_width(static_cast<unsigned long long>(n / kBucketRows))));
+  BoundsExtras extras;
+  unsigned *bucket_starts = nullptr, *bucket_cursors = nullptr;
+  uint2 *bucket_chunks = nullptr;
+  unsigned long long *bucket_words = nullptr;
+  unsigned long long bucket_sequence = 0;
+  if (try_buckets) {
+    Arena &arena = scope.arena();
+    extras.device_copy = scope.alloc<long long>(16);
+    unsigned *totals = scope.alloc<unsigned>(kBucketMax + 4);
+    unsigned *info = totals + kBucketMax;
+    extras.zero = totals;
+    extras.zero_count = kBucketMax + 4;
+    bucket_starts = scope.alloc<unsigned>(kBucketMax + 1);
+    bucket_cursors = scope.alloc<unsigned>(kBucketMax);
+    // a bucket of m rows makes at most m / 8 + 1 pairs
+    bucket_chunks = scope.alloc<uint2>(kBucketMax + static_cast<size_t>(n / 8) + 1);
+    bucket_words = scope.alloc<unsigned long long>(n);
+    bucket_sequence = arena.next_sequence();
+    unsigned *host_out = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned_device()) + kBucketHostOffset);
+    unsigned long long *flag = arena.flag_device(3);
+    const long long *bounds_device = extras.device_copy;
+    extras.enqueue = [=] {
+      const unsigned tiles = static_cast<unsigned>(div_ceil(n, kSortBlock * kBucketItems));
+      bucket_hist_kernel<CT, IT><<<tiles, kSortBlock, 0, stream>>>(
+          coords, batched ? batch_dims : nullptr, batches_in_key, ndim, n, bounds_device, msd_cap,
+          idx_bits, totals, info);
+      check_launch("bucket_hist_kernel");
+      bucket_scan_kernel<<<1, 1024, 0, stream>>>(totals, 1 << msd_cap, info, bucket_starts,
+                                                 bucket_cursors, bucket_chunks, host_out, flag,
+                                                 bucket_sequence);
+      check_launch("bucket_scan_kernel");
+      bucket_deal_kernel<CT, IT><<<tiles, kSortBlock, 0, stream>>>(
+          coords, batched ? batch_dims : nullptr, batches_in_key, ndim, n, bounds_device, msd_cap,
+          idx_bits, info, bucket_starts, bucket_cursors, bucket_words);
+      check_launch("bucket_deal_kernel");
+    };
+  }
+  read_bounds(coords, n, nullptr, 0, ndim, sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64, h_bounds, scope, stream,
+              try_buckets ? &extras : nullptr);
   if (bounds_host_out != nullptr) memcpy(bounds_host_out, h_bounds, sizeof(long long) * 8);
   profile_mark("sort_bounds+sync", stream);
 
@@ -644,6 +1054,30 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
     check_launch("emit_sorted_kernel");
     profile_mark("sort_emit", stream);
     return;
+  }
+
+  if (try_buckets) {
+    // second half: deal and sort, if the layout holds and no bucket is too big
+    CoordSource<CT, IT> src{coords, batched ? batch_dims : nullptr, nullptr, {}};
+    const int bits = single_round_spec(h_bounds, ndim, batches_in_key, src.spec);
+    const BucketLayout lay = bucket_layout(bits, msd_cap, idx_bits);
+    if (lay.ok) {
+      Arena &arena = scope.arena();
+      arena.wait_flag(3, bucket_sequence);
+      volatile unsigned *from_scan =
+          reinterpret_cast<volatile unsigned *>(static_cast<char *>(arena.pinned()) + kBucketHostOffset);
+      const unsigned biggest = from_scan[0];
+      const unsigned pairs = from_scan[1];
+      if (biggest <= static_cast<unsigned>(kBucketCap) && pairs > 0) {
+        const unsigned long long *words = bucket_words;
+        const size_t lds = (static_cast<size_t>(biggest) + 128) * sizeof(unsigned long long);
+        bucket_rank_kernel<CT, IT><<<pairs, kSortBlock, lds, stream>>>(
+            words, bucket_chunks, lay.idx_bits, FinalSink<CT, IT>{coords, ndim, indices_out, sorted_out});
+        check_launch("bucket_rank_kernel");
+        profile_mark("sort_radix", stream);
+        return;
+      }
+    }
   }
 
   int total_passes = 0;

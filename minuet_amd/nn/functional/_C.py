@@ -643,7 +643,20 @@ class Epilogue:
         self.activation, self.negative_slope = activation, negative_slope
 
     def checked(self, num_targets: int, channels: int, dtype: torch.dtype, device) -> "Epilogue":
-        """Copy with operands validated and laid out the way the kernel reads them."""
+        """Copy with operands validated and laid out the way the kernel reads them
+        (the object itself when nothing needs changing)."""
+        scale, shift, residual = self.scale, self.shift, self.residual
+        f32 = torch.float32
+        if ((scale is None or (scale.dtype == f32 and scale.device == device and scale.dim() == 1
+                               and scale.shape[0] == channels and scale.is_contiguous()))
+                and (shift is None or (shift.dtype == f32 and shift.device == device and shift.dim() == 1
+                                       and shift.shape[0] == channels and shift.is_contiguous()))
+                and (residual is None or (residual.dtype == dtype and residual.device == device
+                                          and residual.dim() == 2 and residual.shape[0] == num_targets
+                                          and residual.shape[1] == channels and residual.is_contiguous()
+                                          and residual.data_ptr() % 16 == 0))):
+            return self
+
         def vector(name, t):
             if t is None:
                 return None
@@ -686,7 +699,10 @@ class Epilogue:
 def _host_sizes_arg(sizes_host, num_offsets):
     if sizes_host is None:
         return None, None
-    arr = np.ascontiguousarray(np.asarray(sizes_host, dtype=np.int64))
+    if type(sizes_host) is np.ndarray and sizes_host.dtype == np.int64 and sizes_host.flags.c_contiguous:
+        arr = sizes_host
+    else:
+        arr = np.ascontiguousarray(np.asarray(sizes_host, dtype=np.int64))
     if arr.shape[0] != num_offsets:
         _fail("host copy of kernel_map_sizes has the wrong length")
     return arr, arr.ctypes.data_as(_pi64)
@@ -733,7 +749,7 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
     if gather_index is not None:
         if gather_index.dtype != torch.int32 or gather_index.device != device:
             _fail("gather_index must be an int32 tensor on the device of the features")
-        if kernel_map_sizes_host is None or gather_index.numel() != int(sum(kernel_map_sizes_host)):
+        if kernel_map_sizes_host is None or gather_index.numel() != int(np.sum(kernel_map_sizes_host)):
             _fail("gather_index needs the host sizes and one entry per kernel map hit")
         gather_index = gather_index.contiguous()
     ep = Epilogue() if epilogue is None else epilogue.checked(T, N, weights.dtype, device)
@@ -743,7 +759,7 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
         if kernel_map_order is not None:
             if kernel_map_order_host is None:
                 _fail("packed weights need the host copy of kernel_map_order")
-            keep_order = np.ascontiguousarray(np.asarray(kernel_map_order_host, dtype=np.int64))
+            keep_order, _ = _host_sizes_arg(kernel_map_order_host, O)
             if keep_order.shape[0] != O:
                 _fail("host copy of kernel_map_order has the wrong length")
             order_ptr = keep_order.ctypes.data_as(_pi64)
@@ -824,21 +840,34 @@ def sparse_convolution_forward_implicit(sources: torch.Tensor, weights: torch.Te
     """Output-stationary forward from the dense kernel map ``[O, N_out]`` (int32,
     original offset order): one kernel, no gather / GEMM-output buffers."""
     fn = "sparse_convolution_forward_implicit"
-    _ensure_ndim("sources", sources, 2)
-    _ensure_ndim("weights", weights, 3)
-    _ensure_ndim("kernel_map", kernel_map, 2)
+    device = sources.device
+    dtype = weights.dtype
+    if not (sources.dim() == 2 and weights.dim() == 3 and kernel_map.dim() == 2
+            and kernel_map.shape[0] == weights.shape[0] and sources.shape[1] == weights.shape[1]
+            and weights.device == device and kernel_map.device == device and device.type == "cuda"
+            and kernel_map.dtype == torch.int32 and sources.dtype == dtype and dtype in _FLOAT):
+        # something is off: the checks one by one, for the message
+        _ensure_ndim("sources", sources, 2)
+        _ensure_ndim("weights", weights, 3)
+        _ensure_ndim("kernel_map", kernel_map, 2)
+        _ensure_dim("kernel_map", kernel_map, 0, weights.shape[0])
+        _ensure_dim("sources", sources, 1, weights.shape[1])
+        _common_device([sources, weights, kernel_map])
+        if kernel_map.dtype != torch.int32:
+            _fail("the implicit forward expects an int32 kernel map")
+        if sources.dtype != dtype:
+            _fail(f"Found tensors with two different scalar types ({sources.dtype} != {dtype})")
     O, K, N = weights.shape
-    _ensure_dim("kernel_map", kernel_map, 0, O)
-    _ensure_dim("sources", sources, 1, K)
-    device = _common_device([sources, weights, kernel_map])
-    if kernel_map.dtype != torch.int32:
-        _fail("the implicit forward expects an int32 kernel map")
-    if sources.dtype != weights.dtype:
-        _fail(f"Found tensors with two different scalar types ({sources.dtype} != {weights.dtype})")
-    fcode = _float_code(weights.dtype, fn)
-    S, T = sources.size(0), kernel_map.size(1)
-    sources, weights, kernel_map = sources.contiguous(), weights.contiguous(), kernel_map.contiguous()
-    sources = sources if sources.data_ptr() % 16 == 0 else sources.clone()
+    fcode = _float_code(dtype, fn)
+    S, T = sources.shape[0], kernel_map.shape[1]
+    if not sources.is_contiguous():
+        sources = sources.contiguous()
+    if not weights.is_contiguous():
+        weights = weights.contiguous()
+    if not kernel_map.is_contiguous():
+        kernel_map = kernel_map.contiguous()
+    if sources.data_ptr() % 16:
+        sources = sources.clone()
     out = torch.empty((T, N), dtype=weights.dtype, device=device)
     ep = Epilogue() if epilogue is None else epilogue.checked(T, N, weights.dtype, device)
     if packed_weights is not None:

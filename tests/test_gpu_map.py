@@ -53,6 +53,50 @@ def test_arg_sort_large_two_item_paths():
     np.testing.assert_array_equal(host(got).astype(np.int64), orc.arg_sort_coordinates(c))
 
 
+def _check_arg_sort(c, bd=None):
+    got = F.arg_sort_coordinates(dev(c), batch_dims=None if bd is None else dev(bd))
+    np.testing.assert_array_equal(host(got).astype(np.int64), orc.arg_sort_coordinates(c, bd))
+
+
+@pytest.mark.parametrize("n", [2048, 4096, 4097, 40000])
+def test_arg_sort_clustered_clouds(n):
+    # a dense core and two far outliers: the buckets at the core hold hundreds
+    # to thousands of rows (the largest in-LDS sorts), duplicates included
+    rng = np.random.default_rng(n)
+    c = np.rint(rng.normal(0.0, 30.0, size=(n, 3))).astype(np.int32)
+    c[:, 1:] = rng.integers(-40, 40, size=(n, 2))
+    c[0] = (-2000, 0, 0)
+    c[1] = (2000, 0, 0)
+    c[rng.integers(2, n, n // 5)] = c[rng.integers(2, n, n // 5)]
+    _check_arg_sort(c)
+
+
+def test_arg_sort_one_overfull_bucket_takes_the_radix_passes():
+    rng = np.random.default_rng(77)
+    c = rng.integers(0, 40, size=(50000, 3)).astype(np.int32)
+    c[123] = (10 ** 6, 5, 5)
+    _check_arg_sort(c)
+
+
+@pytest.mark.parametrize("width", [29, 30])
+def test_arg_sort_key_and_row_fill_one_word(width):
+    # 4096 rows (12 index bits), 6 bucket bits: with 2 x 29 key bits the rest of
+    # the key and the row index fill 64 bits exactly; one bit more does not fit
+    rng = np.random.default_rng(width)
+    c = rng.integers(0, 2 ** width, size=(4096, 2)).astype(np.int64)
+    c[0] = (0, 0)
+    c[1] = (2 ** width - 1, 2 ** width - 1)
+    c[rng.integers(2, 4096, 300)] = c[rng.integers(2, 4096, 300)]
+    _check_arg_sort(c)
+
+
+def test_arg_sort_batched_many_rows():
+    sizes = [9000, 0, 20000, 1, 13000]
+    bd = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    c = random_cloud(int(bd[-1]), 120, seed=3, lo=-50, duplicates=0.2)
+    _check_arg_sort(c, bd)
+
+
 @pytest.mark.parametrize("batched", [False, True])
 def test_unique(batched):
     bd = np.array([0, 2500, 2500, 6000], dtype=np.int32) if batched else None
