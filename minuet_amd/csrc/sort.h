@@ -1,8 +1,6 @@
 // Building blocks of the coordinate sort that other stages reuse.
 #pragma once
 
-#include <functional>
-
 #include "common.h"
 
 namespace mnt {
@@ -11,18 +9,8 @@ namespace mnt {
 // out[0..3] = min of a, out[4..7] = max of a, out[8..15] the same for b
 // (INT64_MAX / INT64_MIN for an empty array).  Two launches, then a wait on
 // a completion flag; the second kernel writes the results into pinned host memory.
-// `extras` (optional): a device copy of the 16 results, counters the fold
-// kernel clears, and work to enqueue behind the fold kernel before the host
-// starts waiting for the results (it then runs while the host wakes up).
-struct BoundsExtras {
-  long long *device_copy = nullptr;
-  unsigned *zero = nullptr;
-  int zero_count = 0;
-  std::function<void()> enqueue;
-};
 void read_bounds(const void *a, int64_t na, const void *b, int64_t nb, int ndim, int coord_dtype,
-                 long long out[16], Scope &scope, hipStream_t stream,
-                 const BoundsExtras *extras = nullptr);
+                 long long out[16], Scope &scope, hipStream_t stream);
 
 // Copies a small host int array to device memory as arguments of a tiny copy
 // kernel: no staging buffer to protect, no synchronisation.

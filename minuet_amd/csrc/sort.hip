@@ -29,7 +29,11 @@ constexpr int kBoundsMaxBlocks = 256;
 template <typename CT>
 __global__ __launch_bounds__(kBoundsBlock) void bounds_kernel(
     const CT *__restrict__ a, long long na, int blocks_a, const CT *__restrict__ b, long long nb,
-    int ndim, long long *__restrict__ partial) {
+    int ndim, long long *__restrict__ partial, unsigned *__restrict__ zero, int zero_count) {
+  // counters of the work that follows, cleared on the way (zero may be null)
+  for (int i = blockIdx.x * kBoundsBlock + threadIdx.x; i < zero_count; i += gridDim.x * kBoundsBlock) {
+    zero[i] = 0u;
+  }
   const bool second = static_cast<int>(blockIdx.x) >= blocks_a;
   const CT *coords = second ? b : a;
   const long long n = second ? nb : na;
@@ -94,10 +98,8 @@ __global__ __launch_bounds__(kBoundsBlock) void bounds_kernel(
 
 __global__ __launch_bounds__(kBoundsBlock) void bounds_fold_kernel(
     const long long *__restrict__ partial, int num_partials, int blocks_a, long long *out,
-    long long *__restrict__ device_copy, unsigned *__restrict__ zero, int zero_count,
     unsigned long long *flag, unsigned long long sequence) {
   const int w = threadIdx.x >> 6;
-  for (int i = threadIdx.x; i < zero_count; i += kBoundsBlock) zero[i] = 0u;
   // thread t takes the partials of workgroups t, t+256, ... of each array
   long long fa[8], fb[8];
 #pragma unroll
@@ -145,7 +147,6 @@ __global__ __launch_bounds__(kBoundsBlock) void bounds_fold_kernel(
       v = is_max ? (u > v ? u : v) : (u < v ? u : v);
     }
     out[threadIdx.x] = v;
-    if (device_copy != nullptr) device_copy[threadIdx.x] = v;
   }
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -155,7 +156,7 @@ __global__ __launch_bounds__(kBoundsBlock) void bounds_fold_kernel(
 }
 
 void read_bounds(const void *a, int64_t na, const void *b, int64_t nb, int ndim, int coord_dtype,
-                 long long out[16], Scope &scope, hipStream_t stream, const BoundsExtras *extras) {
+                 long long out[16], Scope &scope, hipStream_t stream) {
   for (int i = 0; i < 16; ++i) out[i] = (i & 4) ? INT64_MIN : INT64_MAX;
   if (na <= 0 && nb <= 0) return;
   const int blocks_a = na > 0 ? static_cast<int>(std::min<int64_t>(div_ceil(na, kBoundsBlock * 4), kBoundsMaxBlocks)) : 0;
@@ -169,18 +170,15 @@ void read_bounds(const void *a, int64_t na, const void *b, int64_t nb, int ndim,
   if (coord_dtype == MNT_INT32) {
     bounds_kernel<int32_t><<<grid, kBoundsBlock, 0, stream>>>(
         static_cast<const int32_t *>(a), na, blocks_a, static_cast<const int32_t *>(b), nb, ndim,
-        partial);
+        partial, nullptr, 0);
   } else {
     bounds_kernel<int64_t><<<grid, kBoundsBlock, 0, stream>>>(
         static_cast<const int64_t *>(a), na, blocks_a, static_cast<const int64_t *>(b), nb, ndim,
-        partial);
+        partial, nullptr, 0);
   }
   check_launch("bounds_kernel");
-  bounds_fold_kernel<<<1, kBoundsBlock, 0, stream>>>(
-      partial, grid, blocks_a, d_out, extras ? extras->device_copy : nullptr,
-      extras ? extras->zero : nullptr, extras ? extras->zero_count : 0, flag, sequence);
+  bounds_fold_kernel<<<1, kBoundsBlock, 0, stream>>>(partial, grid, blocks_a, d_out, flag, sequence);
   check_launch("bounds_fold_kernel");
-  if (extras && extras->enqueue) extras->enqueue();
   scope.arena().wait_flag(0, sequence);
   if (na > 0) memcpy(out, h_out, sizeof(long long) * 8);
   if (nb > 0) memcpy(out + 8, h_out + 8, sizeof(long long) * 8);
@@ -643,14 +641,55 @@ __host__ __device__ inline BucketLayout bucket_layout(int bits, int msd_cap, int
   return l;
 }
 
-// Key layout from the bounds in device memory.
+// Folds the partial extremes that bounds_kernel left for one array (a row of
+// lo[4], hi[4] per workgroup) into b; every thread of the workgroup gets the
+// result.  s_fold: one row of 8 per wavefront of the caller.
+__device__ __forceinline__ void fold_bounds(const long long *__restrict__ partial, int num_partials,
+                                            long long (*s_fold)[2 * MNT_MAX_NDIM],
+                                            long long (&b)[2 * MNT_MAX_NDIM]) {
+#pragma unroll
+  for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) b[slot] = slot >= MNT_MAX_NDIM ? INT64_MIN : INT64_MAX;
+  for (int blk = threadIdx.x; blk < num_partials; blk += blockDim.x) {
+#pragma unroll
+    for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) {
+      const long long u = partial[static_cast<long long>(blk) * 8 + slot];
+      b[slot] = slot >= MNT_MAX_NDIM ? (u > b[slot] ? u : b[slot]) : (u < b[slot] ? u : b[slot]);
+    }
+  }
+#pragma unroll
+  for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) {
+    for (int off = 32; off > 0; off >>= 1) {
+      const long long u = __shfl_down(b[slot], off);
+      b[slot] = slot >= MNT_MAX_NDIM ? (u > b[slot] ? u : b[slot]) : (u < b[slot] ? u : b[slot]);
+    }
+  }
+  const int w = threadIdx.x >> 6;
+  if (lane_id() == 0) {
+#pragma unroll
+    for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) s_fold[w][slot] = b[slot];
+  }
+  __syncthreads();
+  const int waves = blockDim.x >> 6;
+#pragma unroll
+  for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) {
+    long long v = s_fold[0][slot];
+    for (int ww = 1; ww < waves; ++ww) {
+      const long long u = s_fold[ww][slot];
+      v = slot >= MNT_MAX_NDIM ? (u > v ? u : v) : (u < v ? u : v);
+    }
+    // the same in every lane: say so, which keeps what is derived from it in
+    // scalar registers
+    const unsigned lo32 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
+    const unsigned hi32 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(static_cast<unsigned long long>(v) >> 32));
+    b[slot] = static_cast<long long>((static_cast<unsigned long long>(hi32) << 32) | lo32);
+  }
+}
+
+// Key layout from the folded bounds.
 template <typename CT, typename IT>
 __device__ __forceinline__ BucketLayout layout_on_device(
     const CT *__restrict__ coords, const IT *__restrict__ batch_dims, int num_batches, int ndim,
-    const long long *__restrict__ bounds, int msd_cap, int idx_bits, CoordSource<CT, IT> &src) {
-  long long b[2 * MNT_MAX_NDIM];
-#pragma unroll
-  for (int i = 0; i < 2 * MNT_MAX_NDIM; ++i) b[i] = bounds[i];
+    const long long (&b)[2 * MNT_MAX_NDIM], int msd_cap, int idx_bits, CoordSource<CT, IT> &src) {
   src.coords = coords;
   src.batch_dims = batch_dims;
   src.perm = nullptr;
@@ -662,9 +701,16 @@ __device__ __forceinline__ BucketLayout layout_on_device(
 template <typename CT, typename IT>
 __global__ __launch_bounds__(kSortBlock) void bucket_hist_kernel(
     const CT *__restrict__ coords, const IT *__restrict__ batch_dims, int num_batches, int ndim,
-    long long n, const long long *__restrict__ bounds, int msd_cap, int idx_bits,
-    unsigned *__restrict__ totals, unsigned *__restrict__ info) {
+    long long n, const long long *__restrict__ partial, int num_partials, int msd_cap, int idx_bits,
+    unsigned *__restrict__ totals, unsigned *__restrict__ info, long long *__restrict__ bounds_out) {
   __shared__ unsigned hist[kBucketMax];
+  __shared__ long long s_fold[kSortWaves][2 * MNT_MAX_NDIM];
+  long long bounds[2 * MNT_MAX_NDIM];
+  fold_bounds(partial, num_partials, s_fold, bounds);
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+#pragma unroll
+    for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) bounds_out[slot] = bounds[slot];
+  }
   CoordSource<CT, IT> src;
   const BucketLayout lay =
       layout_on_device<CT, IT>(coords, batch_dims, num_batches, ndim, bounds, msd_cap, idx_bits, src);
@@ -694,16 +740,18 @@ __global__ __launch_bounds__(kSortBlock) void bucket_hist_kernel(
   }
 }
 
-// How many threads share the ranking of one row of a bucket of m rows (as a
-// power of two): small buckets spread a row over 2 or 4 threads so that no
-// lane idles, large ones over 4 to 32 so that no thread scans more than about
-// 256 words.  A workgroup then takes 256 >> split rows.
-__device__ __forceinline__ unsigned bucket_split_log2(unsigned m) {
-  return m <= 64 ? 2u : m <= 128 ? 1u : m <= 256 ? 0u : m <= 1024 ? 2u : m <= 4096 ? 4u : 5u;
+// A bucket of up to 256 rows is ranked by one workgroup, with 1 << mode
+// threads sharing a row so that no lane idles (mode 2, 1, 0 for up to 64, 128,
+// 256 rows).  A larger bucket (mode kBucketSplit) is ranked 256 rows per
+// workgroup after a second split inside LDS.
+constexpr unsigned kBucketSplit = 7;
+
+__device__ __forceinline__ unsigned bucket_mode(unsigned m) {
+  return m <= 64 ? 2u : m <= 128 ? 1u : m <= 256 ? 0u : kBucketSplit;
 }
 
-__device__ __forceinline__ uint2 bucket_chunk_entry(unsigned first_row, unsigned rows, unsigned chunk) {
-  return make_uint2(first_row, rows | (bucket_split_log2(rows) << 13) | (chunk << 16));
+__device__ __forceinline__ unsigned bucket_pieces(unsigned m) {
+  return m == 0 ? 0u : m <= kSortBlock ? 1u : (m + kSortBlock - 1) / kSortBlock;
 }
 
 // One workgroup: bucket starts (exclusive scan of the totals, starts[buckets]
@@ -711,98 +759,96 @@ __device__ __forceinline__ uint2 bucket_chunk_entry(unsigned first_row, unsigned
 // ranking kernel runs over, info[1] = whether the bucket sort goes ahead, and
 // for the host the largest bucket (all ones when the layout does not hold)
 // and the number of pairs.
-// chunks[i] = {first row of the bucket, rows of the bucket | split << 13 |
+// chunks[i] = {first row of the bucket, rows of the bucket | mode << 13 |
 // chunk << 16}.
 __global__ __launch_bounds__(1024) void bucket_scan_kernel(
     const unsigned *__restrict__ totals, int buckets, unsigned *__restrict__ info,
     unsigned *__restrict__ starts, unsigned *__restrict__ cursors, uint2 *__restrict__ chunks,
+    const long long *__restrict__ folded, long long *host_bounds,
     unsigned *host_out, unsigned long long *flag, unsigned long long sequence) {
   constexpr int kPer = kBucketMax / 1024;
-  constexpr unsigned kShared = 1024;          // buckets of several chunks listed by whole wavefronts
   __shared__ unsigned long long wave_both[1024 / kWave];
-  __shared__ unsigned s_max, s_shared;
-  __shared__ unsigned shared_first[kShared], shared_rows[kShared], shared_at[kShared];
+  __shared__ unsigned wave_shared[1024 / kWave];
+  __shared__ unsigned s_max;
   const int t = threadIdx.x;
-  if (t == 0) {
-    s_max = 0;
-    s_shared = 0;
-  }
+  if (t == 0) s_max = 0;
   unsigned v[kPer];
-  unsigned sum = 0, biggest = 0, pieces = 0;
+  unsigned sum = 0, biggest = 0, singles = 0, shared = 0;
 #pragma unroll
   for (int j = 0; j < kPer; ++j) {
     const int d = t * kPer + j;
     v[j] = d < buckets ? totals[d] : 0u;
     sum += v[j];
     biggest = v[j] > biggest ? v[j] : biggest;
-    const unsigned rows = kSortBlock >> bucket_split_log2(v[j]);
-    pieces += v[j] <= kBucketCap ? (v[j] + rows - 1) / rows : 0u;
+    const unsigned mine = v[j] <= kBucketCap ? bucket_pieces(v[j]) : 0u;
+    singles += mine == 1 ? 1u : 0u;
+    shared += mine > 1 ? mine : 0u;
   }
-  // both scans in one sweep: rows in the low half, chunks in the high half
-  // (fewer than 2^31 rows, so the low half never carries into the high one)
+  // three scans in two sweeps: rows in the low half and one-workgroup buckets
+  // in the high half of one word (fewer than 2^31 rows, so the low half never
+  // carries into the high one), workgroups of shared buckets in another
   const unsigned long long mine_both =
-      static_cast<unsigned long long>(sum) | (static_cast<unsigned long long>(pieces) << 32);
+      static_cast<unsigned long long>(sum) | (static_cast<unsigned long long>(singles) << 32);
   unsigned long long inclusive = mine_both;
+  unsigned shared_inclusive = shared;
   for (int off = 1; off < kWave; off <<= 1) {
     const unsigned long long u = __shfl_up(inclusive, off);
-    if (static_cast<int>(lane_id()) >= off) inclusive += u;
+    const unsigned u2 = __shfl_up(shared_inclusive, off);
+    if (static_cast<int>(lane_id()) >= off) {
+      inclusive += u;
+      shared_inclusive += u2;
+    }
   }
   for (int off = 32; off > 0; off >>= 1) {
     const unsigned u = __shfl_down(biggest, off);
     biggest = u > biggest ? u : biggest;
   }
-  if (lane_id() == kWave - 1) wave_both[t >> 6] = inclusive;
-  __syncthreads();                            // also orders the clearing of s_max and s_shared
+  if (lane_id() == kWave - 1) {
+    wave_both[t >> 6] = inclusive;
+    wave_shared[t >> 6] = shared_inclusive;
+  }
+  __syncthreads();                            // also orders the clearing of s_max
   if (lane_id() == 0 && biggest != 0) atomicMax(&s_max, biggest);
   unsigned long long before = 0, all_both = 0;
+  unsigned shared_before = 0, all_shared = 0;
 #pragma unroll
   for (int w = 0; w < 1024 / kWave; ++w) {
     const unsigned long long x = wave_both[w];
+    const unsigned x2 = wave_shared[w];
     before += w < (t >> 6) ? x : 0ull;
+    shared_before += w < (t >> 6) ? x2 : 0u;
     all_both += x;
+    all_shared += x2;
   }
   const unsigned long long exclusive = before + inclusive - mine_both;
   unsigned run = static_cast<unsigned>(exclusive);
-  unsigned piece = static_cast<unsigned>(exclusive >> 32);
+  // the workgroups of shared buckets run longest and come first in the list
+  unsigned shared_at = shared_before + shared_inclusive - shared;
+  unsigned single_at = all_shared + static_cast<unsigned>(exclusive >> 32);
 #pragma unroll
   for (int j = 0; j < kPer; ++j) {
     const int d = t * kPer + j;
     if (d < buckets) {
       starts[d] = run;
       cursors[d] = 0u;
-      if (v[j] != 0 && v[j] <= kBucketCap) {
-        const unsigned rows = kSortBlock >> bucket_split_log2(v[j]);
-        const unsigned mine = (v[j] + rows - 1) / rows;
-        const unsigned slot = mine == 1 ? kShared : atomicAdd(&s_shared, 1u);
-        if (mine == 1) {
-          chunks[piece] = bucket_chunk_entry(run, v[j], 0);
-        } else if (slot < kShared) {
-          shared_first[slot] = run;
-          shared_rows[slot] = v[j];
-          shared_at[slot] = piece;
-        } else {
-          for (unsigned c = 0; c < mine; ++c) chunks[piece + c] = bucket_chunk_entry(run, v[j], c);
-        }
-        piece += mine;
+      if (v[j] <= kBucketCap) {
+        const unsigned mine = bucket_pieces(v[j]);
+        const unsigned head = v[j] | (bucket_mode(v[j]) << 13);
+        if (mine == 1) chunks[single_at++] = make_uint2(run, head);
+        for (unsigned c = 0; mine > 1 && c < mine; ++c) chunks[shared_at++] = make_uint2(run, head | (c << 16));
       }
     }
     run += v[j];
   }
   if (t == 1023) starts[buckets] = static_cast<unsigned>(all_both);
   __syncthreads();
-  const unsigned listed = s_shared < kShared ? s_shared : kShared;
-  for (unsigned h = t >> 6; h < listed; h += 1024 / kWave) {
-    const unsigned rows = kSortBlock >> bucket_split_log2(shared_rows[h]);
-    const unsigned mine = (shared_rows[h] + rows - 1) / rows;
-    for (unsigned c = t & (kWave - 1); c < mine; c += kWave) {
-      chunks[shared_at[h] + c] = bucket_chunk_entry(shared_first[h], shared_rows[h], c);
-    }
-  }
   if (t == 0) {
     const bool go = info[0] != 0 && s_max <= kBucketCap;
     info[1] = go ? 1u : 0u;
+#pragma unroll
+    for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) host_bounds[slot] = folded[slot];
     host_out[0] = info[0] != 0 ? s_max : 0xffffffffu;
-    host_out[1] = static_cast<unsigned>(all_both >> 32);
+    host_out[1] = all_shared + static_cast<unsigned>(all_both >> 32);
     __threadfence_system();
     __hip_atomic_store(flag, sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
@@ -813,11 +859,14 @@ __global__ __launch_bounds__(1024) void bucket_scan_kernel(
 template <typename CT, typename IT>
 __global__ __launch_bounds__(kSortBlock) void bucket_deal_kernel(
     const CT *__restrict__ coords, const IT *__restrict__ batch_dims, int num_batches, int ndim,
-    long long n, const long long *__restrict__ bounds, int msd_cap, int idx_bits_,
+    long long n, const long long *__restrict__ folded, int msd_cap, int idx_bits_,
     const unsigned *__restrict__ info, const unsigned *__restrict__ starts,
     unsigned *__restrict__ cursors, unsigned long long *__restrict__ words) {
   __shared__ unsigned hist[kBucketMax];
   if (info[1] == 0) return;
+  long long bounds[2 * MNT_MAX_NDIM];
+#pragma unroll
+  for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) bounds[slot] = folded[slot];
   CoordSource<CT, IT> src;
   const BucketLayout lay =
       layout_on_device<CT, IT>(coords, batch_dims, num_batches, ndim, bounds, msd_cap, idx_bits_, src);
@@ -879,38 +928,115 @@ __global__ __launch_bounds__(kSortBlock) void bucket_deal_kernel(
   }
 }
 
-// One workgroup per (bucket, chunk of rows): stages the whole bucket in LDS,
-// then 1 << split threads per row count the words below that row's word, each
-// over an interleaved share of the bucket; the sum is the row's place in the
-// bucket, and the row is written to its final place.
+// One workgroup per (bucket, chunk of rows): stages the whole bucket in LDS
+// and writes its chunk of rows to their final places.
+//
+// Up to 256 rows: 1 << mode threads per row count the words below that row's
+// word, each over an interleaved share of the bucket; the sum is the row's
+// place in the bucket.
+//
+// More rows: the bucket is first split again by the top 8 bits of its words
+// (a counting sort into LDS: histogram, scan, scatter by cursor, which every
+// workgroup of the bucket repeats for itself); a row then only counts inside
+// its own part, whose rows the other parts precede or follow as a whole.
+// word_bits = width of a word (rest of the key and row index).
 template <typename CT, typename IT>
 __global__ __launch_bounds__(kSortBlock) void bucket_rank_kernel(
     const unsigned long long *__restrict__ words, const uint2 *__restrict__ chunks, int idx_bits,
-    FinalSink<CT, IT> sink) {
+    int word_bits, FinalSink<CT, IT> sink) {
   extern __shared__ __align__(16) unsigned long long s_words[];
+  __shared__ unsigned part_cursor[kSortBlock], part_start[kSortBlock + 1], wave_sums[kSortWaves];
   const unsigned tid = threadIdx.x;
   const uint2 entry = chunks[blockIdx.x];
   const unsigned start = entry.x;
   const unsigned m = entry.y & 0x1fffu;
-  const unsigned split = (entry.y >> 13) & 7u;
+  const unsigned mode = (entry.y >> 13) & 7u;
   const unsigned chunk = entry.y >> 16;
-  // words are read four at a time by each of the 1 << split sharers
-  const unsigned group = 4u << split;
-  const unsigned padded = (m + group - 1u) / group * group;
-  for (unsigned i = tid; i < padded; i += kSortBlock) s_words[i] = i < m ? words[start + i] : ~0ull;
-  __syncthreads();
-  const unsigned part = tid & ((1u << split) - 1u);
-  const unsigned e = chunk * (kSortBlock >> split) + (tid >> split);
-  const unsigned long long mine = e < m ? s_words[e] : 0ull;
-  unsigned rank = 0;
-  for (unsigned j = 4u * part; j < padded; j += group) {
-    const unsigned long long a = s_words[j], b = s_words[j + 1], c = s_words[j + 2], d = s_words[j + 3];
-    rank += (a < mine ? 1u : 0u) + (b < mine ? 1u : 0u) + (c < mine ? 1u : 0u) + (d < mine ? 1u : 0u);
-  }
-  // the sharers of a row sit in neighbouring lanes
-  for (unsigned off = 1; off < (1u << split); off <<= 1) rank += __shfl_xor(rank, off);
   const unsigned long long idx_mask = (1ull << idx_bits) - 1ull;
-  if (e < m && part == 0) sink.store(start + rank, 0ull, static_cast<unsigned>(mine & idx_mask));
+
+  if (mode != kBucketSplit) {
+    // words are read four at a time by each of the 1 << mode sharers
+    const unsigned group = 4u << mode;
+    const unsigned padded = (m + group - 1u) / group * group;
+    for (unsigned i = tid; i < padded; i += kSortBlock) s_words[i] = i < m ? words[start + i] : ~0ull;
+    __syncthreads();
+    const unsigned part = tid & ((1u << mode) - 1u);
+    const unsigned e = tid >> mode;
+    const unsigned long long mine = e < m ? s_words[e] : 0ull;
+    unsigned rank = 0;
+    for (unsigned j = 4u * part; j < padded; j += group) {
+      const unsigned long long a = s_words[j], b = s_words[j + 1], c = s_words[j + 2], d = s_words[j + 3];
+      rank += (a < mine ? 1u : 0u) + (b < mine ? 1u : 0u) + (c < mine ? 1u : 0u) + (d < mine ? 1u : 0u);
+    }
+    // the sharers of a row sit in neighbouring lanes
+    for (unsigned off = 1; off < (1u << mode); off <<= 1) rank += __shfl_xor(rank, off);
+    if (e < m && part == 0) sink.store(start + rank, 0ull, static_cast<unsigned>(mine & idx_mask));
+    return;
+  }
+
+  const int part_bits = word_bits < 8 ? word_bits : 8;
+  const int part_shift = word_bits - part_bits;
+  part_cursor[tid] = 0;
+  __syncthreads();
+  // the thread's words (every 256th of the bucket) stay in registers for both
+  // sweeps; their loads are all in flight together
+  constexpr unsigned kMaxPerThread = (kBucketCap + kSortBlock - 1) / kSortBlock;
+  unsigned long long w[kMaxPerThread];
+#pragma unroll
+  for (unsigned k = 0; k < kMaxPerThread; ++k) {
+    const unsigned i = k * kSortBlock + tid;
+    w[k] = 0ull;
+    if (k * kSortBlock < m && i < m) w[k] = words[start + i];
+  }
+#pragma unroll
+  for (unsigned k = 0; k < kMaxPerThread; ++k) {
+    const unsigned i = k * kSortBlock + tid;
+    if (k * kSortBlock < m && i < m) atomicAdd(&part_cursor[static_cast<unsigned>(w[k] >> part_shift)], 1u);
+  }
+  __syncthreads();
+  {
+    const unsigned count = part_cursor[tid];
+    unsigned inclusive = count;
+    for (int off = 1; off < kWave; off <<= 1) {
+      const unsigned u = __shfl_up(inclusive, off);
+      if (static_cast<int>(lane_id()) >= off) inclusive += u;
+    }
+    if (lane_id() == kWave - 1) wave_sums[tid >> 6] = inclusive;
+    __syncthreads();
+    unsigned before = 0;
+    for (unsigned ww = 0; ww < (tid >> 6); ++ww) before += wave_sums[ww];
+    part_start[tid] = before + inclusive - count;
+    part_cursor[tid] = before + inclusive - count;
+    if (tid == kSortBlock - 1) part_start[kSortBlock] = before + inclusive;
+  }
+  __syncthreads();
+#pragma unroll
+  for (unsigned k = 0; k < kMaxPerThread; ++k) {
+    const unsigned i = k * kSortBlock + tid;
+    if (k * kSortBlock < m && i < m) {
+      s_words[atomicAdd(&part_cursor[static_cast<unsigned>(w[k] >> part_shift)], 1u)] = w[k];
+    }
+  }
+  __syncthreads();
+  // rows are handed out by their place in the dealt bucket: the order inside a
+  // part of the LDS copy differs from workgroup to workgroup
+  const unsigned e = chunk * kSortBlock + tid;
+  if (e < m) {
+    const unsigned long long mine = words[start + e];
+    const unsigned part = static_cast<unsigned>(mine >> part_shift);
+    const unsigned lo = part_start[part], hi = part_start[part + 1];
+    unsigned rank = lo;
+    unsigned j = lo;
+    for (; j + 8 <= hi; j += 8) {              // eight reads in flight, not one
+      unsigned long long x[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) x[u] = s_words[j + u];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) rank += x[u] < mine ? 1u : 0u;
+    }
+    for (; j < hi; ++j) rank += s_words[j] < mine ? 1u : 0u;
+    sink.store(start + rank, 0ull, static_cast<unsigned>(mine & idx_mask));
+  }
 }
 
 // Largest cloud the bucket sort takes (MINUET_BUCKET_SORT_MAX_ROWS overrides;
@@ -957,50 +1083,52 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
 
   profile_mark("enter:arg_sort", stream);
   long long h_bounds[16];
-  // bucket sort, first half: histogram and scan enqueued behind the bounds
+  // bucket sort, first half: bounds partials, bucket histogram, scan and the
+  // dealing step in a row; the scan kernel hands the bounds to the host
   const int batches_in_key = batched ? static_cast<int>(num_batches) : 1;
   const bool try_buckets = n >= kBucketMinN && n <= bucket_sort_max_rows();
   const int idx_bits = bit_width(static_cast<unsigned long long>(n - 1));
   const int msd_cap = std::max(1, std::min(kBucketMaxBits, bit_width(static_cast<unsigned long long>(n / kBucketRows))));
-  BoundsExtras extras;
-  unsigned *bucket_starts = nullptr, *bucket_cursors = nullptr;
+  unsigned *bucket_starts = nullptr;
   uint2 *bucket_chunks = nullptr;
   unsigned long long *bucket_words = nullptr;
-  unsigned long long bucket_sequence = 0;
   if (try_buckets) {
     Arena &arena = scope.arena();
-    extras.device_copy = scope.alloc<long long>(16);
     unsigned *totals = scope.alloc<unsigned>(kBucketMax + 4);
     unsigned *info = totals + kBucketMax;
-    extras.zero = totals;
-    extras.zero_count = kBucketMax + 4;
     bucket_starts = scope.alloc<unsigned>(kBucketMax + 1);
-    bucket_cursors = scope.alloc<unsigned>(kBucketMax);
-    // a bucket of m rows makes at most m / 8 + 1 pairs
-    bucket_chunks = scope.alloc<uint2>(kBucketMax + static_cast<size_t>(n / 8) + 1);
+    unsigned *cursors = scope.alloc<unsigned>(kBucketMax);
+    // a bucket of m rows makes at most m / 256 + 1 pairs
+    bucket_chunks = scope.alloc<uint2>(kBucketMax + static_cast<size_t>(n / kSortBlock) + 1);
     bucket_words = scope.alloc<unsigned long long>(n);
-    bucket_sequence = arena.next_sequence();
+    const int num_partials = static_cast<int>(std::min<int64_t>(div_ceil(n, kBoundsBlock * 4), kBoundsMaxBlocks));
+    long long *partial = scope.alloc<long long>(static_cast<size_t>(num_partials) * 8);
+    long long *folded = scope.alloc<long long>(2 * MNT_MAX_NDIM);
+    const unsigned long long sequence = arena.next_sequence();
+    long long *host_bounds = static_cast<long long *>(arena.pinned_device());
     unsigned *host_out = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned_device()) + kBucketHostOffset);
-    unsigned long long *flag = arena.flag_device(3);
-    const long long *bounds_device = extras.device_copy;
-    extras.enqueue = [=] {
-      const unsigned tiles = static_cast<unsigned>(div_ceil(n, kSortBlock * kBucketItems));
-      bucket_hist_kernel<CT, IT><<<tiles, kSortBlock, 0, stream>>>(
-          coords, batched ? batch_dims : nullptr, batches_in_key, ndim, n, bounds_device, msd_cap,
-          idx_bits, totals, info);
-      check_launch("bucket_hist_kernel");
-      bucket_scan_kernel<<<1, 1024, 0, stream>>>(totals, 1 << msd_cap, info, bucket_starts,
-                                                 bucket_cursors, bucket_chunks, host_out, flag,
-                                                 bucket_sequence);
-      check_launch("bucket_scan_kernel");
-      bucket_deal_kernel<CT, IT><<<tiles, kSortBlock, 0, stream>>>(
-          coords, batched ? batch_dims : nullptr, batches_in_key, ndim, n, bounds_device, msd_cap,
-          idx_bits, info, bucket_starts, bucket_cursors, bucket_words);
-      check_launch("bucket_deal_kernel");
-    };
+    const IT *dims = batched ? batch_dims : nullptr;
+    bounds_kernel<CT><<<num_partials, kBoundsBlock, 0, stream>>>(coords, n, num_partials, nullptr, 0, ndim,
+                                                                 partial, totals, kBucketMax + 4);
+    check_launch("bounds_kernel");
+    const unsigned tiles = static_cast<unsigned>(div_ceil(n, kSortBlock * kBucketItems));
+    bucket_hist_kernel<CT, IT><<<tiles, kSortBlock, 0, stream>>>(
+        coords, dims, batches_in_key, ndim, n, partial, num_partials, msd_cap, idx_bits, totals, info,
+        folded);
+    check_launch("bucket_hist_kernel");
+    bucket_scan_kernel<<<1, 1024, 0, stream>>>(totals, 1 << msd_cap, info, bucket_starts, cursors,
+                                               bucket_chunks, folded, host_bounds,
+                                               host_out, arena.flag_device(3), sequence);
+    check_launch("bucket_scan_kernel");
+    bucket_deal_kernel<CT, IT><<<tiles, kSortBlock, 0, stream>>>(
+        coords, dims, batches_in_key, ndim, n, folded, msd_cap, idx_bits, info, bucket_starts, cursors,
+        bucket_words);
+    check_launch("bucket_deal_kernel");
+    arena.wait_flag(3, sequence);
+    memcpy(h_bounds, arena.pinned(), sizeof(long long) * 8);
+  } else {
+    read_bounds(coords, n, nullptr, 0, ndim, sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64, h_bounds, scope, stream);
   }
-  read_bounds(coords, n, nullptr, 0, ndim, sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64, h_bounds, scope, stream,
-              try_buckets ? &extras : nullptr);
   if (bounds_host_out != nullptr) memcpy(bounds_host_out, h_bounds, sizeof(long long) * 8);
   profile_mark("sort_bounds+sync", stream);
 
@@ -1063,7 +1191,6 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
     const BucketLayout lay = bucket_layout(bits, msd_cap, idx_bits);
     if (lay.ok) {
       Arena &arena = scope.arena();
-      arena.wait_flag(3, bucket_sequence);
       volatile unsigned *from_scan =
           reinterpret_cast<volatile unsigned *>(static_cast<char *>(arena.pinned()) + kBucketHostOffset);
       const unsigned biggest = from_scan[0];
@@ -1072,7 +1199,8 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
         const unsigned long long *words = bucket_words;
         const size_t lds = (static_cast<size_t>(biggest) + 128) * sizeof(unsigned long long);
         bucket_rank_kernel<CT, IT><<<pairs, kSortBlock, lds, stream>>>(
-            words, bucket_chunks, lay.idx_bits, FinalSink<CT, IT>{coords, ndim, indices_out, sorted_out});
+            words, bucket_chunks, lay.idx_bits, lay.shift + lay.idx_bits,
+            FinalSink<CT, IT>{coords, ndim, indices_out, sorted_out});
         check_launch("bucket_rank_kernel");
         profile_mark("sort_radix", stream);
         return;

@@ -71,6 +71,16 @@ def test_arg_sort_clustered_clouds(n):
     _check_arg_sort(c)
 
 
+@pytest.mark.parametrize("distinct,extent", [(3, 2), (1, 1), (40, 5000)])
+def test_arg_sort_many_copies_of_few_rows(distinct, extent):
+    # thousands of equal rows: the order among them is the input order
+    rng = np.random.default_rng(distinct)
+    points = rng.integers(-extent, extent, size=(distinct, 3)).astype(np.int32)
+    c = points[rng.integers(0, distinct, 7000)]
+    c[:500] = rng.integers(-extent, extent, size=(500, 3))
+    _check_arg_sort(c)
+
+
 def test_arg_sort_one_overfull_bucket_takes_the_radix_passes():
     rng = np.random.default_rng(77)
     c = rng.integers(0, 40, size=(50000, 3)).astype(np.int32)
