@@ -54,11 +54,17 @@ __device__ __forceinline__ bool is_batch_end(long long end, const IT *__restrict
 // number of dimensions: slots past ndim re-read coordinate 0, so all loads
 // are issued together instead of one after another.
 template <typename CT>
+__device__ __forceinline__ void load_row_raw(const CT *__restrict__ row, int ndim,
+                                             CT (&raw)[MNT_MAX_NDIM]) {
+#pragma unroll
+  for (int k = 0; k < MNT_MAX_NDIM; ++k) raw[k] = row[k < ndim ? k : 0];
+}
+
+template <typename CT>
 __device__ __forceinline__ void load_row(const CT *__restrict__ row, int ndim,
                                          long long (&c)[MNT_MAX_NDIM]) {
   CT raw[MNT_MAX_NDIM];
-#pragma unroll
-  for (int k = 0; k < MNT_MAX_NDIM; ++k) raw[k] = row[k < ndim ? k : 0];
+  load_row_raw<CT>(row, ndim, raw);
 #pragma unroll
   for (int k = 0; k < MNT_MAX_NDIM; ++k) c[k] = static_cast<long long>(raw[k]);
 }

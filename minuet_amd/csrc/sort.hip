@@ -243,11 +243,18 @@ struct CoordSource {
     const long long row = perm ? static_cast<long long>(perm[i]) : i;
     long long c[MNT_MAX_NDIM];
     load_row<CT>(coords + row * spec.ndim, spec.ndim, c);
+    pack(row, c, key, val);
+  }
+  // Key of row `row` from its coordinates c (fetched earlier, e.g. before the
+  // spec was known).
+  template <typename VT>
+  __device__ __forceinline__ void pack(long long row, const VT (&c)[MNT_MAX_NDIM],
+                                       unsigned long long &key, unsigned &val) const {
     unsigned long long k64 = 0;
 #pragma unroll
     for (int k = 0; k < MNT_MAX_NDIM; ++k) {
       // fields that are not part of this round (or past ndim) have mask 0
-      const unsigned long long v = static_cast<unsigned long long>(c[k]) - spec.lo[k];
+      const unsigned long long v = static_cast<unsigned long long>(static_cast<long long>(c[k])) - spec.lo[k];
       k64 |= (v & spec.mask[k]) << spec.shift[k];
     }
     if (spec.mask[MNT_MAX_NDIM]) {
@@ -580,10 +587,9 @@ void radix_sort_pairs(unsigned long long *&keys, unsigned *&vals, unsigned long 
 // bucket beyond the LDS capacity (strong clustering) takes the radix passes
 // instead; the dealing step sees that for itself and does nothing.
 
-constexpr int kBucketMaxBits = 12;
+constexpr int kBucketMaxBits = 13;
 constexpr int kBucketMax = 1 << kBucketMaxBits;
 constexpr int kBucketCap = 8064;              // rows of the largest bucket: 64 KiB of LDS with padding
-constexpr int kBucketItems = 4;               // rows per thread when dealing
 constexpr int kBucketRows = 128;              // rows per bucket aimed at
 constexpr int64_t kBucketMinN = 2048;
 constexpr size_t kBucketHostOffset = 384;     // pinned block: largest bucket
@@ -642,45 +648,26 @@ __host__ __device__ inline BucketLayout bucket_layout(int bits, int msd_cap, int
 }
 
 // Folds the partial extremes that bounds_kernel left for one array (a row of
-// lo[4], hi[4] per workgroup) into b; every thread of the workgroup gets the
-// result.  s_fold: one row of 8 per wavefront of the caller.
+// lo[4], hi[4] per workgroup, at most 64 rows) into b.  Every wavefront does
+// the whole fold for itself: no LDS, no barrier.
+constexpr int kBucketBoundsBlocks = 64;
 __device__ __forceinline__ void fold_bounds(const long long *__restrict__ partial, int num_partials,
-                                            long long (*s_fold)[2 * MNT_MAX_NDIM],
                                             long long (&b)[2 * MNT_MAX_NDIM]) {
+  const int lane = lane_id();
+  const int row = lane < num_partials ? lane : 0;          // a repeated row changes no extreme
 #pragma unroll
-  for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) b[slot] = slot >= MNT_MAX_NDIM ? INT64_MIN : INT64_MAX;
-  for (int blk = threadIdx.x; blk < num_partials; blk += blockDim.x) {
-#pragma unroll
-    for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) {
-      const long long u = partial[static_cast<long long>(blk) * 8 + slot];
-      b[slot] = slot >= MNT_MAX_NDIM ? (u > b[slot] ? u : b[slot]) : (u < b[slot] ? u : b[slot]);
-    }
-  }
+  for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) b[slot] = partial[row * 8 + slot];
 #pragma unroll
   for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) {
     for (int off = 32; off > 0; off >>= 1) {
-      const long long u = __shfl_down(b[slot], off);
+      const long long u = __shfl_xor(b[slot], off);
       b[slot] = slot >= MNT_MAX_NDIM ? (u > b[slot] ? u : b[slot]) : (u < b[slot] ? u : b[slot]);
-    }
-  }
-  const int w = threadIdx.x >> 6;
-  if (lane_id() == 0) {
-#pragma unroll
-    for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) s_fold[w][slot] = b[slot];
-  }
-  __syncthreads();
-  const int waves = blockDim.x >> 6;
-#pragma unroll
-  for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) {
-    long long v = s_fold[0][slot];
-    for (int ww = 1; ww < waves; ++ww) {
-      const long long u = s_fold[ww][slot];
-      v = slot >= MNT_MAX_NDIM ? (u > v ? u : v) : (u < v ? u : v);
     }
     // the same in every lane: say so, which keeps what is derived from it in
     // scalar registers
-    const unsigned lo32 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
-    const unsigned hi32 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(static_cast<unsigned long long>(v) >> 32));
+    const unsigned lo32 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(b[slot]));
+    const unsigned hi32 =
+        __builtin_amdgcn_readfirstlane(static_cast<unsigned>(static_cast<unsigned long long>(b[slot]) >> 32));
     b[slot] = static_cast<long long>((static_cast<unsigned long long>(hi32) << 32) | lo32);
   }
 }
@@ -698,15 +685,22 @@ __device__ __forceinline__ BucketLayout layout_on_device(
 }
 
 // Rows per bucket; info[0] tells the scan kernel whether the layout holds.
-template <typename CT, typename IT>
+template <typename CT, typename IT, int kBucketItems>
 __global__ __launch_bounds__(kSortBlock) void bucket_hist_kernel(
     const CT *__restrict__ coords, const IT *__restrict__ batch_dims, int num_batches, int ndim,
     long long n, const long long *__restrict__ partial, int num_partials, int msd_cap, int idx_bits,
     unsigned *__restrict__ totals, unsigned *__restrict__ info, long long *__restrict__ bounds_out) {
   __shared__ unsigned hist[kBucketMax];
-  __shared__ long long s_fold[kSortWaves][2 * MNT_MAX_NDIM];
+  // the rows first: their loads need nothing from the bounds
+  const long long base = static_cast<long long>(blockIdx.x) * (kSortBlock * kBucketItems);
+  CT c[kBucketItems][MNT_MAX_NDIM];
+#pragma unroll
+  for (int r = 0; r < kBucketItems; ++r) {
+    const long long i = base + r * kSortBlock + threadIdx.x;
+    load_row_raw<CT>(coords + (i < n ? i : n - 1) * ndim, ndim, c[r]);
+  }
   long long bounds[2 * MNT_MAX_NDIM];
-  fold_bounds(partial, num_partials, s_fold, bounds);
+  fold_bounds(partial, num_partials, bounds);
   if (blockIdx.x == 0 && threadIdx.x == 0) {
 #pragma unroll
     for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) bounds_out[slot] = bounds[slot];
@@ -719,24 +713,18 @@ __global__ __launch_bounds__(kSortBlock) void bucket_hist_kernel(
   const int buckets = 1 << lay.msd_bits;
   for (int d = threadIdx.x; d < buckets; d += kSortBlock) hist[d] = 0;
   __syncthreads();
-  const long long base = static_cast<long long>(blockIdx.x) * (kSortBlock * kBucketItems);
-  unsigned long long key[kBucketItems];
 #pragma unroll
   for (int r = 0; r < kBucketItems; ++r) {
     const long long i = base + r * kSortBlock + threadIdx.x;
+    unsigned long long key;
     unsigned val;
-    key[r] = 0;
-    if (i < n) src.load(i, key[r], val);
-  }
-#pragma unroll
-  for (int r = 0; r < kBucketItems; ++r) {
-    const long long i = base + r * kSortBlock + threadIdx.x;
-    if (i < n) atomicAdd(&hist[static_cast<unsigned>(key[r] >> lay.shift)], 1u);
+    src.pack(i, c[r], key, val);
+    if (i < n) atomicAdd(&hist[static_cast<unsigned>(key >> lay.shift)], 1u);
   }
   __syncthreads();
   for (int d = threadIdx.x; d < buckets; d += kSortBlock) {
-    const unsigned c = hist[d];
-    if (c != 0) atomicAdd(&totals[d], c);
+    const unsigned count = hist[d];
+    if (count != 0) atomicAdd(&totals[d], count);
   }
 }
 
@@ -755,7 +743,7 @@ __device__ __forceinline__ unsigned bucket_pieces(unsigned m) {
 }
 
 // One workgroup: bucket starts (exclusive scan of the totals, starts[buckets]
-// = n), cleared cursors, the list of (bucket, chunk of rows) pairs the
+// = n), the cursors of the dealing step (a copy of the starts), the list of (bucket, chunk of rows) pairs the
 // ranking kernel runs over, info[1] = whether the bucket sort goes ahead, and
 // for the host the largest bucket (all ones when the layout does not hold)
 // and the number of pairs.
@@ -830,7 +818,7 @@ __global__ __launch_bounds__(1024) void bucket_scan_kernel(
     const int d = t * kPer + j;
     if (d < buckets) {
       starts[d] = run;
-      cursors[d] = 0u;
+      cursors[d] = run;                       // the dealing step hands out places from here
       if (v[j] <= kBucketCap) {
         const unsigned mine = bucket_pieces(v[j]);
         const unsigned head = v[j] | (bucket_mode(v[j]) << 13);
@@ -856,39 +844,41 @@ __global__ __launch_bounds__(1024) void bucket_scan_kernel(
 
 // Deals the rows of one tile into their buckets as (rest of key, row) words;
 // nothing to do when the scan kernel called the bucket sort off (info[1]).
-template <typename CT, typename IT>
+template <typename CT, typename IT, int kBucketItems>
 __global__ __launch_bounds__(kSortBlock) void bucket_deal_kernel(
     const CT *__restrict__ coords, const IT *__restrict__ batch_dims, int num_batches, int ndim,
     long long n, const long long *__restrict__ folded, int msd_cap, int idx_bits_,
-    const unsigned *__restrict__ info, const unsigned *__restrict__ starts,
-    unsigned *__restrict__ cursors, unsigned long long *__restrict__ words) {
+    const unsigned *__restrict__ info, unsigned *__restrict__ cursors,
+    unsigned long long *__restrict__ words) {
   __shared__ unsigned hist[kBucketMax];
-  if (info[1] == 0) return;
+  const int tid = threadIdx.x;
+  // the rows first: their loads wait for nothing
+  const long long base = static_cast<long long>(blockIdx.x) * (kSortBlock * kBucketItems);
+  CT c[kBucketItems][MNT_MAX_NDIM];
+#pragma unroll
+  for (int r = 0; r < kBucketItems; ++r) {
+    const long long i = base + r * kSortBlock + tid;
+    load_row_raw<CT>(coords + (i < n ? i : n - 1) * ndim, ndim, c[r]);
+  }
+  const unsigned go = info[1];
   long long bounds[2 * MNT_MAX_NDIM];
 #pragma unroll
   for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) bounds[slot] = folded[slot];
+  if (go == 0) return;
   CoordSource<CT, IT> src;
   const BucketLayout lay =
       layout_on_device<CT, IT>(coords, batch_dims, num_batches, ndim, bounds, msd_cap, idx_bits_, src);
   const int shift = lay.shift, idx_bits = lay.idx_bits;
   const int buckets = 1 << lay.msd_bits;
-  const int tid = threadIdx.x;
   for (int d = tid; d < buckets; d += kSortBlock) hist[d] = 0;
   __syncthreads();
-  const long long base = static_cast<long long>(blockIdx.x) * (kSortBlock * kBucketItems);
   const unsigned long long rest_mask = (1ull << shift) - 1ull;
   unsigned long long key[kBucketItems];
   unsigned row[kBucketItems], place[kBucketItems];
 #pragma unroll
   for (int r = 0; r < kBucketItems; ++r) {
     const long long i = base + r * kSortBlock + tid;
-    key[r] = 0;
-    row[r] = 0;
-    if (i < n) src.load(i, key[r], row[r]);
-  }
-#pragma unroll
-  for (int r = 0; r < kBucketItems; ++r) {
-    const long long i = base + r * kSortBlock + tid;
+    src.pack(i, c[r], key[r], row[r]);
     place[r] = 0;
     if (i < n) place[r] = atomicAdd(&hist[static_cast<unsigned>(key[r] >> shift)], 1u);
   }
@@ -896,7 +886,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_deal_kernel(
   // a range of every bucket this tile has rows for: counts fetched first, then
   // all cursor updates in flight together
   constexpr int kPer = kBucketMax / kSortBlock;
-  unsigned count[kPer], first[kPer], got[kPer];
+  unsigned count[kPer], got[kPer];
 #pragma unroll
   for (int j = 0; j < kPer; ++j) {
     const int d = j * kSortBlock + tid;
@@ -905,17 +895,13 @@ __global__ __launch_bounds__(kSortBlock) void bucket_deal_kernel(
 #pragma unroll
   for (int j = 0; j < kPer; ++j) {
     const int d = j * kSortBlock + tid;
-    first[j] = 0;
     got[j] = 0;
-    if (count[j] != 0) {
-      first[j] = starts[d];
-      got[j] = atomicAdd(&cursors[d], count[j]);
-    }
+    if (count[j] != 0) got[j] = atomicAdd(&cursors[d], count[j]);
   }
 #pragma unroll
   for (int j = 0; j < kPer; ++j) {
     const int d = j * kSortBlock + tid;
-    if (count[j] != 0) hist[d] = first[j] + got[j];
+    if (count[j] != 0) hist[d] = got[j];
   }
   __syncthreads();
 #pragma unroll
@@ -1045,7 +1031,7 @@ static int64_t bucket_sort_max_rows() {
   static const int64_t value = [] {
     const char *text = getenv("MINUET_BUCKET_SORT_MAX_ROWS");
     if (text != nullptr && *text != 0) return static_cast<int64_t>(atoll(text));
-    return static_cast<int64_t>(1) << 19;
+    return static_cast<int64_t>(1) << 21;
   }();
   return value;
 }
@@ -1101,7 +1087,7 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
     // a bucket of m rows makes at most m / 256 + 1 pairs
     bucket_chunks = scope.alloc<uint2>(kBucketMax + static_cast<size_t>(n / kSortBlock) + 1);
     bucket_words = scope.alloc<unsigned long long>(n);
-    const int num_partials = static_cast<int>(std::min<int64_t>(div_ceil(n, kBoundsBlock * 4), kBoundsMaxBlocks));
+    const int num_partials = static_cast<int>(std::min<int64_t>(div_ceil(n, kBoundsBlock * 4), kBucketBoundsBlocks));
     long long *partial = scope.alloc<long long>(static_cast<size_t>(num_partials) * 8);
     long long *folded = scope.alloc<long long>(2 * MNT_MAX_NDIM);
     const unsigned long long sequence = arena.next_sequence();
@@ -1111,18 +1097,30 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
     bounds_kernel<CT><<<num_partials, kBoundsBlock, 0, stream>>>(coords, n, num_partials, nullptr, 0, ndim,
                                                                  partial, totals, kBucketMax + 4);
     check_launch("bounds_kernel");
-    const unsigned tiles = static_cast<unsigned>(div_ceil(n, kSortBlock * kBucketItems));
-    bucket_hist_kernel<CT, IT><<<tiles, kSortBlock, 0, stream>>>(
-        coords, dims, batches_in_key, ndim, n, partial, num_partials, msd_cap, idx_bits, totals, info,
-        folded);
+    // rows per thread of the histogram and dealing kernels: 4, or 16 for a large cloud
+    const bool large = n > (int64_t(1) << 18);
+    const unsigned tiles = static_cast<unsigned>(div_ceil(n, kSortBlock * (large ? 16 : 4)));
+    if (large) {
+      bucket_hist_kernel<CT, IT, 16><<<tiles, kSortBlock, 0, stream>>>(
+          coords, dims, batches_in_key, ndim, n, partial, num_partials, msd_cap, idx_bits, totals, info,
+          folded);
+    } else {
+      bucket_hist_kernel<CT, IT, 4><<<tiles, kSortBlock, 0, stream>>>(
+          coords, dims, batches_in_key, ndim, n, partial, num_partials, msd_cap, idx_bits, totals, info,
+          folded);
+    }
     check_launch("bucket_hist_kernel");
     bucket_scan_kernel<<<1, 1024, 0, stream>>>(totals, 1 << msd_cap, info, bucket_starts, cursors,
                                                bucket_chunks, folded, host_bounds,
                                                host_out, arena.flag_device(3), sequence);
     check_launch("bucket_scan_kernel");
-    bucket_deal_kernel<CT, IT><<<tiles, kSortBlock, 0, stream>>>(
-        coords, dims, batches_in_key, ndim, n, folded, msd_cap, idx_bits, info, bucket_starts, cursors,
-        bucket_words);
+    if (large) {
+      bucket_deal_kernel<CT, IT, 16><<<tiles, kSortBlock, 0, stream>>>(
+          coords, dims, batches_in_key, ndim, n, folded, msd_cap, idx_bits, info, cursors, bucket_words);
+    } else {
+      bucket_deal_kernel<CT, IT, 4><<<tiles, kSortBlock, 0, stream>>>(
+          coords, dims, batches_in_key, ndim, n, folded, msd_cap, idx_bits, info, cursors, bucket_words);
+    }
     check_launch("bucket_deal_kernel");
     arena.wait_flag(3, sequence);
     memcpy(h_bounds, arena.pinned(), sizeof(long long) * 8);
@@ -1130,7 +1128,7 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
     read_bounds(coords, n, nullptr, 0, ndim, sizeof(CT) == 4 ? MNT_INT32 : MNT_INT64, h_bounds, scope, stream);
   }
   if (bounds_host_out != nullptr) memcpy(bounds_host_out, h_bounds, sizeof(long long) * 8);
-  profile_mark("sort_bounds+sync", stream);
+  profile_mark(try_buckets ? "sort_bounds+deal+sync" : "sort_bounds+sync", stream);
 
   // fields from least to most significant: dims ndim-1 .. 0, then the batch id
   int widths[MNT_MAX_NDIM + 1];
@@ -1202,7 +1200,7 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
             words, bucket_chunks, lay.idx_bits, lay.shift + lay.idx_bits,
             FinalSink<CT, IT>{coords, ndim, indices_out, sorted_out});
         check_launch("bucket_rank_kernel");
-        profile_mark("sort_radix", stream);
+        profile_mark("sort_rank", stream);
         return;
       }
     }
