@@ -149,10 +149,20 @@ __device__ __forceinline__ void resolve_chunk(
 // p + j is at least win[p] + j; so once p = lower_bound(first query of the
 // group) is known, every query of the group can only sit in win[p .. p+span]:
 // one search plus span+1 independent LDS reads resolve the whole group.
+//
+// Small tables (the usual 27 offsets) travel as kernel arguments (`carried`,
+// tables == nullptr), which saves the launch that would upload them; the last
+// wavefront copies them into LDS with uniform (scalar) reads while the first
+// two look for the window.
+constexpr int kCarriedInts = 160;
+struct CarriedTables {
+  int v[kCarriedInts];
+};
+
 template <typename CT, typename BT, typename OT>
 __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     KeyReader<CT, BT> src, KeyReader<CT, BT> tgt, Frame frame, const int *__restrict__ tables,
-    int num_groups, int num_offsets, long long delta_min, long long delta_max,
+    CarriedTables carried, int num_groups, int num_offsets, long long delta_min, long long delta_max,
     OT *__restrict__ kernel_map, unsigned *__restrict__ tile_counts, int num_tiles) {
   extern __shared__ __align__(16) unsigned s_dynamic[];
   __shared__ unsigned long long win[kWindowChunk + kWindowPad];
@@ -169,7 +179,21 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
   const long long t0 = static_cast<long long>(blockIdx.x) * kTargetsPerTile;
   const long long t_end = t0 + kTargetsPerTile < num_targets ? t0 + kTargetsPerTile : num_targets;
 
-  for (int i = tid; i < 4 * num_groups + 2 * num_offsets; i += kQueryThreads) s_dynamic[i] = tables[i];
+  if (tables != nullptr) {
+    for (int i = tid; i < 4 * num_groups + 2 * num_offsets; i += kQueryThreads) s_dynamic[i] = tables[i];
+  } else if (w == kQueryThreads / kWave - 1) {
+    const int count = 4 * num_groups + 2 * num_offsets;
+#pragma unroll
+    for (int i0 = 0; i0 < kCarriedInts; i0 += kWave) {
+      if (i0 < count) {                                     // uniform
+        // lane l takes entry i0 + l: 64 selects on scalar operands
+        int mine = 0;
+#pragma unroll
+        for (int l = 0; l < kWave; ++l) mine = static_cast<int>(lane_id()) == l ? carried.v[i0 + l < kCarriedInts ? i0 + l : 0] : mine;
+        if (i0 + static_cast<int>(lane_id()) < count) s_dynamic[i0 + lane_id()] = static_cast<unsigned>(mine);
+      }
+    }
+  }
   for (int o = tid; o < num_offsets; o += kQueryThreads) s_counts[o] = 0;
 
   // ---- window of sources that can match any (offset, target) pair of the tile:
@@ -263,51 +287,55 @@ __global__ __launch_bounds__(kQueryBlock) void count_tiles_kernel(
 __global__ __launch_bounds__(256) void tile_scan_kernel(unsigned *__restrict__ tile_counts,
                                                         int num_tiles,
                                                         unsigned *__restrict__ row_sizes) {
-  __shared__ unsigned partial[256];
+  __shared__ unsigned wave_sums[256 / kWave];
   unsigned *row = tile_counts + static_cast<long long>(blockIdx.x) * num_tiles;
   const int t = threadIdx.x;
+  const int lane = lane_id();
   const int chunk = (num_tiles + 255) / 256;
   const int lo = t * chunk;
   const int hi = lo + chunk < num_tiles ? lo + chunk : num_tiles;
   unsigned sum = 0;
   for (int i = lo; i < hi; ++i) sum += row[i];
-  partial[t] = sum;
-  __syncthreads();
-  for (int off = 1; off < 256; off <<= 1) {
-    unsigned v = t >= off ? partial[t - off] : 0;
-    __syncthreads();
-    partial[t] += v;
-    __syncthreads();
+  unsigned inclusive = sum;
+  for (int off = 1; off < kWave; off <<= 1) {
+    const unsigned u = __shfl_up(inclusive, off);
+    if (lane >= off) inclusive += u;
   }
-  unsigned run = partial[t] - sum;
+  if (lane == kWave - 1) wave_sums[t >> 6] = inclusive;
+  __syncthreads();
+  unsigned before = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < 256 / kWave; ++w) {
+    const unsigned x = wave_sums[w];
+    before += w < (t >> 6) ? x : 0u;
+    total += x;
+  }
+  unsigned run = before + inclusive - sum;
   for (int i = lo; i < hi; ++i) {
     unsigned v = row[i];
     row[i] = run;
     run += v;
   }
-  if (t == 255) row_sizes[blockIdx.x] = partial[255];
+  if (t == 0) row_sizes[blockIdx.x] = total;
 }
 
-// One workgroup, launched after tile_scan_kernel: the row order from the row
-// totals, stable ascending by size (reorder) or identity, its inverse, the
-// sizes in row order and their exclusive prefix.
+// The row order from the row totals, stable ascending by size (reorder) or
+// identity, its inverse, the sizes in row order and their exclusive prefix;
+// run by one whole workgroup.
 // plan layout (unsigned): order[O] | position_of[O] | sorted_sizes[O] | prefix[O+1];
 // the first three blocks are mirrored into plan_host (pinned host memory) and
-// the sequence flag tells the host that they are there.  (A separate launch
-// instead of a "last workgroup" ticket inside tile_scan_kernel: the
-// device-wide fence every workgroup would need costs more than the launch.)
-__global__ __launch_bounds__(256) void map_plan_kernel(const unsigned *__restrict__ row_sizes,
-                                                       int num_offsets, int reorder,
-                                                       unsigned *__restrict__ plan,
-                                                       unsigned *__restrict__ plan_host,
-                                                       unsigned long long *flag,
-                                                       unsigned long long sequence) {
+// the sequence flag tells the host that they are there.
+__device__ __forceinline__ void plan_from_sizes(const unsigned *row_sizes, int num_offsets, int reorder,
+                                                unsigned *__restrict__ plan,
+                                                unsigned *__restrict__ plan_host,
+                                                unsigned long long *flag,
+                                                unsigned long long sequence) {
   const int t = threadIdx.x;
   unsigned *order = plan;
   unsigned *position_of = plan + num_offsets;
   unsigned *sorted_sizes = plan + 2 * num_offsets;
   unsigned *prefix = plan + 3 * num_offsets;
-  for (int o = t; o < num_offsets; o += 256) {
+  for (int o = t; o < num_offsets; o += blockDim.x) {
     const unsigned mine = row_sizes[o];
     int pos = o;
     if (reorder) {
@@ -326,6 +354,9 @@ __global__ __launch_bounds__(256) void map_plan_kernel(const unsigned *__restric
       plan_host[2 * num_offsets + pos] = mine;
     }
   }
+  // thread 0 raises the flag behind a system-scope fence, which covers the
+  // host writes of its own wavefront; the other wavefronts see to theirs
+  if (plan_host != nullptr && t >= kWave && t < num_offsets) __threadfence_system();
   __syncthreads();
   if (t == 0) {
     unsigned total = 0;
@@ -339,6 +370,19 @@ __global__ __launch_bounds__(256) void map_plan_kernel(const unsigned *__restric
       __hip_atomic_store(flag, sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
   }
+}
+
+// One workgroup, launched after tile_scan_kernel.  (A separate launch instead
+// of a "last workgroup" ticket inside tile_scan_kernel: the device-wide fence
+// every workgroup would need costs more than the launch.  One workgroup doing
+// both jobs was measured slower than the two launches as well.)
+__global__ __launch_bounds__(256) void map_plan_kernel(const unsigned *__restrict__ row_sizes,
+                                                       int num_offsets, int reorder,
+                                                       unsigned *__restrict__ plan,
+                                                       unsigned *__restrict__ plan_host,
+                                                       unsigned long long *flag,
+                                                       unsigned long long sequence) {
+  plan_from_sizes(row_sizes, num_offsets, reorder, plan, plan_host, flag, sequence);
 }
 
 template <typename T>
@@ -530,9 +574,12 @@ static void launch_query(const QueryArgs &a, const QueryPlan &plan, const int *d
   KeyReader<CT, BT> tgt{static_cast<const CT *>(a.targets), static_cast<const BT *>(a.target_batch_dims),
                         static_cast<int>(a.num_batches), a.num_targets};
   const size_t dyn = sizeof(unsigned) * (plan.tables.size() + static_cast<size_t>(num_offsets) + 4);
+  CarriedTables carried;
+  memset(&carried, 0, sizeof(carried));
+  if (d_tables == nullptr) memcpy(carried.v, plan.tables.data(), sizeof(int) * plan.tables.size());
   query_kernel<CT, BT, OT><<<num_tiles, kQueryThreads, dyn, stream>>>(
-      src, tgt, plan.frame, d_tables, plan.num_groups, num_offsets, plan.delta_min, plan.delta_max,
-      kernel_map, tile_counts, num_tiles);
+      src, tgt, plan.frame, d_tables, carried, plan.num_groups, num_offsets, plan.delta_min,
+      plan.delta_max, kernel_map, tile_counts, num_tiles);
   check_launch("query_kernel");
 }
 
@@ -569,14 +616,17 @@ static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t n
   profile_mark("query_bounds+sync", stream);
   QueryPlan plan = make_plan(bounds, bounds + 8, offsets_host, num_offsets, a.ndim,
                              batched ? a.num_batches : 1);
-  // Upload the tables as kernel arguments of a tiny copy kernel: nothing to
-  // keep alive on the host and no staging buffer another call could overwrite.
+  // Large tables are uploaded as kernel arguments of a tiny copy kernel: nothing
+  // to keep alive on the host and no staging buffer another call could overwrite.
   const int no = static_cast<int>(num_offsets);
   MNT_CHECK(plan.tables.size() * sizeof(int) + sizeof(unsigned) * (num_offsets + 4) <= 24 * 1024,
             "too many kernel offsets (%lld) for the query kernel's table space",
             static_cast<long long>(num_offsets));
-  int *d_tables = scope.alloc<int>(plan.tables.size());
-  upload_ints(plan.tables, d_tables, stream);
+  int *d_tables = nullptr;                 // small tables ride in the kernel arguments
+  if (plan.tables.size() > static_cast<size_t>(kCarriedInts)) {
+    d_tables = scope.alloc<int>(plan.tables.size());
+    upload_ints(plan.tables, d_tables, stream);
+  }
   QueryArgs b = a;
   if (!batched) {
     b.source_batch_dims = nullptr;

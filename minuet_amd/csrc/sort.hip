@@ -146,7 +146,7 @@ __global__ __launch_bounds__(kBoundsBlock) void bounds_fold_kernel(
       const long long u = s_fold[ww][threadIdx.x];
       v = is_max ? (u > v ? u : v) : (u < v ? u : v);
     }
-    out[threadIdx.x] = v;
+    out[threadIdx.x] = v;                     // wavefront 0, as is the thread that raises the flag
   }
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -648,15 +648,25 @@ __host__ __device__ inline BucketLayout bucket_layout(int bits, int msd_cap, int
 }
 
 // Folds the partial extremes that bounds_kernel left for one array (a row of
-// lo[4], hi[4] per workgroup, at most 64 rows) into b.  Every wavefront does
-// the whole fold for itself: no LDS, no barrier.
-constexpr int kBucketBoundsBlocks = 64;
+// lo[4], hi[4] per workgroup, at most 128 rows) into b.  Every wavefront does
+// the whole fold for itself, two rows per lane: no LDS, no barrier.
+constexpr int kBucketBoundsBlocks = 128;
 __device__ __forceinline__ void fold_bounds(const long long *__restrict__ partial, int num_partials,
                                             long long (&b)[2 * MNT_MAX_NDIM]) {
   const int lane = lane_id();
   const int row = lane < num_partials ? lane : 0;          // a repeated row changes no extreme
+  const int row2 = lane + kWave < num_partials ? lane + kWave : 0;
+  long long b2[2 * MNT_MAX_NDIM];
 #pragma unroll
-  for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) b[slot] = partial[row * 8 + slot];
+  for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) {
+    b[slot] = partial[row * 8 + slot];
+    b2[slot] = partial[row2 * 8 + slot];
+  }
+#pragma unroll
+  for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) {
+    b[slot] = slot >= MNT_MAX_NDIM ? (b2[slot] > b[slot] ? b2[slot] : b[slot])
+                                   : (b2[slot] < b[slot] ? b2[slot] : b[slot]);
+  }
 #pragma unroll
   for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) {
     for (int off = 32; off > 0; off >>= 1) {
