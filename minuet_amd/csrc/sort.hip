@@ -753,8 +753,8 @@ __device__ __forceinline__ unsigned bucket_pieces(unsigned m) {
 }
 
 // One workgroup: bucket starts (exclusive scan of the totals, starts[buckets]
-// = n), the cursors of the dealing step (a copy of the starts), the list of (bucket, chunk of rows) pairs the
-// ranking kernel runs over, info[1] = whether the bucket sort goes ahead, and
+// = n), the cursors of the dealing step (a copy of the starts), the list of
+// (bucket, chunk of rows) pairs the ranking kernel runs over, info[1] = whether the bucket sort goes ahead, and
 // for the host the largest bucket (all ones when the layout does not hold)
 // and the number of pairs.
 // chunks[i] = {first row of the bucket, rows of the bucket | mode << 13 |
@@ -769,13 +769,14 @@ __global__ __launch_bounds__(1024) void bucket_scan_kernel(
   __shared__ unsigned wave_shared[1024 / kWave];
   __shared__ unsigned s_max;
   const int t = threadIdx.x;
+  const int per = (buckets + 1023) / 1024;    // consecutive buckets of one thread
   if (t == 0) s_max = 0;
   unsigned v[kPer];
   unsigned sum = 0, biggest = 0, singles = 0, shared = 0;
 #pragma unroll
   for (int j = 0; j < kPer; ++j) {
-    const int d = t * kPer + j;
-    v[j] = d < buckets ? totals[d] : 0u;
+    const int d = t * per + j;
+    v[j] = j < per && d < buckets ? totals[d] : 0u;
     sum += v[j];
     biggest = v[j] > biggest ? v[j] : biggest;
     const unsigned mine = v[j] <= kBucketCap ? bucket_pieces(v[j]) : 0u;
@@ -825,8 +826,8 @@ __global__ __launch_bounds__(1024) void bucket_scan_kernel(
   unsigned single_at = all_shared + static_cast<unsigned>(exclusive >> 32);
 #pragma unroll
   for (int j = 0; j < kPer; ++j) {
-    const int d = t * kPer + j;
-    if (d < buckets) {
+    const int d = t * per + j;
+    if (j < per && d < buckets) {
       starts[d] = run;
       cursors[d] = run;                       // the dealing step hands out places from here
       if (v[j] <= kBucketCap) {
