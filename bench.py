@@ -213,8 +213,16 @@ def extras(device, with_config5, section="all"):
             net(x4)
         lat = _time_stats(forward, 5, 50)
         kept = _time_stats(lambda: net(x4), 5, 50)
+        # the same pass with cached maps, replayed as one HIP graph
+        try:
+            graphed = minuet.capture_forward(lambda: net(x4))
+            replayed = _time_stats(graphed.replay, 5, 50)
+            del graphed
+        except Exception as error:          # reported, never fatal for the headline
+            replayed = {"error": str(error)[:200]}
         out["config4_unet_fp16"] = {"voxels": int(s4.shape[0]), "batch": 2, "cold_cache": lat,
                                     "kernel_maps_cached": kept,
+                                    "kernel_maps_cached_graph_replay": replayed,
                                     "forward_ms_cold_cache": lat["ms_median"]}
         del net, cache4, x4
     if section == "unet":

@@ -12,3 +12,4 @@ from .utils.helpers import set_kernel_map_cache
 from .utils.helpers import autotune
 from .utils.helpers import load_tunable_config
 from .utils.helpers import dump_tunable_config
+from .utils.graphs import capture_forward
