@@ -333,8 +333,11 @@ int mnt_time_gemm(int allow_shortcut_matmul, int64_t parallel, int has_threshold
  * [O, Cin, Cout] in the same offset order.  No gather or GEMM-output buffer is
  * written: each wavefront keeps 32 output rows in its matrix accumulators and
  * walks the offsets.  Requires Cin * sizeof(element) to be a multiple of 16
- * and at most 128, Cout % 4 == 0 and Cout <= 128; it pays for small channel counts, where the three-kernel
- * form is bound by the buffer traffic.  The epilogue arguments are those of
+ * and at most 2048, Cout % 4 == 0 and Cout <= 512.  Rows beyond 128 bytes are
+ * walked in chunks and more than 128 output channels in groups of 128; the
+ * form pays for rows of up to 128 bytes and up to 128 output channels, where
+ * the three-kernel form is bound by its buffer traffic, and loses beyond
+ * (its matrix work covers the empty (offset, target) pairs too).  The epilogue arguments are those of
  * mnt_sparse_convolution_forward_fused; packed_weights (nullable) is the
  * output of mnt_pack_weights for `weights`.  Results agree with the other forms to
  * rounding (sums are kept in fp32 over all offsets and rounded once).

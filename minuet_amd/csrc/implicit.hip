@@ -14,10 +14,14 @@
 // are along the sorted target order.  Sums are kept in fp32 across all offsets
 // in ascending offset order and rounded once, after the epilogue.
 //
+// Rows wider than one step of K (128 or 256 bytes) are walked in chunks: the
+// pipeline's unit is then an (offset, chunk) pair instead of an offset.  More
+// than 128 output channels are split into groups of 128 over blockIdx.y, each
+// group reading the source rows again (through L2).
+//
 // Compared with the three-kernel form this trades HBM traffic (no buffer rows
-// written and read back) for matrix work on empty rows, which pays while the
-// channel counts are small; the host entry point leaves the choice to the
-// caller.
+// written and read back) for matrix work on empty rows; the host entry point
+// leaves the choice to the caller.
 #include <algorithm>
 
 #include "conv_device.h"
@@ -27,12 +31,14 @@ namespace mnt {
 
 constexpr int kImplicitBlock = 256;
 constexpr int kImplicitTargets = 128;     // per workgroup, 32 per wavefront
-constexpr int kImplicitMaxBlocks = 4;     // 32-channel output blocks (128 channels)
+constexpr int kImplicitMaxBlocks = 4;     // 32-channel output blocks per channel group (128 channels)
+constexpr int kImplicitMaxGroups = 4;     // channel groups (512 channels)
+constexpr int kImplicitMaxRowBytes = 2048;
 constexpr int64_t kImplicitWideTargets = 1 << 16;   // from here on: two target blocks per wavefront
 
-// wt: packed weights [O][Np][KC] (W^T, K-contiguous, zero-padded to one
-// 128-byte chunk per row; see pack_weights_kernel).  Requires
-// K * sizeof(T) <= 128, K % (16 / sizeof(T)) == 0 and N % 4 == 0.
+// wt: packed weights [O][rows][Kp] (W^T, K-contiguous, rows = output channels
+// padded to a multiple of 32, Kp = K padded to a multiple of 128 bytes; see
+// pack_weights_kernel).  Requires K % (16 / sizeof(T)) == 0 and N % 4 == 0.
 // Register sets of the pipeline: 16-byte pieces of one thread's share of a
 // weight tile, and of one lane's source row.
 template <int N>
@@ -89,24 +95,34 @@ __device__ __forceinline__ void finish_four(float (&v)[4], const Epilogue &ep, l
   *reinterpret_cast<V *>(out + (t * N + ch) * static_cast<long long>(sizeof(T))) = raw;
 }
 
-// KS: 32-byte steps of K that hold data (source rows are at most KS * 32 bytes).
+// KS: 32-byte steps of K per pipeline stage.  A source row takes `chunks`
+// stages of KS * 32 bytes (Kp * sizeof(T) must be a multiple of that when
+// chunks > 1).  packed_row = Kp, packed_rows = rows of one offset in wt.
 // MW: 32-target blocks per wavefront.  With MW = 2 a wavefront owns 64 targets
 // and a workgroup 256: every weight fragment read from LDS feeds two matrix
 // operations and the weight tiles are staged half as often per target, at the
 // price of twice the accumulators and source-row registers.
 template <typename T, int NB, int KS, int MW>
-__global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
+__device__ __forceinline__ void implicit_forward_body(
     const T *__restrict__ sources, unsigned source_bytes, const T *__restrict__ wt,
     const int *__restrict__ kernel_map, long long num_targets, int num_offsets, int K, int N,
-    unsigned char *__restrict__ out, Epilogue ep) {
+    int chunks, int packed_row, int packed_rows, unsigned char *__restrict__ out, const Epilogue &ep) {
   constexpr int EPC = 16 / static_cast<int>(sizeof(T));
-  constexpr int KC = kChunkBytes / static_cast<int>(sizeof(T));
   constexpr int kSteps = KS;
   constexpr int Np = NB * 32;
-  constexpr int kRowPieces = 2 * KS;                     // 16-byte pieces of a weight row in use
+  constexpr int kStageBytes = KS * 32;                   // bytes of K per stage
+  constexpr int kStageElems = kStageBytes / static_cast<int>(sizeof(T));
+  constexpr int kRowPieces = 2 * KS;                     // 16-byte pieces of a weight row per stage
   constexpr int kWPieces = (Np * kRowPieces + kImplicitBlock - 1) / kImplicitBlock;
-  constexpr int kBufferBytes = Np * kLdsRowBytes;
+  // LDS rows of staged weights: padded by 16 bytes against bank conflicts, or,
+  // for the widest stage (where two padded buffers would not fit 64 KiB), left
+  // unpadded with the 16-byte pieces of row n stored at position p ^ (n % 16)
+  constexpr bool kSwizzle = KS == 8;
+  constexpr int kLdsRow = kSwizzle ? kStageBytes : kStageBytes + 16;
+  constexpr int kBufferBytes = Np * kLdsRow;
   __shared__ __align__(16) unsigned char w_lds[2 * kBufferBytes];
+  const int num_stages = num_offsets * chunks;
+  const int first_channel = blockIdx.y * Np;             // channel group of this workgroup
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -135,25 +151,33 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
   // Every global load below is unconditional (addresses are clamped, lanes
   // without a source use an out-of-range buffer offset), so that the loads of
   // later stages never have to be waited for early.
-  auto load_index = [&](int o) -> Pieces2<MW> {
+  // stage s belongs to offset s / chunks and covers chunk s % chunks of the rows
+  auto offset_of = [&](int s) -> int { return chunks == 1 ? s : s / chunks; };
+  auto load_index = [&](int s) -> Pieces2<MW> {
     Pieces2<MW> set;
-    const long long row = static_cast<long long>(o < num_offsets ? o : num_offsets - 1) * num_targets;
+    const long long row = static_cast<long long>(offset_of(s < num_stages ? s : num_stages - 1)) * num_targets;
 #pragma unroll
     for (int m = 0; m < MW; ++m) set.v[m] = kernel_map[row + t_safe[m]];
     return set;
   };
-  auto entry = [&](const Pieces2<MW> &set, int m, int o) -> int {
-    return (t_ok[m] && o < num_offsets) ? set.v[m] : -1;
+  auto entry = [&](const Pieces2<MW> &set, int m, int s) -> int {
+    return (t_ok[m] && s < num_stages) ? set.v[m] : -1;
   };
   // piece i of this thread: 16 bytes of weight row (piece / kRowPieces) at
   // position (piece % kRowPieces); threads past the tile repeat its last piece
-  auto load_w = [&](int o) -> Pieces<kWPieces> {
-    const T *base = wt + static_cast<long long>(o < num_offsets ? o : num_offsets - 1) * Np * KC;
+  auto load_w = [&](int s) -> Pieces<kWPieces> {
+    const int stage = s < num_stages ? s : num_stages - 1;
+    const int o = offset_of(stage);
+    const int c = stage - o * chunks;
+    const T *base = wt + (static_cast<long long>(o) * packed_rows + first_channel) * packed_row +
+                    c * kStageElems;
     Pieces<kWPieces> set;
 #pragma unroll
     for (int i = 0; i < kWPieces; ++i) {
       const int piece = min(tid + i * kImplicitBlock, Np * kRowPieces - 1);
-      set.v[i] = *reinterpret_cast<const uint4 *>(base + (piece / kRowPieces) * KC +
+      // a narrower last channel group repeats the last packed row (its outputs are never stored)
+      const int row = min(piece / kRowPieces, packed_rows - 1 - first_channel);
+      set.v[i] = *reinterpret_cast<const uint4 *>(base + static_cast<long long>(row) * packed_row +
                                                   (piece % kRowPieces) * EPC);
     }
     return set;
@@ -162,8 +186,9 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
 #pragma unroll
     for (int i = 0; i < kWPieces; ++i) {
       const int piece = min(tid + i * kImplicitBlock, Np * kRowPieces - 1);
-      *reinterpret_cast<uint4 *>(w_lds + buffer * kBufferBytes + (piece / kRowPieces) * kLdsRowBytes +
-                                 (piece % kRowPieces) * 16) = set.v[i];
+      const int row = piece / kRowPieces;
+      const int at = kSwizzle ? ((piece % kRowPieces) ^ (row & (kRowPieces - 1))) : piece % kRowPieces;
+      *reinterpret_cast<uint4 *>(w_lds + buffer * kBufferBytes + row * kLdsRow + at * 16) = set.v[i];
     }
   };
   // Source rows come through a buffer resource: lanes without a source (and
@@ -172,14 +197,15 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
   const __amdgpu_buffer_rsrc_t source_buffer = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<T *>(sources), 0, source_bytes, 0x00020000);
   const unsigned row_bytes = static_cast<unsigned>(K) * sizeof(T);
-  auto load_a = [&](const Pieces2<MW> &indices, int o) -> Pieces<KS * MW> {
+  auto load_a = [&](const Pieces2<MW> &indices, int s) -> Pieces<KS * MW> {
     Pieces<KS * MW> set;
+    const unsigned chunk_at = chunks == 1 ? 0u : static_cast<unsigned>(s - offset_of(s) * chunks) * kStageBytes;
 #pragma unroll
     for (int m = 0; m < MW; ++m) {
-      const int index = entry(indices, m, o);
+      const int index = entry(indices, m, s);
 #pragma unroll
       for (int kk = 0; kk < kSteps; ++kk) {
-        const unsigned at = (kk * 2 + h) * 16u;
+        const unsigned at = chunk_at + (kk * 2 + h) * 16u;
         const unsigned offset =
             (index >= 0 && at < row_bytes) ? static_cast<unsigned>(index) * row_bytes + at : kNoRow;
         const uint4v v = __builtin_amdgcn_raw_buffer_load_b128(source_buffer, offset, 0, 0);
@@ -189,9 +215,10 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
     return set;
   };
 
-  // Software pipeline over the offsets: while offset o is multiplied, the
-  // source rows of offset o+2 and the weights of offset o+3 are already on
-  // their way, and kernel-map entries are read five offsets ahead.  The loop
+  // Software pipeline over the stages (offsets, or chunks of offsets): while
+  // stage o is multiplied, the source rows of stage o+2 and the weights of
+  // stage o+3 are already on their way, and kernel-map entries are read five
+  // stages ahead.  The loop
   // is unrolled by six so that the roles of the register sets (three sets of
   // source rows, three of weights, six kernel-map entries) rotate without
   // copies: a register is never touched while its load is in flight.
@@ -226,10 +253,10 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
     if (any) {                                                                                     \
       const unsigned char *w_buf = w_lds + (o & 1) * kBufferBytes;                                 \
       _Pragma("unroll") for (int kk = 0; kk < kSteps; ++kk) {                                      \
-        const int off = kk * 32 + h * 16;                                                          \
+        const int off = (kSwizzle ? ((kk * 2 + h) ^ (r & (kRowPieces - 1))) : kk * 2 + h) * 16;     \
         _Pragma("unroll") for (int b = 0; b < NB; ++b) {                                           \
           const uint4 chan =                                                                       \
-              *reinterpret_cast<const uint4 *>(w_buf + (b * 32 + r) * kLdsRowBytes + off);         \
+              *reinterpret_cast<const uint4 *>(w_buf + (b * 32 + r) * kLdsRow + off);              \
           _Pragma("unroll") for (int m = 0; m < MW; ++m) {                                         \
             if (MW == 1 || live[m]) acc[m][b] = Mfma<T>::run(chan, A_CUR.v[m * KS + kk], acc[m][b]); \
           }                                                                                        \
@@ -238,7 +265,7 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
     }                                                                                              \
     store_w((o + 1) & 1, W_STORE);                                                                 \
     __syncthreads();                                                                               \
-    if (++o == num_offsets) break;                                                                 \
+    if (++o == num_stages) break;                                                                  \
   }
   while (true) {
     MNT_STAGE(a0, a2, w0, w2, m0, m2, m5)
@@ -257,7 +284,7 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
     for (int b = 0; b < NB; ++b) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int ch = b * 32 + q * 8 + h * 4;
+        const int ch = first_channel + b * 32 + q * 8 + h * 4;
         if (ch >= N) continue;               // N % 4 == 0: a group of four is all in or all out
         float v[4];
 #pragma unroll
@@ -266,6 +293,28 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
       }
     }
   }
+}
+
+template <typename T, int NB, int KS, int MW>
+__global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
+    const T *__restrict__ sources, unsigned source_bytes, const T *__restrict__ wt,
+    const int *__restrict__ kernel_map, long long num_targets, int num_offsets, int K, int N,
+    int chunks, int packed_row, int packed_rows, unsigned char *__restrict__ out, Epilogue ep) {
+  implicit_forward_body<T, NB, KS, MW>(sources, source_bytes, wt, kernel_map, num_targets, num_offsets, K, N,
+                                       chunks, packed_row, packed_rows, out, ep);
+}
+
+// The 256-byte stage keeps three sets of source-row and weight registers of
+// twice the size in flight: one wavefront per SIMD, with the whole register
+// file, instead of spills.
+template <typename T, int NB>
+__global__ __launch_bounds__(kImplicitBlock) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void implicit_forward_wide_rows_kernel(
+    const T *__restrict__ sources, unsigned source_bytes, const T *__restrict__ wt,
+    const int *__restrict__ kernel_map, long long num_targets, int num_offsets, int K, int N,
+    int chunks, int packed_row, int packed_rows, unsigned char *__restrict__ out, Epilogue ep) {
+  implicit_forward_body<T, NB, 8, 1>(sources, source_bytes, wt, kernel_map, num_targets, num_offsets, K, N,
+                                     chunks, packed_row, packed_rows, out, ep);
 }
 
 // inverse[o][m] = t for every hit kernel_map[o][t] = m (at most one t per
@@ -311,35 +360,48 @@ static void implicit_typed(const T *sources, const T *weights, const T *packed, 
     check_launch("pack_weights_kernel");
     profile_mark("pack_weights", stream);
   }
-  const unsigned grid = static_cast<unsigned>(div_ceil(Tn, kImplicitTargets));
   const unsigned source_bytes = static_cast<unsigned>(S * K * sizeof(T));
+  // stage width: 64 or 128 bytes for narrow rows; wider rows go in chunks of 256
+  // bytes where the padded row is a multiple of that, else of 128
+  const int row_bytes = Kp * static_cast<int>(sizeof(T));
+  const int stage_bytes = K * sizeof(T) <= 64 ? 64 : row_bytes <= 128 ? 128 : row_bytes % 256 == 0 ? 256 : 128;
+  const int chunks = row_bytes <= 128 ? 1 : row_bytes / stage_bytes;
+  // channel groups of up to 128 channels; the last group may be narrower
+  const int groups = static_cast<int>(div_ceil(Np, 32 * kImplicitMaxBlocks));
+  const int blocks = groups > 1 ? kImplicitMaxBlocks : Np / 32;
   // Two target blocks per wavefront where that measured faster: 16-bit
-  // features, 33..64 output channels, and enough targets to fill the chip that
-  // way.  (With one channel block the compiler's register allocation leaves
-  // too few wavefronts per SIMD; in fp32 the matrix work dominates anyway.)
-  const bool wide = sizeof(T) == 2 && Np == 64 && Tn >= kImplicitWideTargets;
-  const unsigned grid_wide = static_cast<unsigned>(div_ceil(Tn, kImplicitTargets * 2));
-#define MNT_IMPLICIT(NB, KS, MW, GRID)                                                             \
-  implicit_forward_kernel<T, NB, KS, MW><<<GRID, kImplicitBlock, 0, stream>>>(                     \
+  // features, 33..64 output channels, rows of one stage, and enough targets to
+  // fill the chip that way.  (With one channel block the compiler's register
+  // allocation leaves too few wavefronts per SIMD; in fp32 the matrix work
+  // dominates anyway.)
+  const bool wide = sizeof(T) == 2 && Np == 64 && chunks == 1 && stage_bytes <= 128 && Tn >= kImplicitWideTargets;
+  const dim3 grid(static_cast<unsigned>(div_ceil(Tn, kImplicitTargets * (wide ? 2 : 1))),
+                  static_cast<unsigned>(groups));
+#define MNT_IMPLICIT(NB, KS, MW)                                                                   \
+  implicit_forward_kernel<T, NB, KS, MW><<<grid, kImplicitBlock, 0, stream>>>(                     \
       sources, source_bytes, wt, kernel_map, Tn, static_cast<int>(O), static_cast<int>(K),         \
-      static_cast<int>(N), reinterpret_cast<unsigned char *>(out), ep)
-#define MNT_IMPLICIT_KS(NB, MW, GRID)     \
-  if (K * sizeof(T) <= 64) {              \
-    MNT_IMPLICIT(NB, 2, MW, GRID);        \
+      static_cast<int>(N), chunks, Kp, Np, reinterpret_cast<unsigned char *>(out), ep)
+#define MNT_IMPLICIT_KS(NB, MW)           \
+  if (stage_bytes == 64) {                \
+    MNT_IMPLICIT(NB, 2, MW);              \
+  } else if (stage_bytes == 128) {        \
+    MNT_IMPLICIT(NB, 4, MW);              \
   } else {                                \
-    MNT_IMPLICIT(NB, 4, MW, GRID);        \
+    implicit_forward_wide_rows_kernel<T, NB><<<grid, kImplicitBlock, 0, stream>>>(                 \
+        sources, source_bytes, wt, kernel_map, Tn, static_cast<int>(O), static_cast<int>(K),       \
+        static_cast<int>(N), chunks, Kp, Np, reinterpret_cast<unsigned char *>(out), ep);          \
   }
-  switch (Np / 32) {
-    case 1: MNT_IMPLICIT_KS(1, 1, grid); break;
+  switch (blocks) {
+    case 1: MNT_IMPLICIT_KS(1, 1); break;
     case 2:
       if (wide) {
-        MNT_IMPLICIT_KS(2, 2, grid_wide);
+        MNT_IMPLICIT_KS(2, 2);
       } else {
-        MNT_IMPLICIT_KS(2, 1, grid);
+        MNT_IMPLICIT_KS(2, 1);
       }
       break;
-    case 3: MNT_IMPLICIT_KS(3, 1, grid); break;
-    default: MNT_IMPLICIT_KS(4, 1, grid); break;
+    case 3: MNT_IMPLICIT_KS(3, 1); break;
+    default: MNT_IMPLICIT_KS(4, 1); break;
   }
 #undef MNT_IMPLICIT_KS
 #undef MNT_IMPLICIT
@@ -366,11 +428,11 @@ extern "C" int mnt_sparse_convolution_forward_implicit(
     MNT_CHECK(S * K * esize < static_cast<int64_t>(kNoRow),
               "source features of %lld bytes exceed the 4 GiB a buffer resource addresses",
               (long long)(S * K * esize));
-    MNT_CHECK((K * esize) % 16 == 0 && K * esize <= kChunkBytes && N % 4 == 0 &&
-                  N <= 32 * kImplicitMaxBlocks,
+    MNT_CHECK((K * esize) % 16 == 0 && K * esize <= kImplicitMaxRowBytes && N % 4 == 0 &&
+                  N <= 32 * kImplicitMaxBlocks * kImplicitMaxGroups,
               "Unsupported channel counts for the implicit forward: Cin = %lld (rows must be a multiple "
               "of 16 bytes, at most %d), Cout = %lld (a multiple of 4, at most %d)",
-              (long long)K, kChunkBytes, (long long)N, 32 * kImplicitMaxBlocks);
+              (long long)K, kImplicitMaxRowBytes, (long long)N, 32 * kImplicitMaxBlocks * kImplicitMaxGroups);
     MNT_CHECK(activation >= MNT_ACT_NONE && activation <= MNT_ACT_RELU6, "unknown activation code %d",
               activation);
     MNT_CHECK(reinterpret_cast<uintptr_t>(sources) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&

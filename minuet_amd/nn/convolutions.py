@@ -494,7 +494,9 @@ class SparseConv(Module):
         if (features.is_cuda and not needs_grad
                 and self._tunable_config.get("dataflow", "auto") != "gather_gemm_scatter"
                 and features.dtype == weights.dtype
-                and _C.implicit_forward_supported(self.in_channels, self.out_channels, weights.dtype)):
+                and _C.implicit_forward_supported(self.in_channels, self.out_channels, weights.dtype)
+                # wider layers are plain library GEMM territory
+                and self.in_channels * weights.dtype.itemsize <= 128 and self.out_channels <= 128):
             rows = features.shape[0]
             identity = self._identity_map
             if identity is None or identity.shape[1] < rows or identity.device != features.device:

@@ -822,14 +822,16 @@ def kernel_map_invert(kernel_map: torch.Tensor, num_sources: int) -> torch.Tenso
     return inverse
 
 
-IMPLICIT_MAX_TARGET_FEATURES = 128
+IMPLICIT_MAX_TARGET_FEATURES = 512
+IMPLICIT_MAX_SOURCE_ROW_BYTES = 2048
 
 
 def implicit_forward_supported(num_source_features: int, num_target_features: int,
                                dtype: torch.dtype) -> bool:
     """Shapes ``sparse_convolution_forward_implicit`` accepts."""
     row_bytes = num_source_features * dtype.itemsize
-    return (row_bytes % 16 == 0 and row_bytes <= 128 and num_target_features % 4 == 0
+    return (row_bytes % 16 == 0 and row_bytes <= IMPLICIT_MAX_SOURCE_ROW_BYTES
+            and num_target_features % 4 == 0
             and num_target_features <= IMPLICIT_MAX_TARGET_FEATURES)
 
 

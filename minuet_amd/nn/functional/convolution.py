@@ -30,13 +30,15 @@ def prefers_implicit(num_offsets: int, num_source_features: int, num_target_feat
                      dtype: torch.dtype) -> bool:
     """Whether ``dataflow="auto"`` takes the single-kernel form for a layer of
     this shape: it must fit that kernel, and it must be the faster one, which
-    measurements say it is for 16-bit features.  fp32 matrix work is 16x dearer,
-    so there it only pays where most (offset, target) pairs are hits, i.e. for
-    small layers with strided 2^D kernels."""
+    measurements say it is for 16-bit features with source rows of up to 128
+    bytes and up to 128 output channels (beyond that its matrix work on empty
+    (offset, target) pairs outweighs the buffer traffic it saves).  fp32 matrix
+    work is 16x dearer, so there it only pays where most (offset, target) pairs
+    are hits, i.e. for small layers with strided 2^D kernels."""
     if not _C.implicit_forward_supported(num_source_features, num_target_features, dtype):
         return False
     if dtype != torch.float32:
-        return True
+        return num_source_features * dtype.itemsize <= 128 and num_target_features <= 128
     return num_offsets <= 8 and num_source_features * num_target_features <= 1024
 
 

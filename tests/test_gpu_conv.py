@@ -154,12 +154,16 @@ def test_forward_epilogue(kind, activation):
     (3, 1, 8, 32, 5000, 20), (3, 1, 24, 48, 4000, 20), (5, 1, 16, 16, 3000, 16),
     (3, 1, 32, 100, 3000, 16), (3, 1, 56, 40, 2000, 12), (1, 1, 32, 12, 999, 12),
     (7, 1, 16, 8, 1500, 10),
+    # rows wider than one pipeline stage (chunks of 256 or 128 bytes) and more
+    # than 128 output channels (channel groups, the last one narrower)
+    (3, 1, 128, 128, 4000, 20), (3, 1, 256, 64, 3000, 16), (2, 2, 128, 256, 6000, 30),
+    (3, 1, 160, 32, 2000, 12), (3, 1, 96, 200, 2000, 12), (3, 1, 72, 300, 1500, 12),
 ])
 def test_forward_implicit(kind, kernel, stride, cin, cout, n, extent):
     """The single-kernel output-stationary forward against the float64 oracle:
     dense kernel map in the original offset order, no rank tables."""
     if not _C.implicit_forward_supported(cin, cout, TORCH[kind]):
-        pytest.skip("source rows wider than the 128 bytes this form stages")
+        pytest.skip("a shape this form does not take")
     src, sbd, tgt, tbd, off, feats, weights = make_layer_case(4, n, extent, kernel, cin, cout, kind, stride)
     kmap = orc.query_sorted_index_with_offsets(src, tgt, off, sbd, tbd)
     esm, etm, eorder, esizes, _ = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=True)
@@ -186,9 +190,10 @@ def test_forward_implicit(kind, kernel, stride, cin, cout, n, extent):
 def test_forward_implicit_rejects_unsupported_shapes():
     assert not _C.implicit_forward_supported(4, 32, torch.float16)       # 8-byte rows
     assert not _C.implicit_forward_supported(32, 30, torch.float16)
-    assert not _C.implicit_forward_supported(32, 256, torch.float16)
-    assert not _C.implicit_forward_supported(128, 32, torch.float16)     # 256-byte rows
-    assert not _C.implicit_forward_supported(64, 32, torch.float32)
+    assert not _C.implicit_forward_supported(32, 516, torch.float16)
+    assert not _C.implicit_forward_supported(1032, 32, torch.float16)    # rows beyond 2048 bytes
+    assert _C.implicit_forward_supported(128, 256, torch.float16)
+    assert _C.implicit_forward_supported(64, 32, torch.float32)
     kmap = torch.full((27, 10), -1, dtype=torch.int32, device="cuda")
     with pytest.raises(RuntimeError, match="Unsupported channel counts"):
         _C.sparse_convolution_forward_implicit(torch.zeros(10, 4, device="cuda").half(),
