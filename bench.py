@@ -26,7 +26,7 @@ HBM_PEAK_GBS = 8000.0
 # WRITE_SIZE of rocprofv3 --pmc, each scaled by what the counter reads for a
 # plain 256 MiB device copy (2.000 and 1.000); the dense kernel map the kernel
 # writes accounts for 21.6 MB of it.
-QUERY_TRAFFIC_BYTES = 30.68e6
+QUERY_TRAFFIC_BYTES = 30.79e6
 
 
 def map_step(_C, coords_dev, offsets):
@@ -321,6 +321,7 @@ def main():
 
     bytes_map = 12 * n + 12 * n + 4 * n + 8 * nnz + 4 * offsets.shape[0]
     bytes_query = 12 * n + 8 * nnz
+    bytes_dense = 12 * n + 4 * offsets.shape[0] * n
     query_ms = stage_ms.get("query", float("nan"))
     achieved = bytes_query / (query_ms * 1e-3) / 1e9 if query_ms == query_ms and query_ms > 0 else None
     result = {
@@ -347,6 +348,10 @@ def main():
                      "frac": None if achieved is None else round(achieved / HBM_PEAK_GBS, 5),
                      "traffic": QUERY_TRAFFIC_BYTES if args.scale == 1.0 else None,
                      "algorithmic_bytes": bytes_query,
+                     # the same launch priced with the dense map M[O, T] as its output, which is
+                     # what it writes and what the reference's query function returns
+                     "dense_form": {"algorithmic_bytes": bytes_dense,
+                                    "achieved": None if achieved is None else round(bytes_dense / (query_ms * 1e-3) / 1e9, 2)},
                      "avg_launch_ms": None if achieved is None else round(query_ms, 5),
                      "map_step": {"algorithmic_bytes": bytes_map,
                                   "device_ms": round(device_ms, 4),
