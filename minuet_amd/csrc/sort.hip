@@ -589,7 +589,8 @@ void radix_sort_pairs(unsigned long long *&keys, unsigned *&vals, unsigned long 
 
 constexpr int kBucketMaxBits = 13;
 constexpr int kBucketMax = 1 << kBucketMaxBits;
-constexpr int kBucketCap = 8064;              // rows of the largest bucket: 64 KiB of LDS with padding
+constexpr int kBucketCap = 7680;              // rows of the largest bucket: its words, their padding and
+                                              // the ranking kernel's tables fit 64 KiB of LDS
 constexpr int kBucketRows = 128;              // rows per bucket aimed at
 constexpr int64_t kBucketMinN = 2048;
 constexpr size_t kBucketHostOffset = 384;     // pinned block: largest bucket

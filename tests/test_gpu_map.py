@@ -81,6 +81,18 @@ def test_arg_sort_many_copies_of_few_rows(distinct, extent):
     _check_arg_sort(c)
 
 
+@pytest.mark.parametrize("copies", [7600, 7680, 7681])
+def test_arg_sort_bucket_at_the_lds_capacity(copies):
+    # one bucket right at (and just past) the largest size the in-LDS ranking
+    # takes; the rows around it are spread so thinly that they share no bucket
+    rng = np.random.default_rng(copies)
+    c = np.empty((copies + 400, 3), dtype=np.int32)
+    c[:copies] = (5, 5, 5)
+    c[copies:] = rng.integers(100000, 2000000, size=(400, 3))
+    c = c[rng.permutation(len(c))]
+    _check_arg_sort(c)
+
+
 def test_arg_sort_one_overfull_bucket_takes_the_radix_passes():
     rng = np.random.default_rng(77)
     c = rng.integers(0, 40, size=(50000, 3)).astype(np.int32)
