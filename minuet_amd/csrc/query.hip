@@ -32,6 +32,7 @@ constexpr int kWindowChunk = 4096;
 constexpr int kWindowPad = 64;            // sentinel keys behind a full chunk
 constexpr int kGroupSpan = 4;             // key span of one offset group
 constexpr int kGroupsInFlight = 3;
+constexpr int kDirectoryRows = 14000;     // 16-bit entries of the row directory (dynamic LDS)
 
 
 template <typename CT, typename BT>
@@ -72,17 +73,55 @@ __device__ __forceinline__ long long wave_lower_bound(const KeyReader<CT, BT> &s
   return lo;
 }
 
+// Settles the queries of one group against the candidates cand[0 .. span]
+// read from window position p on: writes the map entries this workgroup's
+// chunk is responsible for and counts the hits per offset.  The group and
+// member tables hold the same values for every lane; they are moved to scalar
+// registers, so that the loop, the row offsets of the map and the deltas are
+// scalar work.  d0 = q0 - base (wraps to a huge value when q0 < base, which
+// the range test then rejects like any other query outside the window).
+template <typename K, typename OT, bool kWholeWindow>
+__device__ __forceinline__ void settle_group(
+    const K (&cand)[kGroupSpan + 1], int p, unsigned long long q0, unsigned long long d0,
+    const int4 &group, long long c0, bool valid, unsigned long long first_key,
+    unsigned long long next_first, const int2 *s_members, unsigned *s_counts, bool count_hits,
+    OT *__restrict__ column, long long num_targets) {
+  constexpr unsigned long long kLimit = static_cast<unsigned long long>(static_cast<K>(~static_cast<K>(0)));
+  const int first_member = __builtin_amdgcn_readfirstlane(group.z);
+  const int members = __builtin_amdgcn_readfirstlane(group.w);
+  const OT found_base = static_cast<OT>(c0 + p);
+  for (int m = 0; m < members; ++m) {
+    const int2 member = s_members[first_member + m];
+    const unsigned step = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(member.x));
+    const int o = __builtin_amdgcn_readfirstlane(member.y);
+    const unsigned long long d = d0 + step;
+    bool mine = valid;
+    if (!kWholeWindow) {                       // several chunks: this one answers for its own key range only
+      const unsigned long long q = q0 + step;
+      mine = mine && q >= first_key && q < next_first;
+    }
+    const K q_rel = static_cast<K>(d);
+    int at = -1;
+#pragma unroll
+    for (int x = 0; x <= kGroupSpan; ++x) at = cand[x] == q_rel ? x : at;
+    const bool hit = mine && d < kLimit && at >= 0;
+    if (mine) column[static_cast<long long>(o) * num_targets] = hit ? found_base + static_cast<OT>(at) : static_cast<OT>(-1);
+    const unsigned hits = __popcll(__ballot(hit));
+    if (count_hits && hits != 0 && lane_id() == 0) atomicAdd(&s_counts[o], hits);
+  }
+}
+
 // Resolves every (offset, target) pair of the tile against the window chunk
 // staged in LDS as keys of type K relative to `base` (K = 32 bits when the
 // chunk's key range allows, which halves the LDS traffic of the searches).
 // A query outside [base, base + max K) cannot match and is forced to miss.
-template <typename K, typename OT>
+template <typename K, typename OT, bool kWholeWindow>
 __device__ __forceinline__ void resolve_chunk(
     const K *__restrict__ win, int top, unsigned long long base, long long c0,
-    unsigned long long key, bool valid, bool is_first, bool is_last,
-    unsigned long long first_key, unsigned long long next_first, const int4 *s_groups,
-    const int2 *s_members, int num_groups, unsigned *s_counts, bool count_hits, long long t,
-    long long num_targets, OT *__restrict__ kernel_map) {
+    unsigned long long key, bool valid, unsigned long long first_key, unsigned long long next_first,
+    const int4 *s_groups, const int2 *s_members, int num_groups, unsigned *s_counts, bool count_hits,
+    long long t, long long num_targets, OT *__restrict__ kernel_map) {
+  OT *column = kernel_map + t;
   constexpr unsigned long long kLimit = static_cast<unsigned long long>(static_cast<K>(~static_cast<K>(0)));
   for (int g0 = 0; g0 < num_groups; g0 += kGroupsInFlight) {
     // lower bound of the first query of up to three groups, in lockstep
@@ -116,26 +155,67 @@ __device__ __forceinline__ void resolve_chunk(
       K cand[kGroupSpan + 1];
 #pragma unroll
       for (int x = 0; x <= kGroupSpan; ++x) cand[x] = win[p + x];
-      for (int m = 0; m < group[j].w; ++m) {
-        const int2 member = s_members[group[j].z + m];
-        const unsigned long long q = q0[j] + static_cast<unsigned long long>(member.x);
-        const bool mine = valid && (is_first || q >= first_key) && (is_last || q < next_first);
-        const unsigned long long d = q - base;
-        const bool in_range = q >= base && d < kLimit;
-        const K q_rel = static_cast<K>(d);
-        int at = -1;
-#pragma unroll
-        for (int x = 0; x <= kGroupSpan; ++x) at = cand[x] == q_rel ? x : at;
-        const bool hit = mine && in_range && at >= 0;
-        const int o = member.y;
-        if (mine) {
-          kernel_map[static_cast<long long>(o) * num_targets + t] =
-              hit ? static_cast<OT>(c0 + p + at) : static_cast<OT>(-1);
-        }
-        const unsigned hits = __popcll(__ballot(hit));
-        if (count_hits && hits != 0 && lane_id() == 0) atomicAdd(&s_counts[o], hits);
-      }
+      settle_group<K, OT, kWholeWindow>(cand, p, q0[j], q0[j] - base, group[j], c0, valid, first_key,
+                                        next_first, s_members, s_counts, count_hits, column, num_targets);
     }
+  }
+}
+
+// The same with a row directory instead of the binary search.  Keys that
+// differ only in their last coordinate (a "row": same batch, same leading
+// coordinates) are neighbours in the window; dir[b] holds 1 + the window
+// position of the first key of row b (0: the row is empty), b = relative key
+// >> zbits.  All queries of a group lie in one row, so a group costs one
+// directory read and four candidate reads; only when the row is longer than
+// four keys and the queries may sit further on does a binary search inside
+// the row (at most zbits steps) follow.  Needs 32-bit relative keys whose
+// base is the start of a row, and at least 3 bits of last coordinate (then
+// the deltas of a group, at most kGroupSpan apart, never leave the row).
+template <typename OT, bool kWholeWindow>
+__device__ __forceinline__ void resolve_chunk_rows(
+    const unsigned *__restrict__ win, const unsigned short *__restrict__ dir, int len, int zbits,
+    unsigned num_rows, unsigned long long base, long long c0, unsigned long long key, bool valid,
+    unsigned long long first_key, unsigned long long next_first, const int4 *s_groups,
+    const int2 *s_members, int num_groups, unsigned *s_counts, bool count_hits, long long t,
+    long long num_targets, OT *__restrict__ kernel_map) {
+  OT *column = kernel_map + t;
+  for (int g = 0; g < num_groups; ++g) {
+    const int4 group = s_groups[g];
+    const unsigned long long first_delta =
+        static_cast<unsigned long long>(static_cast<unsigned>(group.x)) |
+        (static_cast<unsigned long long>(static_cast<unsigned>(group.y)) << 32);
+    const unsigned long long q0 = key + first_delta;
+    const unsigned long long d0 = q0 - base;
+    const unsigned long long row = d0 >> zbits;
+    const bool inside = q0 >= base && row < num_rows;
+    const unsigned start = inside ? dir[row] : 0u;
+    const unsigned q0_rel = static_cast<unsigned>(d0);
+    const unsigned q_last = q0_rel + static_cast<unsigned>(s_members[group.z + group.w - 1].x);
+    int p = start != 0 ? static_cast<int>(start) - 1 : 0;
+    unsigned cand[kGroupSpan + 1];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) cand[x] = win[p + x];
+    cand[4] = 0xffffffffu;
+    if (start != 0 && cand[3] < q_last && (cand[3] >> zbits) == row) {
+      // a long row whose first four keys do not cover the queries: the lower
+      // bound of the first query inside the row, then the usual span of
+      // candidates from there
+      int lo = p;
+      int hi = p + (1 << zbits) < len ? p + (1 << zbits) : len;      // zbits <= 24 here
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (win[mid] < q0_rel) {
+          lo = mid + 1;
+        } else {
+          hi = mid;
+        }
+      }
+      p = lo;
+#pragma unroll
+      for (int x = 0; x <= kGroupSpan; ++x) cand[x] = win[p + x];
+    }
+    settle_group<unsigned, OT, kWholeWindow>(cand, p, q0, d0, group, c0, valid, first_key, next_first,
+                                             s_members, s_counts, count_hits, column, num_targets);
   }
 }
 
@@ -163,14 +243,19 @@ template <typename CT, typename BT, typename OT>
 __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     KeyReader<CT, BT> src, KeyReader<CT, BT> tgt, Frame frame, const int *__restrict__ tables,
     CarriedTables carried, int num_groups, int num_offsets, long long delta_min, long long delta_max,
-    OT *__restrict__ kernel_map, unsigned *__restrict__ tile_counts, int num_tiles) {
+    OT *__restrict__ kernel_map, unsigned *__restrict__ tile_counts, int num_tiles, int dir_rows) {
   extern __shared__ __align__(16) unsigned s_dynamic[];
   __shared__ unsigned long long win[kWindowChunk + kWindowPad];
   __shared__ long long s_bounds[2];
   // dynamic LDS: [group table: 4 words each][member table: 2 words each][hit counts]
+  // [row directory: dir_rows 16-bit entries]
   const int4 *s_groups = reinterpret_cast<const int4 *>(s_dynamic);
   const int2 *s_members = reinterpret_cast<const int2 *>(s_dynamic + 4 * num_groups);
   unsigned *s_counts = s_dynamic + 4 * num_groups + 2 * num_offsets;
+  unsigned *s_dir_words = s_counts + num_offsets;
+  unsigned short *s_dir = reinterpret_cast<unsigned short *>(s_dir_words);
+  // last coordinate: the least significant field of a key
+  const int zbits = frame.width[frame.ndim - 1];
 
   const int tid = threadIdx.x;
   const int w = tid >> 6;
@@ -227,11 +312,27 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     const unsigned long long first_key = len > 0 ? src(c0, frame) : ~0ull;
     const unsigned long long last_key = len > 0 ? src(c1 - 1, frame) : 0ull;
     const unsigned long long next_first = c1 < w_hi ? src(c1, frame) : ~0ull;
-    const bool narrow = len > 0 && last_key - first_key < 0xffffffffull;
+    // relative keys count from the start of the first key's row
+    const bool rows_possible = dir_rows > 0 && zbits >= 3 && zbits <= 24;
+    const unsigned long long base = rows_possible ? first_key & ~((1ull << zbits) - 1ull) : first_key;
+    const bool narrow = len > 0 && last_key - base < 0xffffffffull;
+    const unsigned long long num_rows = narrow && rows_possible ? ((last_key - base) >> zbits) + 1ull : 0ull;
+    const bool by_rows = num_rows != 0 && num_rows <= static_cast<unsigned long long>(dir_rows);
     if (narrow) {
       unsigned *win32 = reinterpret_cast<unsigned *>(win);
+      if (by_rows) {
+        for (int i = tid; i < static_cast<int>((num_rows + 1) >> 1); i += kQueryThreads) s_dir_words[i] = 0u;
+      }
       for (int i = tid; i < fill; i += kQueryThreads) {
-        win32[i] = i < len ? static_cast<unsigned>(src(c0 + i, frame) - first_key) : 0xffffffffu;
+        win32[i] = i < len ? static_cast<unsigned>(src(c0 + i, frame) - base) : 0xffffffffu;
+      }
+      if (by_rows) {
+        __syncthreads();
+        // the first key of every row enters the directory
+        for (int i = tid; i < len; i += kQueryThreads) {
+          const unsigned row = win32[i] >> zbits;
+          if (i == 0 || (win32[i - 1] >> zbits) != row) s_dir[row] = static_cast<unsigned short>(i + 1);
+        }
       }
     } else {
       for (int i = tid; i < fill; i += kQueryThreads) {
@@ -239,18 +340,33 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
       }
     }
     __syncthreads();
-    const bool is_first = c == 0;
-    const bool is_last = c == num_chunks - 1;
-    if (narrow) {
-      resolve_chunk<unsigned, OT>(reinterpret_cast<const unsigned *>(win), top, first_key, c0, key, valid,
-                                  is_first, is_last, first_key, next_first, s_groups, s_members,
-                                  num_groups, s_counts, tile_counts != nullptr, t, num_targets,
-                                  kernel_map);
-    } else {
-      resolve_chunk<unsigned long long, OT>(win, top, 0ull, c0, key, valid, is_first, is_last, first_key,
-                                            next_first, s_groups, s_members, num_groups, s_counts,
-                                            tile_counts != nullptr, t, num_targets, kernel_map);
+    // a chunk answers for the queries between its first key and the first key
+    // of the next chunk; a window of one chunk answers for all of them
+    const unsigned long long answers_from = c == 0 ? 0ull : first_key;
+    const unsigned long long answers_to = c == num_chunks - 1 ? ~0ull : next_first;
+    const bool counting = tile_counts != nullptr;
+#define MNT_RESOLVE(WHOLE)                                                                         \
+    if (by_rows) {                                                                                 \
+      resolve_chunk_rows<OT, WHOLE>(reinterpret_cast<const unsigned *>(win), s_dir, len, zbits,    \
+                                    static_cast<unsigned>(num_rows), base, c0, key, valid,         \
+                                    answers_from, answers_to, s_groups, s_members, num_groups,     \
+                                    s_counts, counting, t, num_targets, kernel_map);               \
+    } else if (narrow) {                                                                           \
+      resolve_chunk<unsigned, OT, WHOLE>(reinterpret_cast<const unsigned *>(win), top, base, c0,   \
+                                         key, valid, answers_from, answers_to, s_groups,           \
+                                         s_members, num_groups, s_counts, counting, t,             \
+                                         num_targets, kernel_map);                                 \
+    } else {                                                                                       \
+      resolve_chunk<unsigned long long, OT, WHOLE>(win, top, 0ull, c0, key, valid, answers_from,   \
+                                                   answers_to, s_groups, s_members, num_groups,    \
+                                                   s_counts, counting, t, num_targets, kernel_map); \
     }
+    if (num_chunks == 1) {
+      MNT_RESOLVE(true)
+    } else {
+      MNT_RESOLVE(false)
+    }
+#undef MNT_RESOLVE
   }
   if (tile_counts != nullptr) {
     __syncthreads();
@@ -458,6 +574,7 @@ struct QueryPlan {
   std::vector<int> tables;               // group and member tables of query_kernel
   int num_groups;
   long long delta_min, delta_max;
+  bool groups_in_rows;                   // the offsets of every group differ in the last coordinate only
 };
 
 // Builds the packing frame from the coordinate bounds of sources and targets
@@ -530,6 +647,15 @@ static QueryPlan make_plan(const long long *src_bounds, const long long *tgt_bou
       plan.tables[4 * plan.num_groups + 2 * i + 1] = keyed[i].second;
     }
   }
+  plan.groups_in_rows = true;
+  for (int g = 0; g < plan.num_groups; ++g) {
+    const int64_t first = keyed[group_start[g]].second;
+    for (int i = group_start[g] + 1; i < group_start[g + 1]; ++i) {
+      for (int k = 0; k + 1 < ndim; ++k) {
+        if (offsets[keyed[i].second * ndim + k] != offsets[first * ndim + k]) plan.groups_in_rows = false;
+      }
+    }
+  }
   plan.delta_min = num_offsets > 0 ? keyed.front().first : 0;
   plan.delta_max = num_offsets > 0 ? keyed.back().first : 0;
   return plan;
@@ -573,13 +699,18 @@ static void launch_query(const QueryArgs &a, const QueryPlan &plan, const int *d
                         static_cast<int>(a.num_batches), a.num_sources};
   KeyReader<CT, BT> tgt{static_cast<const CT *>(a.targets), static_cast<const BT *>(a.target_batch_dims),
                         static_cast<int>(a.num_batches), a.num_targets};
-  const size_t dyn = sizeof(unsigned) * (plan.tables.size() + static_cast<size_t>(num_offsets) + 4);
+  // room for the row directory where the last coordinate is wide enough for it
+  const bool small_tables = plan.tables.size() * sizeof(int) <= 2048;
+  const int dir_rows =
+      plan.groups_in_rows && small_tables && plan.frame.width[plan.frame.ndim - 1] >= 3 ? kDirectoryRows : 0;
+  const size_t dyn = sizeof(unsigned) * (plan.tables.size() + static_cast<size_t>(num_offsets) + 4) +
+                     sizeof(unsigned short) * static_cast<size_t>(dir_rows);
   CarriedTables carried;
   memset(&carried, 0, sizeof(carried));
   if (d_tables == nullptr) memcpy(carried.v, plan.tables.data(), sizeof(int) * plan.tables.size());
   query_kernel<CT, BT, OT><<<num_tiles, kQueryThreads, dyn, stream>>>(
       src, tgt, plan.frame, d_tables, carried, plan.num_groups, num_offsets, plan.delta_min,
-      plan.delta_max, kernel_map, tile_counts, num_tiles);
+      plan.delta_max, kernel_map, tile_counts, num_tiles, dir_rows);
   check_launch("query_kernel");
 }
 
