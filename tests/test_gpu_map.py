@@ -53,6 +53,13 @@ def test_arg_sort_large_two_item_paths():
     np.testing.assert_array_equal(host(got).astype(np.int64), orc.arg_sort_coordinates(c))
 
 
+def test_arg_sort_beyond_the_bucket_sort_takes_the_radix_passes():
+    # more rows than the bucket sort accepts: radix passes with 16 keys per thread
+    c = random_cloud(2_200_000, 1200, seed=10, lo=-600)
+    got = F.arg_sort_coordinates(dev(c))
+    np.testing.assert_array_equal(host(got).astype(np.int64), orc.arg_sort_coordinates(c))
+
+
 def _check_arg_sort(c, bd=None):
     got = F.arg_sort_coordinates(dev(c), batch_dims=None if bd is None else dev(bd))
     np.testing.assert_array_equal(host(got).astype(np.int64), orc.arg_sort_coordinates(c, bd))
