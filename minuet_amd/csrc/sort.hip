@@ -579,10 +579,11 @@ void radix_sort_pairs(unsigned long long *&keys, unsigned *&vals, unsigned long 
 // and the order inside a bucket needs no stability from the dealing step:
 // cursors handed out by atomics will do.
 //
-// The bucket histogram, its scan and the dealing step are enqueued behind the
-// bounds kernels, before the host waits for the bounds; the kernels work out
-// the key layout from the bounds in device memory.  The host then learns the
-// bounds, the largest bucket and the number of ranking workgroups at once and
+// The bucket histogram, its scan and the dealing step are enqueued right
+// behind bounds_kernel, with no wait in between: the histogram kernel folds
+// the partial bounds itself and the kernels work out the key layout on the
+// device.  The host waits once, for the scan kernel, which hands it the
+// bounds, the largest bucket and the number of ranking workgroups, and
 // launches the ranking while the dealing step still runs.  A cloud with a
 // bucket beyond the LDS capacity (strong clustering) takes the radix passes
 // instead; the dealing step sees that for itself and does nothing.
@@ -755,8 +756,9 @@ __device__ __forceinline__ unsigned bucket_pieces(unsigned m) {
 
 // One workgroup: bucket starts (exclusive scan of the totals, starts[buckets]
 // = n), the cursors of the dealing step (a copy of the starts), the list of
-// (bucket, chunk of rows) pairs the ranking kernel runs over, info[1] = whether the bucket sort goes ahead, and
-// for the host the largest bucket (all ones when the layout does not hold)
+// (bucket, chunk of rows) pairs the ranking kernel runs over, info[1] =
+// whether the bucket sort goes ahead, and for the host the bounds, the
+// largest bucket (all ones when the layout does not hold)
 // and the number of pairs.
 // chunks[i] = {first row of the bucket, rows of the bucket | mode << 13 |
 // chunk << 16}.

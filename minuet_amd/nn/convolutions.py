@@ -112,6 +112,16 @@ class KernelMapCache(object):
         self._coordinates_cache[target_stride] = entry
         return entry
 
+    def coordinates_at(self, coordinates: torch.Tensor, stride, batch_dims: Optional[torch.Tensor]):
+        """What ``get_target_coordinates`` returns for a layer of stride 1: the
+        entry of the level ``stride`` (a tuple of ints), which these coordinates
+        open if it is new."""
+        entry = self._coordinates_cache.get(stride)
+        if entry is None:
+            entry = (coordinates, stride, batch_dims)
+            self._coordinates_cache[stride] = entry
+        return entry
+
     def _map_key(self, ndim, source_stride, target_stride, kernel_size, kernel_dilation, transposed):
         raw = (ndim, source_stride, target_stride, kernel_size, kernel_dilation, transposed)
         try:
@@ -233,15 +243,17 @@ class KernelMapCache(object):
                        else source_batch_dims.dtype)
         cast = (lambda t: t) if index_dtype == torch.int32 else (lambda t: t.to(index_dtype))
         sizes = cast(built["sizes"])
-        sizes.host_sizes = tuple(int(v) for v in built["sizes_host"])
+        # host copies as the library takes them (contiguous int64), made once
+        sizes.host_sizes = np.ascontiguousarray(built["sizes_host"], dtype=np.int64)
         order = cast(built["order"]) if reorder else None
         if order is not None:
-            order.host_order = tuple(int(v) for v in built["order_host"])
+            order.host_order = np.ascontiguousarray(built["order_host"], dtype=np.int64)
         source_masks, target_masks = cast(built["source_masks"]), cast(built["target_masks"])
         # buffer row -> feature row on either side of the map: what a layer
         # (forward or transposed) gathers through
         source_masks.gather_index = built["in_idx"]
         target_masks.gather_index = built["out_idx"]
+        built["in_idx"].num_hits = built["out_idx"].num_hits = int(sizes.host_sizes.sum())
         # source row per (offset, target) in the original offset order: what
         # the single-kernel dataflow walks
         target_masks.kernel_map = built["kernel_map"]
@@ -300,6 +312,7 @@ class SparseConv(Module):
         self._identity_map = None
         self._packed = None
         self._routes = dict()
+        self._trivial = None
 
     @property
     def _allow_shortcut_matmul(self) -> bool:
@@ -313,7 +326,20 @@ class SparseConv(Module):
 
     @property
     def is_trivial(self) -> bool:
-        return all(x == 1 for x in self.stride + self.dilation + self.kernel_size)
+        return self._shape_flags()[0]
+
+    @property
+    def _unit_stride(self) -> bool:
+        return self._shape_flags()[1]
+
+    def _shape_flags(self):
+        """(1x1x1 kernel with stride and dilation 1, stride 1), worked out once
+        per setting of the three tuples."""
+        shape = (self.stride, self.dilation, self.kernel_size)
+        if self._trivial is None or self._trivial[0] != shape:
+            self._trivial = (shape, (all(x == 1 for x in self.stride + self.dilation + self.kernel_size),
+                                     all(x == 1 for x in self.stride)))
+        return self._trivial[1]
 
     def extra_repr(self) -> str:
         parts = [f"{self.in_channels}, {self.out_channels}, kernel_size={self.kernel_size}"]
@@ -495,8 +521,9 @@ class SparseConv(Module):
                 and self._tunable_config.get("dataflow", "auto") != "gather_gemm_scatter"
                 and features.dtype == weights.dtype
                 and _C.implicit_forward_supported(self.in_channels, self.out_channels, weights.dtype)
+                # measured against torch.mm plus a separate epilogue pass up to these widths;
                 # wider layers are plain library GEMM territory
-                and self.in_channels * weights.dtype.itemsize <= 128 and self.out_channels <= 128):
+                and self.in_channels * weights.dtype.itemsize <= 512 and self.out_channels <= 128):
             rows = features.shape[0]
             identity = self._identity_map
             if identity is None or identity.shape[1] < rows or identity.device != features.device:
@@ -528,10 +555,14 @@ class SparseConv(Module):
             cache = self._kernel_map_cache
             if cache is None:
                 raise ValueError("Kernel map cache must be specified")
-            coordinates, stride, batch_dims = cache.get_target_coordinates(
-                transposed=self.transposed, source_coordinates=inputs.C,
-                source_batch_dims=inputs.batch_dims, source_stride=inputs.stride,
-                kernel_stride=self.stride)
+            if self._unit_stride and type(inputs.stride) is tuple:
+                coordinates, stride, batch_dims = cache.coordinates_at(inputs.C, inputs.stride,
+                                                                       inputs.batch_dims)
+            else:
+                coordinates, stride, batch_dims = cache.get_target_coordinates(
+                    transposed=self.transposed, source_coordinates=inputs.C,
+                    source_batch_dims=inputs.batch_dims, source_stride=inputs.stride,
+                    kernel_stride=self.stride)
             map_args = dict(transposed=self.transposed, source_coordinates=inputs.C,
                             source_stride=inputs.stride, source_batch_dims=inputs.batch_dims,
                             target_coordinates=coordinates, target_stride=stride,

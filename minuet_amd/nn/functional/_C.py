@@ -705,7 +705,7 @@ def _host_sizes_arg(sizes_host, num_offsets):
         arr = np.ascontiguousarray(np.asarray(sizes_host, dtype=np.int64))
     if arr.shape[0] != num_offsets:
         _fail("host copy of kernel_map_sizes has the wrong length")
-    return arr, arr.ctypes.data_as(_pi64)
+    return arr, ctypes.cast(arr.__array_interface__["data"][0], _pi64)
 
 
 def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: int,
@@ -749,7 +749,9 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
     if gather_index is not None:
         if gather_index.dtype != torch.int32 or gather_index.device != device:
             _fail("gather_index must be an int32 tensor on the device of the features")
-        if kernel_map_sizes_host is None or gather_index.numel() != int(np.sum(kernel_map_sizes_host)):
+        hits = getattr(gather_index, "num_hits", None)      # noted by KernelMapCache next to the index
+        if kernel_map_sizes_host is None or gather_index.numel() != (
+                int(np.sum(kernel_map_sizes_host)) if hits is None else hits):
             _fail("gather_index needs the host sizes and one entry per kernel map hit")
         gather_index = gather_index.contiguous()
     ep = Epilogue() if epilogue is None else epilogue.checked(T, N, weights.dtype, device)
@@ -759,10 +761,7 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
         if kernel_map_order is not None:
             if kernel_map_order_host is None:
                 _fail("packed weights need the host copy of kernel_map_order")
-            keep_order, _ = _host_sizes_arg(kernel_map_order_host, O)
-            if keep_order.shape[0] != O:
-                _fail("host copy of kernel_map_order has the wrong length")
-            order_ptr = keep_order.ctypes.data_as(_pi64)
+            keep_order, order_ptr = _host_sizes_arg(kernel_map_order_host, O)
     with _on(device):
         _check(load_library().mnt_sparse_convolution_forward_fused(
             int(gather_tile_size), int(scatter_tile_size), 1 if allow_shortcut_matmul else 0,

@@ -26,9 +26,14 @@ __all__ = ["batch_norm_affine", "conv_norm_act", "FusedSequential", "fuse_conv_n
 def batch_norm_affine(norm: torch.nn.BatchNorm1d):
     """``(scale, shift)`` in fp32 with ``norm(x) == x * scale + shift`` in
     evaluation mode.  Cached on the module until one of its tensors changes."""
-    tensors = (norm.running_mean, norm.running_var, norm.weight, norm.bias)
-    key = tuple((t.data_ptr(), t._version) if t is not None else None for t in tensors)
-    cached = getattr(norm, "_minuet_affine", None)
+    # straight from the module's dictionaries: nn.Module.__getattr__ is the slow way in
+    buffers, parameters = norm._buffers, norm._parameters
+    mean, var = buffers["running_mean"], buffers["running_var"]
+    weight, bias = parameters["weight"], parameters["bias"]
+    key = (mean.data_ptr(), mean._version, var.data_ptr(), var._version,
+           None if weight is None else (weight.data_ptr(), weight._version),
+           None if bias is None else (bias.data_ptr(), bias._version))
+    cached = norm.__dict__.get("_minuet_affine")
     if cached is not None and cached[0] == key:
         return cached[1], cached[2]
     with torch.no_grad():
@@ -38,7 +43,7 @@ def batch_norm_affine(norm: torch.nn.BatchNorm1d):
         shift = -norm.running_mean.float() * scale
         if norm.bias is not None:
             shift = shift + norm.bias.float()
-    norm._minuet_affine = (key, scale, shift)
+    norm.__dict__["_minuet_affine"] = (key, scale, shift)
     return scale, shift
 
 
@@ -54,7 +59,7 @@ def _activation_of(module):
 
 def _foldable(norm) -> bool:
     return (isinstance(norm, torch.nn.BatchNorm1d) and not norm.training
-            and norm.running_mean is not None)
+            and norm._buffers.get("running_mean") is not None)
 
 
 def conv_norm_act(conv: SparseConv, norm: Optional[torch.nn.BatchNorm1d], act: Optional[nn.Module],
