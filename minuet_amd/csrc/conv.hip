@@ -433,7 +433,7 @@ struct MetaInArguments {
   __device__ __forceinline__ int operator()(int i) const { return table->v[meta_at + i]; }
 };
 
-template <typename T, typename TC, int NB, bool VEC, typename Meta>
+template <typename T, typename TC, int NB, bool VEC, int CH, typename Meta>
 __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *__restrict__ c,
                                                   const T *__restrict__ wt, const Meta &entry, int K,
                                                   int N, int Kp, int Np,
@@ -441,33 +441,59 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
   constexpr int EPC = 16 / static_cast<int>(sizeof(T));        // elements per 16-byte piece
   constexpr int KC = kChunkBytes / static_cast<int>(sizeof(T));
   constexpr int TN = NB * 32;
-  __shared__ __align__(16) unsigned char b_lds[TN * kLdsRowBytes];
+  constexpr int kLdsChunks = CH > 0 ? CH : 1;
+  // the output pass turns one 32 x 32 block per wavefront around in the same memory
+  constexpr int kTurnRow = 32 * static_cast<int>(sizeof(TC)) + 16;
+  constexpr int kTurnBytes = 32 * kTurnRow;
+  constexpr int kWeightBytes = kLdsChunks * TN * kLdsRowBytes;
+  constexpr int kLdsBytes = kWeightBytes > 4 * kTurnBytes ? kWeightBytes : 4 * kTurnBytes;
+  __shared__ __align__(16) unsigned char b_lds[kLdsBytes];
 
   const int G = entry(0);
   const int at_prefix = 1, at_start = at_prefix + G + 1, at_rows = at_start + G + 1, at_weight = at_rows + G,
             at_list = at_weight + G;
 
-  const int tile = blockIdx.x;
-  int lo = 0, hi = G - 1;
-  while (lo < hi) {
-    const int mid = (lo + hi + 1) >> 1;
-    if (entry(at_prefix + mid) <= tile) {
-      lo = mid;
-    } else {
-      hi = mid - 1;
-    }
-  }
-  const int g = lo;
-  const int r0 = (tile - entry(at_prefix + g)) * kGemmRows;
-  const int valid = min(kGemmRows, entry(at_rows + g) - r0);
-  const long long row_base = static_cast<long long>(entry(at_start + g)) + r0;
-  const int n0 = blockIdx.y * TN;
-  const T *w_base = wt + (static_cast<long long>(entry(at_weight + g)) * Np + n0) * Kp;
-  const int list_at = entry(at_list + g);
-
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wv = tid >> 6;
+  const int tile = blockIdx.x;
+  int g_prefix, g_rows, g_start, g_weight, g_list;
+  if (G <= kWave) {
+    // One trip to memory instead of a search of dependent reads: lane i
+    // fetches the entries of group i, a ballot over the tile prefix finds the
+    // group of this tile, and its lane hands the entries to everyone.
+    const int i = min(lane, G - 1);
+    const int prefix = entry(at_prefix + i), rows = entry(at_rows + i), start = entry(at_start + i),
+              weight = entry(at_weight + i), list = entry(at_list + i);
+    const int g = __popcll(__ballot(lane < G && prefix <= tile)) - 1;
+    g_prefix = __builtin_amdgcn_readlane(prefix, g);
+    g_rows = __builtin_amdgcn_readlane(rows, g);
+    g_start = __builtin_amdgcn_readlane(start, g);
+    g_weight = __builtin_amdgcn_readlane(weight, g);
+    g_list = __builtin_amdgcn_readlane(list, g);
+  } else {
+    int lo = 0, hi = G - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (entry(at_prefix + mid) <= tile) {
+        lo = mid;
+      } else {
+        hi = mid - 1;
+      }
+    }
+    g_prefix = entry(at_prefix + lo);
+    g_rows = entry(at_rows + lo);
+    g_start = entry(at_start + lo);
+    g_weight = entry(at_weight + lo);
+    g_list = entry(at_list + lo);
+  }
+  const int r0 = (tile - g_prefix) * kGemmRows;
+  const int valid = min(kGemmRows, g_rows - r0);
+  const long long row_base = static_cast<long long>(g_start) + r0;
+  const int n0 = blockIdx.y * TN;
+  const T *w_base = wt + (static_cast<long long>(g_weight) * Np + n0) * Kp;
+  const int list_at = g_list;
+
   const int r = lane & 31;
   const int h = lane >> 5;
   const int row = wv * 32 + r;
@@ -490,8 +516,6 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
   // chunk i+1 are loaded into registers while chunk i is multiplied.
   constexpr int kSteps = kChunkBytes / 32;
   constexpr int kWPieces = (TN * 8 + kGemmBlock - 1) / kGemmBlock;
-  uint4 frag[kSteps], frag_next[kSteps];
-  uint4 wpiece[kWPieces];
 
   auto load_a = [&](int k0, uint4 (&dst)[kSteps]) {
 #pragma unroll
@@ -512,7 +536,7 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
       dst[kk] = v;
     }
   };
-  auto load_w = [&](int k0) {
+  auto load_w = [&](int k0, uint4 (&wpiece)[kWPieces]) {
 #pragma unroll
     for (int i = 0; i < kWPieces; ++i) {
       const int piece = tid + i * kGemmBlock;
@@ -526,39 +550,110 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
     }
   };
 
-  load_a(0, frag);
-  load_w(0);
-  for (int k0 = 0; k0 < Kp; k0 += KC) {
-    if (k0 > 0) __syncthreads();                   // previous chunk of W^T fully consumed
+  auto store_w = [&](int chunk, const uint4 (&wpiece)[kWPieces]) {
 #pragma unroll
     for (int i = 0; i < kWPieces; ++i) {
       const int piece = tid + i * kGemmBlock;
       if (piece < TN * 8) {
-        *reinterpret_cast<uint4 *>(b_lds + (piece >> 3) * kLdsRowBytes + (piece & 7) * 16) = wpiece[i];
+        *reinterpret_cast<uint4 *>(b_lds + chunk * (TN * kLdsRowBytes) + (piece >> 3) * kLdsRowBytes +
+                                   (piece & 7) * 16) = wpiece[i];
       }
     }
-    __syncthreads();
-    const bool more = k0 + KC < Kp;
-    if (more) {
-      load_a(k0 + KC, frag_next);
-      load_w(k0 + KC);
-    }
+  };
+  auto multiply = [&](int chunk, const uint4 (&frag)[kSteps]) {
 #pragma unroll
     for (int kk = 0; kk < kSteps; ++kk) {
       const int off = kk * 32 + h * 16;
 #pragma unroll
       for (int b = 0; b < NB; ++b) {
-        const uint4 chan_frag = *reinterpret_cast<const uint4 *>(b_lds + (b * 32 + r) * kLdsRowBytes + off);
+        const uint4 chan_frag = *reinterpret_cast<const uint4 *>(b_lds + chunk * (TN * kLdsRowBytes) +
+                                                                 (b * 32 + r) * kLdsRowBytes + off);
         acc[b] = Mfma<T>::run(chan_frag, frag[kk], acc[b]);
       }
     }
-    if (more) {
+  };
+
+  if constexpr (CH > 0) {
+    // K of CH chunks (Kp == CH * KC): every load of the tile is issued at
+    // once, so the tile pays for one trip to memory instead of one per chunk.
+    uint4 frags[CH][kSteps];
+    uint4 wpieces[CH][kWPieces];
 #pragma unroll
-      for (int kk = 0; kk < kSteps; ++kk) frag[kk] = frag_next[kk];
+    for (int c = 0; c < CH; ++c) load_w(c * KC, wpieces[c]);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) load_a(c * KC, frags[c]);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) store_w(c, wpieces[c]);
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < CH; ++c) multiply(c, frags[c]);
+  } else {
+    uint4 frag[kSteps], frag_next[kSteps];
+    uint4 wpiece[kWPieces];
+    load_a(0, frag);
+    load_w(0, wpiece);
+    for (int k0 = 0; k0 < Kp; k0 += KC) {
+      if (k0 > 0) __syncthreads();                   // previous chunk of W^T fully consumed
+      store_w(0, wpiece);
+      __syncthreads();
+      const bool more = k0 + KC < Kp;
+      if (more) {
+        load_a(k0 + KC, frag_next);
+        load_w(k0 + KC, wpiece);
+      }
+      multiply(0, frag);
+      if (more) {
+#pragma unroll
+        for (int kk = 0; kk < kSteps; ++kk) frag[kk] = frag_next[kk];
+      }
     }
   }
 
-  if (row_ok) {
+  // Output.  A lane holds 4 consecutive channels of one row per accumulator
+  // group, and neighbouring lanes hold different rows: stored as they are,
+  // every lane's 8 or 16 bytes are a write request of their own.  Where rows
+  // are whole 16-byte pieces each wavefront turns its 32 x 32 blocks around in
+  // LDS first, so that a store instruction covers rows in contiguous pieces of
+  // 64 bytes (16-bit buffers) or 128 (32-bit).
+  if (VEC && (static_cast<long long>(N) * sizeof(TC)) % 16 == 0) {
+    constexpr int EPV = 16 / static_cast<int>(sizeof(TC));       // channels per 16-byte piece
+    constexpr int kRowPieces = 32 / EPV;                          // pieces of a block's row
+    constexpr int kPieces = 32 * kRowPieces / kWave;              // per lane and block
+    __syncthreads();                                              // every product has read its weights
+    unsigned char *turn = b_lds + wv * kTurnBytes;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      if (n0 + b * 32 >= N) break;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        TC four[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) four[x] = static_cast<TC>(acc[b][q * 4 + x]);
+        unsigned char *at = turn + r * kTurnRow + (q * 8 + h * 4) * static_cast<int>(sizeof(TC));
+        if (sizeof(TC) == 2) {
+          *reinterpret_cast<uint2 *>(at) = *reinterpret_cast<const uint2 *>(four);
+        } else {
+          *reinterpret_cast<uint4 *>(at) = *reinterpret_cast<const uint4 *>(four);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int i = 0; i < kPieces; ++i) {
+        const int piece = lane + i * kWave;
+        const int pr = piece / kRowPieces, part = piece % kRowPieces;
+        const int ch = n0 + b * 32 + part * EPV;
+        const uint4 v = *reinterpret_cast<const uint4 *>(turn + pr * kTurnRow + part * 16);
+        if (wv * 32 + pr < valid && ch < N) {                     // N % EPV == 0: a piece is all in or all out
+          *reinterpret_cast<uint4 *>(c + (row_base + wv * 32 + pr) * N + ch) = v;
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+  } else if (row_ok) {
     TC *dst = c + (row_base + row) * N;
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
@@ -585,16 +680,16 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
   }
 }
 
-template <typename T, typename TC, int NB, bool VEC>
+template <typename T, typename TC, int NB, bool VEC, int CH>
 __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
     const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt,
     const int *__restrict__ meta, int K, int N, int Kp, int Np,
     const int *__restrict__ gather_index) {
-  grouped_gemm_body<T, TC, NB, VEC>(a, c, wt, MetaInMemory{meta}, K, N, Kp, Np, gather_index);
+  grouped_gemm_body<T, TC, NB, VEC, CH>(a, c, wt, MetaInMemory{meta}, K, N, Kp, Np, gather_index);
 }
 
 // The same with the tables as a by-value argument.
-template <typename T, typename TC, int NB, bool VEC>
+template <typename T, typename TC, int NB, bool VEC, int CH>
 __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_riding_kernel(
     const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt, int K, int N, int Kp, int Np,
     const int *__restrict__ gather_index, PlanChunk table, int table_count, int meta_at,
@@ -602,8 +697,8 @@ __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_riding_kernel(
   if (blockIdx.x == 0 && blockIdx.y == 0) {
     for (int i = threadIdx.x; i < table_count; i += kGemmBlock) table_out[i] = table.v[i];
   }
-  grouped_gemm_body<T, TC, NB, VEC>(a, c, wt, MetaInArguments{&table, meta_at}, K, N, Kp, Np,
-                                    gather_index);
+  grouped_gemm_body<T, TC, NB, VEC, CH>(a, c, wt, MetaInArguments{&table, meta_at}, K, N, Kp, Np,
+                                        gather_index);
 }
 
 // ---------------------------------------------------------- host launchers ----
@@ -751,23 +846,40 @@ static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int 
                            int Kp, int Np, bool vec, const int *gather_index, const RidingTable &riding,
                            hipStream_t stream) {
   dim3 grid(num_tiles, static_cast<unsigned>(div_ceil(Np, NB * 32)));
+  // rows of one or two chunks are loaded whole, ahead of the first product
+  const int chunks = Kp / (kChunkBytes / static_cast<int>(sizeof(T)));
+  const int held = vec && chunks <= 2 ? chunks : 0;
   if (riding.ints != nullptr) {
     PlanChunk chunk;
     const int count = static_cast<int>(riding.ints->size());
     std::memcpy(chunk.v, riding.ints->data(), count * sizeof(int));
-    if (vec) {
-      grouped_gemm_riding_kernel<T, TC, NB, true><<<grid, kGemmBlock, 0, stream>>>(
-          a, c, wt, K, N, Kp, Np, gather_index, chunk, count, riding.meta_at, riding.out);
+#define MNT_RIDING(VEC, CH)                                                                 \
+  grouped_gemm_riding_kernel<T, TC, NB, VEC, CH><<<grid, kGemmBlock, 0, stream>>>(          \
+      a, c, wt, K, N, Kp, Np, gather_index, chunk, count, riding.meta_at, riding.out)
+    if (held == 1) {
+      MNT_RIDING(true, 1);
+    } else if (held == 2) {
+      MNT_RIDING(true, 2);
+    } else if (vec) {
+      MNT_RIDING(true, 0);
     } else {
-      grouped_gemm_riding_kernel<T, TC, NB, false><<<grid, kGemmBlock, 0, stream>>>(
-          a, c, wt, K, N, Kp, Np, gather_index, chunk, count, riding.meta_at, riding.out);
+      MNT_RIDING(false, 0);
     }
-  } else if (vec) {
-    grouped_gemm_kernel<T, TC, NB, true><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np,
-                                                                          gather_index);
+#undef MNT_RIDING
   } else {
-    grouped_gemm_kernel<T, TC, NB, false><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np,
-                                                                           gather_index);
+#define MNT_PLAIN(VEC, CH)                                                                  \
+  grouped_gemm_kernel<T, TC, NB, VEC, CH><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np, \
+                                                                           gather_index)
+    if (held == 1) {
+      MNT_PLAIN(true, 1);
+    } else if (held == 2) {
+      MNT_PLAIN(true, 2);
+    } else if (vec) {
+      MNT_PLAIN(true, 0);
+    } else {
+      MNT_PLAIN(false, 0);
+    }
+#undef MNT_PLAIN
   }
 }
 

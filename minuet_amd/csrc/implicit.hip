@@ -14,7 +14,7 @@
 // are along the sorted target order.  Sums are kept in fp32 across all offsets
 // in ascending offset order and rounded once, after the epilogue.
 //
-// Rows wider than one step of K (128 or 256 bytes) are walked in chunks: the
+// Rows wider than one step of K (128 bytes) are walked in chunks: the
 // pipeline's unit is then an (offset, chunk) pair instead of an offset.  More
 // than 128 output channels are split into groups of 128 over blockIdx.y, each
 // group reading the source rows again (through L2).
@@ -95,6 +95,43 @@ __device__ __forceinline__ void finish_four(float (&v)[4], const Epilogue &ep, l
   *reinterpret_cast<V *>(out + (t * N + ch) * static_cast<long long>(sizeof(T))) = raw;
 }
 
+// The same for one 16-byte piece of an output row (E = 16 / sizeof(T)
+// consecutive channels from `ch` on), its sums given in fp32.
+template <typename T, int E>
+__device__ __forceinline__ void finish_piece(float (&v)[E], const Epilogue &ep, long long t, int ch, int N,
+                                             unsigned char *__restrict__ out) {
+  if (ep.scale != nullptr) {
+#pragma unroll
+    for (int x = 0; x < E; ++x) v[x] *= ep.scale[ch + x];
+  }
+  if (ep.shift != nullptr) {
+#pragma unroll
+    for (int x = 0; x < E; ++x) v[x] += ep.shift[ch + x];
+  }
+  if (ep.residual != nullptr) {
+    const uint4 raw = *reinterpret_cast<const uint4 *>(static_cast<const unsigned char *>(ep.residual) +
+                                                       (t * N + ch) * static_cast<long long>(sizeof(T)));
+    const T *e = reinterpret_cast<const T *>(&raw);
+#pragma unroll
+    for (int x = 0; x < E; ++x) v[x] += to_float(e[x]);
+  }
+  if (ep.activation == MNT_ACT_RELU) {
+#pragma unroll
+    for (int x = 0; x < E; ++x) v[x] = fmaxf(v[x], 0.0f);
+  } else if (ep.activation == MNT_ACT_LEAKY_RELU) {
+#pragma unroll
+    for (int x = 0; x < E; ++x) v[x] = v[x] > 0.0f ? v[x] : v[x] * ep.slope;
+  } else if (ep.activation == MNT_ACT_RELU6) {
+#pragma unroll
+    for (int x = 0; x < E; ++x) v[x] = fminf(fmaxf(v[x], 0.0f), 6.0f);
+  }
+  uint4 raw;
+  T *e = reinterpret_cast<T *>(&raw);
+#pragma unroll
+  for (int x = 0; x < E; ++x) e[x] = static_cast<T>(v[x]);
+  *reinterpret_cast<uint4 *>(out + (t * N + ch) * static_cast<long long>(sizeof(T))) = raw;
+}
+
 // KS: 32-byte steps of K per pipeline stage.  A source row takes `chunks`
 // stages of KS * 32 bytes (Kp * sizeof(T) must be a multiple of that when
 // chunks > 1).  packed_row = Kp, packed_rows = rows of one offset in wt.
@@ -114,13 +151,14 @@ __device__ __forceinline__ void implicit_forward_body(
   constexpr int kStageElems = kStageBytes / static_cast<int>(sizeof(T));
   constexpr int kRowPieces = 2 * KS;                     // 16-byte pieces of a weight row per stage
   constexpr int kWPieces = (Np * kRowPieces + kImplicitBlock - 1) / kImplicitBlock;
-  // LDS rows of staged weights: padded by 16 bytes against bank conflicts, or,
-  // for the widest stage (where two padded buffers would not fit 64 KiB), left
-  // unpadded with the 16-byte pieces of row n stored at position p ^ (n % 16)
-  constexpr bool kSwizzle = KS == 8;
-  constexpr int kLdsRow = kSwizzle ? kStageBytes : kStageBytes + 16;
+  // LDS rows of staged weights are padded by 16 bytes against bank conflicts
+  constexpr int kLdsRow = kStageBytes + 16;
   constexpr int kBufferBytes = Np * kLdsRow;
-  __shared__ __align__(16) unsigned char w_lds[2 * kBufferBytes];
+  // the output pass turns one 32 x 32 block of fp32 sums per wavefront around in the same memory
+  constexpr int kTurnRow = 32 * 4 + 16;
+  constexpr int kTurnBytes = 32 * kTurnRow;
+  constexpr int kLdsBytes = 2 * kBufferBytes > 4 * kTurnBytes ? 2 * kBufferBytes : 4 * kTurnBytes;
+  __shared__ __align__(16) unsigned char w_lds[kLdsBytes];
   const int num_stages = num_offsets * chunks;
   const int first_channel = blockIdx.y * Np;             // channel group of this workgroup
 
@@ -187,8 +225,8 @@ __device__ __forceinline__ void implicit_forward_body(
     for (int i = 0; i < kWPieces; ++i) {
       const int piece = min(tid + i * kImplicitBlock, Np * kRowPieces - 1);
       const int row = piece / kRowPieces;
-      const int at = kSwizzle ? ((piece % kRowPieces) ^ (row & (kRowPieces - 1))) : piece % kRowPieces;
-      *reinterpret_cast<uint4 *>(w_lds + buffer * kBufferBytes + row * kLdsRow + at * 16) = set.v[i];
+      *reinterpret_cast<uint4 *>(w_lds + buffer * kBufferBytes + row * kLdsRow + (piece % kRowPieces) * 16) =
+          set.v[i];
     }
   };
   // Source rows come through a buffer resource: lanes without a source (and
@@ -253,7 +291,7 @@ __device__ __forceinline__ void implicit_forward_body(
     if (any) {                                                                                     \
       const unsigned char *w_buf = w_lds + (o & 1) * kBufferBytes;                                 \
       _Pragma("unroll") for (int kk = 0; kk < kSteps; ++kk) {                                      \
-        const int off = (kSwizzle ? ((kk * 2 + h) ^ (r & (kRowPieces - 1))) : kk * 2 + h) * 16;     \
+        const int off = (kk * 2 + h) * 16;                                                         \
         _Pragma("unroll") for (int b = 0; b < NB; ++b) {                                           \
           const uint4 chan =                                                                       \
               *reinterpret_cast<const uint4 *>(w_buf + (b * 32 + r) * kLdsRow + off);              \
@@ -277,6 +315,58 @@ __device__ __forceinline__ void implicit_forward_body(
   }
 #undef MNT_STAGE
 
+  // Output.  A lane holds 4 consecutive channels of one target per accumulator
+  // group and neighbouring lanes hold different targets: written as they are,
+  // every lane's few bytes are a request of their own.  Where output rows are
+  // whole 16-byte pieces each wavefront turns its 32 x 32 blocks around in LDS
+  // (free after the last stage's barrier), so that one store instruction
+  // covers rows in contiguous pieces of 64 bytes (128 in fp32), and the
+  // residual is read the same way.
+  if ((static_cast<long long>(N) * sizeof(T)) % 16 == 0) {
+    constexpr int EPV = 16 / static_cast<int>(sizeof(T));
+    constexpr int kOutPieces = 32 / EPV;                          // 16-byte pieces of a block's output row
+    constexpr int kPieces = 32 * kOutPieces / 64;                 // per lane and block
+    unsigned char *turn = w_lds + wv * kTurnBytes;
+#pragma unroll
+    for (int m = 0; m < MW; ++m) {
+      const long long block_t0 = static_cast<long long>(blockIdx.x) * (kImplicitTargets * MW) + (wv * MW + m) * 32;
+      if (block_t0 >= num_targets) break;
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        if (first_channel + b * 32 >= N) break;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          *reinterpret_cast<float4 *>(turn + r * kTurnRow + (q * 8 + h * 4) * 4) =
+              make_float4(acc[m][b][q * 4], acc[m][b][q * 4 + 1], acc[m][b][q * 4 + 2], acc[m][b][q * 4 + 3]);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int i = 0; i < kPieces; ++i) {
+          const int piece = lane + i * 64;
+          const int pr = piece / kOutPieces, part = piece % kOutPieces;
+          const int ch = first_channel + b * 32 + part * EPV;
+          float v[EPV];
+#pragma unroll
+          for (int x = 0; x < EPV; x += 4) {
+            const float4 f = *reinterpret_cast<const float4 *>(turn + pr * kTurnRow + (part * EPV + x) * 4);
+            v[x] = f.x;
+            v[x + 1] = f.y;
+            v[x + 2] = f.z;
+            v[x + 3] = f.w;
+          }
+          if (block_t0 + pr < num_targets && ch < N) {            // N % EPV == 0: a piece is all in or all out
+            finish_piece<T, EPV>(v, ep, block_t0 + pr, ch, N, out);
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int m = 0; m < MW; ++m) {
     if (!t_ok[m]) continue;
@@ -302,19 +392,6 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
     int chunks, int packed_row, int packed_rows, unsigned char *__restrict__ out, Epilogue ep) {
   implicit_forward_body<T, NB, KS, MW>(sources, source_bytes, wt, kernel_map, num_targets, num_offsets, K, N,
                                        chunks, packed_row, packed_rows, out, ep);
-}
-
-// The 256-byte stage keeps three sets of source-row and weight registers of
-// twice the size in flight: one wavefront per SIMD, with the whole register
-// file, instead of spills.
-template <typename T, int NB>
-__global__ __launch_bounds__(kImplicitBlock) __attribute__((amdgpu_waves_per_eu(1, 1)))
-void implicit_forward_wide_rows_kernel(
-    const T *__restrict__ sources, unsigned source_bytes, const T *__restrict__ wt,
-    const int *__restrict__ kernel_map, long long num_targets, int num_offsets, int K, int N,
-    int chunks, int packed_row, int packed_rows, unsigned char *__restrict__ out, Epilogue ep) {
-  implicit_forward_body<T, NB, 8, 1>(sources, source_bytes, wt, kernel_map, num_targets, num_offsets, K, N,
-                                     chunks, packed_row, packed_rows, out, ep);
 }
 
 // inverse[o][m] = t for every hit kernel_map[o][t] = m (at most one t per
@@ -361,10 +438,11 @@ static void implicit_typed(const T *sources, const T *weights, const T *packed, 
     profile_mark("pack_weights", stream);
   }
   const unsigned source_bytes = static_cast<unsigned>(S * K * sizeof(T));
-  // stage width: 64 or 128 bytes for narrow rows; wider rows go in chunks of 256
-  // bytes where the padded row is a multiple of that, else of 128
+  // stage width: 64 bytes for rows up to that, else 128; wider rows go in
+  // chunks of 128 bytes (stages of 256 measured two to three times slower:
+  // their registers leave one wavefront per SIMD)
   const int row_bytes = Kp * static_cast<int>(sizeof(T));
-  const int stage_bytes = K * sizeof(T) <= 64 ? 64 : row_bytes <= 128 ? 128 : row_bytes % 256 == 0 ? 256 : 128;
+  const int stage_bytes = K * sizeof(T) <= 64 ? 64 : 128;
   const int chunks = row_bytes <= 128 ? 1 : row_bytes / stage_bytes;
   // channel groups of up to 128 channels; the last group may be narrower
   const int groups = static_cast<int>(div_ceil(Np, 32 * kImplicitMaxBlocks));
@@ -384,12 +462,8 @@ static void implicit_typed(const T *sources, const T *weights, const T *packed, 
 #define MNT_IMPLICIT_KS(NB, MW)           \
   if (stage_bytes == 64) {                \
     MNT_IMPLICIT(NB, 2, MW);              \
-  } else if (stage_bytes == 128) {        \
-    MNT_IMPLICIT(NB, 4, MW);              \
   } else {                                \
-    implicit_forward_wide_rows_kernel<T, NB><<<grid, kImplicitBlock, 0, stream>>>(                 \
-        sources, source_bytes, wt, kernel_map, Tn, static_cast<int>(O), static_cast<int>(K),       \
-        static_cast<int>(N), chunks, Kp, Np, reinterpret_cast<unsigned char *>(out), ep);          \
+    MNT_IMPLICIT(NB, 4, MW);              \
   }
   switch (blocks) {
     case 1: MNT_IMPLICIT_KS(1, 1); break;
