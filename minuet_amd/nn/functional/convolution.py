@@ -31,14 +31,19 @@ def prefers_implicit(num_offsets: int, num_source_features: int, num_target_feat
     """Whether ``dataflow="auto"`` takes the single-kernel form for a layer of
     this shape: it must fit that kernel, and it must be the faster one, which
     measurements say it is for 16-bit features with source rows of up to 128
-    bytes and up to 128 output channels (beyond that its matrix work on empty
-    (offset, target) pairs outweighs the buffer traffic it saves).  fp32 matrix
-    work is 16x dearer, so there it only pays where most (offset, target) pairs
-    are hits, i.e. for small layers with strided 2^D kernels."""
+    bytes and up to 128 output channels, and for rows of up to 256 bytes with up
+    to 64 output channels under kernels of more than 8 offsets (beyond that its
+    matrix work on empty (offset, target) pairs outweighs the buffer traffic it
+    saves).  fp32 matrix work is 16x dearer, so there it only pays where most
+    (offset, target) pairs are hits, i.e. for small layers with strided 2^D
+    kernels."""
     if not _C.implicit_forward_supported(num_source_features, num_target_features, dtype):
         return False
     if dtype != torch.float32:
-        return num_source_features * dtype.itemsize <= 128 and num_target_features <= 128
+        row_bytes = num_source_features * dtype.itemsize
+        if row_bytes <= 128:
+            return num_target_features <= 128
+        return row_bytes <= 256 and num_target_features <= 64 and num_offsets > 8
     return num_offsets <= 8 and num_source_features * num_target_features <= 1024
 
 
