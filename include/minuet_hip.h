@@ -178,6 +178,26 @@ int mnt_kernel_map_emit(int32_t *source_masks_out, int32_t *target_masks_out,
                         int32_t *in_idx_out, int32_t *out_idx_out,
                         int32_t *sizes_dev_out, int32_t *order_dev_out, void *stream);
 
+/* mnt_kernel_map_query and mnt_kernel_map_emit in one call, for callers that
+ * can hand over the pair lists before their length is known: in_idx_out /
+ * out_idx_out (nullable, together) have room for list_capacity >= O * T
+ * entries each, of which the first nnz = sum(sizes) are written.  The tables
+ * are written while the host waits for the sizes, so the call costs one wait
+ * and no launch after it.  Needs S, T, O > 0.  Same reference code
+ * (minuet/nn/convolutions.py:147-170). */
+int mnt_kernel_map_build(const void *sources, int64_t num_sources,
+                         const void *targets, int64_t num_targets,
+                         const int64_t *offsets_host, int64_t num_offsets,
+                         int ndim, int coord_dtype,
+                         const void *source_batch_dims, const void *target_batch_dims,
+                         int64_t num_batches, int batch_dtype, int reorder,
+                         const int64_t *source_bounds_host, const int64_t *target_bounds_host,
+                         int64_t *bounds_host_out, int32_t *kernel_map_out,
+                         int32_t *source_masks_out, int32_t *target_masks_out,
+                         int32_t *in_idx_out, int32_t *out_idx_out, int64_t list_capacity,
+                         int32_t *sizes_dev_out, int32_t *order_dev_out,
+                         int64_t *sizes_host_out, int64_t *order_host_out, void *stream);
+
 /* Per-offset (in_idx, out_idx) pair lists from a dense int32 kernel map: for row
  * o the hits in target order are written at list positions
  * cumsum_host[o] .. cumsum_host[o]+sizes[o]-1 (cumsum_host[O+1], HOST, exclusive

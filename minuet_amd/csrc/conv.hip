@@ -186,7 +186,8 @@ __global__ __launch_bounds__(256) void scatter_wide_kernel(const TB *__restrict_
   // sub-batch at a time (all loads of a batch in flight together), then
   // summed in offset order
   constexpr int kMasks = 32;
-  constexpr int kRows = NV * NBV <= 2 ? 8 : 4;
+  // rows in flight per lane group: 2 to 5 measure the same, more cost a wavefront of occupancy
+  constexpr int kRows = 4;
   for (int o0 = 0; o0 < num_offsets; o0 += kMasks) {
     int d[kMasks];
 #pragma unroll
@@ -321,7 +322,8 @@ __global__ __launch_bounds__(kScatterBlock) void scatter_kernel(
     __syncthreads();
   }
 
-  constexpr int kRows = NV * NBV <= 2 ? 8 : 4;
+  // rows in flight per lane group: 2 to 5 measure the same, more cost a wavefront of occupancy
+  constexpr int kRows = 4;
   const int groups = kScatterBlock / lanes_per_row;
   const int group = tid / lanes_per_row;
   const int lr = tid - group * lanes_per_row;

@@ -831,11 +831,9 @@ struct MapState {
 // Second half of the first phase of a kernel-map build: per-offset sizes and
 // the stable size order from the per-tile hit counts, mirrored into pinned
 // host memory (past the bounds slots), then the state the emit call reads.
-static void finish_sizes(Arena &arena, const MapState &state, unsigned *tile_counts,
-                         unsigned *row_sizes, unsigned *plan, int64_t *sizes_host_out,
-                         int64_t *order_host_out, hipStream_t stream) {
+static unsigned long long enqueue_sizes(Arena &arena, const MapState &state, unsigned *tile_counts,
+                                        unsigned *row_sizes, unsigned *plan, hipStream_t stream) {
   const int64_t num_offsets = state.num_offsets;
-  unsigned *h_plan = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned()) + Arena::kPlanOffset);
   unsigned *d_plan_host = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned_device()) + Arena::kPlanOffset);
   const unsigned long long sequence = arena.next_sequence();
   tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, state.num_tiles,
@@ -844,12 +842,27 @@ static void finish_sizes(Arena &arena, const MapState &state, unsigned *tile_cou
   map_plan_kernel<<<1, 256, 0, stream>>>(row_sizes, static_cast<int>(num_offsets), state.reorder, plan,
                                          d_plan_host, arena.flag_device(1), sequence);
   check_launch("map_plan_kernel");
+  return sequence;
+}
+
+// Waits for the sizes enqueued under `sequence` and hands them to the host arrays.
+static void collect_sizes(Arena &arena, unsigned long long sequence, int64_t num_offsets,
+                          int64_t *sizes_host_out, int64_t *order_host_out) {
+  const unsigned *h_plan =
+      reinterpret_cast<const unsigned *>(static_cast<char *>(arena.pinned()) + Arena::kPlanOffset);
   arena.wait_flag(1, sequence);
-  profile_mark("map_sizes_order+sync", stream);
   for (int64_t j = 0; j < num_offsets; ++j) {
     order_host_out[j] = h_plan[j];
     sizes_host_out[j] = h_plan[2 * num_offsets + j];
   }
+}
+
+static void finish_sizes(Arena &arena, const MapState &state, unsigned *tile_counts,
+                         unsigned *row_sizes, unsigned *plan, int64_t *sizes_host_out,
+                         int64_t *order_host_out, hipStream_t stream) {
+  const unsigned long long sequence = enqueue_sizes(arena, state, tile_counts, row_sizes, plan, stream);
+  collect_sizes(arena, sequence, state.num_offsets, sizes_host_out, order_host_out);
+  profile_mark("map_sizes_order+sync", stream);
   memcpy(arena.map_state, &state, sizeof(state));
   arena.map_state_valid = true;
 }
@@ -1027,6 +1040,62 @@ extern "C" int mnt_kernel_map_query(const void *sources, int64_t num_sources, co
                 kernel_map_out, MNT_INT32, tile_counts, scope, stream);
     }
     finish_sizes(arena, state, tile_counts, row_sizes, plan, sizes_host_out, order_host_out, stream);
+  });
+}
+
+extern "C" int mnt_kernel_map_build(const void *sources, int64_t num_sources, const void *targets,
+                                    int64_t num_targets, const int64_t *offsets_host,
+                                    int64_t num_offsets, int ndim, int coord_dtype,
+                                    const void *source_batch_dims, const void *target_batch_dims,
+                                    int64_t num_batches, int batch_dtype, int reorder,
+                                    const int64_t *source_bounds_host,
+                                    const int64_t *target_bounds_host, int64_t *bounds_host_out,
+                                    int32_t *kernel_map_out, int32_t *source_masks_out,
+                                    int32_t *target_masks_out, int32_t *in_idx_out,
+                                    int32_t *out_idx_out, int64_t list_capacity,
+                                    int32_t *sizes_dev_out, int32_t *order_dev_out,
+                                    int64_t *sizes_host_out, int64_t *order_host_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    QueryArgs a{sources, num_sources, targets, num_targets, ndim, coord_dtype,
+                source_batch_dims, target_batch_dims, num_batches, batch_dtype};
+    check_query_args(a, num_offsets);
+    MNT_CHECK(offsets_host != nullptr && sizes_host_out != nullptr && order_host_out != nullptr, "null argument");
+    MNT_CHECK(num_sources > 0 && num_targets > 0 && num_offsets > 0,
+              "mnt_kernel_map_build needs sources, targets and offsets (use mnt_kernel_map_query / _emit "
+              "for empty operands)");
+    MNT_CHECK(kernel_map_out != nullptr, "kernel_map_out is null");
+    MNT_CHECK((in_idx_out == nullptr) == (out_idx_out == nullptr), "in_idx_out and out_idx_out go together");
+    MNT_CHECK(in_idx_out == nullptr || list_capacity >= num_offsets * num_targets,
+              "list_capacity = %lld cannot hold every (offset, target) pair (%lld)",
+              (long long)list_capacity, (long long)(num_offsets * num_targets));
+    MNT_CHECK(sizeof(unsigned) * 3 * num_offsets + 1024 <= Arena::kPinnedBytes,
+              "too many kernel offsets (%lld)", static_cast<long long>(num_offsets));
+    Arena &arena = Arena::of(stream);
+    arena.map_state_valid = false;
+    const int num_tiles = static_cast<int>(div_ceil(num_targets, kTargetsPerTile));
+    const size_t words = static_cast<size_t>(num_offsets) * num_tiles + num_offsets + 4 * num_offsets + 1;
+    char *keep = static_cast<char *>(arena.persistent(1, 256 + words * sizeof(unsigned)));
+    unsigned *tile_counts = reinterpret_cast<unsigned *>(keep + 256);
+    unsigned *row_sizes = tile_counts + static_cast<size_t>(num_offsets) * num_tiles;
+    unsigned *plan = row_sizes + num_offsets;
+    const MapState state{num_sources, num_targets, num_offsets, num_tiles, reorder, kernel_map_out};
+    if (bounds_host_out != nullptr) {
+      for (int i = 0; i < 16; ++i) bounds_host_out[i] = (i & 4) ? INT64_MIN : INT64_MAX;
+    }
+    {
+      Scope scope(stream);
+      run_query(a, offsets_host, num_offsets, source_bounds_host, target_bounds_host, bounds_host_out,
+                kernel_map_out, MNT_INT32, tile_counts, scope, stream);
+    }
+    // the tables are written while the host waits for the sizes
+    const unsigned long long sequence = enqueue_sizes(arena, state, tile_counts, row_sizes, plan, stream);
+    const int no = static_cast<int>(num_offsets);
+    enqueue_emit<int32_t>(kernel_map_out, num_sources, num_targets, no, tile_counts, num_tiles, plan + no,
+                          plan + 3 * no, source_masks_out, target_masks_out, in_idx_out, out_idx_out,
+                          stream, plan, sizes_dev_out, order_dev_out);
+    collect_sizes(arena, sequence, num_offsets, sizes_host_out, order_host_out);
+    profile_mark("map_sizes_order+emit+sync", stream);
   });
 }
 

@@ -55,6 +55,9 @@ SIGNATURES = {
     "mnt_kernel_map_query": (_int, [_vp, _i64, _vp, _i64, _pi64, _i64, _int, _int, _vp, _vp, _i64,
                                     _int, _int, _pi64, _pi64, _pi64, _vp, _pi64, _pi64, _vp]),
     "mnt_kernel_map_emit": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "mnt_kernel_map_build": (_int, [_vp, _i64, _vp, _i64, _pi64, _i64, _int, _int, _vp, _vp, _i64,
+                                    _int, _int, _pi64, _pi64, _pi64, _vp, _vp, _vp, _vp, _vp, _i64,
+                                    _vp, _vp, _pi64, _pi64, _vp]),
     "mnt_kernel_map_dense": (_int, [_vp, _i64, _vp, _i64, _pi64, _i64, _int, _int, _vp, _vp, _i64, _int,
                                     _pi64, _pi64, _pi64, _vp, _vp]),
     "mnt_kernel_map_tables": (_int, [_vp, _i64, _i64, _i64, _int, _pi64, _pi64, _vp]),
@@ -417,6 +420,11 @@ def cuda_compute_kernel_map_masks(num_sources: int, kernel_map: torch.Tensor,
     return source_masks, target_masks
 
 
+# Pair lists are allocated for their worst case (and the call spared a launch
+# after its wait) while both lists together stay below this many bytes.
+PAIR_LIST_SLACK_BYTES = 256 << 20
+
+
 def kernel_map_build(sources: torch.Tensor, targets: torch.Tensor, offsets_host: np.ndarray,
                      source_batch_dims: Optional[torch.Tensor],
                      target_batch_dims: Optional[torch.Tensor], reorder: bool,
@@ -464,13 +472,41 @@ def kernel_map_build(sources: torch.Tensor, targets: torch.Tensor, offsets_host:
         tmask = torch.empty((num_offsets, num_targets), dtype=torch.int32, device=device)
     sizes_dev = torch.empty((num_offsets,), dtype=torch.int32, device=device)
     order_dev = torch.empty((num_offsets,), dtype=torch.int32, device=device)
+    num_batches = source_batch_dims.numel() - 1 if source_batch_dims is not None else 1
+    # Pair lists whose worst case (every (offset, target) pair a hit) is small
+    # are handed over before their length is known: the tables are then written
+    # while the host waits for the sizes, in one call.
+    capacity = num_offsets * num_targets
+    one_call = (num_sources > 0 and num_targets > 0 and num_offsets > 0
+                and (not want_lists or capacity * 8 <= PAIR_LIST_SLACK_BYTES))
     with _on(device):
         stream = _stream(device)
+        if one_call:
+            if want_lists:
+                both = torch.empty((2, capacity), dtype=torch.int32, device=device)
+            _check(lib.mnt_kernel_map_build(
+                _ptr(sources), num_sources, _ptr(targets), num_targets,
+                offs.ctypes.data_as(_pi64), num_offsets, ndim, ccode, _ptr(source_batch_dims),
+                _ptr(target_batch_dims), num_batches, bcode, 1 if reorder else 0,
+                None if sb is None else sb.ctypes.data_as(_pi64),
+                None if tb is None else tb.ctypes.data_as(_pi64), bounds.ctypes.data_as(_pi64),
+                _ptr(dense), _ptr(smask), _ptr(tmask),
+                _ptr(both[0]) if want_lists else None, _ptr(both[1]) if want_lists else None, capacity,
+                _ptr(sizes_dev), _ptr(order_dev), sizes_host.ctypes.data_as(_pi64),
+                order_host.ctypes.data_as(_pi64), stream))
+            if want_lists:
+                nnz = int(sizes_host.sum())
+                in_idx, out_idx = both[0, :nnz], both[1, :nnz]
+            result.update(sizes_host=sizes_host, order_host=order_host, sizes=sizes_dev, order=order_dev,
+                          bounds=bounds, source_masks=smask, target_masks=tmask, in_idx=in_idx,
+                          out_idx=out_idx)
+            if want_dense:
+                result["kernel_map"] = dense
+            return result
         _check(lib.mnt_kernel_map_query(
             _ptr(sources), num_sources, _ptr(targets), num_targets,
             offs.ctypes.data_as(_pi64), num_offsets, ndim, ccode, _ptr(source_batch_dims),
-            _ptr(target_batch_dims),
-            source_batch_dims.numel() - 1 if source_batch_dims is not None else 1, bcode,
+            _ptr(target_batch_dims), num_batches, bcode,
             1 if reorder else 0,
             None if sb is None else sb.ctypes.data_as(_pi64),
             None if tb is None else tb.ctypes.data_as(_pi64), bounds.ctypes.data_as(_pi64),
