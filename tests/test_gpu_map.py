@@ -346,6 +346,49 @@ def test_dense_then_tables_equals_full_build(reorder, kernel, stride, batched):
     np.testing.assert_array_equal(host(tables["out_idx"]), eout)
 
 
+@pytest.mark.parametrize("reorder", [True, False])
+@pytest.mark.parametrize("kernel,stride,batched", [(3, 1, True), (2, 2, False)])
+def test_one_call_build_equals_two_calls(monkeypatch, reorder, kernel, stride, batched):
+    """mnt_kernel_map_build (lists sized for their worst case, tables written
+    while the host waits) against mnt_kernel_map_query + _emit and the oracle."""
+    src, sbd, tgt, tbd, off = _query_case(23, 20000, 40, -5, kernel, stride, batched=batched)
+    args = (dev(src), dev(tgt), off.astype(np.int64), dev(sbd), dev(tbd), reorder)
+    kw = dict(want_masks=True, want_lists=True, want_dense=True)
+    one = _C.kernel_map_build(*args, **kw)
+    assert one["in_idx"].untyped_storage().nbytes() >= 8 * off.shape[0] * tgt.shape[0]   # the one-call form ran
+    monkeypatch.setattr(_C, "PAIR_LIST_SLACK_BYTES", 0)
+    two = _C.kernel_map_build(*args, **kw)
+    assert two["in_idx"].untyped_storage().nbytes() == 8 * int(two["sizes_host"].sum())
+    for key in ("sizes_host", "order_host", "bounds"):
+        np.testing.assert_array_equal(one[key], two[key])
+    for key in ("sizes", "order", "source_masks", "target_masks", "in_idx", "out_idx", "kernel_map"):
+        assert torch.equal(one[key], two[key]), key
+    esm, etm, eorder, esizes, em = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=reorder)
+    ein, eout, _ = orc.kernel_map_pair_lists(em)
+    np.testing.assert_array_equal(host(one["in_idx"]), ein)
+    np.testing.assert_array_equal(host(one["out_idx"]), eout)
+    np.testing.assert_array_equal(host(one["source_masks"]), esm)
+
+
+def test_one_call_build_rejects_short_lists():
+    cloud = random_cloud(500, 16, seed=5)
+    off = orc.generate_kernel_offsets(3, 3, 1, 1).astype(np.int64)
+    c = dev(cloud)
+    dense = torch.empty((27, 500), dtype=torch.int32, device=c.device)
+    lists = torch.empty((2, 100), dtype=torch.int32, device=c.device)
+    sizes = np.zeros(27, dtype=np.int64)
+    order = np.zeros(27, dtype=np.int64)
+    lib = _C.load_library()
+    with _C._on(c.device):
+        status = lib.mnt_kernel_map_build(
+            _C._ptr(c), 500, _C._ptr(c), 500, off.ctypes.data_as(_C._pi64), 27, 3, 0, None, None, 1, 0, 1,
+            None, None, None, _C._ptr(dense), None, None, _C._ptr(lists[0]), _C._ptr(lists[1]), 100,
+            None, None, sizes.ctypes.data_as(_C._pi64), order.ctypes.data_as(_C._pi64), _C._stream(c.device))
+    assert status != 0
+    with pytest.raises(RuntimeError, match="list_capacity"):
+        _C._check(status)
+
+
 def test_dense_and_tables_empty_inputs():
     off = orc.generate_kernel_offsets(3, 3, 1, 1).astype(np.int64)
     cloud = random_cloud(40, 4, seed=2)
