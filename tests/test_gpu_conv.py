@@ -154,7 +154,7 @@ def test_forward_epilogue(kind, activation):
     (3, 1, 8, 32, 5000, 20), (3, 1, 24, 48, 4000, 20), (5, 1, 16, 16, 3000, 16),
     (3, 1, 32, 100, 3000, 16), (3, 1, 56, 40, 2000, 12), (1, 1, 32, 12, 999, 12),
     (7, 1, 16, 8, 1500, 10),
-    # rows wider than one pipeline stage (chunks of 256 or 128 bytes) and more
+    # rows wider than one pipeline stage (chunks of 128 bytes) and more
     # than 128 output channels (channel groups, the last one narrower)
     (3, 1, 128, 128, 4000, 20), (3, 1, 256, 64, 3000, 16), (2, 2, 128, 256, 6000, 30),
     (3, 1, 160, 32, 2000, 12), (3, 1, 96, 200, 2000, 12), (3, 1, 72, 300, 1500, 12),
