@@ -110,6 +110,19 @@ int mnt_target_coordinates_count(const void *source_coords, int64_t n, int ndim,
 int mnt_target_coordinates_fill(void *target_coords_out, void *target_batch_dims_out,
                                 void *stream);
 
+/* Both phases in one call for a caller that hands over room for the worst case:
+ * target_coords_out holds capacity >= n rows, of which the first
+ * *num_targets_out are written (there are never more targets than sources).
+ * The coordinates are written while the host waits for the count, so nothing
+ * is launched after the wait.  Needs n > 0.  Same reference expression
+ * (minuet/nn/convolutions.py:84-99). */
+int mnt_target_coordinates(const void *source_coords, int64_t n, int ndim, int coord_dtype,
+                           const int64_t *target_stride, const void *batch_dims,
+                           int64_t num_batches, int index_dtype,
+                           const int64_t *source_bounds_host, void *target_coords_out,
+                           int64_t capacity, void *target_batch_dims_out,
+                           int64_t *num_targets_out, void *stream);
+
 /* ---- Map: query -------------------------------------------------------- */
 
 /* Dense kernel map: kernel_map_out[o*T + t] = j with sources[j] == targets[t] +

@@ -395,10 +395,14 @@ struct TargetState {
   int tiles;
 };
 
+// early_out (nullable): room for n target rows; the targets (and early_dims_out,
+// the new batch boundaries) are then written while the host waits for the
+// count, and no second call follows.
 template <typename CT, typename IT>
 static void target_count_typed(const CT *coords, int64_t n, int ndim, const int64_t *target_stride,
                                const IT *batch_dims, int64_t num_batches,
-                               const int64_t *source_bounds, int64_t *count_out, hipStream_t stream) {
+                               const int64_t *source_bounds, int64_t *count_out, hipStream_t stream,
+                               CT *early_out = nullptr, IT *early_dims_out = nullptr) {
   Arena &arena = Arena::of(stream);
   arena.pending.valid = false;
   const bool batched = batch_dims != nullptr && num_batches > 1;
@@ -455,8 +459,14 @@ static void target_count_typed(const CT *coords, int64_t n, int ndim, const int6
       const unsigned long long sequence = arena.next_sequence();
       bitmap_scan_kernel<<<1, 1024, 0, stream>>>(tile_bases, tiles, d, arena.flag_device(2), sequence);
       check_launch("bitmap_scan_kernel");
+      if (early_out != nullptr) {
+        bitmap_emit_kernel<CT, IT><<<tiles, kScanBlock, 0, stream>>>(
+            bitmap, words, tile_bases, tiles, spec, early_out, batched ? early_dims_out : nullptr);
+        check_launch("bitmap_emit_kernel");
+      }
       arena.wait_flag(2, sequence);
       *count_out = static_cast<int64_t>(*h);
+      if (early_out != nullptr) return;
       TargetState state;
       memset(&state, 0, sizeof(state));
       state.spec = spec;
@@ -507,9 +517,15 @@ static void target_count_typed(const CT *coords, int64_t n, int ndim, const int6
     key_rank_kernel<<<tiles, kScanBlock, 0, stream>>>(kept_keys, n, tile_sums, rank, d, arena.flag_device(2),
                                                      sequence);
     check_launch("key_rank_kernel");
+    if (early_out != nullptr) {
+      emit_targets_kernel<CT, IT><<<grid, 256, 0, stream>>>(kept_keys, rank, n, spec, batch_dims, early_out,
+                                                            batched ? early_dims_out : nullptr);
+      check_launch("emit_targets_kernel");
+    }
     arena.wait_flag(2, sequence);
     *count_out = static_cast<int64_t>(*h);
   }
+  if (early_out != nullptr) return;
   auto &p = arena.pending;
   p.valid = true;
   p.count = *count_out;
@@ -654,6 +670,36 @@ extern "C" int mnt_target_coordinates_count(const void *source_coords, int64_t n
   target_count_typed<CT, IT>(static_cast<const CT *>(source_coords), n, ndim, target_stride,      \
                              static_cast<const IT *>(batch_dims), num_batches, source_bounds_host, \
                              num_targets_out, stream)
+    MNT_DISPATCH_CI(coord_dtype, index_dtype, MNT_CALL);
+#undef MNT_CALL
+  });
+}
+
+extern "C" int mnt_target_coordinates(const void *source_coords, int64_t n, int ndim, int coord_dtype,
+                                      const int64_t *target_stride, const void *batch_dims,
+                                      int64_t num_batches, int index_dtype,
+                                      const int64_t *source_bounds_host, void *target_coords_out,
+                                      int64_t capacity, void *target_batch_dims_out,
+                                      int64_t *num_targets_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MNT_CHECK(ndim >= 1 && ndim <= MNT_MAX_NDIM, "ndim must be in [1, %d] but found %d",
+              MNT_MAX_NDIM, ndim);
+    MNT_CHECK(n > 0 && n <= INT32_MAX, "number of coordinates %lld out of range (the one-call form needs "
+              "at least one)", static_cast<long long>(n));
+    MNT_CHECK(target_stride != nullptr && num_targets_out != nullptr && target_coords_out != nullptr,
+              "null argument");
+    MNT_CHECK(capacity >= n, "capacity = %lld rows cannot hold the targets of %lld sources",
+              static_cast<long long>(capacity), static_cast<long long>(n));
+    int_size(coord_dtype);
+    int_size(index_dtype);
+    if (batch_dims == nullptr) num_batches = 1;
+    MNT_CHECK(num_batches <= 1 || target_batch_dims_out != nullptr, "target_batch_dims_out is null");
+#define MNT_CALL(CT, IT)                                                                        \
+  target_count_typed<CT, IT>(static_cast<const CT *>(source_coords), n, ndim, target_stride,      \
+                             static_cast<const IT *>(batch_dims), num_batches, source_bounds_host, \
+                             num_targets_out, stream, static_cast<CT *>(target_coords_out),       \
+                             static_cast<IT *>(target_batch_dims_out))
     MNT_DISPATCH_CI(coord_dtype, index_dtype, MNT_CALL);
 #undef MNT_CALL
   });

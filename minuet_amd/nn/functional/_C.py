@@ -48,6 +48,8 @@ SIGNATURES = {
     "mnt_target_coordinates_count": (_int, [_vp, _i64, _int, _int, _pi64, _vp, _i64, _int, _pi64, _pi64,
                                             _vp]),
     "mnt_target_coordinates_fill": (_int, [_vp, _vp, _vp]),
+    "mnt_target_coordinates": (_int, [_vp, _i64, _int, _int, _pi64, _vp, _i64, _int, _pi64, _vp, _i64,
+                                      _vp, _pi64, _vp]),
     "mnt_query_sorted_index_with_offsets": (_int, [_vp, _i64, _vp, _i64, _vp, _i64, _int, _int,
                                                    _vp, _vp, _i64, _int, _vp, _int, _vp]),
     "mnt_compute_kernel_map_sizes": (_int, [_vp, _i64, _i64, _int, _vp, _vp]),
@@ -317,6 +319,18 @@ def target_coordinates(coordinates: torch.Tensor, batch_dims: Optional[torch.Ten
     stride = (ctypes.c_int64 * ndim)(*[int(s) for s in target_stride])
     count = ctypes.c_int64(0)
     lib = load_library()
+    num_batches = batch_dims.numel() - 1 if batch_dims is not None else 1
+    known_arg = None if known is None else known.ctypes.data_as(_pi64)
+    if n > 0:
+        # room for the worst case (no two sources share a target): the rows are
+        # written while the host waits for their number, in one call
+        with _on(device):
+            room = torch.empty((n, ndim), dtype=coordinates.dtype, device=device)
+            out_dims = torch.empty_like(batch_dims) if batch_dims is not None else None
+            _check(lib.mnt_target_coordinates(
+                _ptr(coordinates), n, ndim, ccode, stride, _ptr(batch_dims), num_batches, icode,
+                known_arg, _ptr(room), n, _ptr(out_dims), ctypes.byref(count), _stream(device)))
+        return room[:count.value], out_dims
     with _on(device):
         _check(lib.mnt_target_coordinates_count(
             _ptr(coordinates), n, ndim, ccode, stride, _ptr(batch_dims),

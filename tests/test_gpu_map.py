@@ -181,6 +181,58 @@ def test_target_coordinates_bitmap_and_sorted_forms(extent, batches):
                 np.testing.assert_array_equal(host(got_bd), exp_bd)
 
 
+def _target_coordinates_two_calls(c, bd, stride):
+    """mnt_target_coordinates_count + _fill through the C-ABI (the library's
+    one-call form is what ``_C.target_coordinates`` takes for n > 0)."""
+    import ctypes
+    n, ndim = c.shape
+    lib = _C.load_library()
+    strides = (ctypes.c_int64 * ndim)(*stride)
+    count = ctypes.c_int64(0)
+    with _C._on(c.device):
+        _C._check(lib.mnt_target_coordinates_count(
+            _C._ptr(c), n, ndim, 0, strides, _C._ptr(bd), bd.numel() - 1 if bd is not None else 1, 0,
+            None, ctypes.byref(count), _C._stream(c.device)))
+        out = torch.empty((count.value, ndim), dtype=c.dtype, device=c.device)
+        out_bd = torch.empty_like(bd) if bd is not None else None
+        _C._check(lib.mnt_target_coordinates_fill(_C._ptr(out), _C._ptr(out_bd), _C._stream(c.device)))
+    return out, out_bd
+
+
+@pytest.mark.parametrize("extent,batches", [(40, 3), (1 << 20, 2)])
+def test_target_coordinates_one_call_equals_two_calls(extent, batches):
+    """Bitmap form (narrow key range) and sorted form (wide): the one-call entry
+    point writes, into room for n rows, what count + fill write."""
+    rng = np.random.default_rng(7 + extent)
+    n = 5000
+    c = rng.integers(-extent, extent, size=(n, 3)).astype(np.int32)
+    bd = np.concatenate([[0], np.sort(rng.integers(0, n, size=batches - 1)), [n]]).astype(np.int32)
+    c, bd = sorted_unique(c, bd)
+    for stride in ((2, 2, 2), (1, 4, 8)):
+        one, one_bd = _C.target_coordinates(dev(c), dev(bd), stride)
+        assert one.untyped_storage().nbytes() == c.shape[0] * 3 * 4          # the one-call form ran
+        two, two_bd = _target_coordinates_two_calls(dev(c), dev(bd), stride)
+        assert torch.equal(one, two) and torch.equal(one_bd, two_bd)
+        exp, exp_bd = orc.target_coordinates(c, bd, stride)
+        np.testing.assert_array_equal(host(one), exp)
+        np.testing.assert_array_equal(host(one_bd), exp_bd)
+
+
+def test_target_coordinates_one_call_rejects_short_room():
+    import ctypes
+    c = dev(sorted_unique(random_cloud(300, 12, seed=3), None)[0])
+    n = c.shape[0]
+    room = torch.empty((n - 1, 3), dtype=torch.int32, device=c.device)
+    count = ctypes.c_int64(0)
+    with _C._on(c.device):
+        status = _C.load_library().mnt_target_coordinates(
+            _C._ptr(c), n, 3, 0, (ctypes.c_int64 * 3)(2, 2, 2), None, 1, 0, None, _C._ptr(room), n - 1,
+            None, ctypes.byref(count), _C._stream(c.device))
+    assert status != 0
+    with pytest.raises(RuntimeError, match="capacity"):
+        _C._check(status)
+
+
 def _query_case(seed, n, extent, lo, kernel, stride=1, batched=False, cdtype=np.int32, idtype=np.int32):
     bd = None
     if batched:
