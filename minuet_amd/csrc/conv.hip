@@ -402,7 +402,10 @@ constexpr int kMaxChannelBlocks = 4;    // 32-channel blocks per workgroup (128 
 // One workgroup multiplies 128 buffer rows of one offset by that offset's
 // weights: out^T = W^T x A^T.  The first MFMA operand holds 32 output
 // channels, the second 32 data rows, so every lane ends up with 4 consecutive
-// channels of ONE data row per accumulator group and stores them as one vector.
+// channels of ONE data row per accumulator group (how the rows are written:
+// see the output pass at the end of the kernel).  CH > 0: K is exactly CH
+// chunks of 128 bytes (CH <= 2) and the whole tile is loaded before the first
+// product; CH == 0: any K, one chunk ahead.
 //
 // A never passes through LDS: lane (r, h) of a wavefront loads, for step kk of
 // a 128-byte chunk of row r, the 16 bytes at offset 32*kk + 16*h — exactly its
