@@ -53,10 +53,9 @@ struct Pieces2 {
 
 typedef unsigned uint4v __attribute__((ext_vector_type(4)));
 
-// Buffer offset that is out of range for every source tensor this kernel
-// accepts, and stays so with the few hundred bytes a load adds to it: such a
-// load returns zeros without touching memory.
-constexpr unsigned kNoRow = 0xFFFFF000u;
+// Source tensors stay below this many bytes: rows are addressed through 32-bit
+// buffer offsets.
+constexpr unsigned kMaxSourceBytes = 0xFFFFF000u;
 
 // One output row's worth of epilogue and store: four consecutive channels of
 // target t held by this lane.
@@ -260,9 +259,8 @@ __device__ __forceinline__ void implicit_forward_body(
       *reinterpret_cast<uint4 *>(w_lds + buffer * kBufferBytes + w_put[i]) = set.v[i];
     }
   };
-  // Source rows come through a buffer resource: pieces past the end of a row
-  // use an out-of-range offset, which yields the zeros the product needs and
-  // no memory access.
+  // Source rows come through a buffer resource (32-bit offsets, a scalar part
+  // for what all lanes share).
   const __amdgpu_buffer_rsrc_t source_buffer = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<T *>(sources), 0, source_bytes, 0x00020000);
   const unsigned row_bytes = static_cast<unsigned>(K) * sizeof(T);
@@ -273,16 +271,17 @@ __device__ __forceinline__ void implicit_forward_body(
 #pragma unroll
     for (int m = 0; m < MW; ++m) {
       const int index = (t_ok[m] && live) ? indices.v[m] : -1;
-      const unsigned row_at = index >= 0 ? static_cast<unsigned>(index) * row_bytes + h * 16u : kNoRow;
+      const unsigned row_at = static_cast<unsigned>(index) * row_bytes + h * 16u;
 #pragma unroll
       for (int kk = 0; kk < kSteps; ++kk) {
-        // the step's place in the row is the same for all lanes: it rides in the scalar offset
-        unsigned offset = row_at;
-        if (!PLAIN && chunk_at + (kk * 2 + h) * 16u >= row_bytes) offset = kNoRow;
-        // lanes without a source sit the load out (an out-of-range lane still
-        // takes its turn in the address unit: 7 to 10 % of a layer at 200k voxels)
+        // Lanes without a source, and pieces past the end of a ragged row, sit
+        // the load out and keep zeros (a lane that loads out of range still
+        // takes its turn in the address unit: 7 to 10 % of a layer at 200k
+        // voxels).  The step's place in the row is the same for all lanes: it
+        // rides in the scalar offset.
+        const bool take = index >= 0 && (PLAIN || chunk_at + (kk * 2 + h) * 16u < row_bytes);
         uint4v v = {0u, 0u, 0u, 0u};
-        if (index >= 0) v = __builtin_amdgcn_raw_buffer_load_b128(source_buffer, offset, chunk_at + kk * 32u, 0);
+        if (take) v = __builtin_amdgcn_raw_buffer_load_b128(source_buffer, row_at, chunk_at + kk * 32u, 0);
         set.v[m * KS + kk] = make_uint4(v.x, v.y, v.z, v.w);
       }
     }
@@ -548,7 +547,7 @@ extern "C" int mnt_sparse_convolution_forward_implicit(
                   O <= 65535,
               "bad shape S=%lld T=%lld O=%lld Cin=%lld Cout=%lld", (long long)S, (long long)T,
               (long long)O, (long long)K, (long long)N);
-    MNT_CHECK(S * K * esize < static_cast<int64_t>(kNoRow),
+    MNT_CHECK(S * K * esize < static_cast<int64_t>(kMaxSourceBytes),
               "source features of %lld bytes exceed the 4 GiB a buffer resource addresses",
               (long long)(S * K * esize));
     MNT_CHECK((K * esize) % 16 == 0 && K * esize <= kImplicitMaxRowBytes && N % 4 == 0 &&
