@@ -152,3 +152,19 @@ def test_random_unique_points():
     with pytest.raises(ValueError):
         random_unique_points(2, 10, 0, 2)
     assert len({tuple(p) for p in random_unique_points(2, 9, 0, 2).tolist()}) == 9
+
+
+def test_auto_dataflow_rule():
+    """Which layer shapes ``dataflow="auto"`` sends to the single-kernel form:
+    16-bit rows of up to 128 bytes with up to 128 output channels, rows of up
+    to 256 bytes with up to 64 output channels under kernels of more than 8
+    offsets, and small fp32 layers with 2^D kernels."""
+    prefers = minuet.nn.functional.prefers_implicit
+    half, single = torch.float16, torch.float32
+    assert prefers(27, 32, 32, half) and prefers(27, 64, 128, half) and prefers(8, 64, 128, torch.bfloat16)
+    assert not prefers(27, 64, 256, half)                 # too many output channels
+    assert prefers(27, 128, 64, half) and not prefers(27, 128, 128, half)
+    assert not prefers(8, 128, 64, half)                  # strided 2^3 kernel: one hit in eight
+    assert not prefers(27, 256, 64, half)                 # 512-byte rows
+    assert not prefers(27, 30, 32, half)                  # rows not a multiple of 16 bytes
+    assert prefers(8, 32, 32, single) and not prefers(27, 32, 32, single) and not prefers(8, 64, 64, single)
