@@ -148,6 +148,24 @@ int mnt_compute_kernel_map_sizes(const void *kernel_map, int64_t num_offsets,
                                  int64_t num_targets, int index_dtype, void *sizes_out,
                                  void *stream);
 
+/* mnt_compute_kernel_map_sizes for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): same arguments, same kernels, same result, but the per-(offset,
+ * tile of 512 targets) hit counts live in a device array that is part of the
+ * library image (MNT_STATIC_SCRATCH_WORDS 32-bit words, held by every GPU the
+ * library runs on until the process ends) instead of the scratch arena.  The
+ * call makes no hipMalloc / hipFree and touches no arena; a map that needs more
+ * than num_offsets * (ceil(num_targets / 512) + 1) <= MNT_STATIC_SCRATCH_WORDS
+ * words is refused with an error.  All calls on one GPU share the array:
+ * calls that overlap on one GPU (two streams, two threads) race; calls on one
+ * stream are ordered.  The first call on a device looks the array's address
+ * up and should be made outside stream capture.  No counterpart in the
+ * reference, which allocates from its buffer pool in every call. */
+#define MNT_STATIC_SCRATCH_WORDS (1u << 20)
+int mnt_compute_kernel_map_sizes_static(const void *kernel_map, int64_t num_offsets,
+                                        int64_t num_targets, int index_dtype, void *sizes_out,
+                                        void *stream);
+
 /* Rank tables: target_masks[o,t] = rank of the hit among the hits of row o in
  * target order, source_masks[o, kernel_map[o,t]] = the same rank, -1 elsewhere.
  * Replaces cuda_compute_kernel_map_masks,

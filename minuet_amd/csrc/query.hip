@@ -19,6 +19,7 @@
 // hiding), the others by walking forward from there.  Hits are counted per
 // offset with wavefront ballots.
 #include <algorithm>
+#include <mutex>
 
 #include "device_utils.h"
 #include "sort.h"
@@ -1188,5 +1189,78 @@ extern "C" int mnt_kernel_map_emit(int32_t *source_masks_out, int32_t *target_ma
                           plan + 3 * no, source_masks_out, target_masks_out, in_idx_out, out_idx_out,
                           stream, plan, sizes_dev_out, order_dev_out);
     profile_mark("map_emit", stream);
+  });
+}
+
+// ---- the sizes of a kernel map without any allocation ------------------------
+//
+// Same kernels as mnt_compute_kernel_map_sizes; the per-(row, tile) hit counts
+// and the row totals live in a file-scope device array instead of the arena.
+// Each GPU holds its own copy of the array for the life of the process; its
+// address is looked up once per device and kept.
+
+namespace mnt {
+
+constexpr size_t kStaticScratchWords = MNT_STATIC_SCRATCH_WORDS;   // 4 MiB per GPU
+static __device__ __align__(256) unsigned scratch[kStaticScratchWords];
+
+constexpr int kMaxDevices = 64;
+static unsigned *g_scratch_address[kMaxDevices] = {nullptr};
+static std::mutex g_scratch_mutex;
+
+// Device address of the current device's copy of `scratch` (the array's name
+// is only a host-side stand-in and must never reach a kernel).
+static unsigned *static_scratch() {
+  int device = 0;
+  MNT_HIP(hipGetDevice(&device));
+  MNT_CHECK(device >= 0 && device < kMaxDevices, "device index %d out of range", device);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_address[device] == nullptr) {
+    void *address = nullptr;
+    MNT_HIP(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
+    MNT_CHECK(address != nullptr, "the static scratch array has no device address");
+    g_scratch_address[device] = static_cast<unsigned *>(address);
+  }
+  return g_scratch_address[device];
+}
+
+}  // namespace mnt
+
+extern "C" int mnt_compute_kernel_map_sizes_static(const void *kernel_map, int64_t num_offsets,
+                                                   int64_t num_targets, int index_dtype,
+                                                   void *sizes_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    int_size(index_dtype);
+    MNT_CHECK(num_offsets >= 0 && num_targets >= 0 && num_targets <= INT32_MAX && num_offsets <= 65535,
+              "bad shape O=%lld T=%lld", (long long)num_offsets, (long long)num_targets);
+    if (num_offsets == 0) return;
+    MNT_CHECK(sizes_out != nullptr, "sizes_out is null");
+    if (num_targets == 0) {
+      // a fill kernel, not a memset node: the call may be under stream capture
+      if (index_dtype == MNT_INT32) enqueue_fill<int32_t>(static_cast<int32_t *>(sizes_out), num_offsets, 0, stream);
+      else enqueue_fill<int64_t>(static_cast<int64_t *>(sizes_out), num_offsets, 0, stream);
+      return;
+    }
+    MNT_CHECK(kernel_map != nullptr, "kernel_map is null");
+    const int num_tiles = static_cast<int>(div_ceil(num_targets, kTargetsPerTile));
+    const size_t words = static_cast<size_t>(num_offsets) * num_tiles + static_cast<size_t>(num_offsets);
+    MNT_CHECK(words <= kStaticScratchWords,
+              "mnt_compute_kernel_map_sizes_static: %lld offsets x %d tiles of %d targets need %zu words "
+              "of scratch, the static array holds %zu (use mnt_compute_kernel_map_sizes)",
+              (long long)num_offsets, num_tiles, kTargetsPerTile, words, kStaticScratchWords);
+    unsigned *base = static_scratch();
+    unsigned *tile_counts = base;                  // every word in use is written by count_tiles_kernel
+    unsigned *row_sizes = base + static_cast<size_t>(num_offsets) * num_tiles;
+    enqueue_count_tiles(kernel_map, index_dtype, num_offsets, num_targets, tile_counts, num_tiles, stream);
+    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes);
+    check_launch("tile_scan_kernel");
+    const unsigned grid = grid_for(num_offsets, 256);
+    if (index_dtype == MNT_INT32) {
+      export_sizes_kernel<int32_t><<<grid, 256, 0, stream>>>(row_sizes, static_cast<int>(num_offsets), static_cast<int32_t *>(sizes_out));
+    } else {
+      export_sizes_kernel<int64_t><<<grid, 256, 0, stream>>>(row_sizes, static_cast<int>(num_offsets), static_cast<int64_t *>(sizes_out));
+    }
+    check_launch("export_sizes_kernel");
   });
 }

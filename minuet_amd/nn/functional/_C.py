@@ -53,6 +53,7 @@ SIGNATURES = {
     "mnt_query_sorted_index_with_offsets": (_int, [_vp, _i64, _vp, _i64, _vp, _i64, _int, _int,
                                                    _vp, _vp, _i64, _int, _vp, _int, _vp]),
     "mnt_compute_kernel_map_sizes": (_int, [_vp, _i64, _i64, _int, _vp, _vp]),
+    "mnt_compute_kernel_map_sizes_static": (_int, [_vp, _i64, _i64, _int, _vp, _vp]),
     "mnt_compute_kernel_map_masks": (_int, [_vp, _i64, _i64, _i64, _int, _vp, _vp, _vp]),
     "mnt_kernel_map_query": (_int, [_vp, _i64, _vp, _i64, _pi64, _i64, _int, _int, _vp, _vp, _i64,
                                     _int, _int, _pi64, _pi64, _pi64, _vp, _pi64, _pi64, _vp]),
@@ -415,6 +416,26 @@ def cuda_compute_kernel_map_sizes(kernel_map: torch.Tensor) -> torch.Tensor:
             _ptr(kernel_map), kernel_map.size(0), kernel_map.size(1), icode, _ptr(sizes),
             _stream(device)))
     return sizes
+
+
+STATIC_SCRATCH_WORDS = 1 << 20
+
+
+def compute_kernel_map_sizes_static(kernel_map: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """:func:`cuda_compute_kernel_map_sizes` through the entry point that
+    allocates nothing: ``out`` ([O], dtype of ``kernel_map``) is written in
+    place and the counts live in the library's static device array, so maps
+    beyond ``O * (ceil(T / 512) + 1) <= STATIC_SCRATCH_WORDS`` are refused."""
+    _ensure_ndim("kernel_map", kernel_map, 2)
+    device = _common_device([kernel_map, out])
+    icode = _int_code(_common_dtype([kernel_map, out]), "tensor", "compute_kernel_map_sizes_static")
+    if not kernel_map.is_contiguous() or not out.is_contiguous() or out.numel() != kernel_map.size(0):
+        _fail("compute_kernel_map_sizes_static needs contiguous tensors and one output entry per offset")
+    with _on(device):
+        _check(load_library().mnt_compute_kernel_map_sizes_static(
+            _ptr(kernel_map), kernel_map.size(0), kernel_map.size(1), icode, _ptr(out),
+            _stream(device)))
+    return out
 
 
 def cuda_compute_kernel_map_masks(num_sources: int, kernel_map: torch.Tensor,
