@@ -30,10 +30,9 @@ QUERY_TRAFFIC_BYTES = 30.79e6
 
 
 def map_step(_C, coords_dev, offsets):
-    _, sorted_dev, bounds = _C.sort_coordinates(coords_dev, return_bounds=True)
-    built = _C.kernel_map_build(sorted_dev, sorted_dev, offsets, None, None, reorder=False,
-                                want_masks=False, want_lists=True, source_bounds=bounds,
-                                target_bounds=bounds)
+    """One Map step: unsorted voxels -> sorted voxels -> per-offset pair lists in
+    the order KernelMapCache keeps them (rows by ascending size), one library call."""
+    _, sorted_dev, built = _C.sorted_kernel_map_lists(coords_dev, offsets, reorder=True)
     return sorted_dev, built
 
 
@@ -296,7 +295,7 @@ def main():
     assert np.array_equal(sorted_dev.cpu().numpy(), ref_sorted)
     import c_oracle
     ref_map = c_oracle.query(ref_sorted, ref_sorted, offsets32)
-    ein, eout = c_oracle.pair_lists(ref_map)
+    ein, eout, _ = orc.kernel_map_pair_lists(ref_map[orc.stable_size_order(orc.compute_kernel_map_sizes(ref_map))])
     assert np.array_equal(built["in_idx"].cpu().numpy(), ein)
     assert np.array_equal(built["out_idx"].cpu().numpy(), eout)
 

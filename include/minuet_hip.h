@@ -229,6 +229,55 @@ int mnt_kernel_map_build(const void *sources, int64_t num_sources,
                          int32_t *sizes_dev_out, int32_t *order_dev_out,
                          int64_t *sizes_host_out, int64_t *order_host_out, void *stream);
 
+/* The pair lists alone, for callers that need neither the dense map nor the rank
+ * tables: arguments as mnt_kernel_map_build without kernel_map_out and the
+ * two tables; in_idx_out / out_idx_out have room for list_capacity >= O * T
+ * entries each, of which the first nnz = sum(sizes) are written.  The query
+ * keeps each wavefront's hits compacted in scratch instead of writing the
+ * dense map, and one more launch moves them to their list positions, so the
+ * dense [O, T] map is neither written nor read back.  One wait (sizes and
+ * order; the lists are being written meanwhile), one more only when bounds
+ * are missing.  Needs S, T, O > 0.  Same reference code
+ * (minuet/nn/convolutions.py:147-170, with the lists taking the place of the
+ * rank tables of csrc/minuet/cuda/functions/scan.cu:292-365). */
+int mnt_kernel_map_lists(const void *sources, int64_t num_sources,
+                         const void *targets, int64_t num_targets,
+                         const int64_t *offsets_host, int64_t num_offsets,
+                         int ndim, int coord_dtype,
+                         const void *source_batch_dims, const void *target_batch_dims,
+                         int64_t num_batches, int batch_dtype, int reorder,
+                         const int64_t *source_bounds_host, const int64_t *target_bounds_host,
+                         int64_t *bounds_host_out,
+                         int32_t *in_idx_out, int32_t *out_idx_out, int64_t list_capacity,
+                         int32_t *sizes_dev_out, int32_t *order_dev_out,
+                         int64_t *sizes_host_out, int64_t *order_host_out, void *stream);
+
+/* The Map step of a stride-1 (submanifold) layer on raw input in ONE call:
+ * arg-sort of coords[n, ndim] (one cloud, no batch_dims) as
+ * mnt_arg_sort_coordinates does it (indices_out int32 [n], sorted_coords_out
+ * [n, ndim]) followed by the pair lists of the kernel map of the sorted cloud
+ * onto itself as mnt_kernel_map_lists builds them (offsets_host int64 [O, ndim],
+ * lists with room for list_capacity >= O * n entries, sizes / order on the
+ * device and on the host).  bounds_host_out (8 x int64) receives the
+ * coordinate minima [0..3] and maxima [4..7].
+ * For clouds of 2 048 .. 2 097 152 rows and up to 64 offsets the whole step is
+ * a chain of six launches (bounds, bucket histogram, dealing, ranking, query,
+ * list placing) that never returns to the host in between: key layouts, bucket
+ * starts and the query plan are worked out on the device, and the host waits
+ * once, for the sizes.  A cloud the chain declines (a bucket beyond 4 096
+ * rows, keys that do not fit a word) and every other shape go through the two
+ * separate entry points inside this call; the results are the same.
+ * Replaces F.arg_sort_coordinates (minuet/nn/functional/indexing.py:14-56)
+ * followed by the miss path of KernelMapCache.get_kernel_map
+ * (minuet/nn/convolutions.py:147-170). */
+int mnt_sorted_kernel_map_lists(const void *coords, int64_t n, int ndim, int coord_dtype,
+                                const int64_t *offsets_host, int64_t num_offsets, int reorder,
+                                int32_t *indices_out, void *sorted_coords_out,
+                                int32_t *in_idx_out, int32_t *out_idx_out, int64_t list_capacity,
+                                int32_t *sizes_dev_out, int32_t *order_dev_out,
+                                int64_t *bounds_host_out, int64_t *sizes_host_out,
+                                int64_t *order_host_out, void *stream);
+
 /* Per-offset (in_idx, out_idx) pair lists from a dense int32 kernel map: for row
  * o the hits in target order are written at list positions
  * cumsum_host[o] .. cumsum_host[o]+sizes[o]-1 (cumsum_host[O+1], HOST, exclusive

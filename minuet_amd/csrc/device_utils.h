@@ -17,6 +17,13 @@ __device__ __forceinline__ unsigned long long lanes_below() {
   return (1ull << lane_id()) - 1ull;
 }
 
+// A 64-bit value that is the same in every lane, moved to scalar registers.
+__device__ __forceinline__ long long uniform64(long long v) {
+  const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
+  const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(static_cast<unsigned long long>(v) >> 32));
+  return static_cast<long long>((static_cast<unsigned long long>(hi) << 32) | lo);
+}
+
 // Batch of row i: the g with dims[g] <= i < dims[g+1] (dims has num_batches+1
 // entries).  Rows at or past dims[num_batches] land in the last batch.
 template <typename IT>

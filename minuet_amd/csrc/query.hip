@@ -22,6 +22,7 @@
 #include <mutex>
 
 #include "device_utils.h"
+#include "query_plan.h"
 #include "sort.h"
 
 namespace mnt {
@@ -49,6 +50,12 @@ struct KeyReader {
   }
 };
 
+// Width of the last coordinate's field, the least significant one of a key
+// (no indexing by a run-time value: the frame stays in registers).
+__device__ __forceinline__ int last_width(const Frame &f) {
+  return f.ndim == 1 ? f.width[0] : f.ndim == 2 ? f.width[1] : f.ndim == 3 ? f.width[2] : f.width[3];
+}
+
 // First index in [lo, hi) whose key is >= q (hi if none), found by one
 // wavefront probing 64 equally spaced rows per step.  All lanes must call
 // with the same arguments.
@@ -74,6 +81,23 @@ __device__ __forceinline__ long long wave_lower_bound(const KeyReader<CT, BT> &s
   return lo;
 }
 
+// Where a query launch that feeds the pair lists leaves its hits (the dense
+// map is not written then).  A wavefront owns 64 consecutive targets; the
+// hits it finds under offset o are stored compacted, in target order, at the
+// start of the wavefront's own 64 slots of stage[o, :], and the ballot that
+// says which of its targets they belong to goes to masks[o, wavefront].  A
+// tile whose source window takes several chunks cannot compact (a later chunk
+// may answer for a lower target): it marks itself in tile_mode and writes
+// every target's slot, -1 for a miss, like a row of the dense map.
+struct HitSink {
+  int *stage;                      // [O, T]
+  unsigned long long *masks;       // [O, ceil(T / 64)]
+  unsigned *row_totals;            // [O], zero before the launch; hits are added with atomics
+  unsigned *tile_mode;             // [tiles]: 0 = compacted, 1 = a slot per target
+  long long num_wave_tiles;        // ceil(T / 64)
+  int num_offsets;
+};
+
 // Settles the queries of one group against the candidates cand[0 .. span]
 // read from window position p on: writes the map entries this workgroup's
 // chunk is responsible for and counts the hits per offset.  The group and
@@ -81,12 +105,12 @@ __device__ __forceinline__ long long wave_lower_bound(const KeyReader<CT, BT> &s
 // registers, so that the loop, the row offsets of the map and the deltas are
 // scalar work.  d0 = q0 - base (wraps to a huge value when q0 < base, which
 // the range test then rejects like any other query outside the window).
-template <typename K, typename OT, bool kWholeWindow>
+template <typename K, typename OT, bool kWholeWindow, bool kLists>
 __device__ __forceinline__ void settle_group(
     const K (&cand)[kGroupSpan + 1], int p, unsigned long long q0, unsigned long long d0,
     const int4 &group, long long c0, bool valid, unsigned long long first_key,
     unsigned long long next_first, const int2 *s_members, unsigned *s_counts, bool count_hits,
-    OT *__restrict__ column, long long num_targets) {
+    OT *__restrict__ column, long long num_targets, const HitSink &sink, long long t) {
   constexpr unsigned long long kLimit = static_cast<unsigned long long>(static_cast<K>(~static_cast<K>(0)));
   const int first_member = __builtin_amdgcn_readfirstlane(group.z);
   const int members = __builtin_amdgcn_readfirstlane(group.w);
@@ -106,8 +130,22 @@ __device__ __forceinline__ void settle_group(
 #pragma unroll
     for (int x = 0; x <= kGroupSpan; ++x) at = cand[x] == q_rel ? x : at;
     const bool hit = mine && d < kLimit && at >= 0;
-    if (mine) column[static_cast<long long>(o) * num_targets] = hit ? found_base + static_cast<OT>(at) : static_cast<OT>(-1);
-    const unsigned hits = __popcll(__ballot(hit));
+    const unsigned long long votes = __ballot(hit);
+    if (kLists) {
+      const long long row = static_cast<long long>(o) * num_targets;
+      const long long wave_t0 = t - lane_id();
+      if (kWholeWindow) {
+        if (hit) sink.stage[row + wave_t0 + __popcll(votes & lanes_below())] = static_cast<int>(found_base) + at;
+        if (lane_id() == 0 && wave_t0 < num_targets) {
+          sink.masks[static_cast<long long>(o) * sink.num_wave_tiles + (wave_t0 >> 6)] = votes;
+        }
+      } else {
+        if (mine) sink.stage[row + t] = hit ? static_cast<int>(found_base) + at : -1;
+      }
+    } else {
+      if (mine) column[static_cast<long long>(o) * num_targets] = hit ? found_base + static_cast<OT>(at) : static_cast<OT>(-1);
+    }
+    const unsigned hits = __popcll(votes);
     if (count_hits && hits != 0 && lane_id() == 0) atomicAdd(&s_counts[o], hits);
   }
 }
@@ -116,12 +154,12 @@ __device__ __forceinline__ void settle_group(
 // staged in LDS as keys of type K relative to `base` (K = 32 bits when the
 // chunk's key range allows, which halves the LDS traffic of the searches).
 // A query outside [base, base + max K) cannot match and is forced to miss.
-template <typename K, typename OT, bool kWholeWindow>
+template <typename K, typename OT, bool kWholeWindow, bool kLists>
 __device__ __forceinline__ void resolve_chunk(
     const K *__restrict__ win, int top, unsigned long long base, long long c0,
     unsigned long long key, bool valid, unsigned long long first_key, unsigned long long next_first,
     const int4 *s_groups, const int2 *s_members, int num_groups, unsigned *s_counts, bool count_hits,
-    long long t, long long num_targets, OT *__restrict__ kernel_map) {
+    long long t, long long num_targets, OT *__restrict__ kernel_map, const HitSink &sink) {
   OT *column = kernel_map + t;
   constexpr unsigned long long kLimit = static_cast<unsigned long long>(static_cast<K>(~static_cast<K>(0)));
   for (int g0 = 0; g0 < num_groups; g0 += kGroupsInFlight) {
@@ -156,8 +194,9 @@ __device__ __forceinline__ void resolve_chunk(
       K cand[kGroupSpan + 1];
 #pragma unroll
       for (int x = 0; x <= kGroupSpan; ++x) cand[x] = win[p + x];
-      settle_group<K, OT, kWholeWindow>(cand, p, q0[j], q0[j] - base, group[j], c0, valid, first_key,
-                                        next_first, s_members, s_counts, count_hits, column, num_targets);
+      settle_group<K, OT, kWholeWindow, kLists>(cand, p, q0[j], q0[j] - base, group[j], c0, valid,
+                                                first_key, next_first, s_members, s_counts, count_hits,
+                                                column, num_targets, sink, t);
     }
   }
 }
@@ -172,51 +211,160 @@ __device__ __forceinline__ void resolve_chunk(
 // the row (at most zbits steps) follow.  Needs 32-bit relative keys whose
 // base is the start of a row, and at least 3 bits of last coordinate (then
 // the deltas of a group, at most kGroupSpan apart, never leave the row).
-template <typename OT, bool kWholeWindow>
+// settle_group for the form the list builds spend their time in: 32-bit
+// relative keys, a window of one chunk, hits going to the staging slots.  The
+// member entries were read together with the candidates (a group has at most
+// kGroupSpan + 1 members: unique deltas within a span of kGroupSpan), the loop
+// is unrolled and compares are 32 bits wide.  With kCollect the ballot of
+// offset o is not stored here but parked in lane o of `votes` (up to 64
+// offsets); the caller stores all of them with one instruction at the end.
+template <bool kCollect>
+__device__ __forceinline__ void settle_group_staged(
+    const unsigned (&cand)[kGroupSpan + 1], int p, unsigned long long d0, const int2 (&member)[kGroupSpan + 1],
+    int members, long long c0, bool inside, unsigned *s_counts, long long num_targets,
+    const HitSink &sink, long long wave_t0, unsigned &votes_lo, unsigned &votes_hi) {
+  const unsigned q0_rel = static_cast<unsigned>(d0);
+  // the largest step of a group is kGroupSpan: one test of the key range for all members
+  const bool low = inside && (d0 >> 32) == 0ull && q0_rel < 0xffffffffu - kGroupSpan;
+  const int found_base = static_cast<int>(c0) + p;
+#pragma unroll
+  for (int m = 0; m <= kGroupSpan; ++m) {
+    if (m >= members) break;                    // uniform
+    const unsigned step = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(member[m].x));
+    const int o = __builtin_amdgcn_readfirstlane(member[m].y);
+    const unsigned q_rel = q0_rel + step;
+    int at = -1;
+#pragma unroll
+    for (int x = 0; x <= kGroupSpan; ++x) at = cand[x] == q_rel ? x : at;
+    const bool hit = low && at >= 0;
+    const unsigned long long votes = __builtin_amdgcn_ballot_w64(hit);
+    const unsigned lo = static_cast<unsigned>(votes), hi = static_cast<unsigned>(votes >> 32);
+    const unsigned rank = __builtin_amdgcn_mbcnt_hi(hi, __builtin_amdgcn_mbcnt_lo(lo, 0u));
+    // the row and the wavefront's first slot are the same in every lane: the
+    // store takes them as its scalar base and the rank as its 32-bit offset
+    int *slots = sink.stage + (static_cast<long long>(o) * num_targets + wave_t0);
+    if (hit) slots[rank] = found_base + at;
+    if (kCollect) {
+      const bool keeper = static_cast<int>(lane_id()) == o;
+      votes_lo = keeper ? lo : votes_lo;
+      votes_hi = keeper ? hi : votes_hi;
+    } else if (lane_id() == 0 && wave_t0 < num_targets) {
+      sink.masks[static_cast<long long>(o) * sink.num_wave_tiles + (wave_t0 >> 6)] = votes;
+      atomicAdd(&s_counts[o], static_cast<unsigned>(__popcll(votes)));
+    }
+  }
+}
+
+template <typename OT, bool kWholeWindow, bool kLists>
 __device__ __forceinline__ void resolve_chunk_rows(
     const unsigned *__restrict__ win, const unsigned short *__restrict__ dir, int len, int zbits,
     unsigned num_rows, unsigned long long base, long long c0, unsigned long long key, bool valid,
     unsigned long long first_key, unsigned long long next_first, const int4 *s_groups,
     const int2 *s_members, int num_groups, unsigned *s_counts, bool count_hits, long long t,
-    long long num_targets, OT *__restrict__ kernel_map) {
+    long long num_targets, OT *__restrict__ kernel_map, const HitSink &sink) {
   OT *column = kernel_map + t;
-  for (int g = 0; g < num_groups; ++g) {
-    const int4 group = s_groups[g];
-    const unsigned long long first_delta =
-        static_cast<unsigned long long>(static_cast<unsigned>(group.x)) |
-        (static_cast<unsigned long long>(static_cast<unsigned>(group.y)) << 32);
-    const unsigned long long q0 = key + first_delta;
-    const unsigned long long d0 = q0 - base;
-    const unsigned long long row = d0 >> zbits;
-    const bool inside = q0 >= base && row < num_rows;
-    const unsigned start = inside ? dir[row] : 0u;
-    const unsigned q0_rel = static_cast<unsigned>(d0);
-    const unsigned q_last = q0_rel + static_cast<unsigned>(s_members[group.z + group.w - 1].x);
-    int p = start != 0 ? static_cast<int>(start) - 1 : 0;
-    unsigned cand[kGroupSpan + 1];
+  constexpr bool kStaged = kWholeWindow && kLists;
+  // staged form: up to 64 offsets leave their ballots in the lanes of one
+  // register pair; they are stored once, after the last group
+  const bool collect = kStaged && sink.num_offsets <= kWave;
+  const long long wave_t0 = uniform64(t - lane_id());
+  unsigned votes_lo = 0, votes_hi = 0;
+  // three groups in lockstep: their directory reads, then their candidate
+  // reads, are in flight together
+  for (int g0 = 0; g0 < num_groups; g0 += kGroupsInFlight) {
+    int4 group[kGroupsInFlight];
+    unsigned long long q0[kGroupsInFlight], d0[kGroupsInFlight], row[kGroupsInFlight];
+    unsigned start[kGroupsInFlight], q_last[kGroupsInFlight];
+    int2 member[kGroupsInFlight][kGroupSpan + 1];
+    bool inside[kGroupsInFlight];
 #pragma unroll
-    for (int x = 0; x < 4; ++x) cand[x] = win[p + x];
-    cand[4] = 0xffffffffu;
-    if (start != 0 && cand[3] < q_last && (cand[3] >> zbits) == row) {
-      // a long row whose first four keys do not cover the queries: the lower
-      // bound of the first query inside the row, then the usual span of
-      // candidates from there
-      int lo = p;
-      int hi = p + (1 << zbits) < len ? p + (1 << zbits) : len;      // zbits <= 24 here
-      while (lo < hi) {
-        const int mid = (lo + hi) >> 1;
-        if (win[mid] < q0_rel) {
-          lo = mid + 1;
-        } else {
-          hi = mid;
-        }
+    for (int j = 0; j < kGroupsInFlight; ++j) {
+      group[j] = s_groups[g0 + j < num_groups ? g0 + j : num_groups - 1];
+      const unsigned long long first_delta =
+          static_cast<unsigned long long>(static_cast<unsigned>(group[j].x)) |
+          (static_cast<unsigned long long>(static_cast<unsigned>(group[j].y)) << 32);
+      q0[j] = key + first_delta;
+      d0[j] = q0[j] - base;
+      row[j] = d0[j] >> zbits;
+      inside[j] = valid && q0[j] >= base && row[j] < num_rows;
+      start[j] = inside[j] ? dir[row[j]] : 0u;
+      // entries past the group's last member repeat the last one
+#pragma unroll
+      for (int m = 0; m <= kGroupSpan; ++m) {
+        member[j][m] = s_members[group[j].z + (m < group[j].w ? m : group[j].w - 1)];
       }
-      p = lo;
-#pragma unroll
-      for (int x = 0; x <= kGroupSpan; ++x) cand[x] = win[p + x];
+      q_last[j] = static_cast<unsigned>(d0[j]) + static_cast<unsigned>(member[j][kGroupSpan].x);
     }
-    settle_group<unsigned, OT, kWholeWindow>(cand, p, q0, d0, group, c0, valid, first_key, next_first,
-                                             s_members, s_counts, count_hits, column, num_targets);
+    int p[kGroupsInFlight];
+    unsigned cand[kGroupsInFlight][kGroupSpan + 1];
+#pragma unroll
+    for (int j = 0; j < kGroupsInFlight; ++j) {
+      p[j] = start[j] != 0 ? static_cast<int>(start[j]) - 1 : 0;
+#pragma unroll
+      for (int x = 0; x < 4; ++x) cand[j][x] = win[p[j] + x];
+      cand[j][4] = 0xffffffffu;
+    }
+#pragma unroll
+    for (int j = 0; j < kGroupsInFlight; ++j) {
+      if (g0 + j >= num_groups) continue;       // uniform across the workgroup
+      const unsigned q0_rel = static_cast<unsigned>(d0[j]);
+      if (start[j] != 0 && cand[j][3] < q_last[j] && (cand[j][3] >> zbits) == row[j]) {
+        // a long row whose first four keys do not cover the queries.  In a row
+        // without holes (a wall: every height occupied) the first query sits
+        // as far behind the row's first key as their last coordinates differ:
+        // look there first and keep the place if its neighbours confirm that
+        // it is the lower bound; search the row otherwise.
+        const int last = len - 1;
+        int guess = p[j] + (q0_rel > cand[j][0] ? static_cast<int>(q0_rel - cand[j][0]) : 0);
+        guess = guess < last ? guess : last;
+        const unsigned before = win[guess > 0 ? guess - 1 : 0];
+        unsigned at[kGroupSpan + 1];
+#pragma unroll
+        for (int x = 0; x <= kGroupSpan; ++x) at[x] = win[guess + x];
+        if ((guess == 0 || before < q0_rel) && at[0] >= q0_rel) {
+          p[j] = guess;
+        } else {
+          int lo = p[j];
+          int hi = p[j] + (1 << zbits) < len ? p[j] + (1 << zbits) : len;      // zbits <= 24 here
+          while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (win[mid] < q0_rel) {
+              lo = mid + 1;
+            } else {
+              hi = mid;
+            }
+          }
+          p[j] = lo;
+#pragma unroll
+          for (int x = 0; x <= kGroupSpan; ++x) at[x] = win[lo + x];
+        }
+#pragma unroll
+        for (int x = 0; x <= kGroupSpan; ++x) cand[j][x] = at[x];
+      }
+      if (kStaged) {
+        const int members = __builtin_amdgcn_readfirstlane(group[j].w);
+        if (collect) {
+          settle_group_staged<true>(cand[j], p[j], d0[j], member[j], members, c0, inside[j], s_counts,
+                                    num_targets, sink, wave_t0, votes_lo, votes_hi);
+        } else {
+          settle_group_staged<false>(cand[j], p[j], d0[j], member[j], members, c0, inside[j], s_counts,
+                                     num_targets, sink, wave_t0, votes_lo, votes_hi);
+        }
+      } else {
+        settle_group<unsigned, OT, kWholeWindow, kLists>(cand[j], p[j], q0[j], d0[j], group[j], c0, valid,
+                                                         first_key, next_first, s_members, s_counts,
+                                                         count_hits, column, num_targets, sink, t);
+      }
+    }
+  }
+  if (collect && wave_t0 < num_targets) {
+    // lane o holds the ballot of offset o
+    const int o = lane_id();
+    if (o < sink.num_offsets) {
+      const unsigned long long votes = (static_cast<unsigned long long>(votes_hi) << 32) | votes_lo;
+      sink.masks[static_cast<long long>(o) * sink.num_wave_tiles + (wave_t0 >> 6)] = votes;
+      atomicAdd(&s_counts[o], static_cast<unsigned>(__popcll(votes)));
+    }
   }
 }
 
@@ -240,12 +388,35 @@ struct CarriedTables {
   int v[kCarriedInts];
 };
 
-template <typename CT, typename BT, typename OT>
+template <typename CT, typename BT, typename OT, bool kLists>
 __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     KeyReader<CT, BT> src, KeyReader<CT, BT> tgt, Frame frame, const int *__restrict__ tables,
     CarriedTables carried, int num_groups, int num_offsets, long long delta_min, long long delta_max,
-    OT *__restrict__ kernel_map, unsigned *__restrict__ tile_counts, int num_tiles, int dir_rows) {
+    OT *__restrict__ kernel_map, unsigned *__restrict__ tile_counts, int num_tiles, int dir_rows,
+    HitSink sink, const DevicePlan *__restrict__ device_plan) {
   extern __shared__ __align__(16) unsigned s_dynamic[];
+  if (device_plan != nullptr) {
+    // a launch inside a chain that never went back to the host: the verdict of
+    // the launches before it and the plan come from device memory.  The values
+    // are the same in every lane; saying so keeps them in scalar registers.
+    const int verdict = device_plan->verdict;
+#pragma unroll
+    for (int k = 0; k < MNT_MAX_NDIM; ++k) {
+      frame.lo[k] = uniform64(device_plan->frame.lo[k]);
+      frame.shift[k] = __builtin_amdgcn_readfirstlane(device_plan->frame.shift[k]);
+      frame.width[k] = __builtin_amdgcn_readfirstlane(device_plan->frame.width[k]);
+    }
+    frame.batch_shift = __builtin_amdgcn_readfirstlane(device_plan->frame.batch_shift);
+    frame.batch_width = 0;
+    frame.total_bits = __builtin_amdgcn_readfirstlane(device_plan->frame.total_bits);
+    tables = device_plan->tables;
+    num_groups = __builtin_amdgcn_readfirstlane(device_plan->num_groups);
+    delta_min = uniform64(device_plan->delta_min);
+    delta_max = uniform64(device_plan->delta_max);
+    const int in_rows = __builtin_amdgcn_readfirstlane(device_plan->groups_in_rows);
+    if (__builtin_amdgcn_readfirstlane(verdict) != 0) return;
+    dir_rows = in_rows != 0 && last_width(frame) >= 3 ? dir_rows : 0;
+  }
   __shared__ unsigned long long win[kWindowChunk + kWindowPad];
   __shared__ long long s_bounds[2];
   // dynamic LDS: [group table: 4 words each][member table: 2 words each][hit counts]
@@ -256,7 +427,7 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
   unsigned *s_dir_words = s_counts + num_offsets;
   unsigned short *s_dir = reinterpret_cast<unsigned short *>(s_dir_words);
   // last coordinate: the least significant field of a key
-  const int zbits = frame.width[frame.ndim - 1];
+  const int zbits = last_width(frame);
 
   const int tid = threadIdx.x;
   const int w = tid >> 6;
@@ -348,19 +519,22 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     const bool counting = tile_counts != nullptr;
 #define MNT_RESOLVE(WHOLE)                                                                         \
     if (by_rows) {                                                                                 \
-      resolve_chunk_rows<OT, WHOLE>(reinterpret_cast<const unsigned *>(win), s_dir, len, zbits,    \
-                                    static_cast<unsigned>(num_rows), base, c0, key, valid,         \
-                                    answers_from, answers_to, s_groups, s_members, num_groups,     \
-                                    s_counts, counting, t, num_targets, kernel_map);               \
+      resolve_chunk_rows<OT, WHOLE, kLists>(reinterpret_cast<const unsigned *>(win), s_dir, len,   \
+                                            zbits, static_cast<unsigned>(num_rows), base, c0, key, \
+                                            valid, answers_from, answers_to, s_groups, s_members,  \
+                                            num_groups, s_counts, counting, t, num_targets,        \
+                                            kernel_map, sink);                                     \
     } else if (narrow) {                                                                           \
-      resolve_chunk<unsigned, OT, WHOLE>(reinterpret_cast<const unsigned *>(win), top, base, c0,   \
-                                         key, valid, answers_from, answers_to, s_groups,           \
-                                         s_members, num_groups, s_counts, counting, t,             \
-                                         num_targets, kernel_map);                                 \
+      resolve_chunk<unsigned, OT, WHOLE, kLists>(reinterpret_cast<const unsigned *>(win), top,     \
+                                                 base, c0, key, valid, answers_from, answers_to,   \
+                                                 s_groups, s_members, num_groups, s_counts,        \
+                                                 counting, t, num_targets, kernel_map, sink);      \
     } else {                                                                                       \
-      resolve_chunk<unsigned long long, OT, WHOLE>(win, top, 0ull, c0, key, valid, answers_from,   \
-                                                   answers_to, s_groups, s_members, num_groups,    \
-                                                   s_counts, counting, t, num_targets, kernel_map); \
+      resolve_chunk<unsigned long long, OT, WHOLE, kLists>(win, top, 0ull, c0, key, valid,         \
+                                                           answers_from, answers_to, s_groups,     \
+                                                           s_members, num_groups, s_counts,        \
+                                                           counting, t, num_targets, kernel_map,   \
+                                                           sink);                                  \
     }
     if (num_chunks == 1) {
       MNT_RESOLVE(true)
@@ -372,9 +546,12 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
   if (tile_counts != nullptr) {
     __syncthreads();
     for (int o = tid; o < num_offsets; o += kQueryThreads) {
-      tile_counts[static_cast<long long>(o) * num_tiles + blockIdx.x] = s_counts[o];
+      const unsigned hits = s_counts[o];
+      tile_counts[static_cast<long long>(o) * num_tiles + blockIdx.x] = hits;
+      if (kLists && hits != 0) atomicAdd(&sink.row_totals[o], hits);
     }
   }
+  if (kLists && tid == 0) sink.tile_mode[blockIdx.x] = num_chunks == 1 ? 0u : 1u;
 }
 
 // Hit counts of every (row, tile of 512 targets) of an existing dense map.
@@ -557,6 +734,146 @@ __global__ __launch_bounds__(kQueryBlock) void emit_kernel(
   }
 }
 
+
+// Final pair lists from the staged hits of a lists-mode query launch.  Row o
+// of the lists starts where the rows ordered before it end (ascending hit
+// count with ties in offset order when reorder is set, offset order
+// otherwise); inside the row the tiles follow each other.  A workgroup takes
+// kPlaceTiles consecutive tiles of one offset: it works out the list position
+// of its first hit from the row totals and the tile counts before it (every
+// workgroup sums those for itself; there is no scan pass), then each
+// wavefront copies its tiles 64 targets at a time: the ballot says which
+// targets hit, their sources are read from the staging slots and both go to
+// consecutive list entries.  Workgroup (0, 0) also ranks the rows for the
+// host (plan_from_sizes) and writes the device copies of sizes and order.
+constexpr int kPlaceTiles = 4;
+constexpr int kPlaceBlock = 256;
+
+__global__ __launch_bounds__(kPlaceBlock) void place_kernel(
+    const int *__restrict__ stage, const unsigned long long *__restrict__ masks,
+    const unsigned *__restrict__ tile_counts, const unsigned *__restrict__ row_totals,
+    const unsigned *__restrict__ tile_mode, long long num_targets, int num_offsets, int num_tiles,
+    long long num_wave_tiles, int reorder, int *__restrict__ in_idx, int *__restrict__ out_idx,
+    unsigned *__restrict__ plan, unsigned *__restrict__ plan_host, unsigned long long *flag,
+    unsigned long long sequence, int *__restrict__ sizes_out, int *__restrict__ order_out,
+    const DevicePlan *__restrict__ chain_plan, const long long *__restrict__ folded_bounds,
+    long long *chain_host) {
+  __shared__ unsigned s_partial[kPlaceBlock / kWave];
+  const int tid = threadIdx.x;
+  const int lane = lane_id();
+  const int w = tid >> 6;
+  const int o = blockIdx.y;
+  const int tile0 = blockIdx.x * kPlaceTiles;
+  if (chain_plan != nullptr) {
+    // end of a chain of launches: the host learns the chain's verdict and the
+    // coordinate bounds together with the sizes
+    const int verdict = chain_plan->verdict;
+    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) {
+#pragma unroll
+      for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) chain_host[slot] = folded_bounds[slot];
+      chain_host[2 * MNT_MAX_NDIM] = static_cast<long long>(verdict);
+      if (verdict != 0) {
+        __threadfence_system();
+        __hip_atomic_store(flag, sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
+    }
+    if (verdict != 0) return;
+  }
+  if (blockIdx.x == 0 && blockIdx.y == 0) {
+    plan_from_sizes(row_totals, num_offsets, reorder, plan, plan_host, flag, sequence);
+    for (int j = tid; j < num_offsets; j += kPlaceBlock) {
+      if (order_out) order_out[j] = static_cast<int>(plan[j]);
+      if (sizes_out) sizes_out[j] = static_cast<int>(plan[2 * num_offsets + j]);
+    }
+  }
+  // list position of the first hit of (o, tile0): rows before row o, tiles before tile0
+  const unsigned mine = row_totals[o];
+  unsigned before = 0;
+  for (int p = tid; p < num_offsets; p += kPlaceBlock) {
+    const unsigned other = row_totals[p];
+    const bool first = reorder ? (other < mine || (other == mine && p < o)) : p < o;
+    before += first ? other : 0u;
+  }
+  const unsigned *counts = tile_counts + static_cast<long long>(o) * num_tiles;
+  for (int i = tid; i < tile0; i += kPlaceBlock) before += counts[i];
+  for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off);
+  if (lane == 0) s_partial[w] = before;
+  __syncthreads();
+  unsigned base = 0;
+#pragma unroll
+  for (int ww = 0; ww < kPlaceBlock / kWave; ++ww) base += s_partial[ww];
+  // tiles of this workgroup: exclusive prefix of their counts
+  const int my_tile = tile0 + lane;
+  const unsigned count = lane < kPlaceTiles && my_tile < num_tiles ? counts[my_tile] : 0u;
+  unsigned inclusive = count;
+  for (int off = 1; off < kPlaceTiles; off <<= 1) {
+    const unsigned u = __shfl_up(inclusive, off);
+    if (lane >= off) inclusive += u;
+  }
+  const unsigned exclusive = inclusive - count;
+  const long long row = static_cast<long long>(o) * num_targets;
+  const unsigned long long below = lanes_below();
+  for (int j = w; j < kPlaceTiles; j += kPlaceBlock / kWave) {
+    const int tile = tile0 + j;
+    if (tile >= num_tiles) break;                                   // uniform per wavefront
+    const unsigned tile_hits = __shfl(count, j);
+    if (tile_hits == 0) continue;
+    unsigned at = base + __shfl(exclusive, j);
+    const long long t_tile = static_cast<long long>(tile) * kTargetsPerTile;
+    constexpr int kSegments = kTargetsPerTile / kWave;
+    if (tile_mode[tile] == 0) {
+      // lane s holds the ballot of segment s and the hits before it
+      const long long wave_tile = (t_tile >> 6) + lane;
+      const unsigned long long my_mask =
+          lane < kSegments && wave_tile < num_wave_tiles
+              ? masks[static_cast<long long>(o) * num_wave_tiles + wave_tile] : 0ull;
+      const unsigned my_hits = __popcll(my_mask);
+      unsigned seg_inclusive = my_hits;
+      for (int off = 1; off < kSegments; off <<= 1) {
+        const unsigned u = __shfl_up(seg_inclusive, off);
+        if (lane >= off) seg_inclusive += u;
+      }
+      const unsigned seg_exclusive = seg_inclusive - my_hits;
+      int found[kSegments];
+      unsigned rank[kSegments];
+      bool hit[kSegments];
+#pragma unroll
+      for (int s = 0; s < kSegments; ++s) {
+        const unsigned long long mask = __shfl(my_mask, s);
+        hit[s] = (mask >> lane) & 1ull;
+        const unsigned r = __popcll(mask & below);
+        rank[s] = at + __shfl(seg_exclusive, s) + r;
+        found[s] = hit[s] ? stage[row + t_tile + s * kWave + r] : -1;
+      }
+#pragma unroll
+      for (int s = 0; s < kSegments; ++s) {
+        if (hit[s]) {
+          in_idx[rank[s]] = found[s];
+          out_idx[rank[s]] = static_cast<int>(t_tile + s * kWave + lane);
+        }
+      }
+    } else {
+      int found[kSegments];
+#pragma unroll
+      for (int s = 0; s < kSegments; ++s) {
+        const long long t = t_tile + s * kWave + lane;
+        found[s] = t < num_targets ? stage[row + t] : -1;
+      }
+#pragma unroll
+      for (int s = 0; s < kSegments; ++s) {
+        const bool hit = found[s] != -1;
+        const unsigned long long mask = __ballot(hit);
+        if (hit) {
+          const unsigned r = at + __popcll(mask & below);
+          in_idx[r] = found[s];
+          out_idx[r] = static_cast<int>(t_tile + s * kWave + lane);
+        }
+        at += __popcll(mask);
+      }
+    }
+  }
+}
+
 template <typename IT>
 __global__ __launch_bounds__(256) void export_sizes_kernel(const unsigned *__restrict__ sizes,
                                                            int n, IT *__restrict__ out) {
@@ -692,10 +1009,10 @@ static void check_query_args(const QueryArgs &a, int64_t num_offsets) {
   }
 }
 
-template <typename CT, typename BT, typename OT>
+template <typename CT, typename BT, typename OT, bool kLists>
 static void launch_query(const QueryArgs &a, const QueryPlan &plan, const int *d_tables,
                          int num_offsets, OT *kernel_map, unsigned *tile_counts, int num_tiles,
-                         hipStream_t stream) {
+                         const HitSink &sink, hipStream_t stream) {
   KeyReader<CT, BT> src{static_cast<const CT *>(a.sources), static_cast<const BT *>(a.source_batch_dims),
                         static_cast<int>(a.num_batches), a.num_sources};
   KeyReader<CT, BT> tgt{static_cast<const CT *>(a.targets), static_cast<const BT *>(a.target_batch_dims),
@@ -709,9 +1026,9 @@ static void launch_query(const QueryArgs &a, const QueryPlan &plan, const int *d
   CarriedTables carried;
   memset(&carried, 0, sizeof(carried));
   if (d_tables == nullptr) memcpy(carried.v, plan.tables.data(), sizeof(int) * plan.tables.size());
-  query_kernel<CT, BT, OT><<<num_tiles, kQueryThreads, dyn, stream>>>(
+  query_kernel<CT, BT, OT, kLists><<<num_tiles, kQueryThreads, dyn, stream>>>(
       src, tgt, plan.frame, d_tables, carried, plan.num_groups, num_offsets, plan.delta_min,
-      plan.delta_max, kernel_map, tile_counts, num_tiles, dir_rows);
+      plan.delta_max, kernel_map, tile_counts, num_tiles, dir_rows, sink, nullptr);
   check_launch("query_kernel");
 }
 
@@ -736,10 +1053,12 @@ static void resolve_bounds(const QueryArgs &a, const int64_t *source_bounds, con
 
 // Runs the query into kernel_map (element type out_dtype) and, when tile_counts
 // is given, the per-(offset, tile) hit counts.  offsets_host: int64 [O, ndim].
+// With a sink the hits are staged for the pair lists instead and kernel_map
+// is not touched (tile_counts is needed then).
 static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t num_offsets,
                       const int64_t *source_bounds, const int64_t *target_bounds,
                       int64_t *bounds_out, void *kernel_map, int out_dtype, unsigned *tile_counts,
-                      Scope &scope, hipStream_t stream) {
+                      Scope &scope, hipStream_t stream, const HitSink *sink = nullptr) {
   const int num_tiles = static_cast<int>(div_ceil(a.num_targets, kTargetsPerTile));
   const bool batched = a.source_batch_dims != nullptr && a.num_batches > 1;
   profile_mark("enter:query", stream);
@@ -768,9 +1087,21 @@ static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t n
   const bool c32 = a.coord_dtype == MNT_INT32;
   const bool b32 = !batched || a.batch_dtype == MNT_INT32;
   const bool o32 = out_dtype == MNT_INT32;
-#define MNT_Q(CT, BT, OT)                                                                 \
-  launch_query<CT, BT, OT>(b, plan, d_tables, no, static_cast<OT *>(kernel_map), tile_counts, \
-                           num_tiles, stream)
+  if (sink != nullptr) {
+#define MNT_QL(CT, BT)                                                                          \
+  launch_query<CT, BT, int32_t, true>(b, plan, d_tables, no, nullptr, tile_counts, num_tiles, *sink, stream)
+    if (c32 && b32) MNT_QL(int32_t, int32_t);
+    else if (c32) MNT_QL(int32_t, int64_t);
+    else if (b32) MNT_QL(int64_t, int32_t);
+    else MNT_QL(int64_t, int64_t);
+#undef MNT_QL
+    profile_mark("query", stream);
+    return;
+  }
+  const HitSink none{nullptr, nullptr, nullptr, nullptr, 0, 0};
+#define MNT_Q(CT, BT, OT)                                                                        \
+  launch_query<CT, BT, OT, false>(b, plan, d_tables, no, static_cast<OT *>(kernel_map), tile_counts, \
+                                  num_tiles, none, stream)
   if (c32 && b32 && o32) MNT_Q(int32_t, int32_t, int32_t);
   else if (c32 && b32) MNT_Q(int32_t, int32_t, int64_t);
   else if (c32 && o32) MNT_Q(int32_t, int64_t, int32_t);
@@ -1097,6 +1428,195 @@ extern "C" int mnt_kernel_map_build(const void *sources, int64_t num_sources, co
                           stream, plan, sizes_dev_out, order_dev_out);
     collect_sizes(arena, sequence, num_offsets, sizes_host_out, order_host_out);
     profile_mark("map_sizes_order+emit+sync", stream);
+  });
+}
+
+extern "C" int mnt_kernel_map_lists(const void *sources, int64_t num_sources, const void *targets,
+                                    int64_t num_targets, const int64_t *offsets_host,
+                                    int64_t num_offsets, int ndim, int coord_dtype,
+                                    const void *source_batch_dims, const void *target_batch_dims,
+                                    int64_t num_batches, int batch_dtype, int reorder,
+                                    const int64_t *source_bounds_host,
+                                    const int64_t *target_bounds_host, int64_t *bounds_host_out,
+                                    int32_t *in_idx_out, int32_t *out_idx_out, int64_t list_capacity,
+                                    int32_t *sizes_dev_out, int32_t *order_dev_out,
+                                    int64_t *sizes_host_out, int64_t *order_host_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    QueryArgs a{sources, num_sources, targets, num_targets, ndim, coord_dtype,
+                source_batch_dims, target_batch_dims, num_batches, batch_dtype};
+    check_query_args(a, num_offsets);
+    MNT_CHECK(offsets_host != nullptr && sizes_host_out != nullptr && order_host_out != nullptr, "null argument");
+    MNT_CHECK(num_sources > 0 && num_targets > 0 && num_offsets > 0,
+              "mnt_kernel_map_lists needs sources, targets and offsets (use mnt_kernel_map_query / _emit "
+              "for empty operands)");
+    MNT_CHECK(in_idx_out != nullptr && out_idx_out != nullptr, "in_idx_out / out_idx_out is null");
+    MNT_CHECK(list_capacity >= num_offsets * num_targets,
+              "list_capacity = %lld cannot hold every (offset, target) pair (%lld)",
+              (long long)list_capacity, (long long)(num_offsets * num_targets));
+    MNT_CHECK(sizeof(unsigned) * 3 * num_offsets + 1024 <= Arena::kPinnedBytes,
+              "too many kernel offsets (%lld)", static_cast<long long>(num_offsets));
+    Arena &arena = Arena::of(stream);
+    arena.map_state_valid = false;
+    if (bounds_host_out != nullptr) {
+      for (int i = 0; i < 16; ++i) bounds_host_out[i] = (i & 4) ? INT64_MIN : INT64_MAX;
+    }
+    Scope scope(stream);
+    const int no = static_cast<int>(num_offsets);
+    const int num_tiles = static_cast<int>(div_ceil(num_targets, kTargetsPerTile));
+    const int64_t num_wave_tiles = div_ceil(num_targets, kWave);
+    int *stage = scope.alloc<int>(static_cast<size_t>(num_offsets) * num_targets);
+    unsigned long long *masks = scope.alloc<unsigned long long>(static_cast<size_t>(num_offsets) * num_wave_tiles);
+    unsigned *tile_counts = scope.alloc<unsigned>(static_cast<size_t>(num_offsets) * num_tiles);
+    unsigned *tile_mode = scope.alloc<unsigned>(num_tiles);
+    unsigned *row_totals = scope.alloc<unsigned>(num_offsets);
+    unsigned *plan = scope.alloc<unsigned>(4 * num_offsets + 1);
+    enqueue_fill<unsigned>(row_totals, num_offsets, 0u, stream);
+    const HitSink sink{stage, masks, row_totals, tile_mode, num_wave_tiles, no};
+    run_query(a, offsets_host, num_offsets, source_bounds_host, target_bounds_host, bounds_host_out,
+              nullptr, MNT_INT32, tile_counts, scope, stream, &sink);
+    unsigned *d_plan_host = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned_device()) + Arena::kPlanOffset);
+    const unsigned long long sequence = arena.next_sequence();
+    dim3 grid(static_cast<unsigned>(div_ceil(num_tiles, kPlaceTiles)), static_cast<unsigned>(num_offsets));
+    place_kernel<<<grid, kPlaceBlock, 0, stream>>>(stage, masks, tile_counts, row_totals, tile_mode,
+                                                   num_targets, no, num_tiles, num_wave_tiles, reorder,
+                                                   in_idx_out, out_idx_out, plan, d_plan_host,
+                                                   arena.flag_device(1), sequence, sizes_dev_out,
+                                                   order_dev_out, nullptr, nullptr, nullptr);
+    check_launch("place_kernel");
+    collect_sizes(arena, sequence, num_offsets, sizes_host_out, order_host_out);
+    profile_mark("map_place+sync", stream);
+  });
+}
+
+// ---- sort -> query -> pair lists as one chain of six launches and one wait ----
+
+namespace mnt {
+
+constexpr size_t kChainHostOffset = 128;      // pinned block: bounds (8 words), then the chain's verdict
+
+template <typename CT>
+static void launch_query_chain(const CT *sorted, int64_t n, int ndim, int num_offsets,
+                               unsigned *tile_counts, int num_tiles, const HitSink &sink,
+                               const DevicePlan *plan, hipStream_t stream) {
+  KeyReader<CT, int32_t> rows{sorted, nullptr, 1, n};
+  Frame frame;
+  memset(&frame, 0, sizeof(frame));
+  frame.ndim = ndim;
+  CarriedTables carried;
+  memset(&carried, 0, sizeof(carried));
+  // LDS for the largest tables these offsets can make and for the row directory
+  const size_t dyn = sizeof(unsigned) * (6 * static_cast<size_t>(num_offsets) + num_offsets + 4) +
+                     sizeof(unsigned short) * static_cast<size_t>(kDirectoryRows);
+  query_kernel<CT, int32_t, int32_t, true><<<num_tiles, kQueryThreads, dyn, stream>>>(
+      rows, rows, frame, nullptr, carried, 0, num_offsets, 0, 0, nullptr, tile_counts, num_tiles,
+      kDirectoryRows, sink, plan);
+  check_launch("query_kernel");
+}
+
+}  // namespace mnt
+
+extern "C" int mnt_sorted_kernel_map_lists(const void *coords, int64_t n, int ndim, int coord_dtype,
+                                           const int64_t *offsets_host, int64_t num_offsets,
+                                           int reorder, int32_t *indices_out, void *sorted_coords_out,
+                                           int32_t *in_idx_out, int32_t *out_idx_out,
+                                           int64_t list_capacity, int32_t *sizes_dev_out,
+                                           int32_t *order_dev_out, int64_t *bounds_host_out,
+                                           int64_t *sizes_host_out, int64_t *order_host_out,
+                                           void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MNT_CHECK(ndim >= 1 && ndim <= MNT_MAX_NDIM, "ndim must be in [1, %d] but found %d", MNT_MAX_NDIM, ndim);
+    MNT_CHECK(n > 0 && n <= INT32_MAX, "number of coordinates %lld out of range", static_cast<long long>(n));
+    MNT_CHECK(num_offsets > 0 && num_offsets <= 65535, "number of offsets %lld out of range",
+              static_cast<long long>(num_offsets));
+    int_size(coord_dtype);
+    MNT_CHECK(coords != nullptr && offsets_host != nullptr && indices_out != nullptr &&
+                  sorted_coords_out != nullptr && in_idx_out != nullptr && out_idx_out != nullptr &&
+                  bounds_host_out != nullptr && sizes_host_out != nullptr && order_host_out != nullptr,
+              "null argument");
+    MNT_CHECK(list_capacity >= num_offsets * n,
+              "list_capacity = %lld cannot hold every (offset, target) pair (%lld)",
+              (long long)list_capacity, (long long)(num_offsets * n));
+    bool small_offsets = true;
+    for (int64_t i = 0; i < num_offsets * ndim; ++i) {
+      small_offsets = small_offsets && offsets_host[i] >= INT32_MIN / 2 && offsets_host[i] <= INT32_MAX / 2;
+    }
+    if (small_offsets && chain_sort_takes(n, 1, static_cast<int>(num_offsets))) {
+      profile_mark("enter:map_chain", stream);
+      Arena &arena = Arena::of(stream);
+      arena.map_state_valid = false;
+      Scope scope(stream);
+      const int no = static_cast<int>(num_offsets);
+      const int buckets = 1 << chain_sort_msd_bits(n);
+      const int num_tiles = static_cast<int>(div_ceil(n, kTargetsPerTile));
+      const int64_t num_wave_tiles = div_ceil(n, kWave);
+      ChainSortBuffers buf;
+      buf.partial = scope.alloc<long long>(128 * 8);
+      buf.folded = scope.alloc<long long>(2 * MNT_MAX_NDIM);
+      buf.counter_words = 2 * buckets + no;
+      buf.counters = scope.alloc<unsigned>(buf.counter_words);
+      buf.info = scope.alloc<unsigned>(4);
+      buf.status = scope.alloc<unsigned>(4);
+      buf.chunks = scope.alloc<uint2>(chain_sort_max_pairs(n));
+      buf.words = scope.alloc<unsigned long long>(n);
+      buf.plan = scope.alloc<DevicePlan>(1);
+      unsigned *row_totals = buf.counters + 2 * buckets;
+      int *stage = scope.alloc<int>(static_cast<size_t>(num_offsets) * n);
+      unsigned long long *masks = scope.alloc<unsigned long long>(static_cast<size_t>(num_offsets) * num_wave_tiles);
+      unsigned *tile_counts = scope.alloc<unsigned>(static_cast<size_t>(num_offsets) * num_tiles);
+      unsigned *tile_mode = scope.alloc<unsigned>(num_tiles);
+      unsigned *plan = scope.alloc<unsigned>(4 * num_offsets + 1);
+      OffsetTable table;
+      memset(&table, 0, sizeof(table));
+      for (int o = 0; o < no; ++o) {
+        for (int k = 0; k < ndim; ++k) table.v[o][k] = static_cast<int>(offsets_host[o * ndim + k]);
+      }
+      enqueue_chain_sort(coords, n, ndim, coord_dtype, indices_out, sorted_coords_out, buf, table, no, stream);
+      const HitSink sink{stage, masks, row_totals, tile_mode, num_wave_tiles, no};
+      if (coord_dtype == MNT_INT32) {
+        launch_query_chain<int32_t>(static_cast<const int32_t *>(sorted_coords_out), n, ndim, no, tile_counts,
+                                    num_tiles, sink, buf.plan, stream);
+      } else {
+        launch_query_chain<int64_t>(static_cast<const int64_t *>(sorted_coords_out), n, ndim, no, tile_counts,
+                                    num_tiles, sink, buf.plan, stream);
+      }
+      profile_mark("query", stream);
+      char *pinned_device = static_cast<char *>(arena.pinned_device());
+      unsigned *d_plan_host = reinterpret_cast<unsigned *>(pinned_device + Arena::kPlanOffset);
+      long long *d_chain_host = reinterpret_cast<long long *>(pinned_device + kChainHostOffset);
+      const unsigned long long sequence = arena.next_sequence();
+      dim3 grid(static_cast<unsigned>(div_ceil(num_tiles, kPlaceTiles)), static_cast<unsigned>(num_offsets));
+      place_kernel<<<grid, kPlaceBlock, 0, stream>>>(stage, masks, tile_counts, row_totals, tile_mode, n, no,
+                                                     num_tiles, num_wave_tiles, reorder, in_idx_out,
+                                                     out_idx_out, plan, d_plan_host, arena.flag_device(1),
+                                                     sequence, sizes_dev_out, order_dev_out, buf.plan,
+                                                     buf.folded, d_chain_host);
+      check_launch("place_kernel");
+      arena.wait_flag(1, sequence);
+      const long long *h_chain = reinterpret_cast<const long long *>(static_cast<char *>(arena.pinned()) + kChainHostOffset);
+      profile_mark("map_place+sync", stream);
+      if (h_chain[2 * MNT_MAX_NDIM] == 0) {
+        const unsigned *h_plan = reinterpret_cast<const unsigned *>(static_cast<char *>(arena.pinned()) + Arena::kPlanOffset);
+        for (int64_t j = 0; j < num_offsets; ++j) {
+          order_host_out[j] = h_plan[j];
+          sizes_host_out[j] = h_plan[2 * num_offsets + j];
+        }
+        memcpy(bounds_host_out, h_chain, sizeof(long long) * 2 * MNT_MAX_NDIM);
+        return;
+      }
+      // the chain declined (strong clustering, keys too wide): the calls below start over
+    }
+    if (mnt_arg_sort_coordinates(coords, n, ndim, coord_dtype, nullptr, 1, MNT_INT32, indices_out,
+                                 sorted_coords_out, bounds_host_out, stream_) != 0) {
+      throw Error{mnt_last_error()};
+    }
+    if (mnt_kernel_map_lists(sorted_coords_out, n, sorted_coords_out, n, offsets_host, num_offsets, ndim,
+                             coord_dtype, nullptr, nullptr, 1, MNT_INT32, reorder, bounds_host_out,
+                             bounds_host_out, nullptr, in_idx_out, out_idx_out, list_capacity,
+                             sizes_dev_out, order_dev_out, sizes_host_out, order_host_out, stream_) != 0) {
+      throw Error{mnt_last_error()};
+    }
   });
 }
 

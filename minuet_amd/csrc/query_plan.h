@@ -1,0 +1,166 @@
+// The query plan of a stride-1 kernel map worked out on the device: packing
+// frame, key deltas of the offsets in ascending order and their groups, as
+// make_plan() in query.hip builds them on the host from coordinate bounds
+// that it had to wait for.  A chain of launches that never returns to the
+// host (sort -> query -> lists) lets one wavefront of an earlier kernel write
+// this block instead; the query kernel reads it from device memory.
+#pragma once
+
+#include "device_utils.h"
+
+namespace mnt {
+
+constexpr int kPlanGroupSpan = 4;                // key span of one offset group (kGroupSpan of the query)
+constexpr int kPlanMaxOffsets = 64;              // one lane per offset
+constexpr int kPlanInts = 6 * kPlanMaxOffsets;   // 4 words per group + 2 per member
+
+// Kernel offsets as launch arguments (rows past the count are ignored).
+struct OffsetTable {
+  int v[kPlanMaxOffsets][MNT_MAX_NDIM];
+};
+
+struct DevicePlan {
+  Frame frame;
+  long long delta_min, delta_max;
+  int num_groups;
+  int groups_in_rows;       // every group's offsets differ in the last coordinate only
+  int verdict;              // 0: go; otherwise the chain stops (sort declined, or keys beyond 63 bits)
+  int num_offsets;
+  int tables[kPlanInts];    // groups (first delta low / high, first member, members), then members (step, offset)
+};
+
+struct PlanScratch {        // LDS of the wavefront that builds the plan
+  int inverse[kPlanMaxOffsets];              // offset at each place of the ascending delta order
+};
+
+__device__ __forceinline__ int plan_bits(unsigned long long range) {
+  return range == 0 ? 0 : 64 - __builtin_clzll(range);
+}
+
+// Run by ONE whole wavefront.  bounds = lo[4], hi[4] of the cloud (sources and
+// targets are the same rows); the frame leaves room for every offset on both
+// sides of every field, so key(q + offset) == key(q) + delta(offset).
+// `declined` is the verdict of the launches before (non-zero: stop).
+__device__ __forceinline__ void make_plan_on_device(const long long *__restrict__ bounds,
+                                                    const OffsetTable &offsets, int num_offsets,
+                                                    int ndim, unsigned declined, PlanScratch &lds,
+                                                    DevicePlan *__restrict__ out) {
+  const int lane = lane_id();
+  // lane o takes offset o: selects on scalar operands, no indexed access to the arguments
+  int d[MNT_MAX_NDIM] = {0, 0, 0, 0};
+#pragma unroll
+  for (int l = 0; l < kPlanMaxOffsets; ++l) {
+#pragma unroll
+    for (int k = 0; k < MNT_MAX_NDIM; ++k) d[k] = lane == l ? offsets.v[l][k] : d[k];
+  }
+  const bool live = lane < num_offsets;
+  Frame f;
+  int bits = 0;
+  int reach_lo[MNT_MAX_NDIM], reach_hi[MNT_MAX_NDIM];
+#pragma unroll
+  for (int k = 0; k < MNT_MAX_NDIM; ++k) {
+    int lo = live && k < ndim ? d[k] : 0, hi = lo;
+    for (int off = 32; off > 0; off >>= 1) {
+      const int a = __shfl_xor(lo, off), b = __shfl_xor(hi, off);
+      lo = a < lo ? a : lo;
+      hi = b > hi ? b : hi;
+    }
+    reach_lo[k] = lo < 0 ? lo : 0;
+    reach_hi[k] = hi > 0 ? hi : 0;
+  }
+  bool fits = true;
+#pragma unroll
+  for (int k = MNT_MAX_NDIM - 1; k >= 0; --k) {
+    f.lo[k] = 0;
+    f.shift[k] = 0;
+    f.width[k] = 0;
+    if (k < ndim) {
+      // coordinates are at most 64-bit and the reach is small: a range that wraps is caught below
+      const long long lo = bounds[k] + reach_lo[k];
+      const long long hi = bounds[MNT_MAX_NDIM + k] + reach_hi[k];
+      const unsigned long long range = static_cast<unsigned long long>(hi) - static_cast<unsigned long long>(lo);
+      fits = fits && hi >= lo && lo <= bounds[k] && hi >= bounds[MNT_MAX_NDIM + k] && range < (1ull << 63);
+      f.lo[k] = lo;
+      f.width[k] = plan_bits(range);
+      f.shift[k] = bits < 63 ? bits : 63;
+      bits += f.width[k];
+    }
+  }
+  f.batch_width = 0;
+  f.batch_shift = bits < 63 ? bits : 63;
+  f.ndim = ndim;
+  f.total_bits = bits;
+  fits = fits && bits <= 63;
+
+  long long delta = 0;
+#pragma unroll
+  for (int k = 0; k < MNT_MAX_NDIM; ++k) {
+    if (k < ndim) {
+      delta += static_cast<long long>(static_cast<unsigned long long>(static_cast<long long>(d[k])) << f.shift[k]);
+    }
+  }
+  // place among the offsets in ascending delta order (ties keep offset order)
+  int place = 0;
+  for (int p = 0; p < num_offsets; ++p) {
+    const long long other = __shfl(delta, p);
+    place += (other < delta || (other == delta && p < lane)) ? 1 : 0;
+  }
+  // lane i takes over the offset of place i; from here on lanes are places
+  if (live) lds.inverse[place] = lane;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  const int origin = live ? lds.inverse[lane] : lane;
+  const long long mine = __shfl(delta, origin);
+  int lead[MNT_MAX_NDIM];
+#pragma unroll
+  for (int k = 0; k < MNT_MAX_NDIM; ++k) lead[k] = __shfl(d[k], origin);
+  // first place whose delta lies beyond this one's group span (num_offsets if none)
+  int next = num_offsets;
+  for (int p = num_offsets - 1; p >= 0; --p) {
+    const long long other = __shfl(mine, p);
+    next = p > lane && other - mine > kPlanGroupSpan ? p : next;
+  }
+  // the greedy grouping follows those links from place 0
+  unsigned long long starts = 0;
+  int num_groups = 0;
+  for (int cur = 0; cur < num_offsets; cur = __shfl(next, cur)) {
+    starts |= 1ull << cur;
+    ++num_groups;
+  }
+  const unsigned long long upto = starts & ((2ull << lane) - 1ull);
+  const int group = __popcll(upto) - 1;
+  const int first_place = live ? 63 - __builtin_clzll(upto) : 0;
+  const long long first_delta = __shfl(mine, first_place);
+  bool same_row = true;
+#pragma unroll
+  for (int k = 0; k < MNT_MAX_NDIM; ++k) {
+    const int other = __shfl(lead[k], first_place);
+    same_row = same_row && (k + 1 >= ndim || other == lead[k]);
+  }
+  const bool in_rows = __ballot(live && !same_row) == 0ull;
+  if (live) {
+    out->tables[4 * num_groups + 2 * lane + 0] = static_cast<int>(mine - first_delta);
+    out->tables[4 * num_groups + 2 * lane + 1] = origin;
+    if ((starts >> lane) & 1ull) {
+      const unsigned long long first = static_cast<unsigned long long>(mine);
+      out->tables[4 * group + 0] = static_cast<int>(static_cast<unsigned>(first & 0xffffffffull));
+      out->tables[4 * group + 1] = static_cast<int>(static_cast<unsigned>(first >> 32));
+      out->tables[4 * group + 2] = lane;
+      out->tables[4 * group + 3] = next - lane;
+    }
+  }
+  const long long delta_min = __shfl(mine, 0);
+  const long long delta_max = __shfl(mine, num_offsets > 0 ? num_offsets - 1 : 0);
+  if (lane == 0) {
+    out->frame = f;
+    out->delta_min = num_offsets > 0 ? delta_min : 0;
+    out->delta_max = num_offsets > 0 ? delta_max : 0;
+    out->num_groups = num_groups;
+    out->groups_in_rows = in_rows ? 1 : 0;
+    out->verdict = declined != 0 ? static_cast<int>(declined) : (fits ? 0 : 2);
+    out->num_offsets = num_offsets;
+  }
+}
+
+}  // namespace mnt

@@ -34,4 +34,38 @@ void radix_sort_pairs(unsigned long long *&keys, unsigned *&vals, unsigned long 
                       unsigned *&vals_alt, int64_t n, int bits, unsigned *counts,
                       hipStream_t stream);
 
+// ---- the bucket sort as a chain of launches that never waits for the host ----
+
+struct OffsetTable;
+struct DevicePlan;
+
+// Device memory of one chain (all of it scratch).  `counters` is cleared by
+// the first launch: totals[buckets] | cursors[buckets] | whatever the caller
+// keeps behind them (counter_words in all).
+struct ChainSortBuffers {
+  long long *partial;            // [128 * 8] partial extremes
+  long long *folded;             // [8] coordinate minima, then maxima
+  unsigned *counters;
+  int counter_words;
+  unsigned *info;                // [4]
+  unsigned *status;              // [4]: [0] set by the dealing kernel (non-zero: the sort declined),
+                                 // [2] number of (bucket, chunk) pairs of the ranking launch
+  uint2 *chunks;                 // [chain_sort_max_pairs(n)]
+  unsigned long long *words;     // [n]
+  DevicePlan *plan;              // query plan written by the ranking launch (nullable)
+};
+
+// Whether the chain takes a cloud of n rows (one batch) with this many offsets;
+// the final word is the chain's own (status[0]), known once it has run.
+bool chain_sort_takes(int64_t n, int64_t num_batches, int num_offsets);
+// log2 of the number of buckets the chain uses for n rows, and the most
+// (bucket, chunk) pairs its ranking launch can have.
+int chain_sort_msd_bits(int64_t n);
+int64_t chain_sort_max_pairs(int64_t n);
+// Enqueues bounds -> histogram -> dealing -> ranking (int32 permutation and
+// sorted rows); the ranking launch also writes the query plan for `offsets`.
+void enqueue_chain_sort(const void *coords, int64_t n, int ndim, int coord_dtype, int32_t *indices_out,
+                        void *sorted_out, const ChainSortBuffers &buf, const OffsetTable &offsets,
+                        int num_offsets, hipStream_t stream);
+
 }  // namespace mnt

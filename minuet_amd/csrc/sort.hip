@@ -10,6 +10,7 @@
 #include <vector>
 
 #include "device_utils.h"
+#include "query_plan.h"
 
 namespace mnt {
 
@@ -940,14 +941,18 @@ __global__ __launch_bounds__(kSortBlock) void bucket_deal_kernel(
 // workgroup of the bucket repeats for itself); a row then only counts inside
 // its own part, whose rows the other parts precede or follow as a whole.
 // word_bits = width of a word (rest of the key and row index).
+struct RankShared {
+  unsigned part_cursor[kSortBlock], part_start[kSortBlock + 1], wave_sums[kSortWaves];
+};
+
 template <typename CT, typename IT>
-__global__ __launch_bounds__(kSortBlock) void bucket_rank_kernel(
-    const unsigned long long *__restrict__ words, const uint2 *__restrict__ chunks, int idx_bits,
-    int word_bits, FinalSink<CT, IT> sink) {
-  extern __shared__ __align__(16) unsigned long long s_words[];
-  __shared__ unsigned part_cursor[kSortBlock], part_start[kSortBlock + 1], wave_sums[kSortWaves];
+__device__ __forceinline__ void rank_bucket_chunk(
+    const unsigned long long *__restrict__ words, const uint2 entry, int idx_bits, int word_bits,
+    const FinalSink<CT, IT> &sink, unsigned long long *s_words, RankShared &sh) {
+  unsigned (&part_cursor)[kSortBlock] = sh.part_cursor;
+  unsigned (&part_start)[kSortBlock + 1] = sh.part_start;
+  unsigned (&wave_sums)[kSortWaves] = sh.wave_sums;
   const unsigned tid = threadIdx.x;
-  const uint2 entry = chunks[blockIdx.x];
   const unsigned start = entry.x;
   const unsigned m = entry.y & 0x1fffu;
   const unsigned mode = (entry.y >> 13) & 7u;
@@ -1039,6 +1044,15 @@ __global__ __launch_bounds__(kSortBlock) void bucket_rank_kernel(
   }
 }
 
+template <typename CT, typename IT>
+__global__ __launch_bounds__(kSortBlock) void bucket_rank_kernel(
+    const unsigned long long *__restrict__ words, const uint2 *__restrict__ chunks, int idx_bits,
+    int word_bits, FinalSink<CT, IT> sink) {
+  extern __shared__ __align__(16) unsigned long long s_words[];
+  __shared__ RankShared sh;
+  rank_bucket_chunk<CT, IT>(words, chunks[blockIdx.x], idx_bits, word_bits, sink, s_words, sh);
+}
+
 // Largest cloud the bucket sort takes (MINUET_BUCKET_SORT_MAX_ROWS overrides;
 // 0 switches it off).
 static int64_t bucket_sort_max_rows() {
@@ -1072,6 +1086,272 @@ __global__ __launch_bounds__(256) void emit_sorted_kernel(const CT *__restrict__
 
 static int bit_width(unsigned long long range) {
   return range == 0 ? 0 : 64 - __builtin_clzll(range);
+}
+
+// ------------------------------------ bucket sort without a host round trip ----
+//
+// The same sort enqueued as four launches that need nothing from the host
+// (bounds -> histogram -> dealing -> ranking), for a chain that goes on to
+// query the sorted rows: the dealing kernel scans the bucket totals for itself
+// (every workgroup repeats the scan of at most 8192 counters; there is no scan
+// launch), the ranking kernel takes one bucket per workgroup whatever its
+// size, so its grid is known beforehand.  What the host would have decided
+// after its wait is decided on the device and left in `status`: a word that
+// every later kernel of the chain reads first and that the host looks at once,
+// at the end.  status[0] != 0: the cloud does not fit this sort (key wider than
+// a word, or a bucket beyond kChainBucketCap rows); nothing was written.
+
+constexpr int kChainBucketCap = 4096;         // rows of the largest bucket (32 KiB of LDS)
+
+// Dealing with the scan folded in.  LDS: s_hist[buckets], s_starts[buckets + 1].
+template <typename CT, typename IT, int kBucketItems>
+__global__ __launch_bounds__(kSortBlock) void bucket_deal_scan_kernel(
+    const CT *__restrict__ coords, int ndim, long long n, const long long *__restrict__ folded,
+    int msd_cap, int idx_bits_, const unsigned *__restrict__ info,
+    const unsigned *__restrict__ totals, unsigned *__restrict__ cursors,
+    uint2 *__restrict__ chunks_out, unsigned *__restrict__ status,
+    unsigned long long *__restrict__ words) {
+  extern __shared__ __align__(16) unsigned s_deal[];
+  __shared__ unsigned long long s_wave[kSortWaves];
+  __shared__ unsigned s_wave_shared[kSortWaves], s_wave_max[kSortWaves];
+  const int tid = threadIdx.x;
+  const int lane = lane_id();
+  const int buckets = 1 << msd_cap;
+  unsigned *s_hist = s_deal;
+  unsigned *s_starts = s_deal + buckets;
+  // the rows first: their loads wait for nothing
+  const long long base = static_cast<long long>(blockIdx.x) * (kSortBlock * kBucketItems);
+  CT c[kBucketItems][MNT_MAX_NDIM];
+#pragma unroll
+  for (int r = 0; r < kBucketItems; ++r) {
+    const long long i = base + r * kSortBlock + tid;
+    load_row_raw<CT>(coords + (i < n ? i : n - 1) * ndim, ndim, c[r]);
+  }
+  // bucket starts: thread t scans the consecutive buckets [t * per, (t + 1) * per)
+  constexpr int kPer = kBucketMax / kSortBlock;
+  const int per = (buckets + kSortBlock - 1) / kSortBlock;
+  unsigned v[kPer];
+  unsigned sum = 0, biggest = 0, singles = 0, shared = 0;
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int d = tid * per + j;
+    v[j] = j < per && d < buckets ? totals[d] : 0u;
+    sum += v[j];
+    biggest = v[j] > biggest ? v[j] : biggest;
+    const unsigned pieces = bucket_pieces(v[j]);
+    singles += pieces == 1 ? 1u : 0u;
+    shared += pieces > 1 ? pieces : 0u;
+  }
+  const unsigned layout_ok = info[0];
+  long long bounds[2 * MNT_MAX_NDIM];
+#pragma unroll
+  for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) bounds[slot] = folded[slot];
+  // rows in the low half and one-workgroup buckets in the high half of one word
+  // (fewer than 2^31 rows), workgroups of shared buckets in another
+  const unsigned long long mine_both =
+      static_cast<unsigned long long>(sum) | (static_cast<unsigned long long>(singles) << 32);
+  unsigned long long inclusive = mine_both;
+  unsigned shared_inclusive = shared;
+  for (int off = 1; off < kWave; off <<= 1) {
+    const unsigned long long u = __shfl_up(inclusive, off);
+    const unsigned u2 = __shfl_up(shared_inclusive, off);
+    if (lane >= off) {
+      inclusive += u;
+      shared_inclusive += u2;
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned u = __shfl_xor(biggest, off);
+    biggest = u > biggest ? u : biggest;
+  }
+  if (lane == kWave - 1) {
+    s_wave[tid >> 6] = inclusive;
+    s_wave_shared[tid >> 6] = shared_inclusive;
+  }
+  if (lane == 0) s_wave_max[tid >> 6] = biggest;
+  for (int d = tid; d < buckets; d += kSortBlock) s_hist[d] = 0;
+  __syncthreads();
+  unsigned long long before = 0, all_both = 0;
+  unsigned shared_before = 0, all_shared = 0, all_max = 0;
+#pragma unroll
+  for (int w = 0; w < kSortWaves; ++w) {
+    before += w < (tid >> 6) ? s_wave[w] : 0ull;
+    shared_before += w < (tid >> 6) ? s_wave_shared[w] : 0u;
+    all_both += s_wave[w];
+    all_shared += s_wave_shared[w];
+    all_max = s_wave_max[w] > all_max ? s_wave_max[w] : all_max;
+  }
+  const bool go = layout_ok != 0 && all_max <= static_cast<unsigned>(kChainBucketCap);
+  if (blockIdx.x == 0 && tid == 0) {
+    status[0] = go ? 0u : 1u;
+    status[2] = go ? all_shared + static_cast<unsigned>(all_both >> 32) : 0u;      // pairs of the ranking launch
+  }
+  if (!go) return;                               // the same verdict in every workgroup
+  {
+    const unsigned long long exclusive = before + inclusive - mine_both;
+    unsigned run = static_cast<unsigned>(exclusive);
+    // the workgroups of shared buckets run longest and come first in the list
+    unsigned shared_at = shared_before + shared_inclusive - shared;
+    unsigned single_at = all_shared + static_cast<unsigned>(exclusive >> 32);
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      const int d = tid * per + j;
+      if (j < per && d < buckets) {
+        s_starts[d] = run;
+        if (blockIdx.x == 0) {
+          const unsigned pieces = bucket_pieces(v[j]);
+          const unsigned head = v[j] | (bucket_mode(v[j]) << 13);
+          if (pieces == 1) chunks_out[single_at++] = make_uint2(run, head);
+          for (unsigned c = 0; pieces > 1 && c < pieces; ++c) chunks_out[shared_at++] = make_uint2(run, head | (c << 16));
+        }
+      }
+      run += v[j];
+    }
+  }
+  CoordSource<CT, IT> src;
+  const BucketLayout lay = layout_on_device<CT, IT>(coords, nullptr, 1, ndim, bounds, msd_cap, idx_bits_, src);
+  const int shift = lay.shift, idx_bits = lay.idx_bits;
+  const unsigned long long rest_mask = (1ull << shift) - 1ull;
+  unsigned long long key[kBucketItems];
+  unsigned row[kBucketItems], place[kBucketItems];
+#pragma unroll
+  for (int r = 0; r < kBucketItems; ++r) {
+    const long long i = base + r * kSortBlock + tid;
+    src.pack(i, c[r], key[r], row[r]);
+    place[r] = 0;
+    if (i < n) place[r] = atomicAdd(&s_hist[static_cast<unsigned>(key[r] >> shift)], 1u);
+  }
+  __syncthreads();
+  // a range of every bucket this tile has rows for (cursors count from zero)
+  unsigned count[kPer], got[kPer];
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int d = j * kSortBlock + tid;
+    count[j] = d < buckets ? s_hist[d] : 0u;
+  }
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int d = j * kSortBlock + tid;
+    got[j] = 0;
+    if (count[j] != 0) got[j] = atomicAdd(&cursors[d], count[j]);
+  }
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int d = j * kSortBlock + tid;
+    if (count[j] != 0) s_hist[d] = got[j] + s_starts[d];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < kBucketItems; ++r) {
+    const long long i = base + r * kSortBlock + tid;
+    if (i < n) {
+      const unsigned pos = s_hist[static_cast<unsigned>(key[r] >> shift)] + place[r];
+      words[pos] = ((key[r] & rest_mask) << idx_bits) | static_cast<unsigned long long>(row[r]);
+    }
+  }
+}
+
+// bucket_rank_kernel inside the chain: the (bucket, chunk) list and its length
+// come from the dealing launch, so the grid is the largest the list can get
+// and workgroups past its end leave at once; the word width follows from the
+// folded bounds.  Workgroup 0 has no bucket: its first wavefront writes the
+// query plan of the launches that follow.
+template <typename CT, typename IT>
+__global__ __launch_bounds__(kSortBlock) void bucket_rank_chain_kernel(
+    const unsigned long long *__restrict__ words, const uint2 *__restrict__ chunks,
+    const unsigned *__restrict__ pair_count, int max_pairs, const long long *__restrict__ folded,
+    int ndim, int msd_cap, int idx_bits, const unsigned *__restrict__ status, FinalSink<CT, IT> sink,
+    OffsetTable offsets, int num_offsets, DevicePlan *__restrict__ plan_out) {
+  __shared__ __align__(16) unsigned long long s_words[kChainBucketCap + 128];
+  __shared__ RankShared sh;
+  const unsigned declined = status[0];
+  if (blockIdx.x == 0) {
+    // runs whatever the sort's verdict: the plan carries the verdict of the whole chain
+    if (plan_out != nullptr && threadIdx.x < kWave) {
+      PlanScratch &scratch = *reinterpret_cast<PlanScratch *>(s_words);
+      static_assert(sizeof(PlanScratch) <= sizeof(s_words), "plan scratch must fit the word staging area");
+      make_plan_on_device(folded, offsets, num_offsets, ndim, declined, scratch, plan_out);
+    }
+    return;
+  }
+  const unsigned pair = blockIdx.x - 1;
+  const unsigned pairs = pair_count[0];
+  const uint2 entry = chunks[pair];                    // the list has room for max_pairs entries
+  long long bounds[2 * MNT_MAX_NDIM];
+#pragma unroll
+  for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) bounds[slot] = folded[slot];
+  if (declined != 0 || pair >= pairs) return;
+  SortSpec spec;
+  const int key_bits = single_round_spec(bounds, ndim, 1, spec);
+  const BucketLayout lay = bucket_layout(key_bits, msd_cap, idx_bits);
+  rank_bucket_chunk<CT, IT>(words, entry, idx_bits, lay.shift + idx_bits, sink, s_words, sh);
+}
+
+bool chain_sort_takes(int64_t n, int64_t num_batches, int num_offsets) {
+  return n >= kBucketMinN && n <= bucket_sort_max_rows() && n <= (int64_t(1) << 21) && num_batches <= 1 &&
+         num_offsets >= 1 && num_offsets <= kPlanMaxOffsets;
+}
+
+template <typename CT>
+static void enqueue_chain_sort_typed(const CT *coords, int64_t n, int ndim, int32_t *indices_out,
+                                     CT *sorted_out, const ChainSortBuffers &buf,
+                                     const OffsetTable &offsets, int num_offsets, hipStream_t stream) {
+  const int idx_bits = bit_width(static_cast<unsigned long long>(n - 1));
+  const int msd_cap = chain_sort_msd_bits(n);
+  const int buckets = 1 << msd_cap;
+  const int num_partials = static_cast<int>(std::min<int64_t>(div_ceil(n, kBoundsBlock * 4), kBucketBoundsBlocks));
+  bounds_kernel<CT><<<num_partials, kBoundsBlock, 0, stream>>>(coords, n, num_partials, nullptr, 0, ndim,
+                                                               buf.partial, buf.counters, buf.counter_words);
+  check_launch("bounds_kernel");
+  profile_mark("sort_bounds", stream);
+  const bool large = n > (int64_t(1) << 18);
+  const unsigned tiles = static_cast<unsigned>(div_ceil(n, kSortBlock * (large ? 16 : 4)));
+  unsigned *totals = buf.counters;
+  unsigned *cursors = buf.counters + buckets;
+  if (large) {
+    bucket_hist_kernel<CT, int32_t, 16><<<tiles, kSortBlock, 0, stream>>>(
+        coords, nullptr, 1, ndim, n, buf.partial, num_partials, msd_cap, idx_bits, totals, buf.info, buf.folded);
+  } else {
+    bucket_hist_kernel<CT, int32_t, 4><<<tiles, kSortBlock, 0, stream>>>(
+        coords, nullptr, 1, ndim, n, buf.partial, num_partials, msd_cap, idx_bits, totals, buf.info, buf.folded);
+  }
+  check_launch("bucket_hist_kernel");
+  profile_mark("sort_hist", stream);
+  const size_t lds = sizeof(unsigned) * (2 * static_cast<size_t>(buckets));
+  if (large) {
+    bucket_deal_scan_kernel<CT, int32_t, 16><<<tiles, kSortBlock, lds, stream>>>(
+        coords, ndim, n, buf.folded, msd_cap, idx_bits, buf.info, totals, cursors, buf.chunks, buf.status, buf.words);
+  } else {
+    bucket_deal_scan_kernel<CT, int32_t, 4><<<tiles, kSortBlock, lds, stream>>>(
+        coords, ndim, n, buf.folded, msd_cap, idx_bits, buf.info, totals, cursors, buf.chunks, buf.status, buf.words);
+  }
+  check_launch("bucket_deal_scan_kernel");
+  profile_mark("sort_deal", stream);
+  const int max_pairs = static_cast<int>(chain_sort_max_pairs(n));
+  bucket_rank_chain_kernel<CT, int32_t><<<max_pairs + 1, kSortBlock, 0, stream>>>(
+      buf.words, buf.chunks, buf.status + 2, max_pairs, buf.folded, ndim, msd_cap, idx_bits, buf.status,
+      FinalSink<CT, int32_t>{coords, ndim, indices_out, sorted_out}, offsets, num_offsets, buf.plan);
+  check_launch("bucket_rank_chain_kernel");
+  profile_mark("sort_rank", stream);
+}
+
+// A bucket of m rows makes at most m / 256 + 1 pairs.
+int64_t chain_sort_max_pairs(int64_t n) { return (int64_t(1) << chain_sort_msd_bits(n)) + n / kSortBlock + 1; }
+
+int chain_sort_msd_bits(int64_t n) {
+  return std::max(1, std::min(kBucketMaxBits, bit_width(static_cast<unsigned long long>(n / kBucketRows))));
+}
+
+void enqueue_chain_sort(const void *coords, int64_t n, int ndim, int coord_dtype, int32_t *indices_out,
+                        void *sorted_out, const ChainSortBuffers &buf, const OffsetTable &offsets,
+                        int num_offsets, hipStream_t stream) {
+  if (coord_dtype == MNT_INT32) {
+    enqueue_chain_sort_typed<int32_t>(static_cast<const int32_t *>(coords), n, ndim, indices_out,
+                                      static_cast<int32_t *>(sorted_out), buf, offsets, num_offsets, stream);
+  } else {
+    enqueue_chain_sort_typed<int64_t>(static_cast<const int64_t *>(coords), n, ndim, indices_out,
+                                      static_cast<int64_t *>(sorted_out), buf, offsets, num_offsets, stream);
+  }
 }
 
 template <typename CT, typename IT>

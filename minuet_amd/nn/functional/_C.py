@@ -61,6 +61,12 @@ SIGNATURES = {
     "mnt_kernel_map_build": (_int, [_vp, _i64, _vp, _i64, _pi64, _i64, _int, _int, _vp, _vp, _i64,
                                     _int, _int, _pi64, _pi64, _pi64, _vp, _vp, _vp, _vp, _vp, _i64,
                                     _vp, _vp, _pi64, _pi64, _vp]),
+    "mnt_kernel_map_lists": (_int, [_vp, _i64, _vp, _i64, _pi64, _i64, _int, _int, _vp, _vp, _i64,
+                                    _int, _int, _pi64, _pi64, _pi64, _vp, _vp, _i64, _vp, _vp, _pi64,
+                                    _pi64, _vp]),
+    # host arrays are passed as plain addresses here (the call sits on a hot path)
+    "mnt_sorted_kernel_map_lists": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _vp, _vp, _vp,
+                                           _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
     "mnt_kernel_map_dense": (_int, [_vp, _i64, _vp, _i64, _pi64, _i64, _int, _int, _vp, _vp, _i64, _int,
                                     _pi64, _pi64, _pi64, _vp, _vp]),
     "mnt_kernel_map_tables": (_int, [_vp, _i64, _i64, _i64, _int, _pi64, _pi64, _vp]),
@@ -491,7 +497,8 @@ def kernel_map_build(sources: torch.Tensor, targets: torch.Tensor, offsets_host:
     offs = np.ascontiguousarray(np.asarray(offsets_host, dtype=np.int64).reshape(-1, ndim))
     num_offsets = offs.shape[0]
     num_sources, num_targets = sources.size(0), targets.size(0)
-    dense = torch.empty((num_offsets, num_targets), dtype=torch.int32, device=device)
+    lists_only = want_lists and not want_masks and not want_dense
+    dense = None if lists_only else torch.empty((num_offsets, num_targets), dtype=torch.int32, device=device)
     sizes_host = np.zeros(num_offsets, dtype=np.int64)
     order_host = np.zeros(num_offsets, dtype=np.int64)
     bounds = np.zeros(16, dtype=np.int64)
@@ -516,6 +523,24 @@ def kernel_map_build(sources: torch.Tensor, targets: torch.Tensor, offsets_host:
                 and (not want_lists or capacity * 8 <= PAIR_LIST_SLACK_BYTES))
     with _on(device):
         stream = _stream(device)
+        if lists_only and not one_call:
+            dense = torch.empty((num_offsets, num_targets), dtype=torch.int32, device=device)
+        if one_call and lists_only:
+            # the lists alone: the dense map is neither written nor read back
+            both = torch.empty((2, capacity), dtype=torch.int32, device=device)
+            _check(lib.mnt_kernel_map_lists(
+                _ptr(sources), num_sources, _ptr(targets), num_targets,
+                offs.ctypes.data_as(_pi64), num_offsets, ndim, ccode, _ptr(source_batch_dims),
+                _ptr(target_batch_dims), num_batches, bcode, 1 if reorder else 0,
+                None if sb is None else sb.ctypes.data_as(_pi64),
+                None if tb is None else tb.ctypes.data_as(_pi64), bounds.ctypes.data_as(_pi64),
+                _ptr(both[0]), _ptr(both[1]), capacity, _ptr(sizes_dev), _ptr(order_dev),
+                sizes_host.ctypes.data_as(_pi64), order_host.ctypes.data_as(_pi64), stream))
+            nnz = int(sizes_host.sum())
+            result.update(sizes_host=sizes_host, order_host=order_host, sizes=sizes_dev, order=order_dev,
+                          bounds=bounds, source_masks=None, target_masks=None, in_idx=both[0, :nnz],
+                          out_idx=both[1, :nnz])
+            return result
         if one_call:
             if want_lists:
                 both = torch.empty((2, capacity), dtype=torch.int32, device=device)
@@ -559,6 +584,119 @@ def kernel_map_build(sources: torch.Tensor, targets: torch.Tensor, offsets_host:
     if want_dense:
         result["kernel_map"] = dense
     return result
+
+
+class SortedMapLists:
+    """What :func:`sorted_kernel_map_lists` returns: the sorted cloud and the pair
+    lists of its kernel map.  All int32 results live in one device allocation;
+    the tensors handed out (``indices``, ``coordinates``, ``in_idx``, ``out_idx``,
+    ``sizes``, ``order``) are views of it, made when first asked for.  Reads like
+    the dict of :func:`kernel_map_build` (``built["in_idx"]``, ``"sizes_host"``,
+    ``"order_host"``, ``"bounds"`` ...)."""
+    __slots__ = ("_store", "_coords", "_host", "_n", "_ndim", "_num_offsets", "_views")
+
+    def __init__(self, store, coords, host, n, ndim, num_offsets):
+        self._store, self._coords, self._host = store, coords, host
+        self._n, self._ndim, self._num_offsets = n, ndim, num_offsets
+        self._views = {}
+
+    @property
+    def sizes_host(self):
+        return self._host[8:8 + self._num_offsets]
+
+    @property
+    def order_host(self):
+        return self._host[8 + self._num_offsets:]
+
+    @property
+    def nnz(self) -> int:
+        return int(self.sizes_host.sum())
+
+    def _view(self, key):
+        n, no = self._n, self._num_offsets
+        cap = no * n
+        lists = n if self._coords is not None else n * (1 + self._ndim)
+        if key == "indices":
+            return self._store[:n]
+        if key == "coordinates":
+            return self._coords if self._coords is not None else self._store[n:lists].view(n, self._ndim)
+        if key == "in_idx":
+            return self._store[lists:lists + self.nnz]
+        if key == "out_idx":
+            return self._store[lists + cap:lists + cap + self.nnz]
+        if key == "sizes":
+            return self._store[lists + 2 * cap:lists + 2 * cap + no]
+        if key == "order":
+            return self._store[lists + 2 * cap + no:lists + 2 * cap + 2 * no]
+        if key == "sizes_host":
+            return self.sizes_host
+        if key == "order_host":
+            return self.order_host
+        if key == "bounds":
+            return np.concatenate([self._host[:8], self._host[:8]])
+        if key in ("source_masks", "target_masks"):
+            return None
+        raise KeyError(key)
+
+    def __getitem__(self, key):
+        if key not in self._views:
+            self._views[key] = self._view(key)
+        return self._views[key]
+
+    def __contains__(self, key):
+        return key in ("indices", "coordinates", "in_idx", "out_idx", "sizes", "order", "sizes_host",
+                       "order_host", "bounds", "source_masks", "target_masks")
+
+
+def sorted_kernel_map_lists(coordinates: torch.Tensor, offsets_host: np.ndarray, reorder: bool = True):
+    """The Map step of a stride-1 layer on an unsorted cloud (one batch) in one
+    library call: ``sort_coordinates`` then the lists-only ``kernel_map_build``
+    of the sorted cloud onto itself.  Returns ``(indices int32 [n], sorted
+    coordinates, built)`` with ``built`` a :class:`SortedMapLists` that reads
+    like the dict :func:`kernel_map_build` returns for ``want_masks=False,
+    want_lists=True`` (``bounds`` holds the 8 bounds of the cloud twice:
+    sources, then targets)."""
+    if coordinates.dim() != 2:
+        _ensure_ndim("coordinates", coordinates, 2)
+    device = coordinates.device
+    if device.type != "cuda":
+        _common_device([coordinates])
+    n, ndim = coordinates.shape
+    ccode = _INT.get(coordinates.dtype)
+    if ccode is None:
+        _int_code(coordinates.dtype, "coordinate", "sorted_kernel_map_lists")
+    if not 1 <= ndim <= 4:
+        _check_ndim_supported(ndim, "sorted_kernel_map_lists", coordinates.dtype)
+    offs = offsets_host
+    if not (isinstance(offs, np.ndarray) and offs.dtype == np.int64 and offs.ndim == 2
+            and offs.shape[1] == ndim and offs.flags.c_contiguous):
+        offs = np.ascontiguousarray(np.asarray(offsets_host, dtype=np.int64).reshape(-1, ndim))
+    num_offsets = offs.shape[0]
+    if n == 0 or num_offsets == 0:
+        indices, out = sort_coordinates(coordinates)
+        return indices, out, kernel_map_build(out, out, offs, None, None, reorder, want_masks=False,
+                                              want_lists=True)
+    if not coordinates.is_contiguous():
+        coordinates = coordinates.contiguous()
+    capacity = num_offsets * n
+    narrow = ccode == 0
+    lists = n * (1 + ndim) if narrow else n
+    store = torch.empty((lists + 2 * capacity + 2 * num_offsets,), dtype=torch.int32, device=device)
+    coords_out = None if narrow else torch.empty_like(coordinates)
+    host = np.empty(8 + 2 * num_offsets, dtype=np.int64)
+    base = store.data_ptr()
+    hbase = host.ctypes.data
+    with _on(device):
+        status = load_library().mnt_sorted_kernel_map_lists(
+            coordinates.data_ptr(), n, ndim, ccode, offs.ctypes.data, num_offsets,
+            1 if reorder else 0, base, base + 4 * n if narrow else coords_out.data_ptr(),
+            base + 4 * lists, base + 4 * (lists + capacity), capacity,
+            base + 4 * (lists + 2 * capacity), base + 4 * (lists + 2 * capacity + num_offsets),
+            hbase, hbase + 64, hbase + 64 + 8 * num_offsets, _stream(device))
+    if status != 0:
+        _check(status)
+    built = SortedMapLists(store, coords_out, host, n, ndim, num_offsets)
+    return built["indices"], built["coordinates"], built
 
 
 def kernel_map_dense(sources: torch.Tensor, targets: torch.Tensor, offsets_host: np.ndarray,

@@ -455,3 +455,110 @@ def test_dense_and_tables_empty_inputs():
     tables = _C.kernel_map_tables(dense, 40, reorder=False)
     assert tables["sizes_host"].sum() == 0 and (host(tables["source_masks"]) == -1).all()
     assert _C.kernel_map_invert(dense, 40).eq(-1).all()
+
+
+def _check_lists_only(src, sbd, tgt, tbd, off, reorder):
+    built = _C.kernel_map_build(dev(src), dev(tgt), off.astype(np.int64), dev(sbd), dev(tbd),
+                                reorder=reorder, want_masks=False, want_lists=True)
+    assert built["source_masks"] is None and "kernel_map" not in built          # the lists-only form ran
+    _, _, eorder, esizes, em = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=reorder)
+    np.testing.assert_array_equal(built["sizes_host"], esizes.astype(np.int64))
+    np.testing.assert_array_equal(host(built["sizes"]), esizes)
+    expect_order = eorder.astype(np.int64) if reorder else np.arange(off.shape[0])
+    np.testing.assert_array_equal(built["order_host"], expect_order)
+    np.testing.assert_array_equal(host(built["order"]), expect_order)
+    ein, eout, _ = orc.kernel_map_pair_lists(em)
+    np.testing.assert_array_equal(host(built["in_idx"]), ein)
+    np.testing.assert_array_equal(host(built["out_idx"]), eout)
+    return built
+
+
+@pytest.mark.parametrize("reorder", [True, False])
+@pytest.mark.parametrize("kernel,stride,batched,n,extent", [
+    (3, 1, False, 30000, 45), (2, 2, True, 30000, 45), (5, 1, False, 20000, 40), (3, 1, True, 70001, 64),
+    (3, 1, False, 1, 4), (3, 1, False, 513, 9), (7, 1, False, 3000, 14), ((3, 1, 2), 1, False, 5000, 20),
+])
+def test_kernel_map_lists_only(reorder, kernel, stride, batched, n, extent):
+    """Pair lists without the dense map (mnt_kernel_map_lists): compacted staging
+    in the query kernel, placing kernel, sizes and order, against the oracle."""
+    src, sbd, tgt, tbd, off = _query_case(29, n, extent, -extent // 3, kernel, stride, batched=batched)
+    _check_lists_only(src, sbd, tgt, tbd, off, reorder)
+
+
+def test_kernel_map_lists_only_many_chunks_and_int64():
+    # a fully occupied block: the source window of a tile spans several LDS chunks,
+    # so those tiles stage one slot per target instead of compacting
+    g = np.stack(np.meshgrid(np.arange(6), np.arange(40), np.arange(40), indexing="ij"), -1)
+    src = g.reshape(-1, 3).astype(np.int32)
+    off = orc.generate_kernel_offsets(3, 5, 1, 1).astype(np.int32)
+    _check_lists_only(src, None, src, None, off, True)
+    src64, sbd, tgt, tbd, off64 = _query_case(31, 9000, 30, -7, 3, 1, batched=True, cdtype=np.int64,
+                                              idtype=np.int64)
+    _check_lists_only(src64, sbd, tgt, tbd, off64, True)
+    # nothing matches: every size is zero and the lists are empty
+    far = src + np.array([1000, 0, 0], dtype=np.int32)
+    built = _check_lists_only(src, None, far, None, orc.generate_kernel_offsets(3, 3, 1, 1).astype(np.int32), True)
+    assert built["in_idx"].numel() == 0
+
+
+def _check_sorted_lists(cloud, off, reorder=True):
+    """mnt_sorted_kernel_map_lists against the oracle's sort and kernel map."""
+    indices, sorted_dev, built = _C.sorted_kernel_map_lists(dev(cloud), off.astype(np.int64), reorder=reorder)
+    order = orc.arg_sort_coordinates(cloud)
+    ref = cloud[order]
+    assert indices.dtype == torch.int32
+    np.testing.assert_array_equal(host(indices).astype(np.int64), order)
+    np.testing.assert_array_equal(host(sorted_dev), ref)
+    np.testing.assert_array_equal(built["bounds"][:cloud.shape[1]], cloud.min(0))
+    np.testing.assert_array_equal(built["bounds"][4:4 + cloud.shape[1]], cloud.max(0))
+    _, _, eorder, esizes, em = orc.build_kernel_map(ref, None, ref, None, off.astype(cloud.dtype), reorder=reorder)
+    np.testing.assert_array_equal(built["sizes_host"], esizes.astype(np.int64))
+    np.testing.assert_array_equal(host(built["sizes"]), esizes)
+    expect_order = eorder.astype(np.int64) if reorder else np.arange(off.shape[0])
+    np.testing.assert_array_equal(built["order_host"], expect_order)
+    np.testing.assert_array_equal(host(built["order"]), expect_order)
+    ein, eout, _ = orc.kernel_map_pair_lists(em)
+    np.testing.assert_array_equal(host(built["in_idx"]), ein)
+    np.testing.assert_array_equal(host(built["out_idx"]), eout)
+
+
+@pytest.mark.parametrize("reorder", [True, False])
+@pytest.mark.parametrize("n,extent,kernel,cdtype", [
+    (30000, 45, 3, np.int32), (2048, 20, 3, np.int32), (70001, 64, 2, np.int32), (50000, 300, 3, np.int64),
+    (9000, 30, 4, np.int32), (40000, 50, (3, 1, 2), np.int32),
+    # below the chain's smallest cloud and beyond its 64 offsets: the two separate calls inside
+    (600, 9, 3, np.int32), (20000, 40, 5, np.int32),
+])
+def test_sorted_kernel_map_lists(reorder, n, extent, kernel, cdtype):
+    cloud = np.unique(random_cloud(n, extent, seed=41, lo=-extent // 3, dtype=cdtype), axis=0)
+    cloud = cloud[np.random.default_rng(5).permutation(cloud.shape[0])]
+    off = orc.generate_kernel_offsets(3, kernel, 1, 1)
+    _check_sorted_lists(cloud, off, reorder)
+
+
+def test_sorted_kernel_map_lists_lidar_and_clustered():
+    from minuet_amd.synthetic import make_cloud
+    off = orc.generate_kernel_offsets(3, 3, 1, 1)
+    # the generator of configuration 2 at a quarter of its size: planes of constant x make large buckets
+    _check_sorted_lists(make_cloud(2, scale=0.25)["coords"], off)
+    # one dense slab: a bucket far beyond what the chain ranks in LDS, so the chain declines on the device
+    g = np.stack(np.meshgrid(np.arange(2), np.arange(120), np.arange(120), indexing="ij"), -1).reshape(-1, 3)
+    far = np.array([[4000, 0, 0], [-4000, 5, 5]])
+    cloud = np.concatenate([g, far]).astype(np.int32)
+    cloud = cloud[np.random.default_rng(9).permutation(cloud.shape[0])]
+    _check_sorted_lists(cloud, off)
+    # rows that repeat (the sort is stable; the map is that of the rows as they are)
+    dup = random_cloud(5000, 12, seed=3, duplicates=0.3)
+    indices, sorted_dev, _ = _C.sorted_kernel_map_lists(dev(dup), off.astype(np.int64))
+    order = orc.arg_sort_coordinates(dup)
+    np.testing.assert_array_equal(host(indices).astype(np.int64), order)
+    np.testing.assert_array_equal(host(sorted_dev), dup[order])
+
+
+def test_sorted_kernel_map_lists_2d_and_4d():
+    rng = np.random.default_rng(11)
+    for ndim, extent in ((2, 300), (4, 12)):
+        cloud = np.unique(rng.integers(-5, extent, size=(20000, ndim)).astype(np.int32), axis=0)
+        cloud = cloud[rng.permutation(cloud.shape[0])]
+        off = orc.generate_kernel_offsets(ndim, 3 if ndim == 2 else 2, 1, 1)
+        _check_sorted_lists(cloud, off)
