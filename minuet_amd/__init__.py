@@ -13,3 +13,4 @@ from .utils.helpers import autotune
 from .utils.helpers import load_tunable_config
 from .utils.helpers import dump_tunable_config
 from .utils.graphs import capture_forward
+from .utils.helpers import invalidate_cached_weights

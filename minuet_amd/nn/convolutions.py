@@ -74,10 +74,14 @@ class KernelMapCache(object):
     def _known_bounds(self, coordinates: torch.Tensor):
         """Host copy of the per-dimension min / max of a coordinate tensor seen
         before (keyed by its storage), or None."""
-        return self._bounds_cache.get((coordinates.data_ptr(), coordinates.shape[0]))
+        entry = self._bounds_cache.get((coordinates.data_ptr(), coordinates.shape[0]))
+        return None if entry is None else entry[1]
 
     def _remember_bounds(self, coordinates: torch.Tensor, bounds: np.ndarray):
-        self._bounds_cache[(coordinates.data_ptr(), coordinates.shape[0])] = np.array(bounds, dtype=np.int64)
+        # the entry keeps the tensor alive until reset(): its storage cannot be
+        # handed to another tensor while the bounds are filed under its address
+        self._bounds_cache[(coordinates.data_ptr(), coordinates.shape[0])] = (
+            coordinates, np.array(bounds, dtype=np.int64))
 
     def get_target_coordinates(self, source_coordinates: torch.Tensor,
                                source_batch_dims: Optional[torch.Tensor],
@@ -296,6 +300,7 @@ class SparseConv(Module):
         self.transposed = transposed
         factory = {"device": device, "dtype": dtype}
         volume = int(np.prod(self.kernel_size))
+        self._packed = None
         self.kernel = torch.nn.Parameter(torch.empty(volume, in_channels, out_channels, **factory))
         if bias:
             self.bias = torch.nn.Parameter(torch.empty(out_channels, **factory))
@@ -310,7 +315,6 @@ class SparseConv(Module):
                                 "dataflow": "auto"}
         self._tuning_data = None
         self._identity_map = None
-        self._packed = None
         self._routes = dict()
         self._trivial = None
 
@@ -358,9 +362,29 @@ class SparseConv(Module):
         output) channel count (reference: convolutions.py:311-319)."""
         fan = self.out_channels if self.transposed else self.in_channels
         bound = 1.0 / np.sqrt(fan * len(self.kernel))
-        self.kernel.data.uniform_(-bound, bound)
-        if self.bias is not None:
-            self.bias.data.uniform_(-bound, bound)
+        with torch.no_grad():
+            self.kernel.uniform_(-bound, bound)
+            if self.bias is not None:
+                self.bias.uniform_(-bound, bound)
+        self.invalidate_cached_weights()
+
+    def invalidate_cached_weights(self):
+        """Drops the packed copy of ``kernel`` that inference passes keep.  The
+        copy follows the parameter by its storage and version counter, which
+        every in-place operation on the parameter itself bumps; writes through
+        ``kernel.data`` (``kernel.data.copy_(...)``, ``.data.normal_()``) bump
+        nothing, so call this after them (``reset_parameters``, ``load_state_dict``
+        and ``.to()`` / ``.half()`` / ``.cuda()`` do it themselves)."""
+        self._packed = None
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        super()._load_from_state_dict(*args, **kwargs)
+        self.invalidate_cached_weights()
+
+    def _apply(self, fn, *args, **kwargs):
+        result = super()._apply(fn, *args, **kwargs)
+        self.invalidate_cached_weights()
+        return result
 
     def set_kernel_map_cache(self, cache: KernelMapCache):
         self._kernel_map_cache = cache

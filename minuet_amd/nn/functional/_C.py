@@ -317,6 +317,13 @@ def target_coordinates(coordinates: torch.Tensor, batch_dims: Optional[torch.Ten
     library calls.  ``source_bounds`` (8 int64: per-dimension minima, then
     maxima of ``coordinates``) spares their reduction on the device."""
     _ensure_ndim("coordinates", coordinates, 2)
+    if batch_dims is not None and batch_dims.numel() <= 2:
+        # one cloud carrying its boundaries: the library runs it as unbatched and
+        # writes no boundaries, so they are put together here
+        # (minuet/nn/convolutions.py:92-96 returns [0, count] for it)
+        out, _ = target_coordinates(coordinates, None, target_stride, source_bounds)
+        ends = [0, out.shape[0]][:batch_dims.numel()]
+        return out, torch.tensor(ends, dtype=batch_dims.dtype, device=batch_dims.device)
     known = None if source_bounds is None else np.ascontiguousarray(source_bounds, dtype=np.int64)
     device = _common_device([coordinates] + ([batch_dims] if batch_dims is not None else []))
     n, ndim = coordinates.shape

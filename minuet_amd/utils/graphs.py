@@ -9,7 +9,7 @@ graph and replayed with new feature values, which removes the per-layer
 launch cost on the host.  (Not in the reference, whose layers synchronise to
 read the kernel-map sizes back on every call:
 minuet/nn/functional/convolution.py:32-60.)"""
-from typing import Callable, Optional
+from typing import Callable
 
 import torch
 
@@ -31,18 +31,23 @@ class GraphedForward:
         return self.output
 
 
-def capture_forward(forward: Callable[[], object], warmup: int = 3,
-                    stream: Optional["torch.cuda.Stream"] = None) -> GraphedForward:
+def capture_forward(forward: Callable[[], object], warmup: int = 3) -> GraphedForward:
     """Captures ``forward()`` (a callable without arguments that runs the network
     on fixed input tensors and returns its output) in a HIP graph.
 
     The warm-up runs happen on the capture stream first, so that the kernel maps
     are cached, weights are packed and the stream's scratch arena has its final
     size before anything is recorded; a pass that still has to build a kernel
-    map waits on the device and cannot be captured."""
+    map waits on the device and cannot be captured.
+
+    The capture stream is a fresh one that only the returned object knows: the
+    graph's kernels use scratch pointers of that stream's arena, which
+    therefore must not be freed (``cuda_free_buffers`` acts on the arena of
+    the stream that is current, never this one) nor used by other work.  Replays
+    of one ``GraphedForward`` must not overlap (they share that scratch)."""
     if not torch.cuda.is_available():
         raise RuntimeError("[Minuet] graph capture needs a GPU")
-    side = stream if stream is not None else torch.cuda.Stream()
+    side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.no_grad(), torch.cuda.stream(side):
         for _ in range(max(1, warmup)):

@@ -9,7 +9,7 @@ import numpy as np
 from torch.nn import Module
 
 __all__ = ["as_tuple", "generate_kernel_offsets", "set_kernel_map_cache",
-           "dump_tunable_config", "load_tunable_config", "autotune"]
+           "dump_tunable_config", "load_tunable_config", "autotune", "invalidate_cached_weights"]
 
 
 def as_tuple(value, *, size: int = 3, name: Optional[str] = None):
@@ -55,6 +55,21 @@ def set_kernel_map_cache(module: Module, cache):
     for child in module.children():
         set_kernel_map_cache(child, cache=cache)
     return module
+
+
+def invalidate_cached_weights(module: Module):
+    """Drops every derived copy of parameters that inference passes keep below
+    ``module``: packed convolution kernels and the per-channel scale / shift of
+    folded BatchNorm layers.  Those copies follow the parameters by storage and
+    version counter, which writes through ``.data`` do not bump; call this
+    after such writes (no counterpart in the reference, which repacks its
+    weights in every forward, csrc/minuet/cuda/functions/sparse_convolution.cu:526-553)."""
+    for child in module.modules():
+        drop = getattr(child, "invalidate_cached_weights", None)
+        if callable(drop):
+            drop()
+        else:
+            child.__dict__.pop("_minuet_affine", None)
 
 
 def _ensure_directory(path: str):

@@ -482,3 +482,114 @@ def test_autotune_and_timers(tmp_path):
         saved = json.load(fh)
     assert saved["0"]["gather_tile_size"] == cfg["0"]["gather_tile_size"]
     assert F.cuda_buffer_total_size() >= F.cuda_buffer_used_size() >= 0
+
+
+def test_cached_weights_are_dropped_on_request_and_by_the_module_hooks():
+    """Packed kernels and folded BatchNorm constants follow in-place updates of
+    the parameters by themselves; writes through ``.data`` (which bump no
+    version counter) need ``invalidate_cached_weights``; ``reset_parameters``
+    and ``load_state_dict`` drop the copies themselves."""
+    src, sbd, tgt, tbd, off, feats, weights = make_layer_case(21, 3000, 16, 3, 32, 32, "fp16")
+    conv = minuet.nn.SparseConv3d(32, 32, 3, dtype=torch.float16, device="cuda")
+    norm = minuet.nn.BatchNorm(32, device="cuda").eval()
+    net = minuet.nn.FusedSequential(conv, norm, minuet.nn.ReLU()).eval()
+    minuet.set_kernel_map_cache(net, minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda"))
+    x = minuet.SparseTensor(dev(feats).half(), dev(src))
+    rms = lambda t: t.float().pow(2).mean().sqrt().item()
+    close = lambda a, b: (a.float() - b.float()).abs().max().item() <= 2e-2 * max(rms(b), 1e-6)
+    with torch.no_grad():
+        for flow in ("gather_gemm_scatter", "implicit"):
+            conv.tunable_config["dataflow"] = flow
+            a = conv(x).F.clone()
+            conv.kernel.data.mul_(2.0)                 # no version bump: the packed copy is stale
+            conv.invalidate_cached_weights()
+            assert close(conv(x).F, 2 * a.float())
+            conv.kernel.data.mul_(0.5)
+            minuet.invalidate_cached_weights(net)      # the model-wide form
+            assert close(conv(x).F, a)
+        # reset_parameters after a forward: the output follows the new weights
+        before = conv(x).F.clone()
+        conv.reset_parameters()
+        after = conv(x).F
+        conv.invalidate_cached_weights()
+        assert torch.equal(conv(x).F, after) and not torch.equal(after, before)
+        # load_state_dict
+        state = {k: v.clone() for k, v in net.state_dict().items()}
+        y0 = net(x).F.clone()
+        conv.kernel.mul_(3.0)
+        norm.weight.data.fill_(0.25)
+        minuet.invalidate_cached_weights(net)
+        assert not close(net(x).F, y0)
+        net.load_state_dict(state)
+        assert close(net(x).F, y0)
+        # the folded BatchNorm: a .data write shows after invalidation
+        norm.bias.data.add_(1.0)
+        minuet.invalidate_cached_weights(net)
+        y1 = net(x).F
+        ref = torch.relu(norm(conv(x)).F.float())
+        assert close(y1, ref)
+
+
+@pytest.mark.parametrize("kind", ["fp16", "bf16"])
+@pytest.mark.parametrize("cin,cout", [(32, 64), (64, 64), (48, 64), (16, 40)])
+def test_forward_implicit_two_target_blocks_per_wavefront(kind, cin, cout):
+    """Clouds of more than 2^19 targets with 33..64 output channels run the
+    single-kernel forward with two target blocks per wavefront (256 targets per
+    workgroup, a ragged last tile): against the three-kernel dataflow on every
+    row, and against float64 sums written out here on a sample of rows."""
+    dtype = TORCH[kind]
+    n = (1 << 19) + 77
+    rng = np.random.default_rng(77)
+    extent = 300
+    flat = rng.choice(extent ** 3, size=n, replace=False)
+    flat.sort()                                          # lexicographic order of (x, y, z)
+    coords = np.stack([flat // (extent * extent), (flat // extent) % extent, flat % extent], 1).astype(np.int32)
+    off = orc.generate_kernel_offsets(3, 3, 1, 1)
+    c_dev = dev(coords)
+    built = _C.kernel_map_build(c_dev, c_dev, off.astype(np.int64), None, None, reorder=True,
+                                want_masks=True, want_lists=True, want_dense=True)
+    kmap = built["kernel_map"]
+    feats = torch.from_numpy(rng.normal(size=(n, cin))).to(dtype).cuda()
+    weights = torch.from_numpy(rng.normal(size=(27, cin, cout)) / np.sqrt(27 * cin)).to(dtype).cuda()
+    scale = dev(rng.uniform(0.5, 1.5, size=cout).astype(np.float32))
+    shift = dev(rng.uniform(-0.5, 0.5, size=cout).astype(np.float32))
+    residual = torch.from_numpy(rng.normal(size=(n, cout))).to(dtype).cuda()
+    sizes = built["sizes"]
+    sizes.host_sizes = built["sizes_host"]
+    order = built["order"]
+    order.host_order = built["order_host"]
+    source_masks = built["source_masks"]
+    source_masks.gather_index = built["in_idx"]
+    sample = rng.choice(n, size=1500, replace=False)
+    sample[:3] = (0, n - 1, n - 2)                       # the ragged last tile is in the sample
+    # the sampled rows of the kernel map, checked against a search over packed keys
+    keys = flat.astype(np.int64)
+    for o in range(27):
+        q = coords[sample].astype(np.int64) + off[o]
+        inside = ((q >= 0) & (q < extent)).all(1)
+        qk = (q[:, 0] * extent + q[:, 1]) * extent + q[:, 2]
+        pos = np.searchsorted(keys, qk)
+        pos_c = np.minimum(pos, n - 1)
+        hit = inside & (keys[pos_c] == qk)
+        np.testing.assert_array_equal(host(kmap[o, sample]), np.where(hit, pos_c, -1))
+    km = host(kmap[:, sample])
+    f64, w64 = host(feats.double()), host(weights.double())
+    plain = np.zeros((sample.shape[0], cout))
+    for o in range(27):
+        rows = np.nonzero(km[o] >= 0)[0]
+        plain[rows] += f64[km[o, rows]] @ w64[o]
+    fused = np.maximum(plain * host(scale).astype(np.float64) + host(shift).astype(np.float64)
+                       + host(residual.double())[sample], 0.0)
+    for epilogue, ref in ((None, plain), (F.Epilogue(scale, shift, residual, "relu"), fused)):
+        out = _C.sparse_convolution_forward_implicit(feats, weights, kmap, epilogue=epilogue)
+        assert out.shape == (n, cout) and torch.isfinite(out).all()
+        assert_features_close(out[sample], ref, kind)
+        three = F.sparse_convolution_forward(
+            sources=feats, weights=weights, source_masks=source_masks, target_masks=built["target_masks"],
+            kernel_map_order=order, kernel_map_sizes=sizes, gather_tile_size=0, scatter_tile_size=0,
+            allow_shortcut_matmul=True, threshold=-1, epilogue=epilogue, dataflow="gather_gemm_scatter")
+        # two roundings of the same sums: 2e-2 of the RMS, or one unit in the
+        # last place of the largest value where that is more (bf16 keeps 8 bits)
+        diff = (out.float() - three.float()).abs().max().item()
+        ulp = three.float().abs().max().item() * 2.0 ** (-7 if kind == "bf16" else -10)
+        assert diff <= max(2e-2 * three.float().pow(2).mean().sqrt().item(), ulp), diff

@@ -562,3 +562,42 @@ def test_sorted_kernel_map_lists_2d_and_4d():
         cloud = cloud[rng.permutation(cloud.shape[0])]
         off = orc.generate_kernel_offsets(ndim, 3 if ndim == 2 else 2, 1, 1)
         _check_sorted_lists(cloud, off)
+
+
+@pytest.mark.parametrize("idtype", [np.int32, np.int64])
+def test_target_coordinates_one_cloud_with_boundaries(idtype):
+    """A single cloud that still carries batch_dims = [0, n] gets [0, count]
+    back, as the reference's tensor expression gives (convolutions.py:92-96)."""
+    c, _ = sorted_unique(random_cloud(6000, 30, seed=19, lo=-9))
+    bd = np.array([0, c.shape[0]], dtype=idtype)
+    got, got_bd = _C.target_coordinates(dev(c), dev(bd), (2, 2, 2))
+    exp, _ = orc.target_coordinates(c, None, (2, 2, 2))
+    np.testing.assert_array_equal(host(got), exp)
+    assert got_bd.dtype == (torch.int32 if idtype == np.int32 else torch.int64)
+    np.testing.assert_array_equal(host(got_bd), [0, exp.shape[0]])
+    cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+    coords, stride, dims = cache.get_target_coordinates(dev(c), dev(bd), 1, 2)
+    np.testing.assert_array_equal(host(coords), exp)
+    np.testing.assert_array_equal(host(dims), [0, exp.shape[0]])
+
+
+def test_cache_bounds_survive_recycled_storage():
+    """Bounds remembered for a temporary (the contiguous copy of a strided
+    coordinate view) must not be picked up by a later tensor that lands on the
+    recycled address: the cache keeps what it files bounds under alive."""
+    cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+    a, _ = sorted_unique(random_cloud(4000, 20, seed=3, lo=0))
+    wide = torch.zeros((a.shape[0], 6), dtype=torch.int32, device="cuda")
+    wide[:, ::2] = dev(a)
+    view = wide[:, ::2]                                    # not contiguous: the cache works on a copy
+    assert not view.is_contiguous()
+    dense_a = cache.get_dense_kernel_map(view, 1, None, view, 1, None, 3, 1)
+    np.testing.assert_array_equal(host(dense_a), orc.query_sorted_index_with_offsets(
+        a, a, orc.generate_kernel_offsets(3, 3, 1, 1)))
+    # same row count, far larger coordinates, allocated right after the temporary went away
+    b = a[: a.shape[0]].copy()
+    b[:, 0] += 5000
+    b_dev = dev(b)
+    dense_b = cache.get_dense_kernel_map(b_dev, 2, None, b_dev, 2, None, 3, 1)
+    np.testing.assert_array_equal(host(dense_b), orc.query_sorted_index_with_offsets(
+        b, b, orc.generate_kernel_offsets(3, 3, 2, 1)))
