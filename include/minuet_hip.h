@@ -59,6 +59,14 @@ int mnt_buffer_set_page_size(void *stream, size_t bytes); /* cuda_set_buffer_pag
 size_t mnt_buffer_total_size(void *stream);               /* cuda_buffer_total_size */
 size_t mnt_buffer_used_size(void *stream);                /* cuda_buffer_used_size */
 int mnt_reset_error(void);                                /* cuda_reset_error */
+/* cuda_device_reset (csrc/minuet/torch/cuda_memory_buffer.cu:38,47).  The
+ * reference calls cudaDeviceReset(), which also destroys the context PyTorch
+ * allocates from; here the call waits for the device and gives back what the
+ * LIBRARY holds on the current device (the arenas of every stream with their
+ * pages, persistent blocks and pinned staging blocks) and clears the error
+ * state, so that tensors of the process stay valid.  Pending two-phase calls
+ * are forgotten. */
+int mnt_device_reset(void);
 
 /* ---- Map: coordinate sort ---------------------------------------------- */
 

@@ -70,6 +70,9 @@ inline int guarded(Fn &&fn) {
 class Arena {
  public:
   static Arena &of(hipStream_t stream);
+  // Gives back everything the library holds on the current device: the arenas
+  // of all its streams (pages, persistent blocks, pinned staging blocks).
+  static void reset_device();
 
   struct Mark {
     size_t page;
@@ -80,7 +83,7 @@ class Arena {
   Mark mark() const;
   void release(const Mark &m);
   void preallocate(size_t bytes);
-  void free_all();
+  void free_all(bool synchronise = true);
   size_t total() const;
   size_t used() const;
   void set_growth(float g) { growth_ = g; }

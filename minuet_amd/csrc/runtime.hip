@@ -73,8 +73,8 @@ void Arena::preallocate(size_t bytes) {
   add_page(align_up(bytes, page_size_));
 }
 
-void Arena::free_all() {
-  MNT_HIP(hipStreamSynchronize(stream_));
+void Arena::free_all(bool synchronise) {
+  if (synchronise) MNT_HIP(hipStreamSynchronize(stream_));
   for (auto &p : pages_) MNT_HIP(hipFree(p.base));
   pages_.clear();
   cursor_ = 0;
@@ -87,6 +87,27 @@ void Arena::free_all() {
   }
   pending.valid = false;
   map_state_valid = false;
+}
+
+void Arena::reset_device() {
+  int device = 0;
+  MNT_HIP(hipGetDevice(&device));
+  std::lock_guard<std::mutex> lock(g_arena_mutex);
+  for (auto it = g_arenas.begin(); it != g_arenas.end();) {
+    if (it->first.first != device) {
+      ++it;
+      continue;
+    }
+    Arena *arena = it->second;
+    arena->free_all(false);               // the caller has waited for the whole device; the stream may be gone
+    if (arena->pinned_ != nullptr) {
+      MNT_HIP(hipHostFree(arena->pinned_));
+      arena->pinned_ = nullptr;
+      arena->pinned_device_ = nullptr;
+    }
+    delete arena;
+    it = g_arenas.erase(it);
+  }
 }
 
 size_t Arena::total() const {
@@ -245,6 +266,15 @@ int mnt_reset_error(void) {
   (void)hipGetLastError();
   g_last_error.clear();
   return 0;
+}
+
+int mnt_device_reset(void) {
+  return guarded([&] {
+    MNT_HIP(hipDeviceSynchronize());
+    Arena::reset_device();
+    (void)hipGetLastError();
+    g_last_error.clear();
+  });
 }
 
 }  // extern "C"

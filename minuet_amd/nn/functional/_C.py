@@ -42,6 +42,7 @@ SIGNATURES = {
     "mnt_buffer_total_size": (_sz, [_vp]),
     "mnt_buffer_used_size": (_sz, [_vp]),
     "mnt_reset_error": (_int, []),
+    "mnt_device_reset": (_int, []),
     "mnt_arg_sort_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _vp, _pi64, _vp]),
     "mnt_unique_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _pi64, _vp]),
     "mnt_fill_unique_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _int, _vp, _vp]),
@@ -1171,6 +1172,13 @@ def cuda_buffer_total_size() -> int:
 
 def cuda_reset_error():
     load_library().mnt_reset_error()
+
+
+def cuda_device_reset():
+    """csrc/minuet/torch/cuda_memory_buffer.cu:38,47.  Frees everything the library
+    holds on the current device (every stream's arena); unlike the reference's
+    cudaDeviceReset() it leaves the context, and with it every torch tensor, alone."""
+    _check(load_library().mnt_device_reset())
 
 
 def profile_enable(on: bool):

@@ -3,7 +3,7 @@ from . import _C
 
 __all__ = ["cuda_buffer_total_size", "cuda_buffer_used_size", "cuda_free_buffers",
            "cuda_set_buffer_growth", "cuda_set_buffer_page_size", "cuda_preallocate_buffer",
-           "cuda_reset_error"]
+           "cuda_reset_error", "cuda_device_reset"]
 
 
 def cuda_buffer_total_size() -> int:
@@ -35,3 +35,9 @@ def cuda_set_buffer_page_size(page_size: int):
 
 def cuda_reset_error():
     _C.cuda_reset_error()
+
+
+def cuda_device_reset():
+    """Gives back all scratch memory the library holds on the current device
+    (every stream's arena) and clears its error state."""
+    _C.cuda_device_reset()
