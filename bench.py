@@ -22,11 +22,23 @@ for _p in (ROOT, os.path.join(ROOT, "oracle")):
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per query_kernel launch on this workload at scale 1: FETCH_SIZE and
-# WRITE_SIZE of rocprofv3 --pmc, each scaled by what the counter reads for a
-# plain 256 MiB device copy (2.000 and 1.000); the dense kernel map the kernel
-# writes accounts for 21.6 MB of it.
-QUERY_TRAFFIC_BYTES = 30.79e6
+MAP_PROFILE = os.path.join(ROOT, "profiles", "map_step_config2_200k_voxels.md")
+
+
+def measured_traffic(kernel):
+    """HBM bytes per launch of `kernel` on this workload at scale 1, from the
+    committed rocprofv3 summary (FETCH_SIZE + WRITE_SIZE, each scaled by what
+    the counter reads for a plain device copy of known size); None when the
+    summary does not list the kernel."""
+    import re
+    try:
+        text = open(MAP_PROFILE).read()
+    except OSError:
+        return None
+    match = re.search(r"traffic_bytes:\s*(\{.*?\})", text)
+    if not match:
+        return None
+    return json.loads(match.group(1)).get(kernel)
 
 
 def map_step(_C, coords_dev, offsets):
@@ -36,21 +48,55 @@ def map_step(_C, coords_dev, offsets):
     return sorted_dev, built
 
 
-def cpu_baseline(coords, offsets, budget_s=12.0):
-    """The plain-C restatement of the reference algorithm (oracle/oracle_c.c) on
-    the host cores, same cloud, for about `budget_s` seconds."""
-    import c_oracle
-    c_oracle.map_step(coords, offsets)            # warm-up (page faults, thread pool)
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _median_ms(fn, budget_s, most):
+    fn()                                          # warm-up (page faults, thread pool)
     times = []
     start = time.perf_counter()
-    while time.perf_counter() - start < budget_s and len(times) < 200:
+    while time.perf_counter() - start < budget_s and len(times) < most:
         t0 = time.perf_counter()
-        c_oracle.map_step(coords, offsets)
+        fn()
         times.append(time.perf_counter() - t0)
-    return {"value": round(1e3 * float(np.median(times)), 3), "unit": "ms", "cores": c_oracle.num_threads(),
-            "kind": "port",
-            "sample": f"{len(times)} full Map steps (sort, query, sizes, pair lists) of the same "
-                      f"{coords.shape[0]}-voxel cloud; median"}
+    return 1e3 * float(np.median(times)), len(times)
+
+
+def cpu_baseline(coords, offsets, budget_s=10.0):
+    """The plain-C restatement of the reference algorithm (oracle/oracle_c.c) on
+    the host cores: the Map step of the same cloud for about `budget_s` seconds,
+    then the layer of configuration 1 (3x3x3, 32 -> 32 channels, fp32: gather,
+    per-offset GEMM, scatter, with its kernel map built beforehand)."""
+    import c_oracle
+    import minuet_oracle as orc
+    from minuet_amd.synthetic import make_cloud
+    map_ms, map_runs = _median_ms(lambda: c_oracle.map_step(coords, offsets), budget_s, 200)
+    c1 = make_cloud(1)["coords"]
+    _, s1 = c_oracle.arg_sort(c1)
+    dense = c_oracle.query(s1, s1, offsets)
+    sizes = c_oracle.sizes(dense)
+    order = orc.stable_size_order(sizes)
+    sm, tm = c_oracle.masks(dense, s1.shape[0], order)
+    rng = np.random.default_rng(1001)
+    feats = rng.normal(size=(s1.shape[0], 32)).astype(np.float32)
+    weights = (rng.normal(size=(27, 32, 32)) / np.sqrt(27 * 32)).astype(np.float32)
+    layer_ms, layer_runs = _median_ms(
+        lambda: c_oracle.conv_forward(feats, weights, sm, tm, order, sizes[order]), 5.0, 200)
+    return {"value": round(map_ms, 3), "unit": "ms", "cores": c_oracle.num_threads(),
+            "kind": "port", "cpu_model": cpu_model(), "host_cpus": os.cpu_count(),
+            "sample": f"{map_runs} full Map steps (sort, query, sizes, pair lists) of the same "
+                      f"{coords.shape[0]}-voxel cloud; median",
+            "config1_layer_fp32": {"ms": round(layer_ms, 3), "voxels": int(s1.shape[0]),
+                                   "mvoxels_per_s": round(s1.shape[0] / layer_ms / 1e3, 2),
+                                   "sample": f"{layer_runs} forward passes of the configuration-1 layer "
+                                             f"(gather, 27 GEMMs, scatter; kernel map cached); median"}}
 
 
 def _time_ms(fn, warmup, reps):
@@ -86,7 +132,7 @@ def _time_stats(fn, warmup, reps):
 MFMA_PEAK_TFLOPS = {"fp16": 2500.0, "bf16": 2500.0, "fp32": 157.3}
 
 
-def layer_stages(device, config, channels, kernel_size, dtype_name):
+def layer_stages(device, config, channels, kernel_size, dtype_name, tune=False):
     """Gather, grouped GEMM and Scatter timed one by one through the library's
     stage timers (the reference's cuda_time_* interface), then the whole layer
     through both dataflows, with the algorithmic bytes / flops of each."""
@@ -144,6 +190,29 @@ def layer_stages(device, config, channels, kernel_size, dtype_name):
             stats["mvoxels_per_s"] = round(voxels / stats["ms_mean"] / 1e3, 1)
             stats["achieved_TFLOPs"] = round(flops / (stats["ms_mean"] * 1e-3) / 1e12, 1)
             out["layer_" + flow] = stats
+        if tune:
+            # the layer's own autotuner (padding threshold, gather / scatter tile, dataflow)
+            # on this workload, then the layer as tuned
+            conv.tunable_config.update(dataflow="auto", threshold=-1, gather_tile_size=0, scatter_tile_size=0)
+            t0 = time.perf_counter()
+            minuet.autotune(conv, cache, [x])
+            seconds = time.perf_counter() - t0
+            cache.reset()
+            tuned = dict(conv.tunable_config)
+            stats = _time_stats(lambda: conv(x), 10, 50)
+            stats["mvoxels_per_s"] = round(voxels / stats["ms_mean"] / 1e3, 1)
+            # rows of the GEMM buffers under the padding plans the threshold chooses between
+            # (padded rows are laid out, never computed: the kernel's tiles stop at each group's size)
+            sizes_list = [int(v) for v in host_sizes[:-1]]          # the centre offset takes the shortcut
+            plans = {}
+            for name, threshold in (("none (-1)", -1), ("0.5", 0.5), ("one bucket (None)", None)):
+                buckets = _C.generate_padding_buckets(sizes_list, threshold)
+                rows = _C.cumsum_kernel_padded_sizes(sizes_list, buckets)[-1]
+                plans[name] = {"buckets": len(buckets) - 1, "buffer_rows": int(rows),
+                               "padding_waste": round(rows / max(1, sum(sizes_list)) - 1.0, 4)}
+            out["autotune"] = {"seconds": round(seconds, 2), "tuned_config": tuned, "layer_as_tuned": stats,
+                               "padding_plans": plans, "group_sizes_min_median_max": [
+                                   int(host_sizes.min()), int(np.median(host_sizes)), int(host_sizes.max())]}
     return out
 
 
@@ -162,7 +231,7 @@ def extras(device, with_config5, section="all"):
     if section == "layer-kernels":
         return {"config2_layer_kernels_fp16_c64": layer_stages(device, 2, 64, 3, "fp16")}
     if section == "config5":
-        return {"config5_layer_bf16_c64_k5": layer_stages(device, 5, 64, 5, "bf16")}
+        return {"config5_layer_bf16_c64_k5": layer_stages(device, 5, 64, 5, "bf16", tune=True)}
     with torch.no_grad():
         # configuration 1: submanifold 3x3x3, 32 -> 32, fp32
         c1 = torch.from_numpy(make_cloud(1)["coords"]).to(device)
@@ -228,7 +297,7 @@ def extras(device, with_config5, section="all"):
         return {"config4_unet_fp16": out["config4_unet_fp16"]}
     out["config2_layer_kernels_fp16_c64"] = layer_stages(device, 2, 64, 3, "fp16")
     if with_config5:
-        out["config5_layer_bf16_c64_k5"] = layer_stages(device, 5, 64, 5, "bf16")
+        out["config5_layer_bf16_c64_k5"] = layer_stages(device, 5, 64, 5, "bf16", tune=True)
     return out
 
 
@@ -305,6 +374,8 @@ def main():
         map_step(_C, coords_dev, offsets)
     torch.cuda.synchronize()
     wall_ms = 1e3 * (time.perf_counter() - t0) / args.steps
+    # the same step one by one: stream events between the calls, at least 50 of them
+    step_stats = _time_stats(lambda: map_step(_C, coords_dev, offsets), 10, max(50, min(args.steps, 500)))
 
     # per-stage device time from the library's own stream events
     _C.profile_enable(True)
@@ -320,7 +391,6 @@ def main():
 
     bytes_map = 12 * n + 12 * n + 4 * n + 8 * nnz + 4 * offsets.shape[0]
     bytes_query = 12 * n + 8 * nnz
-    bytes_dense = 12 * n + 4 * offsets.shape[0] * n
     query_ms = stage_ms.get("query", float("nan"))
     achieved = bytes_query / (query_ms * 1e-3) / 1e9 if query_ms == query_ms and query_ms > 0 else None
     result = {
@@ -340,17 +410,15 @@ def main():
                                "unsorted unique voxels to per-offset (in,out) int32 lists",
                    "voxels": n, "nnz": nnz, "generator": cloud["note"], "seed": 1002,
                    "bounding_box": [coords.min(0).tolist(), coords.max(0).tolist()],
-                   "mvoxels_per_s": round(n / wall_ms / 1e3, 2)},
+                   "mvoxels_per_s": round(n / wall_ms / 1e3, 2),
+                   "list_order": "rows by ascending size (what KernelMapCache keeps)"},
+        "step_stats": step_stats,
         "roofline": {"bound": "hbm", "kernel": "query_kernel",
                      "achieved": None if achieved is None else round(achieved, 2),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": None if achieved is None else round(achieved / HBM_PEAK_GBS, 5),
-                     "traffic": QUERY_TRAFFIC_BYTES if args.scale == 1.0 else None,
+                     "traffic": measured_traffic("query_kernel") if args.scale == 1.0 else None,
                      "algorithmic_bytes": bytes_query,
-                     # the same launch priced with the dense map M[O, T] as its output, which is
-                     # what it writes and what the reference's query function returns
-                     "dense_form": {"algorithmic_bytes": bytes_dense,
-                                    "achieved": None if achieved is None else round(bytes_dense / (query_ms * 1e-3) / 1e9, 2)},
                      "avg_launch_ms": None if achieved is None else round(query_ms, 5),
                      "map_step": {"algorithmic_bytes": bytes_map,
                                   "device_ms": round(device_ms, 4),

@@ -285,6 +285,12 @@ class SparseConv(Module):
 
     __AVAILABLE_THRESHOLD__ = [-1, *list(np.linspace(0, 2, num=50)), None]
     __NUM_TUNING_ROUNDS__ = 10
+    # The reference times its bucket GEMMs under every threshold because padded
+    # rows are computed there (convolutions.py:367-389).  The grouped GEMM here
+    # stops each group's tiles at the group's size, so the threshold changes the
+    # buffer layout only and the sweep would time the same work 52 times: the
+    # tuner keeps -1 (no padded rows, least scratch) unless this is set.
+    __TUNE_THRESHOLD__ = False
 
     def __init__(self, ndim: int, in_channels: int, out_channels: int, kernel_size,
                  stride=1, dilation=1, bias: bool = False, transposed: bool = False,
@@ -419,7 +425,10 @@ class SparseConv(Module):
             if self.is_trivial or not self._tuning_data:
                 return
             best = None
-            for threshold in self.__AVAILABLE_THRESHOLD__:
+            thresholds = self.__AVAILABLE_THRESHOLD__ if self.__TUNE_THRESHOLD__ else []
+            if not self.__TUNE_THRESHOLD__:
+                self._tunable_config["threshold"] = -1
+            for threshold in thresholds:
                 try:
                     score = self._score(F.cuda_time_gemm, threshold=threshold)
                 except RuntimeError:

@@ -463,6 +463,7 @@ def test_autotune_and_timers(tmp_path):
     minuet.set_kernel_map_cache(net, cache)
     minuet.nn.SparseConv.__NUM_TUNING_ROUNDS__ = 1
     minuet.nn.SparseConv.__AVAILABLE_THRESHOLD__ = [-1, 0.5, None]
+    minuet.nn.SparseConv.__TUNE_THRESHOLD__ = True          # the reference's sweep, off by default here
     path = str(tmp_path / "tuned" / "config.json")
     with torch.no_grad():
         before = net(x).F.clone()
@@ -481,7 +482,13 @@ def test_autotune_and_timers(tmp_path):
     with open(path) as fh:
         saved = json.load(fh)
     assert saved["0"]["gather_tile_size"] == cfg["0"]["gather_tile_size"]
-    assert F.cuda_buffer_total_size() >= F.cuda_buffer_used_size() >= 0
+    # without the sweep the tuner leaves the threshold that pads nothing
+    minuet.nn.SparseConv.__TUNE_THRESHOLD__ = False
+    net[0].tunable_config["threshold"] = 0.5
+    with torch.no_grad():
+        minuet.autotune(net, cache, [x])
+    assert net[0].tunable_config["threshold"] == -1
+    assert F.cuda_buffer_used_size() == 0
 
 
 def test_cached_weights_are_dropped_on_request_and_by_the_module_hooks():
