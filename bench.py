@@ -153,8 +153,9 @@ def layer_stages(device, config, channels, kernel_size, dtype_name, tune=False):
     with torch.no_grad():
         conv.tunable_config["dataflow"] = "gather_gemm_scatter"     # builds the rank tables
         conv(x)
-        source_masks, target_masks, order, sizes = next(iter(cache._kernel_maps_cache.values()))
-        host_sizes = np.asarray(sizes.host_sizes, dtype=np.int64)
+        kernel_map = next(iter(cache._kernel_maps_cache.values()))
+        source_masks, target_masks, order, sizes = kernel_map
+        host_sizes = np.asarray(kernel_map.sizes_host, dtype=np.int64)
         voxels = int(sorted_dev.shape[0])
         nnz = int(host_sizes.sum())
         moved = nnz - voxels                       # the centre offset takes the shortcut

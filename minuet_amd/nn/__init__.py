@@ -1,4 +1,5 @@
 from . import functional
+from .kernel_map import *
 from .convolutions import *
 from .activations import *
 from .normalizations import *

@@ -18,6 +18,7 @@ from torch.nn import Module
 
 from minuet_amd.nn import functional as F
 from minuet_amd.nn.functional import _C
+from minuet_amd.nn.kernel_map import KernelMap
 from minuet_amd.tensors import SparseTensor
 from minuet_amd.utils.helpers import as_tuple, generate_kernel_offsets
 
@@ -48,9 +49,10 @@ class KernelMapCache(object):
         self._device = device
         self._layout = layout
         self._disable_reordering = disable_reordering
-        self._kernel_maps_cache = dict()        # key -> rank tables, order, sizes
+        self._kernel_maps_cache = dict()        # key -> KernelMap of the forward layer
+        self._swapped_maps_cache = dict()       # key -> the same map as its transposed layer reads it
         self._key_memo = dict()
-        self._dense_maps_cache = dict()         # key -> dense kernel map [O, T]
+        self._dense_maps_cache = dict()         # key -> (dense kernel map [O, T], number of sources)
         self._inverse_maps_cache = dict()       # key -> its inverse [O, S] (transposed layers)
         self._coordinates_cache = dict()
         self._bounds_cache = dict()
@@ -67,6 +69,7 @@ class KernelMapCache(object):
     def reset(self):
         self._coordinates_cache.clear()
         self._kernel_maps_cache.clear()
+        self._swapped_maps_cache.clear()
         self._dense_maps_cache.clear()
         self._inverse_maps_cache.clear()
         self._bounds_cache.clear()
@@ -162,8 +165,8 @@ class KernelMapCache(object):
         key, source_stride, kernel_size, kernel_dilation = self._map_key(
             source_coordinates.shape[1], source_stride, target_stride, kernel_size, kernel_dilation,
             transposed)
-        dense = self._dense_maps_cache.get(key)
-        if dense is None:
+        entry = self._dense_maps_cache.get(key)
+        if entry is None:
             if transposed:
                 raise RuntimeError(_TRANSPOSED_FIRST)
             offsets = self._kernel_offsets(source_stride, kernel_size, kernel_dilation)
@@ -177,13 +180,18 @@ class KernelMapCache(object):
             if source_coordinates.shape[0] > 0 and target_coordinates.shape[0] > 0:
                 self._remember_bounds(source_coordinates, bounds[:8])
                 self._remember_bounds(target_coordinates, bounds[8:])
-            dense.num_sources = source_coordinates.shape[0]
-            self._dense_maps_cache[key] = dense
+            entry = (dense, source_coordinates.shape[0])
+            self._dense_maps_cache[key] = entry
         if not transposed:
-            return dense
+            return entry[0]
+        return self._inverse_of(key)
+
+    def _inverse_of(self, key) -> torch.Tensor:
+        """Dense map of the transposed layer of ``key`` ([O, S]), made on first use."""
         inverse = self._inverse_maps_cache.get(key)
         if inverse is None:
-            inverse = _C.kernel_map_invert(dense, dense.num_sources)
+            dense, num_sources = self._dense_maps_cache[key]
+            inverse = _C.kernel_map_invert(dense, num_sources)
             self._inverse_maps_cache[key] = inverse
         return inverse
 
@@ -191,30 +199,29 @@ class KernelMapCache(object):
                        source_batch_dims: Optional[torch.Tensor],
                        target_coordinates: torch.Tensor, target_stride,
                        target_batch_dims: Optional[torch.Tensor], kernel_size, kernel_dilation,
-                       disable_reordering: bool = False, transposed: bool = False):
-        """``(source_masks, target_masks, kernel_map_order, kernel_map_sizes)`` of
-        a layer (reference: convolutions.py:102-173)."""
+                       disable_reordering: bool = False, transposed: bool = False) -> KernelMap:
+        """The layer's :class:`KernelMap`, which unpacks like the reference's tuple
+        ``(source_masks, target_masks, kernel_map_order, kernel_map_sizes)``
+        (reference: convolutions.py:102-173)."""
         key, source_stride, kernel_size, kernel_dilation = self._map_key(
             source_coordinates.shape[1], source_stride, target_stride, kernel_size, kernel_dilation,
             transposed)
-        hit = self._kernel_maps_cache.get(key)
-        if hit is None:
+        cached = self._swapped_maps_cache if transposed else self._kernel_maps_cache
+        hit = cached.get(key)
+        if hit is not None:
+            return hit
+        forward = self._kernel_maps_cache.get(key)
+        if forward is None:
             if transposed and key not in self._dense_maps_cache:
                 raise RuntimeError(_TRANSPOSED_FIRST)
-            hit = self._build_tables(key, source_coordinates, source_batch_dims, target_coordinates,
-                                     target_batch_dims, source_stride, kernel_size, kernel_dilation,
-                                     disable_reordering)
-        source_masks, target_masks, order, sizes = hit
-        if transposed:
-            source_masks, target_masks = target_masks, source_masks
-            if getattr(target_masks, "kernel_map", None) is None:
-                # dense map of the transposed layer, made on first use
-                inverse = self._inverse_maps_cache.get(key)
-                if inverse is None:
-                    inverse = _C.kernel_map_invert(source_masks.kernel_map, target_masks.shape[1])
-                    self._inverse_maps_cache[key] = inverse
-                target_masks.kernel_map = inverse
-        return source_masks, target_masks, order, sizes
+            forward = self._build_tables(key, source_coordinates, source_batch_dims, target_coordinates,
+                                         target_batch_dims, source_stride, kernel_size, kernel_dilation,
+                                         disable_reordering)
+        if not transposed:
+            return forward
+        swapped = forward.swapped(dense=self._inverse_of(key))
+        self._swapped_maps_cache[key] = swapped
+        return swapped
 
     def _build_tables(self, key, source_coordinates, source_batch_dims, target_coordinates,
                       target_batch_dims, source_stride, kernel_size, kernel_dilation,
@@ -224,10 +231,11 @@ class KernelMapCache(object):
         (For a transposed caller the coordinate arguments are the other way
         round, but then the dense map exists and they are not used.)"""
         reorder = not self._disable_reordering and not disable_reordering
-        dense = self._dense_maps_cache.get(key)
-        if dense is not None:
+        entry = self._dense_maps_cache.get(key)
+        if entry is not None:
             # the query ran earlier for a layer that needed the dense map only
-            built = _C.kernel_map_tables(dense, dense.num_sources, reorder=reorder, want_lists=True)
+            dense, num_sources = entry
+            built = _C.kernel_map_tables(dense, num_sources, reorder=reorder, want_lists=True)
         else:
             offsets = self._kernel_offsets(source_stride, kernel_size, kernel_dilation)
             source_coordinates = source_coordinates.contiguous()
@@ -241,29 +249,19 @@ class KernelMapCache(object):
             if source_coordinates.shape[0] > 0 and target_coordinates.shape[0] > 0:
                 self._remember_bounds(source_coordinates, built["bounds"][:8])
                 self._remember_bounds(target_coordinates, built["bounds"][8:])
-            built["kernel_map"].num_sources = source_coordinates.shape[0]
-            self._dense_maps_cache[key] = built["kernel_map"]
+            dense, num_sources = built["kernel_map"], source_coordinates.shape[0]
+            self._dense_maps_cache[key] = (dense, num_sources)
         index_dtype = (source_coordinates.dtype if source_batch_dims is None
                        else source_batch_dims.dtype)
         cast = (lambda t: t) if index_dtype == torch.int32 else (lambda t: t.to(index_dtype))
-        sizes = cast(built["sizes"])
-        # host copies as the library takes them (contiguous int64), made once
-        sizes.host_sizes = np.ascontiguousarray(built["sizes_host"], dtype=np.int64)
-        order = cast(built["order"]) if reorder else None
-        if order is not None:
-            order.host_order = np.ascontiguousarray(built["order_host"], dtype=np.int64)
-        source_masks, target_masks = cast(built["source_masks"]), cast(built["target_masks"])
-        # buffer row -> feature row on either side of the map: what a layer
-        # (forward or transposed) gathers through
-        source_masks.gather_index = built["in_idx"]
-        target_masks.gather_index = built["out_idx"]
-        built["in_idx"].num_hits = built["out_idx"].num_hits = int(sizes.host_sizes.sum())
-        # source row per (offset, target) in the original offset order: what
-        # the single-kernel dataflow walks
-        target_masks.kernel_map = built["kernel_map"]
-        entry = (source_masks, target_masks, order, sizes)
-        self._kernel_maps_cache[key] = entry
-        return entry
+        kernel_map = KernelMap(cast(built["source_masks"]), cast(built["target_masks"]),
+                               cast(built["order"]) if reorder else None, cast(built["sizes"]),
+                               sizes_host=built["sizes_host"],
+                               order_host=built["order_host"] if reorder else None,
+                               in_idx=built["in_idx"], out_idx=built["out_idx"], dense=dense,
+                               num_sources=num_sources, num_targets=dense.shape[1])
+        self._kernel_maps_cache[key] = kernel_map
+        return kernel_map
 
 
 class SparseConv(Module):
@@ -399,9 +397,10 @@ class SparseConv(Module):
     def _score(self, timer, **kwargs):
         times = []
         for _ in range(self.__NUM_TUNING_ROUNDS__):
-            for source_masks, target_masks, sizes in self._tuning_data:
-                times.append(timer(weights=self.kernel, source_masks=source_masks,
-                                   target_masks=target_masks, kernel_map_sizes=sizes,
+            for kernel_map in self._tuning_data:
+                times.append(timer(weights=self.kernel, source_masks=kernel_map.source_masks,
+                                   target_masks=kernel_map.target_masks,
+                                   kernel_map_sizes=kernel_map.kernel_map_sizes,
                                    allow_shortcut_matmul=self._allow_shortcut_matmul, **kwargs))
         return float(np.average(times)) if times else float("inf")
 
@@ -469,15 +468,14 @@ class SparseConv(Module):
         for dataflow in ("gather_gemm_scatter", "implicit"):
             total = 0.0
             try:
-                for source_masks, target_masks, sizes in self._tuning_data:
-                    if dataflow == "implicit" and getattr(target_masks, "kernel_map", None) is None:
+                for kernel_map in self._tuning_data:
+                    if dataflow == "implicit" and kernel_map.dense is None:
                         raise RuntimeError("no dense kernel map")
-                    sources = torch.randn(source_masks.shape[1], self.in_channels,
+                    sources = torch.randn(kernel_map.num_sources, self.in_channels,
                                           device=self.kernel.device).to(self.kernel.dtype)
-                    order = getattr(sizes, "kernel_map_order", None)
+                    order = kernel_map.kernel_map_order
                     call = lambda: F.sparse_convolution_forward(
-                        sources=sources, weights=self.kernel, source_masks=source_masks,
-                        target_masks=target_masks, kernel_map_order=order, kernel_map_sizes=sizes,
+                        sources=sources, weights=self.kernel, kernel_map=kernel_map,
                         gather_tile_size=self._tunable_config["gather_tile_size"],
                         scatter_tile_size=self._tunable_config["scatter_tile_size"],
                         allow_shortcut_matmul=self._allow_shortcut_matmul and order is not None,
@@ -631,14 +629,12 @@ class SparseConv(Module):
     def _forward_tables(self, cache, map_args, sources, epilogue):
         """Gather -> GEMM -> Scatter through the rank tables (the reference's
         dataflow, convolutions.py:470-494)."""
-        source_masks, target_masks, order, sizes = cache.get_kernel_map(**map_args)
+        kernel_map = cache.get_kernel_map(**map_args)
         if self._tuning_data is not None:
-            sizes.kernel_map_order = order
-            self._tuning_data.append((source_masks, target_masks, sizes))
+            self._tuning_data.append(kernel_map)
         weights, packed = self._packed_kernel() if sources.is_cuda else (self.kernel, None)
         return F.sparse_convolution_forward(
-            sources=sources, weights=weights, source_masks=source_masks,
-            target_masks=target_masks, kernel_map_order=order, kernel_map_sizes=sizes,
+            sources=sources, weights=weights, kernel_map=kernel_map,
             gather_tile_size=self._tunable_config["gather_tile_size"],
             scatter_tile_size=self._tunable_config["scatter_tile_size"],
             allow_shortcut_matmul=self._allow_shortcut_matmul,

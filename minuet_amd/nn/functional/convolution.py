@@ -5,6 +5,7 @@ from typing import Optional
 import torch
 
 from . import _C
+from ..kernel_map import KernelMap
 
 __all__ = ["cuda_time_gather", "cuda_time_scatter", "sparse_convolution_forward",
            "cuda_time_gemm", "set_gemm_parallel_level", "Epilogue", "pack_weights",
@@ -78,56 +79,67 @@ def cuda_time_gemm(weights: torch.Tensor, source_masks: torch.Tensor,
 
 
 def sparse_convolution_forward(sources: torch.Tensor, weights: torch.Tensor,
-                               source_masks: torch.Tensor, target_masks: torch.Tensor,
-                               kernel_map_order: Optional[torch.Tensor],
-                               kernel_map_sizes: torch.Tensor, gather_tile_size: int,
-                               scatter_tile_size: int, allow_shortcut_matmul: bool = False,
+                               source_masks: Optional[torch.Tensor] = None,
+                               target_masks: Optional[torch.Tensor] = None,
+                               kernel_map_order: Optional[torch.Tensor] = None,
+                               kernel_map_sizes: Optional[torch.Tensor] = None,
+                               gather_tile_size: int = 0, scatter_tile_size: int = 0,
+                               allow_shortcut_matmul: bool = False,
                                parallel: Optional[int] = None,
                                threshold: Optional[float] = 0,
                                epilogue: Optional[_C.Epilogue] = None,
                                dataflow: str = "auto",
-                               packed_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Output features ``[N_out, C_out]`` of one sparse convolution given the rank
-    tables of its kernel map (reference: convolution.py:110-155).  A host copy
-    of the sizes attached to ``kernel_map_sizes`` as attribute ``host_sizes``
-    (``KernelMapCache`` does that) avoids a device read-back per call; an int32
-    tensor attached to ``source_masks`` as attribute ``gather_index`` (the
-    source row of every buffer row, also from ``KernelMapCache``) lets the GEMM
-    read the source rows directly instead of going through a gather buffer.
-    ``epilogue`` (:class:`Epilogue`) is applied to each output row inside
-    Scatter, before the row is rounded to the feature dtype.
+                               packed_weights: Optional[torch.Tensor] = None,
+                               kernel_map=None) -> torch.Tensor:
+    """Output features ``[N_out, C_out]`` of one sparse convolution
+    (reference: convolution.py:110-155).
 
-    ``dataflow`` chooses between the reference's Gather -> GEMM -> Scatter
-    (``"gather_gemm_scatter"``) and the single-kernel output-stationary form
-    (``"implicit"``), which needs the dense kernel map attached to
-    ``target_masks`` as attribute ``kernel_map`` (``KernelMapCache`` does that)
-    and ``weights`` in their original offset order, as a layer holds them.
+    The kernel map comes either as the reference's four tensors
+    (``source_masks``, ``target_masks``, ``kernel_map_order``,
+    ``kernel_map_sizes``; a 4-tuple from ``KernelMapCache.get_kernel_map``
+    unpacks into them) or as ``kernel_map=`` a :class:`~minuet_amd.nn.KernelMap`,
+    which is what ``KernelMapCache.get_kernel_map`` returns.  With the four
+    tensors alone the call behaves like the reference: Gather, grouped GEMM and
+    Scatter as separate kernels, and the sizes are read back from the device
+    once per call.  A ``KernelMap`` carries host copies of sizes and order, the
+    pair lists and the dense map, with which nothing is read back, the Gather
+    is folded into the GEMM's operand load and ``dataflow`` has a choice:
+
+    ``"gather_gemm_scatter"`` is the reference's dataflow, ``"implicit"`` the
+    single-kernel output-stationary form (needs ``kernel_map.dense`` and
+    ``weights`` in their original offset order, as a layer holds them) and
     ``"auto"`` takes the implicit form where it is the faster one: 16-bit
     features whose rows it can stage, and small fp32 layers with 2^D kernels.
 
-    ``packed_weights`` (``pack_weights(weights)``, kept by the caller while the
-    weights are unchanged) spares the packing pass that otherwise starts every
-    call; with a ``kernel_map_order`` it also needs that tensor's host copy as
-    attribute ``host_order`` (from ``KernelMapCache``) and is ignored without."""
+    ``epilogue`` (:class:`Epilogue`) is applied to each output row before it is
+    rounded to the feature dtype.  ``packed_weights`` (``pack_weights(weights)``,
+    kept by the caller while the weights are unchanged) spares the packing pass
+    that otherwise starts every call; it needs a ``KernelMap`` when the map is
+    reordered (the host copy of the order) and is ignored without."""
     if not sources.is_cuda:
         raise NotImplementedError
     if dataflow not in DATAFLOWS:
         raise ValueError(f"dataflow must be one of {DATAFLOWS}")
-    dense = getattr(target_masks, "kernel_map", None)
+    if kernel_map is None and isinstance(source_masks, KernelMap):
+        kernel_map, source_masks = source_masks, None
+    host_sizes = host_order = gather_index = dense = None
+    if kernel_map is not None:
+        source_masks, target_masks, kernel_map_order, kernel_map_sizes = kernel_map
+        host_sizes, host_order = kernel_map.sizes_host, kernel_map.order_host
+        gather_index = kernel_map.in_idx if host_sizes is not None else None
+        dense = kernel_map.dense
     if dataflow == "implicit" and dense is None:
-        raise ValueError("the implicit dataflow needs target_masks.kernel_map (the dense kernel map)")
+        raise ValueError("the implicit dataflow needs a KernelMap with its dense map")
     if dense is not None and dataflow != "gather_gemm_scatter":
         if dataflow == "implicit" or prefers_implicit(weights.shape[0], weights.shape[1],
                                                       weights.shape[2], weights.dtype):
             return _C.sparse_convolution_forward_implicit(sources, weights, dense, epilogue=epilogue,
                                                           packed_weights=packed_weights)
+    if source_masks is None or target_masks is None or kernel_map_sizes is None:
+        raise ValueError("the Gather-GEMM-Scatter dataflow needs the rank tables and sizes of the kernel map")
     if parallel is None:
         parallel = GEMM_PARALLEL_LEVEL
-    host_sizes = getattr(kernel_map_sizes, "host_sizes", None)
-    gather_index = getattr(source_masks, "gather_index", None) if host_sizes is not None else None
-    host_order = None
     if kernel_map_order is not None:
-        host_order = getattr(kernel_map_order, "host_order", None)
         if host_order is None:
             packed_weights = None
         kernel_map_order = kernel_map_order.contiguous()

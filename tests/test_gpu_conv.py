@@ -47,24 +47,18 @@ def make_layer_case(seed, n, extent, kernel, cin, cout, kind, stride=1, batched=
     return src, sbd, tgt, tbd, off, feats, weights
 
 
-def with_host_sizes(sizes):
-    tensor = dev(sizes)
-    tensor.host_sizes = tuple(int(v) for v in sizes)
-    return tensor
-
-
-def with_gather_index(source_masks, sizes):
-    """Rank table on the device carrying its inverse (buffer row -> source row),
-    derived here from the table itself."""
+def kernel_map_of(source_masks, target_masks, order, sizes):
+    """A KernelMap on the device from the oracle's tables: host copies of sizes
+    and order plus the pair list of source rows (buffer row -> source row),
+    derived here from the rank table itself."""
     start = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
     index = np.full(int(start[-1]), -1, dtype=np.int32)
     for j in range(source_masks.shape[0]):
         hit = np.nonzero(source_masks[j] >= 0)[0]
         index[start[j] + source_masks[j, hit]] = hit
     assert (index >= 0).all()
-    tensor = dev(source_masks)
-    tensor.gather_index = dev(index)
-    return tensor
+    return minuet.nn.KernelMap(dev(source_masks), dev(target_masks), dev(order), dev(sizes),
+                               sizes_host=sizes, order_host=order, in_idx=dev(index))
 
 
 @pytest.mark.parametrize("kind", ["fp32", "fp16", "bf16"])
@@ -88,21 +82,16 @@ def test_forward_functional(kind, kernel, stride, cin, cout, n, extent):
             assert out.dtype == dtype and out.shape == (tgt.shape[0], cout)
             assert_features_close(out, ref, kind)
             # Gather folded into the GEMM: same products, same summation order
+            kernel_map = kernel_map_of(esm, etm, eorder, esizes)
             fused = F.sparse_convolution_forward(
-                sources=dev(feats).to(dtype), weights=dev(weights).to(dtype),
-                source_masks=with_gather_index(esm, esizes), target_masks=dev(etm),
-                kernel_map_order=dev(eorder), kernel_map_sizes=with_host_sizes(esizes),
+                sources=dev(feats).to(dtype), weights=dev(weights).to(dtype), kernel_map=kernel_map,
                 gather_tile_size=0, scatter_tile_size=0,
                 allow_shortcut_matmul=shortcut and stride == 1, threshold=threshold)
             assert torch.equal(fused, out)
             # weights packed ahead of time (in the layer's own offset order)
-            order_dev = dev(eorder)
-            order_dev.host_order = tuple(int(v) for v in eorder)
             w_dev = dev(weights).to(dtype)
             ahead = F.sparse_convolution_forward(
-                sources=dev(feats).to(dtype), weights=w_dev,
-                source_masks=with_gather_index(esm, esizes), target_masks=dev(etm),
-                kernel_map_order=order_dev, kernel_map_sizes=with_host_sizes(esizes),
+                sources=dev(feats).to(dtype), weights=w_dev, kernel_map=kernel_map,
                 gather_tile_size=0, scatter_tile_size=0,
                 allow_shortcut_matmul=shortcut and stride == 1, threshold=threshold,
                 packed_weights=F.pack_weights(w_dev))
@@ -561,12 +550,9 @@ def test_forward_implicit_two_target_blocks_per_wavefront(kind, cin, cout):
     scale = dev(rng.uniform(0.5, 1.5, size=cout).astype(np.float32))
     shift = dev(rng.uniform(-0.5, 0.5, size=cout).astype(np.float32))
     residual = torch.from_numpy(rng.normal(size=(n, cout))).to(dtype).cuda()
-    sizes = built["sizes"]
-    sizes.host_sizes = built["sizes_host"]
-    order = built["order"]
-    order.host_order = built["order_host"]
-    source_masks = built["source_masks"]
-    source_masks.gather_index = built["in_idx"]
+    kernel_map = minuet.nn.KernelMap(built["source_masks"], built["target_masks"], built["order"],
+                                     built["sizes"], sizes_host=built["sizes_host"],
+                                     order_host=built["order_host"], in_idx=built["in_idx"])
     sample = rng.choice(n, size=1500, replace=False)
     sample[:3] = (0, n - 1, n - 2)                       # the ragged last tile is in the sample
     # the sampled rows of the kernel map, checked against a search over packed keys
@@ -592,11 +578,49 @@ def test_forward_implicit_two_target_blocks_per_wavefront(kind, cin, cout):
         assert out.shape == (n, cout) and torch.isfinite(out).all()
         assert_features_close(out[sample], ref, kind)
         three = F.sparse_convolution_forward(
-            sources=feats, weights=weights, source_masks=source_masks, target_masks=built["target_masks"],
-            kernel_map_order=order, kernel_map_sizes=sizes, gather_tile_size=0, scatter_tile_size=0,
+            sources=feats, weights=weights, kernel_map=kernel_map, gather_tile_size=0, scatter_tile_size=0,
             allow_shortcut_matmul=True, threshold=-1, epilogue=epilogue, dataflow="gather_gemm_scatter")
         # two roundings of the same sums: 2e-2 of the RMS, or one unit in the
         # last place of the largest value where that is more (bf16 keeps 8 bits)
         diff = (out.float() - three.float()).abs().max().item()
         ulp = three.float().abs().max().item() * 2.0 ** (-7 if kind == "bf16" else -10)
         assert diff <= max(2e-2 * three.float().pow(2).mean().sqrt().item(), ulp), diff
+
+
+def test_kernel_map_object_is_the_fast_path(monkeypatch):
+    """KernelMapCache returns a KernelMap that unpacks like the reference's
+    4-tuple; handing it to F.sparse_convolution_forward keeps the pass free of
+    read-backs and separate gathers whatever happened to the tables themselves
+    (clones, casts), while the four bare tensors run the reference's way."""
+    src, sbd, tgt, tbd, off, feats, weights = make_layer_case(5, 4000, 18, 3, 32, 32, "fp32")
+    cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+    c = dev(src)
+    kernel_map = cache.get_kernel_map(c, 1, None, c, 1, None, 3, 1)
+    assert isinstance(kernel_map, minuet.nn.KernelMap) and len(kernel_map) == 4
+    source_masks, target_masks, order, sizes = kernel_map                  # the reference's tuple
+    assert kernel_map.nnz == int(host(sizes).sum()) and kernel_map.num_offsets == 27
+    assert kernel_map.in_idx.numel() == kernel_map.nnz and kernel_map.dense.shape == (27, src.shape[0])
+    seen = []
+    real = _C.cuda_sparse_convolution_forward
+
+    def spy(*args, **kwargs):
+        seen.append((kwargs.get("kernel_map_sizes_host") is not None, kwargs.get("gather_index") is not None))
+        return real(*args, **kwargs)
+
+    monkeypatch.setattr(_C, "cuda_sparse_convolution_forward", spy)
+    f, w = dev(feats).float(), dev(weights).float()
+    common = dict(gather_tile_size=0, scatter_tile_size=0, allow_shortcut_matmul=True, threshold=-1,
+                  dataflow="gather_gemm_scatter")
+    a = F.sparse_convolution_forward(f, w, kernel_map=kernel_map, **common)
+    cloned = kernel_map.with_tables(source_masks.clone(), target_masks.clone().contiguous())
+    b = F.sparse_convolution_forward(f, w, kernel_map=cloned, **common)
+    bare = F.sparse_convolution_forward(f, w, source_masks.clone(), target_masks.clone(), order, sizes, 0, 0,
+                                        allow_shortcut_matmul=True, threshold=-1, dataflow="gather_gemm_scatter")
+    positional = F.sparse_convolution_forward(f, w, *kernel_map, 0, 0, allow_shortcut_matmul=True, threshold=-1,
+                                              dataflow="gather_gemm_scatter")
+    assert seen == [(True, True), (True, True), (False, False), (False, False)]
+    assert torch.equal(a, b) and torch.equal(a, bare) and torch.equal(a, positional)
+    esm, etm, eorder, esizes, _ = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=True)
+    assert_features_close(a, orc.sparse_convolution_forward(feats, weights, esm, etm, eorder, esizes), "fp32")
+    with pytest.raises(ValueError, match="dense"):
+        F.sparse_convolution_forward(f, w, source_masks, target_masks, order, sizes, 0, 0, dataflow="implicit")
