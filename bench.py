@@ -183,7 +183,7 @@ def layer_stages(device, config, channels, kernel_size, dtype_name, tune=False):
                                       # rows in and out of the buffers: what bounds it at small widths
                                       **{"hbm_" + k: v for k, v in hbm(2 * nnz * channels * esize, gemm_ms).items()
                                          if k != "ms"}}
-        for flow in ("gather_gemm_scatter", "implicit"):
+        for flow in ("gather_gemm_scatter", "list_driven", "implicit"):
             if flow == "implicit" and not _C.implicit_forward_supported(channels, channels, dtype):
                 continue
             conv.tunable_config["dataflow"] = flow

@@ -286,6 +286,20 @@ int mnt_sorted_kernel_map_lists(const void *coords, int64_t n, int ndim, int coo
                                 int64_t *bounds_host_out, int64_t *sizes_host_out,
                                 int64_t *order_host_out, void *stream);
 
+/* Target-major row lists of a kernel map whose pair lists exist, from its dense
+ * int32 map kernel_map[O, T] (original offset order): row_ptr_out[T + 1] and
+ * out_pos_out[nnz] such that the product of list entry p (list row j in the
+ * order order_host[j] -> offset, NULL = offset order, sizes_host[j] hits each,
+ * hits in target order: the numbering of in_idx / out_idx) belongs at buffer
+ * row out_pos_out[p] and target t owns the consecutive buffer rows
+ * row_ptr_out[t] .. row_ptr_out[t + 1] - 1, in list-row order.  Feeds
+ * mnt_sparse_convolution_forward_rows.  Does not wait for the device.  At most
+ * 1024 offsets.  Takes the place of the rank table target_masks
+ * (csrc/minuet/cuda/functions/scan.cu:292-365) as what Scatter is driven by. */
+int mnt_kernel_map_row_lists(const int32_t *kernel_map, int64_t num_offsets, int64_t num_targets,
+                             const int64_t *sizes_host, const int64_t *order_host,
+                             int32_t *row_ptr_out, int32_t *out_pos_out, void *stream);
+
 /* Per-offset (in_idx, out_idx) pair lists from a dense int32 kernel map: for row
  * o the hits in target order are written at list positions
  * cumsum_host[o] .. cumsum_host[o]+sizes[o]-1 (cumsum_host[O+1], HOST, exclusive
@@ -402,6 +416,32 @@ int mnt_sparse_convolution_forward_fused(int64_t gather_tile, int64_t scatter_ti
                                          const void *packed_weights,
                                          const int64_t *order_host,
                                          void *out, void *stream);
+
+/* The same convolution driven by lists instead of rank tables: the grouped GEMM
+ * reads the source row of list entry p through in_idx[p] (Gather folded into
+ * its operand load) and writes the product to buffer row out_pos[p]; Scatter
+ * then sums, for target t, the CONSECUTIVE buffer rows row_ptr[t] ..
+ * row_ptr[t + 1] - 1 in fp32 and applies the epilogue: no rank table and no
+ * row list is read, the buffer streams through once.  in_idx: the list of
+ * mnt_kernel_map_emit / _lists; out_pos, row_ptr: mnt_kernel_map_row_lists;
+ * sizes_host / order_host (int64[O], order_host NULL = offset order) as those
+ * calls return them; weights [O, Cin, Cout] in the layer's own offset order,
+ * packed_weights (nullable) their mnt_pack_weights form.  Rows are summed in
+ * list-row order, the centre offset with the others (the reference adds it
+ * last as well, sparse_convolution.cu:647-660), so results agree with
+ * mnt_sparse_convolution_forward to rounding.  Epilogue arguments as in
+ * mnt_sparse_convolution_forward_fused.  Same reference code
+ * (csrc/minuet/cuda/functions/sparse_convolution.cu:504-661). */
+int mnt_sparse_convolution_forward_rows(int64_t scatter_tile, const void *sources,
+                                        const void *weights, const int64_t *sizes_host,
+                                        const int64_t *order_host, const int32_t *in_idx,
+                                        const int32_t *out_pos, const int32_t *row_ptr,
+                                        int64_t num_sources, int64_t num_targets,
+                                        int64_t num_offsets, int64_t num_source_features,
+                                        int64_t num_target_features, int float_dtype,
+                                        const float *channel_scale, const float *channel_shift,
+                                        const void *residual, int activation, float negative_slope,
+                                        const void *packed_weights, void *out, void *stream);
 
 /* Weights [O, Cin, Cout] -> the layout the matrix kernels stage:
  * packed[O][Np][Kp] = W^T per offset, K-contiguous, zero-padded to

@@ -383,6 +383,70 @@ __global__ __launch_bounds__(kScatterBlock) void scatter_kernel(
   }
 }
 
+// Scatter of the list-driven dataflow: the GEMM has written its products in
+// target-major order, so target t sums the CONSECUTIVE buffer rows
+// row_ptr[t] .. row_ptr[t + 1] - 1 (in the order of the kernel map's rows, the
+// centre offset last, which is the reference's order of summation,
+// sparse_convolution.cu:642-660) and no rank table or row list is read: the
+// buffer streams through once.  One lane group per target, `tile` targets per
+// workgroup.
+template <typename TB, typename T, int VB, int NV>
+__global__ __launch_bounds__(kScatterBlock) void scatter_rows_kernel(
+    const TB *__restrict__ buffer, unsigned char *__restrict__ targets, const int *__restrict__ row_ptr,
+    long long num_targets, int channels, int lanes_per_row, int tile, Epilogue ep) {
+  typedef typename VecOf<VB>::type V;
+  constexpr int E = VB / static_cast<int>(sizeof(T));
+  constexpr int BB = E * static_cast<int>(sizeof(TB));          // buffer bytes per vector
+  typedef typename VecOf<(BB > 16 ? 16 : BB)>::type BV;
+  constexpr int NBV = BB > 16 ? BB / 16 : 1;
+  constexpr int kRows = 4;                                       // rows in flight per lane group
+  const int tid = static_cast<int>(threadIdx.x);
+  const int groups = kScatterBlock / lanes_per_row;
+  const int group = tid / lanes_per_row;
+  const int lr = tid - group * lanes_per_row;
+  if (group >= groups) return;
+  const long long t0 = static_cast<long long>(blockIdx.x) * tile;
+  for (int tt = group; tt < tile; tt += groups) {
+    const long long t = t0 + tt;
+    if (t >= num_targets) break;
+    const int lo = row_ptr[t], hi = row_ptr[t + 1];
+    float acc[NV][E];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+#pragma unroll
+      for (int k = 0; k < E; ++k) acc[i][k] = 0.0f;
+    }
+    for (int k0 = lo; k0 < hi; k0 += kRows) {
+      BV raw[kRows][NV][NBV];
+#pragma unroll
+      for (int j = 0; j < kRows; ++j) {
+        if (k0 + j < hi) {
+          const TB *src = buffer + static_cast<long long>(k0 + j) * channels;
+#pragma unroll
+          for (int i = 0; i < NV; ++i) {
+            const TB *piece = src + (lr + i * lanes_per_row) * E;
+#pragma unroll
+            for (int v = 0; v < NBV; ++v) raw[j][i][v] = reinterpret_cast<const BV *>(piece)[v];
+          }
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kRows; ++j) {
+        if (k0 + j < hi) {
+#pragma unroll
+          for (int i = 0; i < NV; ++i) {
+            const TB *e = reinterpret_cast<const TB *>(raw[j][i]);
+#pragma unroll
+            for (int k = 0; k < E; ++k) acc[i][k] += to_float(e[k]);
+          }
+        }
+      }
+    }
+    unsigned char *dst = targets + t * channels * static_cast<long long>(sizeof(T));
+    finish_row<T, V, E, NV>(acc, ep, t, channels, lr, lanes_per_row, dst);
+  }
+}
+
 // Element type of the GEMM-output / scatter-input buffer for feature type T.
 // bfloat16 keeps only 8 significant bits, so rounding every partial product
 // to it would cost more accuracy than the output rounding itself.
@@ -420,7 +484,11 @@ constexpr int kMaxChannelBlocks = 4;    // 32-channel blocks per workgroup (128 
 // data row i of group g is then row gather_index[list_start[g] + i] of `a`
 // (the source features) instead of buffer row row_start[g] + i, and no gather
 // buffer exists; a group with list_start < 0 reads row i of `a` itself (the
-// centre offset of the shortcut).  The output rows stay in buffer order.
+// centre offset of the shortcut).  The output rows stay in buffer order,
+// unless `out_pos` (nullable, needs gather_index and no such centre group)
+// says where each goes: the product of list entry p = list_start[g] + i is
+// then written to buffer row out_pos[p] (the target-major layout that the
+// list-driven Scatter sums without an index).
 //
 // The tables reach the kernel either in device memory (grouped_gemm_kernel) or
 // as a by-value argument (grouped_gemm_riding_kernel: meta starts at entry
@@ -442,7 +510,8 @@ template <typename T, typename TC, int NB, bool VEC, int CH, typename Meta>
 __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *__restrict__ c,
                                                   const T *__restrict__ wt, const Meta &entry, int K,
                                                   int N, int Kp, int Np,
-                                                  const int *__restrict__ gather_index) {
+                                                  const int *__restrict__ gather_index,
+                                                  const int *__restrict__ out_pos) {
   constexpr int EPC = 16 / static_cast<int>(sizeof(T));        // elements per 16-byte piece
   constexpr int KC = kChunkBytes / static_cast<int>(sizeof(T));
   constexpr int TN = NB * 32;
@@ -509,6 +578,8 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
                           : (row_ok ? gather_index[static_cast<long long>(list_at) + r0 + row] : 0);
   }
   const T *a_row = a + a_index * K;
+  // where this tile's rows go, for the lists of the output pass (null: buffer order)
+  const int *pos_list = out_pos != nullptr ? out_pos + (static_cast<long long>(list_at) + r0) : nullptr;
 
   floatx16 acc[NB];
 #pragma unroll
@@ -624,6 +695,13 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
     constexpr int EPV = 16 / static_cast<int>(sizeof(TC));       // channels per 16-byte piece
     constexpr int kRowPieces = 32 / EPV;                          // pieces of a block's row
     constexpr int kPieces = 32 * kRowPieces / kWave;              // per lane and block
+    // buffer row of every row piece this lane will write
+    long long out_row[kPieces];
+#pragma unroll
+    for (int i = 0; i < kPieces; ++i) {
+      const int rr = wv * 32 + (lane + i * kWave) / kRowPieces;
+      out_row[i] = pos_list != nullptr ? (rr < valid ? static_cast<long long>(pos_list[rr]) : 0ll) : row_base + rr;
+    }
     __syncthreads();                                              // every product has read its weights
     unsigned char *turn = b_lds + wv * kTurnBytes;
 #pragma unroll
@@ -651,7 +729,7 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
         const int ch = n0 + b * 32 + part * EPV;
         const uint4 v = *reinterpret_cast<const uint4 *>(turn + pr * kTurnRow + part * 16);
         if (wv * 32 + pr < valid && ch < N) {                     // N % EPV == 0: a piece is all in or all out
-          *reinterpret_cast<uint4 *>(c + (row_base + wv * 32 + pr) * N + ch) = v;
+          *reinterpret_cast<uint4 *>(c + out_row[i] * N + ch) = v;
         }
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -659,7 +737,7 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
   } else if (row_ok) {
-    TC *dst = c + (row_base + row) * N;
+    TC *dst = c + (pos_list != nullptr ? static_cast<long long>(pos_list[row]) : row_base + row) * N;
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
 #pragma unroll
@@ -689,8 +767,8 @@ template <typename T, typename TC, int NB, bool VEC, int CH>
 __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
     const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt,
     const int *__restrict__ meta, int K, int N, int Kp, int Np,
-    const int *__restrict__ gather_index) {
-  grouped_gemm_body<T, TC, NB, VEC, CH>(a, c, wt, MetaInMemory{meta}, K, N, Kp, Np, gather_index);
+    const int *__restrict__ gather_index, const int *__restrict__ out_pos) {
+  grouped_gemm_body<T, TC, NB, VEC, CH>(a, c, wt, MetaInMemory{meta}, K, N, Kp, Np, gather_index, out_pos);
 }
 
 // The same with the tables as a by-value argument.
@@ -698,12 +776,12 @@ template <typename T, typename TC, int NB, bool VEC, int CH>
 __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_riding_kernel(
     const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt, int K, int N, int Kp, int Np,
     const int *__restrict__ gather_index, PlanChunk table, int table_count, int meta_at,
-    int *__restrict__ table_out) {
+    int *__restrict__ table_out, const int *__restrict__ out_pos) {
   if (blockIdx.x == 0 && blockIdx.y == 0) {
     for (int i = threadIdx.x; i < table_count; i += kGemmBlock) table_out[i] = table.v[i];
   }
   grouped_gemm_body<T, TC, NB, VEC, CH>(a, c, wt, MetaInArguments{&table, meta_at}, K, N, Kp, Np,
-                                        gather_index);
+                                        gather_index, out_pos);
 }
 
 // ---------------------------------------------------------- host launchers ----
@@ -849,7 +927,7 @@ struct RidingTable {
 template <typename T, typename TC, int NB>
 static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int num_tiles, int K, int N,
                            int Kp, int Np, bool vec, const int *gather_index, const RidingTable &riding,
-                           hipStream_t stream) {
+                           hipStream_t stream, const int *out_pos) {
   dim3 grid(num_tiles, static_cast<unsigned>(div_ceil(Np, NB * 32)));
   // rows of one or two chunks are loaded whole, ahead of the first product
   const int chunks = Kp / (kChunkBytes / static_cast<int>(sizeof(T)));
@@ -860,7 +938,7 @@ static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int 
     std::memcpy(chunk.v, riding.ints->data(), count * sizeof(int));
 #define MNT_RIDING(VEC, CH)                                                                 \
   grouped_gemm_riding_kernel<T, TC, NB, VEC, CH><<<grid, kGemmBlock, 0, stream>>>(          \
-      a, c, wt, K, N, Kp, Np, gather_index, chunk, count, riding.meta_at, riding.out)
+      a, c, wt, K, N, Kp, Np, gather_index, chunk, count, riding.meta_at, riding.out, out_pos)
     if (held == 1) {
       MNT_RIDING(true, 1);
     } else if (held == 2) {
@@ -874,7 +952,7 @@ static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int 
   } else {
 #define MNT_PLAIN(VEC, CH)                                                                  \
   grouped_gemm_kernel<T, TC, NB, VEC, CH><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np, \
-                                                                           gather_index)
+                                                                           gather_index, out_pos)
     if (held == 1) {
       MNT_PLAIN(true, 1);
     } else if (held == 2) {
@@ -891,7 +969,7 @@ static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int 
 template <typename T, typename TC>
 static void launch_gemm(const T *a, TC *c, const T *wt, const int *meta, int num_tiles, int K, int N,
                         int Kp, int Np, const int *gather_index, hipStream_t stream,
-                        const RidingTable &riding = RidingTable()) {
+                        const RidingTable &riding = RidingTable(), const int *out_pos = nullptr) {
   if (num_tiles == 0) return;
   const bool vec = (static_cast<int64_t>(K) * sizeof(T)) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(a) % 16 == 0 && N % 4 == 0 &&
@@ -903,10 +981,10 @@ static void launch_gemm(const T *a, TC *c, const T *wt, const int *meta, int num
   const int blocks = Np / 32;
   const int slices = static_cast<int>(div_ceil(blocks, kMaxChannelBlocks));
   switch (static_cast<int>(div_ceil(blocks, slices))) {
-    case 1: launch_gemm_nb<T, TC, 1>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream); break;
-    case 2: launch_gemm_nb<T, TC, 2>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream); break;
-    case 3: launch_gemm_nb<T, TC, 3>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream); break;
-    default: launch_gemm_nb<T, TC, 4>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream); break;
+    case 1: launch_gemm_nb<T, TC, 1>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream, out_pos); break;
+    case 2: launch_gemm_nb<T, TC, 2>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream, out_pos); break;
+    case 3: launch_gemm_nb<T, TC, 3>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream, out_pos); break;
+    default: launch_gemm_nb<T, TC, 4>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream, out_pos); break;
   }
   check_launch("grouped_gemm_kernel");
 }
@@ -1119,6 +1197,112 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
   profile_mark("scatter", stream);
 }
 
+template <typename TB, typename T>
+static void launch_scatter_rows(const LaneShape &sh, const TB *buffer, void *targets, const int *row_ptr,
+                                int64_t num_targets, int channels, const Epilogue &ep, hipStream_t stream) {
+  if (num_targets == 0) return;
+  MNT_CHECK(sh.lanes_per_row <= kScatterBlock, "feature rows of %d lanes do not fit a workgroup", sh.lanes_per_row);
+  const int groups = std::max(1, kScatterBlock / sh.lanes_per_row);
+  int tile = 64;
+  while (tile > 8 && num_targets / tile < 2048 && tile / 2 >= groups) tile /= 2;
+  tile = std::max(tile, groups);
+  const unsigned grid = static_cast<unsigned>(div_ceil(num_targets, tile));
+#define MNT_S(VB, NV)                                                                     \
+  scatter_rows_kernel<TB, T, VB, NV><<<grid, kScatterBlock, 0, stream>>>(                 \
+      buffer, static_cast<unsigned char *>(targets), row_ptr, num_targets, channels, sh.lanes_per_row, tile, ep)
+#define MNT_SV(VB)                 \
+  switch (sh.nv) {                 \
+    case 1: MNT_S(VB, 1); break;   \
+    case 2: MNT_S(VB, 2); break;   \
+    case 4: MNT_S(VB, 4); break;   \
+    default: MNT_S(VB, 8); break;  \
+  }
+  if (sh.vb == 16) {
+    MNT_SV(16);
+  } else if (sh.vb == 8) {
+    MNT_SV(8);
+  } else if (sh.vb == 4) {
+    MNT_SV(4);
+  } else {
+    if constexpr (sizeof(T) == 2) {
+      MNT_SV(2);
+    } else {
+      MNT_FAIL("feature rows are not aligned to their element size");
+    }
+  }
+#undef MNT_SV
+#undef MNT_S
+  check_launch("scatter_rows_kernel");
+}
+
+// Forward pass of the list-driven dataflow: grouped GEMM reading its rows through
+// in_idx and writing them to out_pos, then the streaming Scatter.
+template <typename T>
+static void forward_rows_typed(int64_t scatter_tile, const ForwardPlan &plan, const T *sources,
+                               const T *weights, const int *in_idx, const int *out_pos,
+                               const int *row_ptr, const Epilogue &epilogue, const T *packed,
+                               const int64_t *order_host, int64_t S, int64_t Tn, int64_t O, int64_t K,
+                               int64_t N, T *out, hipStream_t stream) {
+  Scope scope(stream);
+  const int kc = kChunkBytes / static_cast<int>(sizeof(T));
+  const int Kp = static_cast<int>(div_ceil(K, kc) * kc);
+  const int Np = static_cast<int>(div_ceil(N, 32) * 32);
+  profile_mark("enter:forward", stream);
+  // every group points at the matrix of the offset its row stands for (the
+  // weights are packed in the layer's own offset order)
+  std::vector<int> meta(plan.meta);
+  {
+    const int G = meta[0];
+    int *weight = meta.data() + 1 + (G + 1) + (G + 1) + G;
+    if (order_host != nullptr) {
+      for (int i = 0; i < G; ++i) weight[i] = static_cast<int>(order_host[weight[i]]);
+    }
+  }
+  std::vector<int> ints(plan.row_start);
+  const size_t meta_at = ints.size();
+  ints.insert(ints.end(), meta.begin(), meta.end());
+  int *d_ints = scope.alloc<int>(ints.size());
+  int *d_meta = d_ints + meta_at;
+  const bool fits = ints.size() <= static_cast<size_t>(kPlanInts);
+  RidingTable riding;
+  const T *wt = packed;
+  if (packed != nullptr) {
+    if (fits && plan.num_tiles > 0 && plan.num_tiles <= kRidingMaxTiles) {
+      riding.ints = &ints;
+      riding.meta_at = static_cast<int>(meta_at);
+      riding.out = d_ints;
+    } else {
+      upload_ints(ints, d_ints, stream);
+    }
+  } else {
+    T *fresh = scope.alloc<T>(static_cast<size_t>(O) * Np * Kp);
+    wt = fresh;
+    PlanChunk chunk;
+    int count = 0;
+    if (fits) {
+      count = static_cast<int>(ints.size());
+      std::memcpy(chunk.v, ints.data(), ints.size() * sizeof(int));
+    } else {
+      upload_ints(ints, d_ints, stream);
+    }
+    const long long total = static_cast<long long>(O) * Np * Kp;
+    pack_weights_kernel<T, int32_t><<<grid_for(total, 256, 4096), 256, 0, stream>>>(
+        weights, nullptr, static_cast<int>(O), static_cast<int>(K), static_cast<int>(N), Kp, Np, fresh, chunk,
+        count, d_ints);
+    check_launch("pack_weights_kernel");
+  }
+  profile_mark("pack_weights", stream);
+  typedef typename BufferOf<T>::type TB;
+  const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
+  TB *cbuf = scope.alloc<TB>(rows * N);
+  launch_gemm<T, TB>(sources, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np,
+                     in_idx, stream, riding, out_pos);
+  profile_mark("gemm", stream);
+  const LaneShape ssh = lane_shape(scatter_tile, N, sizeof(T), cbuf, out, "num_target_features");
+  launch_scatter_rows<TB, T>(ssh, cbuf, out, row_ptr, Tn, static_cast<int>(N), epilogue, stream);
+  profile_mark("scatter", stream);
+}
+
 }  // namespace mnt
 
 using namespace mnt;
@@ -1232,6 +1416,59 @@ extern "C" int mnt_sparse_convolution_forward(
       weights, source_masks, target_masks, kernel_map_order, kernel_map_sizes, sizes_host, S, T, O, K,
       N, index_dtype, float_dtype, gather_index, nullptr, nullptr, nullptr, MNT_ACT_NONE, 0.0f, nullptr,
       nullptr, out, stream_);
+}
+
+extern "C" int mnt_sparse_convolution_forward_rows(
+    int64_t scatter_tile, const void *sources, const void *weights, const int64_t *sizes_host,
+    const int64_t *order_host, const int32_t *in_idx, const int32_t *out_pos, const int32_t *row_ptr,
+    int64_t S, int64_t T, int64_t O, int64_t K, int64_t N, int float_dtype, const float *channel_scale,
+    const float *channel_shift, const void *residual, int activation, float negative_slope,
+    const void *packed_weights, void *out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    float_size(float_dtype);
+    MNT_CHECK(S >= 0 && T >= 0 && O >= 0 && K >= 1 && N >= 1 && S <= INT32_MAX && T <= INT32_MAX &&
+                  O <= 65535 && K <= 65536 && N <= 65536,
+              "bad shape S=%lld T=%lld O=%lld Cin=%lld Cout=%lld", (long long)S, (long long)T,
+              (long long)O, (long long)K, (long long)N);
+    MNT_CHECK(activation >= MNT_ACT_NONE && activation <= MNT_ACT_RELU6, "unknown activation code %d",
+              activation);
+    MNT_CHECK(reinterpret_cast<uintptr_t>(residual) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(channel_scale) % 4 == 0 &&
+                  reinterpret_cast<uintptr_t>(channel_shift) % 4 == 0,
+              "epilogue operands are not aligned (residual: 16 bytes, scale / shift: 4 bytes)");
+    MNT_CHECK(reinterpret_cast<uintptr_t>(packed_weights) % 16 == 0, "packed weights are not 16-byte aligned");
+    MNT_CHECK(sizes_host != nullptr, "sizes_host is null");
+    if (T == 0) return;
+    MNT_CHECK(out != nullptr && row_ptr != nullptr, "null argument");
+    int64_t nnz = 0;
+    for (int64_t j = 0; j < O; ++j) {
+      MNT_CHECK(sizes_host[j] >= 0 && sizes_host[j] <= T, "kernel map size %lld of offset %lld is out of range",
+                (long long)sizes_host[j], (long long)j);
+      MNT_CHECK(order_host == nullptr || (order_host[j] >= 0 && order_host[j] < O),
+                "order_host[%lld] is out of range", (long long)j);
+      nnz += sizes_host[j];
+    }
+    MNT_CHECK(nnz == 0 || (in_idx != nullptr && out_pos != nullptr), "the pair lists are missing");
+    MNT_CHECK(nnz == 0 || (sources != nullptr && weights != nullptr), "null operand");
+    // no padding and no shortcut: buffer rows are list positions
+    ForwardPlan plan = make_forward_plan(sizes_host, O, S, T, false, true, -1.0);
+    MNT_CHECK(plan.total_rows == nnz, "the forward plan does not match the pair lists");
+    const Epilogue epilogue = {channel_scale, channel_shift, residual, activation, negative_slope};
+#define MNT_ROWS(FT)                                                                                  \
+  forward_rows_typed<FT>(scatter_tile, plan, static_cast<const FT *>(sources),                        \
+                         static_cast<const FT *>(weights), in_idx, out_pos, row_ptr, epilogue,         \
+                         static_cast<const FT *>(packed_weights), order_host, S, T, O, K, N,           \
+                         static_cast<FT *>(out), stream)
+    if (float_dtype == MNT_FLOAT32) {
+      MNT_ROWS(float);
+    } else if (float_dtype == MNT_FLOAT16) {
+      MNT_ROWS(half_t);
+    } else {
+      MNT_ROWS(bf16_t);
+    }
+#undef MNT_ROWS
+  });
 }
 
 extern "C" int mnt_pack_weights(const void *weights, int64_t O, int64_t K, int64_t N, int float_dtype,

@@ -874,6 +874,95 @@ __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
   }
 }
 
+// Target-major row lists of a kernel map, for the list-driven Scatter.  The
+// pair lists number the hits row by row (list position p = row prefix + rank
+// of the target among the row's hits); here every target gets the run
+// row_ptr[t] .. row_ptr[t + 1] - 1 of a second numbering, by target first and
+// by row (in list order) second, and out_pos[p] says where hit p sits in it.
+// One workgroup per tile of 512 targets, one target per lane:
+//   1. every wavefront ballots its 64 targets against each offset's row of the
+//      dense map and leaves the ballots in LDS; a lane counts its own hits;
+//   2. the counts are scanned (row_ptr) and the ballots of an offset turned
+//      into the rank of each wavefront's first hit;
+//   3. every lane walks the rows in list order and numbers its hits.
+// tables: order[O] (list row j -> offset), list_start[O] (first list position
+// of row j).  tile_bases: exclusive per-offset scan of the per-tile hit counts.
+// Dynamic LDS: O * (64 + 32 + 4) bytes + 64.
+__global__ __launch_bounds__(kQueryThreads) void row_lists_kernel(
+    const int *__restrict__ kernel_map, long long num_targets, int num_offsets,
+    const unsigned *__restrict__ tile_bases, int num_tiles, const int *__restrict__ tables,
+    int *__restrict__ row_ptr, int *__restrict__ out_pos) {
+  extern __shared__ __align__(16) unsigned char s_rows[];
+  constexpr int kWaves = kQueryThreads / kWave;
+  unsigned long long *s_ballot = reinterpret_cast<unsigned long long *>(s_rows);            // [O][waves]
+  unsigned *s_first = reinterpret_cast<unsigned *>(s_ballot + static_cast<size_t>(num_offsets) * kWaves);  // [O][waves]
+  unsigned *s_base = s_first + static_cast<size_t>(num_offsets) * kWaves;                   // [O], by list row
+  unsigned *s_wave = s_base + num_offsets;                                                  // [waves + 2]
+  const int tid = threadIdx.x;
+  const int lane = lane_id();
+  const int w = tid >> 6;
+  const int tile = blockIdx.x;
+  const long long t = static_cast<long long>(tile) * kTargetsPerTile + tid;
+  const bool valid = t < num_targets;
+  const int *order = tables;
+  const int *list_start = tables + num_offsets;
+  if (tid == 0) s_wave[kWaves] = 0;
+  __syncthreads();
+  unsigned count = 0;
+  for (int o = 0; o < num_offsets; ++o) {
+    const bool hit = valid && kernel_map[static_cast<long long>(o) * num_targets + t] != -1;
+    const unsigned long long votes = __builtin_amdgcn_ballot_w64(hit);
+    if (lane == 0) s_ballot[o * kWaves + w] = votes;
+    count += hit ? 1u : 0u;
+  }
+  // hits of this tile before each target, and of all tiles before this one
+  unsigned inclusive = count;
+  for (int off = 1; off < kWave; off <<= 1) {
+    const unsigned u = __shfl_up(inclusive, off);
+    if (lane >= off) inclusive += u;
+  }
+  if (lane == kWave - 1) s_wave[w] = inclusive;
+  unsigned earlier = 0;
+  for (int o = tid; o < num_offsets; o += kQueryThreads) {
+    earlier += tile_bases[static_cast<long long>(o) * num_tiles + tile];
+  }
+  for (int off = 32; off > 0; off >>= 1) earlier += __shfl_xor(earlier, off);
+  if (lane == 0 && earlier != 0) atomicAdd(&s_wave[kWaves], earlier);
+  __syncthreads();
+  for (int j = tid; j < num_offsets; j += kQueryThreads) {
+    // list row j: the rank of each wavefront's first hit, and the list position of the tile's first
+    const int o = order[j];
+    unsigned run = 0;
+#pragma unroll
+    for (int ww = 0; ww < kWaves; ++ww) {
+      s_first[o * kWaves + ww] = run;
+      run += __popcll(s_ballot[o * kWaves + ww]);
+    }
+    s_base[j] = static_cast<unsigned>(list_start[j]) + tile_bases[static_cast<long long>(o) * num_tiles + tile];
+  }
+  unsigned before = s_wave[kWaves];
+  unsigned tile_hits = 0;
+#pragma unroll
+  for (int ww = 0; ww < kWaves; ++ww) {
+    before += ww < w ? s_wave[ww] : 0u;
+    tile_hits += s_wave[ww];
+  }
+  unsigned at = before + inclusive - count;
+  if (valid) row_ptr[t] = static_cast<int>(at);
+  if (t == num_targets - 1) row_ptr[num_targets] = static_cast<int>(s_wave[kWaves] + tile_hits);
+  __syncthreads();
+  const unsigned long long below = lanes_below();
+  for (int j = 0; j < num_offsets; ++j) {
+    const int o = order[j];
+    const unsigned long long votes = s_ballot[o * kWaves + w];
+    if ((votes >> lane) & 1ull) {
+      const unsigned p = s_base[j] + s_first[o * kWaves + w] + __popcll(votes & below);
+      out_pos[p] = static_cast<int>(at);
+      ++at;
+    }
+  }
+}
+
 template <typename IT>
 __global__ __launch_bounds__(256) void export_sizes_kernel(const unsigned *__restrict__ sizes,
                                                            int n, IT *__restrict__ out) {
@@ -1617,6 +1706,53 @@ extern "C" int mnt_sorted_kernel_map_lists(const void *coords, int64_t n, int nd
                              sizes_dev_out, order_dev_out, sizes_host_out, order_host_out, stream_) != 0) {
       throw Error{mnt_last_error()};
     }
+  });
+}
+
+extern "C" int mnt_kernel_map_row_lists(const int32_t *kernel_map, int64_t num_offsets,
+                                        int64_t num_targets, const int64_t *sizes_host,
+                                        const int64_t *order_host, int32_t *row_ptr_out,
+                                        int32_t *out_pos_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MNT_CHECK(num_offsets >= 0 && num_offsets <= 1024 && num_targets >= 0 && num_targets <= INT32_MAX,
+              "bad shape O=%lld T=%lld (at most 1024 offsets)", (long long)num_offsets, (long long)num_targets);
+    MNT_CHECK(row_ptr_out != nullptr, "row_ptr_out is null");
+    if (num_targets == 0 || num_offsets == 0) {
+      enqueue_fill<int32_t>(row_ptr_out, num_targets + 1, 0, stream);
+      return;
+    }
+    MNT_CHECK(kernel_map != nullptr && sizes_host != nullptr, "null argument");
+    int64_t nnz = 0;
+    std::vector<int> tables(2 * num_offsets);
+    std::vector<char> seen(num_offsets, 0);
+    for (int64_t j = 0; j < num_offsets; ++j) {
+      const int64_t o = order_host != nullptr ? order_host[j] : j;
+      MNT_CHECK(o >= 0 && o < num_offsets && !seen[o], "order_host is not a permutation of the offsets");
+      seen[o] = 1;
+      MNT_CHECK(sizes_host[j] >= 0 && sizes_host[j] <= num_targets, "size of list row %lld is out of range",
+                (long long)j);
+      tables[j] = static_cast<int>(o);
+      tables[num_offsets + j] = static_cast<int>(nnz);
+      nnz += sizes_host[j];
+    }
+    MNT_CHECK(nnz <= INT32_MAX, "more than 2^31 - 1 hits");
+    MNT_CHECK(nnz == 0 || out_pos_out != nullptr, "out_pos_out is null");
+    Scope scope(stream);
+    const int num_tiles = static_cast<int>(div_ceil(num_targets, kTargetsPerTile));
+    unsigned *tile_counts = scope.alloc<unsigned>(static_cast<size_t>(num_offsets) * num_tiles);
+    unsigned *row_sizes = scope.alloc<unsigned>(num_offsets);
+    int *d_tables = scope.alloc<int>(tables.size());
+    upload_ints(tables, d_tables, stream);
+    enqueue_count_tiles(kernel_map, MNT_INT32, num_offsets, num_targets, tile_counts, num_tiles, stream);
+    tile_scan_kernel<<<static_cast<unsigned>(num_offsets), 256, 0, stream>>>(tile_counts, num_tiles, row_sizes);
+    check_launch("tile_scan_kernel");
+    const size_t lds = static_cast<size_t>(num_offsets) * (kQueryThreads / kWave) * (sizeof(unsigned long long) + sizeof(unsigned)) +
+                       static_cast<size_t>(num_offsets) * sizeof(unsigned) + 64;
+    row_lists_kernel<<<num_tiles, kQueryThreads, lds, stream>>>(kernel_map, num_targets,
+                                                                static_cast<int>(num_offsets), tile_counts,
+                                                                num_tiles, d_tables, row_ptr_out, out_pos_out);
+    check_launch("row_lists_kernel");
   });
 }
 

@@ -465,12 +465,14 @@ class SparseConv(Module):
         """Times one whole layer per dataflow on the recorded kernel maps (random
         features) and keeps the faster one."""
         best = None
-        for dataflow in ("gather_gemm_scatter", "implicit"):
+        for dataflow in ("gather_gemm_scatter", "list_driven", "implicit"):
             total = 0.0
             try:
                 for kernel_map in self._tuning_data:
                     if dataflow == "implicit" and kernel_map.dense is None:
                         raise RuntimeError("no dense kernel map")
+                    if dataflow == "list_driven" and not kernel_map.ensure_row_lists():
+                        raise RuntimeError("no row lists for this kernel map")
                     sources = torch.randn(kernel_map.num_sources, self.in_channels,
                                           device=self.kernel.device).to(self.kernel.dtype)
                     order = kernel_map.kernel_map_order
@@ -522,7 +524,7 @@ class SparseConv(Module):
         per_piece = 16 // features.element_size()
         pad = -self.in_channels % per_piece
         if (pad == 0 or features.dtype == torch.float32 or not features.is_cuda
-                or self._tunable_config.get("dataflow", "auto") == "gather_gemm_scatter"
+                or self._tunable_config.get("dataflow", "auto") in ("gather_gemm_scatter", "list_driven")
                 or not _C.implicit_forward_supported(self.in_channels + pad, self.out_channels,
                                                      features.dtype)):
             return 0
@@ -532,7 +534,7 @@ class SparseConv(Module):
         """Whether this call runs the single-kernel dataflow: forced by the
         tunable ``dataflow``, or chosen where it is the faster one."""
         dataflow = self._tunable_config.get("dataflow", "auto")
-        if dataflow == "gather_gemm_scatter" or not features.is_cuda:
+        if dataflow in ("gather_gemm_scatter", "list_driven") or not features.is_cuda:
             return False
         if features.dtype != self.kernel.dtype:
             return False
@@ -549,7 +551,7 @@ class SparseConv(Module):
         weights = self.kernel.view(1, self.in_channels, self.out_channels)
         needs_grad = torch.is_grad_enabled() and (features.requires_grad or weights.requires_grad)
         if (features.is_cuda and not needs_grad
-                and self._tunable_config.get("dataflow", "auto") != "gather_gemm_scatter"
+                and self._tunable_config.get("dataflow", "auto") not in ("gather_gemm_scatter", "list_driven")
                 and features.dtype == weights.dtype
                 and _C.implicit_forward_supported(self.in_channels, self.out_channels, weights.dtype)
                 # measured against torch.mm plus a separate epilogue pass up to these widths;
@@ -632,6 +634,10 @@ class SparseConv(Module):
         kernel_map = cache.get_kernel_map(**map_args)
         if self._tuning_data is not None:
             self._tuning_data.append(kernel_map)
+        dataflow = "gather_gemm_scatter"
+        if (self._tunable_config.get("dataflow") == "list_driven" and self._tuning_data is None
+                and sources.is_cuda and kernel_map.ensure_row_lists()):
+            dataflow = "list_driven"
         weights, packed = self._packed_kernel() if sources.is_cuda else (self.kernel, None)
         return F.sparse_convolution_forward(
             sources=sources, weights=weights, kernel_map=kernel_map,
@@ -639,7 +645,7 @@ class SparseConv(Module):
             scatter_tile_size=self._tunable_config["scatter_tile_size"],
             allow_shortcut_matmul=self._allow_shortcut_matmul,
             threshold=self._tunable_config["threshold"], epilogue=epilogue,
-            dataflow="gather_gemm_scatter", packed_weights=packed)
+            dataflow=dataflow, packed_weights=packed)
 
 
 class SparseConv3d(SparseConv):

@@ -68,6 +68,7 @@ SIGNATURES = {
     # host arrays are passed as plain addresses here (the call sits on a hot path)
     "mnt_sorted_kernel_map_lists": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _vp, _vp, _vp,
                                            _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "mnt_kernel_map_row_lists": (_int, [_vp, _i64, _i64, _pi64, _pi64, _vp, _vp, _vp]),
     "mnt_kernel_map_dense": (_int, [_vp, _i64, _vp, _i64, _pi64, _i64, _int, _int, _vp, _vp, _i64, _int,
                                     _pi64, _pi64, _pi64, _vp, _vp]),
     "mnt_kernel_map_tables": (_int, [_vp, _i64, _i64, _i64, _int, _pi64, _pi64, _vp]),
@@ -81,6 +82,9 @@ SIGNATURES = {
                                                     _vp, _vp, _vp, _pi64, _i64, _i64, _i64, _i64,
                                                     _i64, _int, _int, _vp, _vp, _vp, _vp, _int,
                                                     _c.c_float, _vp, _pi64, _vp, _vp]),
+    "mnt_sparse_convolution_forward_rows": (_int, [_i64, _vp, _vp, _pi64, _pi64, _vp, _vp, _vp, _i64, _i64,
+                                                   _i64, _i64, _i64, _int, _vp, _vp, _vp, _int, _c.c_float,
+                                                   _vp, _vp, _vp]),
     "mnt_pack_weights": (_int, [_vp, _i64, _i64, _i64, _int, _vp, _vp]),
     "mnt_sparse_convolution_forward_implicit": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                                                        _int, _vp, _vp, _vp, _int, _c.c_float, _vp,
@@ -783,6 +787,34 @@ def kernel_map_tables(kernel_map: torch.Tensor, num_sources: int, reorder: bool,
                 kernel_map=kernel_map)
 
 
+MAX_ROW_LIST_OFFSETS = 1024
+
+
+def kernel_map_row_lists(kernel_map: torch.Tensor, sizes_host, order_host=None):
+    """``(row_ptr [T + 1], out_pos [nnz])`` (int32) of a dense int32 kernel map
+    whose pair lists are numbered by ``sizes_host`` / ``order_host`` (as
+    :func:`kernel_map_build` returns them): the target-major row lists that
+    :func:`sparse_convolution_forward_rows` is driven by.  Waits for nothing."""
+    _ensure_ndim("kernel_map", kernel_map, 2)
+    device = _common_device([kernel_map])
+    if kernel_map.dtype != torch.int32:
+        _fail("kernel_map_row_lists expects an int32 kernel map")
+    kernel_map = kernel_map.contiguous()
+    num_offsets, num_targets = kernel_map.shape
+    sizes = np.ascontiguousarray(sizes_host, dtype=np.int64)
+    order = None if order_host is None else np.ascontiguousarray(order_host, dtype=np.int64)
+    if sizes.shape[0] != num_offsets or (order is not None and order.shape[0] != num_offsets):
+        _fail("sizes_host / order_host need one entry per offset")
+    row_ptr = torch.empty((num_targets + 1,), dtype=torch.int32, device=device)
+    out_pos = torch.empty((int(sizes.sum()),), dtype=torch.int32, device=device)
+    with _on(device):
+        _check(load_library().mnt_kernel_map_row_lists(
+            _ptr(kernel_map), num_offsets, num_targets, sizes.ctypes.data_as(_pi64),
+            None if order is None else order.ctypes.data_as(_pi64), _ptr(row_ptr), _ptr(out_pos),
+            _stream(device)))
+    return row_ptr, out_pos
+
+
 def kernel_map_pair_lists(kernel_map: torch.Tensor, sizes_host: Sequence[int]):
     """Per-offset (in_idx, out_idx) lists of an int32 dense kernel map."""
     _ensure_ndim("kernel_map", kernel_map, 2)
@@ -966,9 +998,7 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
     if gather_index is not None:
         if gather_index.dtype != torch.int32 or gather_index.device != device:
             _fail("gather_index must be an int32 tensor on the device of the features")
-        hits = getattr(gather_index, "num_hits", None)      # noted by KernelMapCache next to the index
-        if kernel_map_sizes_host is None or gather_index.numel() != (
-                int(np.sum(kernel_map_sizes_host)) if hits is None else hits):
+        if kernel_map_sizes_host is None or gather_index.numel() != int(np.sum(kernel_map_sizes_host)):
             _fail("gather_index needs the host sizes and one entry per kernel map hit")
         gather_index = gather_index.contiguous()
     ep = Epilogue() if epilogue is None else epilogue.checked(T, N, weights.dtype, device)
@@ -988,6 +1018,45 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
             _ptr(kernel_map_sizes), sizes_ptr, S, T, O, K, N, icode, fcode, _ptr(gather_index),
             _ptr(ep.scale), _ptr(ep.shift), _ptr(ep.residual), ACTIVATION_CODES[ep.activation],
             float(ep.negative_slope), _ptr(packed_weights), order_ptr, _ptr(out), _stream(device)))
+    del keep, keep_order
+    return out
+
+
+def sparse_convolution_forward_rows(sources: torch.Tensor, weights: torch.Tensor, sizes_host, order_host,
+                                    in_idx: torch.Tensor, out_pos: torch.Tensor, row_ptr: torch.Tensor,
+                                    scatter_tile_size: int = 0, epilogue: Optional["Epilogue"] = None,
+                                    packed_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The list-driven Gather-GEMM-Scatter (mnt_sparse_convolution_forward_rows):
+    ``in_idx`` / ``out_pos`` [nnz] and ``row_ptr`` [T + 1] int32 on the device,
+    ``sizes_host`` / ``order_host`` int64 on the host (``order_host`` None: rows
+    in offset order), ``weights`` [O, Cin, Cout] in the layer's offset order."""
+    _ensure_ndim("sources", sources, 2)
+    _ensure_ndim("weights", weights, 3)
+    device = _common_device([sources, weights, in_idx, out_pos, row_ptr])
+    fcode = _float_code(_common_dtype([sources, weights]), "sparse_convolution_forward_rows")
+    S, K = sources.shape
+    O, K2, N = weights.shape
+    if K2 != K:
+        _fail(f"The dimension 1 of Tensor weights is expected to be {K} but found {K2}")
+    T = row_ptr.numel() - 1
+    for name, tensor in (("in_idx", in_idx), ("out_pos", out_pos), ("row_ptr", row_ptr)):
+        if tensor.dtype != torch.int32 or not tensor.is_contiguous():
+            _fail(f"{name} must be a contiguous int32 tensor")
+    keep, sizes_ptr = _host_sizes_arg(sizes_host, O)
+    keep_order, order_ptr = (None, None) if order_host is None else _host_sizes_arg(order_host, O)
+    if in_idx.numel() != out_pos.numel() or in_idx.numel() != int(np.asarray(keep).sum()):
+        _fail("in_idx / out_pos need one entry per kernel map hit")
+    ep = Epilogue() if epilogue is None else epilogue.checked(T, N, sources.dtype, device)
+    if packed_weights is not None:
+        _check_packed(packed_weights, weights)
+    sources, weights = sources.contiguous(), weights.contiguous()
+    out = torch.empty((T, N), dtype=sources.dtype, device=device)
+    with _on(device):
+        _check(load_library().mnt_sparse_convolution_forward_rows(
+            int(scatter_tile_size), _ptr(sources), _ptr(weights), sizes_ptr, order_ptr, _ptr(in_idx),
+            _ptr(out_pos), _ptr(row_ptr), S, T, O, K, N, fcode, _ptr(ep.scale), _ptr(ep.shift),
+            _ptr(ep.residual), ACTIVATION_CODES[ep.activation], float(ep.negative_slope),
+            _ptr(packed_weights), _ptr(out), _stream(device)))
     del keep, keep_order
     return out
 

@@ -16,7 +16,7 @@ pack_weights = _C.pack_weights
 Epilogue = _C.Epilogue
 
 GEMM_PARALLEL_LEVEL = 4
-DATAFLOWS = ("auto", "gather_gemm_scatter", "implicit")
+DATAFLOWS = ("auto", "gather_gemm_scatter", "implicit", "list_driven")
 
 
 def set_gemm_parallel_level(level: int):
@@ -111,6 +111,14 @@ def sparse_convolution_forward(sources: torch.Tensor, weights: torch.Tensor,
     ``"auto"`` takes the implicit form where it is the faster one: 16-bit
     features whose rows it can stage, and small fp32 layers with 2^D kernels.
 
+    ``"list_driven"`` is Gather-GEMM-Scatter without the rank tables: the GEMM
+    reads its rows through the pair list and writes its products in
+    target-major order (``KernelMap.row_ptr`` / ``out_pos``, built on first use
+    from the dense map), so that Scatter reads them as one stream.  Scatter
+    gains what the GEMM's scattered row writes lose, so ``"auto"`` never picks
+    it; a layer's autotuner times it beside the other two.  Padding threshold,
+    gather tile and the centre-offset shortcut have no meaning there.
+
     ``epilogue`` (:class:`Epilogue`) is applied to each output row before it is
     rounded to the feature dtype.  ``packed_weights`` (``pack_weights(weights)``,
     kept by the caller while the weights are unchanged) spares the packing pass
@@ -130,11 +138,19 @@ def sparse_convolution_forward(sources: torch.Tensor, weights: torch.Tensor,
         dense = kernel_map.dense
     if dataflow == "implicit" and dense is None:
         raise ValueError("the implicit dataflow needs a KernelMap with its dense map")
-    if dense is not None and dataflow != "gather_gemm_scatter":
+    if dense is not None and dataflow in ("auto", "implicit"):
         if dataflow == "implicit" or prefers_implicit(weights.shape[0], weights.shape[1],
                                                       weights.shape[2], weights.dtype):
             return _C.sparse_convolution_forward_implicit(sources, weights, dense, epilogue=epilogue,
                                                           packed_weights=packed_weights)
+    if dataflow == "list_driven":
+        if kernel_map is None or gather_index is None or not kernel_map.ensure_row_lists():
+            raise ValueError("the list-driven dataflow needs a KernelMap with its dense map and pair lists")
+        # list-driven form: Gather folded into the GEMM, products written in
+        # target-major order, Scatter streams through them (no rank table read)
+        return _C.sparse_convolution_forward_rows(
+            sources, weights, host_sizes, host_order, gather_index, kernel_map.out_pos, kernel_map.row_ptr,
+            scatter_tile_size=scatter_tile_size, epilogue=epilogue, packed_weights=packed_weights)
     if source_masks is None or target_masks is None or kernel_map_sizes is None:
         raise ValueError("the Gather-GEMM-Scatter dataflow needs the rank tables and sizes of the kernel map")
     if parallel is None:

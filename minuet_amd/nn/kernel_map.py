@@ -71,6 +71,20 @@ class KernelMap(tuple):
     def nnz(self) -> Optional[int]:
         return None if self.sizes_host is None else int(self.sizes_host.sum())
 
+    def ensure_row_lists(self) -> bool:
+        """Builds ``row_ptr`` / ``out_pos`` (the target-major row lists of the
+        list-driven dataflow) if they are missing; needs the dense map, the pair
+        lists and the host sizes, at most 1024 offsets.  Waits for nothing on
+        the device.  Returns whether the map has them afterwards."""
+        if self.row_ptr is not None:
+            return True
+        from minuet_amd.nn.functional import _C
+        if (self.dense is None or self.in_idx is None or self.sizes_host is None or not self.dense.is_cuda
+                or not 0 < self.num_offsets <= _C.MAX_ROW_LIST_OFFSETS):
+            return False
+        self.row_ptr, self.out_pos = _C.kernel_map_row_lists(self.dense, self.sizes_host, self.order_host)
+        return True
+
     def swapped(self, dense: Optional[torch.Tensor] = None) -> "KernelMap":
         """The same map read the other way round, as a transposed layer uses it
         (minuet/nn/convolutions.py:135-140 swaps the two rank tables): sources

@@ -461,7 +461,7 @@ def test_autotune_and_timers(tmp_path):
         after = net(x).F
     cfg = minuet.dump_tunable_config(net)
     assert set(cfg["0"].keys()) == {"threshold", "gather_tile_size", "scatter_tile_size", "dataflow"}
-    assert cfg["0"]["dataflow"] in ("gather_gemm_scatter", "implicit")
+    assert cfg["0"]["dataflow"] in ("gather_gemm_scatter", "implicit", "list_driven")
     assert 32 % cfg["0"]["gather_tile_size"] == 0 and 64 % cfg["0"]["scatter_tile_size"] == 0
     # the tuned layer may run the other dataflow: equal to rounding, not bit for bit
     rms = before.float().pow(2).mean().sqrt().item()
@@ -624,3 +624,95 @@ def test_kernel_map_object_is_the_fast_path(monkeypatch):
     assert_features_close(a, orc.sparse_convolution_forward(feats, weights, esm, etm, eorder, esizes), "fp32")
     with pytest.raises(ValueError, match="dense"):
         F.sparse_convolution_forward(f, w, source_masks, target_masks, order, sizes, 0, 0, dataflow="implicit")
+
+
+@pytest.mark.parametrize("kind", ["fp32", "fp16", "bf16"])
+@pytest.mark.parametrize("kernel,stride,cin,cout,n,extent,batched", [
+    (3, 1, 32, 32, 20000, 60, False), (3, 1, 128, 128, 5000, 22, True), (2, 2, 64, 128, 20000, 50, False),
+    (5, 1, 16, 16, 3000, 16, False), (3, 1, 256, 256, 3000, 16, False), (3, 1, 24, 40, 2000, 12, True),
+    (3, 1, 3, 5, 2000, 12, False), (7, 1, 16, 8, 1500, 10, False),
+])
+def test_forward_list_driven(kind, kernel, stride, cin, cout, n, extent, batched):
+    """Gather-GEMM-Scatter driven by lists (pair lists + target-major row lists,
+    no rank table read): the row lists against a plain construction from the
+    oracle's dense map, the output against the float64 oracle and, to rounding,
+    against the table-driven form; with and without an epilogue."""
+    src, sbd, tgt, tbd, off, feats, weights = make_layer_case(8, n, extent, kernel, cin, cout, kind, stride, batched)
+    esm, etm, eorder, esizes, em = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=True)
+    ref = orc.sparse_convolution_forward(feats, weights, esm, etm, eorder, esizes)
+    dtype = TORCH[kind]
+    built = _C.kernel_map_build(dev(src), dev(tgt), off.astype(np.int64), dev(sbd), dev(tbd), reorder=True,
+                                want_masks=True, want_lists=True, want_dense=True)
+    row_ptr, out_pos = _C.kernel_map_row_lists(built["kernel_map"], built["sizes_host"], built["order_host"])
+    # expected lists: hits by target, then by list row; p numbers them by list row, then by target
+    hits_t, hits_j = [], []
+    dense = orc.query_sorted_index_with_offsets(src, tgt, off, sbd, tbd, dtype=np.int32)
+    by_row = dense[eorder]                                  # [list row, target]
+    jj, tt = np.nonzero(by_row >= 0)                        # row-major: by list row, then target = list numbering
+    p_of = {}
+    for p, (j, t) in enumerate(zip(jj, tt)):
+        p_of[(j, t)] = p
+    tt2, jj2 = np.nonzero(by_row.T >= 0)                    # by target, then list row = buffer numbering
+    expect_pos = np.empty(len(jj), dtype=np.int32)
+    for pos, (t, j) in enumerate(zip(tt2, jj2)):
+        expect_pos[p_of[(j, t)]] = pos
+    counts = (by_row >= 0).sum(axis=0)
+    np.testing.assert_array_equal(host(row_ptr), np.concatenate([[0], np.cumsum(counts)]))
+    np.testing.assert_array_equal(host(out_pos), expect_pos)
+    kernel_map = minuet.nn.KernelMap(built["source_masks"], built["target_masks"], built["order"], built["sizes"],
+                                     sizes_host=built["sizes_host"], order_host=built["order_host"],
+                                     in_idx=built["in_idx"], out_idx=built["out_idx"], dense=built["kernel_map"])
+    f, w = dev(feats).to(dtype), dev(weights).to(dtype)
+    tables = F.sparse_convolution_forward(f, w, kernel_map=kernel_map, allow_shortcut_matmul=stride == 1,
+                                          threshold=-1, dataflow="gather_gemm_scatter")
+    assert kernel_map.row_ptr is None
+    lists = F.sparse_convolution_forward(f, w, kernel_map=kernel_map, dataflow="list_driven")
+    assert kernel_map.row_ptr is not None                   # built on first use
+    assert lists.dtype == dtype and lists.shape == (tgt.shape[0], cout)
+    assert_features_close(lists, ref, kind)
+    diff = (lists.float() - tables.float()).abs().max().item()
+    scale_of = tables.float().abs().max().item()
+    assert diff <= max(2e-2 * tables.float().pow(2).mean().sqrt().item() if kind != "fp32" else 0.0,
+                       scale_of * 2.0 ** {"fp32": -20, "fp16": -10, "bf16": -7}[kind]), diff
+    packed = F.sparse_convolution_forward(f, w, kernel_map=kernel_map, dataflow="list_driven",
+                                          packed_weights=F.pack_weights(w))
+    assert torch.equal(packed, lists)
+    rng = np.random.default_rng(5)
+    scale = rng.uniform(0.5, 1.5, size=cout).astype(np.float32)
+    shift = rng.uniform(-0.5, 0.5, size=cout).astype(np.float32)
+    residual = quantise(rng.normal(size=ref.shape), kind)
+    fused = np.maximum(ref * scale.astype(np.float64) + shift.astype(np.float64) + residual, 0.0)
+    out = F.sparse_convolution_forward(f, w, kernel_map=kernel_map, dataflow="list_driven",
+                                       epilogue=F.Epilogue(dev(scale), dev(shift), dev(residual).to(dtype), "relu"))
+    assert_features_close(out, fused, kind)
+
+
+def test_list_driven_layers_in_a_module_chain():
+    """down (stride 2) -> submanifold -> transposed up through the modules with
+    the list-driven dataflow chosen: every layer, the transposed one included,
+    runs without rank tables and agrees with the float64 oracle."""
+    rng = np.random.default_rng(4)
+    c, _ = sorted_unique(random_cloud(12000, 40, seed=9, lo=-11))
+    feats = rng.normal(size=(c.shape[0], 16))
+    down = minuet.nn.SparseConv3d(16, 32, 2, stride=2, dtype=torch.float32, device="cuda")
+    sub = minuet.nn.SparseConv3d(32, 32, 3, dtype=torch.float32, device="cuda")
+    up = minuet.nn.SparseConv(3, 32, 16, 2, stride=2, transposed=True, dtype=torch.float32, device="cuda")
+    cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+    for m in (down, sub, up):
+        m.set_kernel_map_cache(cache)
+        m.tunable_config["dataflow"] = "list_driven"
+    with torch.no_grad():
+        a = down(minuet.SparseTensor(dev(feats).float(), dev(c)))
+        b = sub(a)
+        y = up(b)
+    assert all(km.row_ptr is not None for km in cache._kernel_maps_cache.values())
+    assert all(km.row_ptr is not None for km in cache._swapped_maps_cache.values())
+    r1, c1, _, _ = orc.conv_layer(c, None, feats.astype(np.float32).astype(np.float64),
+                                  host(down.kernel.detach().double()), 2, stride=2)
+    r2, _, _, _ = orc.conv_layer(c1, None, r1, host(sub.kernel.detach().double()), 3, source_stride=2)
+    r3, c3, _, _ = orc.conv_layer(c1, None, r2, host(up.kernel.detach().double()), 2, stride=2,
+                                  source_stride=2, transposed_from=(c, None, 1))
+    np.testing.assert_array_equal(host(y.C), c3)
+    for got, ref in ((a.F, r1), (b.F, r2), (y.F, r3)):
+        err = np.abs(host(got.double()) - ref).max()
+        assert err <= 1e-5 * np.abs(ref).max(), err
