@@ -377,6 +377,13 @@ def main():
     wall_ms = 1e3 * (time.perf_counter() - t0) / args.steps
     # the same step one by one: stream events between the calls, at least 50 of them
     step_stats = _time_stats(lambda: map_step(_C, coords_dev, offsets), 10, max(50, min(args.steps, 500)))
+    # how often a step makes the host wait for the device (the library's own tally)
+    _C.host_wait_stats(reset=True)
+    for _ in range(50):
+        map_step(_C, coords_dev, offsets)
+    waits, waited_s = _C.host_wait_stats(reset=True)
+    step_stats["host_waits_per_step"] = round(waits / 50, 2)
+    step_stats["host_wait_ms_per_step"] = round(1e3 * waited_s / 50, 4)
 
     # per-stage device time from the library's own stream events
     _C.profile_enable(True)

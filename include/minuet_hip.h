@@ -68,6 +68,15 @@ int mnt_reset_error(void);                                /* cuda_reset_error */
  * are forgotten. */
 int mnt_device_reset(void);
 
+/* How often, and for how long in total, library calls of this process have
+ * made the host wait for a result of the device (every such wait is the poll
+ * of one completion flag in pinned memory) since the last reset of the tally.
+ * Either output may be null; reset != 0 clears the tally after reading it.
+ * No counterpart in the reference, whose waits are stream synchronisations
+ * inside its functions (e.g. csrc/minuet/cuda/functions/query_sorted_index.cu:
+ * 13-119, three of them); bench.py reports the figure per Map step. */
+int mnt_host_wait_stats(int64_t *waits_out, int64_t *nanoseconds_out, int reset);
+
 /* ---- Map: coordinate sort ---------------------------------------------- */
 
 /* Stable lexicographic arg-sort of coords[n, ndim] (dimension 0 most

@@ -141,10 +141,21 @@ unsigned long long *Arena::flag_device(int slot) {
                                                 static_cast<size_t>(slot) * 64);
 }
 
+static std::atomic<long long> g_host_waits{0}, g_host_wait_ns{0};
+
 void Arena::wait_flag(int slot, unsigned long long sequence) {
   volatile unsigned long long *flag = reinterpret_cast<volatile unsigned long long *>(
       static_cast<char *>(pinned()) + kFlagOffset + static_cast<size_t>(slot) * 64);
   const auto start = std::chrono::steady_clock::now();
+  struct Tally {
+    std::chrono::steady_clock::time_point since;
+    ~Tally() {
+      g_host_waits.fetch_add(1, std::memory_order_relaxed);
+      g_host_wait_ns.fetch_add(std::chrono::duration_cast<std::chrono::nanoseconds>(
+                                   std::chrono::steady_clock::now() - since).count(),
+                               std::memory_order_relaxed);
+    }
+  } tally{start};
   unsigned spins = 0;
   while (*flag != sequence) {
     if ((++spins & 0x3FFFu) == 0) {
@@ -266,6 +277,17 @@ int mnt_reset_error(void) {
   (void)hipGetLastError();
   g_last_error.clear();
   return 0;
+}
+
+int mnt_host_wait_stats(int64_t *waits_out, int64_t *nanoseconds_out, int reset) {
+  return guarded([&] {
+    if (waits_out != nullptr) *waits_out = g_host_waits.load(std::memory_order_relaxed);
+    if (nanoseconds_out != nullptr) *nanoseconds_out = g_host_wait_ns.load(std::memory_order_relaxed);
+    if (reset) {
+      g_host_waits.store(0, std::memory_order_relaxed);
+      g_host_wait_ns.store(0, std::memory_order_relaxed);
+    }
+  });
 }
 
 int mnt_device_reset(void) {

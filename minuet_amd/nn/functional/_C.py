@@ -43,6 +43,7 @@ SIGNATURES = {
     "mnt_buffer_used_size": (_sz, [_vp]),
     "mnt_reset_error": (_int, []),
     "mnt_device_reset": (_int, []),
+    "mnt_host_wait_stats": (_int, [_pi64, _pi64, _int]),
     "mnt_arg_sort_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _vp, _pi64, _vp]),
     "mnt_unique_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _pi64, _vp]),
     "mnt_fill_unique_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _int, _vp, _vp]),
@@ -1248,6 +1249,15 @@ def cuda_device_reset():
     holds on the current device (every stream's arena); unlike the reference's
     cudaDeviceReset() it leaves the context, and with it every torch tensor, alone."""
     _check(load_library().mnt_device_reset())
+
+
+def host_wait_stats(reset: bool = False):
+    """``(waits, seconds)``: how often and for how long library calls of this
+    process have made the host wait for the device since the tally was last
+    reset (each wait polls one completion flag in pinned memory)."""
+    waits, ns = ctypes.c_int64(0), ctypes.c_int64(0)
+    _check(load_library().mnt_host_wait_stats(ctypes.byref(waits), ctypes.byref(ns), 1 if reset else 0))
+    return waits.value, ns.value * 1e-9
 
 
 def profile_enable(on: bool):

@@ -125,9 +125,10 @@ def test_config5_large_kernel_bf16_properties():
         conv.set_kernel_map_cache(cache)
         feats = torch.randn(n, 64, device="cuda").bfloat16()
         outputs = {}
-        # both dataflows: the single-kernel form ("auto" takes it here) and the
-        # reference's Gather -> grouped GEMM -> Scatter over the 125 skewed groups
-        for flow in ("auto", "gather_gemm_scatter"):
+        # every dataflow: the single-kernel form ("auto" takes it here), the
+        # reference's Gather -> grouped GEMM -> Scatter over the 125 skewed groups,
+        # and its list-driven variant
+        for flow in ("auto", "gather_gemm_scatter", "list_driven"):
             conv.tunable_config["dataflow"] = flow
             with torch.no_grad():
                 y = conv(minuet.SparseTensor(feats, sorted_dev))
@@ -145,6 +146,7 @@ def test_config5_large_kernel_bf16_properties():
             outputs[flow] = y.F.float()
         # the two dataflows round the same fp32 sums once each: 2e-2 of the RMS, or
         # one bf16 unit in the last place of the largest value where that is more
-        diff = (outputs["auto"] - outputs["gather_gemm_scatter"]).abs().max().item()
         rms = outputs["auto"].pow(2).mean().sqrt().item()
-        assert diff <= max(2e-2 * rms, outputs["auto"].abs().max().item() * 2.0 ** -7), diff
+        for flow in ("gather_gemm_scatter", "list_driven"):
+            diff = (outputs["auto"] - outputs[flow]).abs().max().item()
+            assert diff <= max(2e-2 * rms, outputs["auto"].abs().max().item() * 2.0 ** -7), (flow, diff)
