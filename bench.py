@@ -289,11 +289,32 @@ def extras(device, with_config5, section="all"):
             del graphed
         except Exception as error:          # reported, never fatal for the headline
             replayed = {"error": str(error)[:200]}
+        # cold passes again with the cache's look-ahead: from the second pass on the
+        # worker thread builds levels and maps beside the layers (same results)
+        ahead4 = minuet.nn.KernelMapCache(3, torch.int32, device, lookahead=True)
+        minuet.set_kernel_map_cache(net, ahead4)
+
+        passes = [0]
+
+        def forward_ahead():
+            ahead4.reset()
+            net(x4)
+            passes[0] += 1
+        try:
+            lat_ahead = _time_stats(forward_ahead, 5, 50)
+            # the very first pass has no recipe yet and builds everything itself
+            lat_ahead["map_builds_taken_from_the_worker_per_pass"] = round(
+                ahead4.num_ahead_hits / max(1, passes[0] - 1), 1)
+            ahead4.reset()
+        except Exception as error:
+            lat_ahead = {"error": str(error)[:200]}
         out["config4_unet_fp16"] = {"voxels": int(s4.shape[0]), "batch": 2, "cold_cache": lat,
+                                    "cold_cache_lookahead": lat_ahead,
                                     "kernel_maps_cached": kept,
                                     "kernel_maps_cached_graph_replay": replayed,
-                                    "forward_ms_cold_cache": lat["ms_median"]}
-        del net, cache4, x4
+                                    "forward_ms_cold_cache": lat["ms_median"],
+                                    "forward_ms_cold_cache_lookahead": lat_ahead.get("ms_median")}
+        del net, cache4, ahead4, x4
     if section == "unet":
         return {"config4_unet_fp16": out["config4_unet_fp16"]}
     out["config2_layer_kernels_fp16_c64"] = layer_stages(device, 2, 64, 3, "fp16")

@@ -520,6 +520,63 @@ int mnt_sparse_convolution_forward_implicit(const void *sources, const void *wei
 int mnt_kernel_map_invert(const int32_t *kernel_map, int64_t num_offsets, int64_t num_targets,
                           int64_t num_sources, int32_t *inverse_out, void *stream);
 
+/* ---- Map: building a pass's coordinates and kernel maps ahead ------------- */
+
+/* A network that has seen one cloud asks for the same coordinate levels and
+ * kernel maps, in the same order, for the next one.  With the list of those
+ * requests (the items below) the library builds all of them for a new cloud on
+ * a worker thread and a stream of its own while the caller goes on enqueueing
+ * layers: mnt_lookahead_start returns at once, mnt_lookahead_wait(item) blocks
+ * until that item is built, makes `stream` wait for the kernels that wrote it
+ * and returns its size.  Every item is built by the entry point a caller would
+ * use for it (mnt_target_coordinates, mnt_kernel_map_dense,
+ * mnt_kernel_map_tables + mnt_kernel_map_emit, mnt_kernel_map_invert), so the
+ * results are theirs; outputs go to buffers the caller allocated for the worst
+ * case (no level has more rows than level 0).
+ *
+ * Levels: level 0 is the cloud given to mnt_lookahead_start; a COORDS item
+ * makes level `target_level` from level `source_level`.
+ *   MNT_AHEAD_COORDS  stride[ndim]; out0 = coordinates [capacity, ndim],
+ *                     out1 = batch boundaries [num_batches + 1] (batched clouds);
+ *                     size = number of rows.
+ *   MNT_AHEAD_DENSE   source_level, target_level, offsets (host, int64
+ *                     [num_offsets, ndim], alive until the session ends);
+ *                     out0 = kernel map [num_offsets, T] int32 (capacity >=
+ *                     num_offsets * T ints); size = T.
+ *   MNT_AHEAD_TABLES  dense_item, reorder; out0 / out1 = rank tables [O, S] /
+ *                     [O, T], out2 / out3 = pair lists (capacity entries each),
+ *                     out4 / out5 = device sizes / order [O]; host0 / host1 =
+ *                     host sizes / order int64 [O]; size = number of pairs.
+ *   MNT_AHEAD_INVERT  dense_item; out0 = inverse map [O, S]; size = S.
+ * bounds_out (nullable, 8 x int64 per level, -1 flags unknown in
+ * bounds_known_out) receives the coordinate bounds of every level.
+ * One session per process at a time; mnt_lookahead_finish waits for the worker
+ * to go idle (items nobody waited for are still built, or skipped after an
+ * error) and makes `stream` wait for everything it enqueued: call it before
+ * the buffers are released.  An item that fails makes its wait return non-zero
+ * with the message in mnt_last_error(); items that depend on it fail too.
+ * No counterpart in the reference, whose KernelMapCache builds every map when
+ * a layer first asks for it (minuet/nn/convolutions.py:58-173). */
+enum { MNT_AHEAD_COORDS = 0, MNT_AHEAD_DENSE = 1, MNT_AHEAD_TABLES = 2, MNT_AHEAD_INVERT = 3 };
+typedef struct mnt_lookahead_item {
+  int32_t kind;
+  int32_t source_level, target_level, dense_item, reorder;
+  int32_t reserved;
+  int64_t stride[4];
+  const int64_t *offsets;
+  int64_t num_offsets;
+  int64_t capacity;
+  void *out0, *out1, *out2, *out3, *out4, *out5;
+  int64_t *host0, *host1;
+} mnt_lookahead_item;
+int mnt_lookahead_start(const void *coords, int64_t n, int ndim, int coord_dtype,
+                        const void *batch_dims, int64_t num_batches, int index_dtype,
+                        const int64_t *bounds_host, const mnt_lookahead_item *items,
+                        int num_items, int num_levels, int64_t *bounds_out,
+                        int32_t *bounds_known_out, void *stream);
+int mnt_lookahead_wait(int item, void *stream, int64_t *size_out);
+int mnt_lookahead_finish(void *stream);
+
 /* ---- stage timing -------------------------------------------------------- */
 
 /* mnt_profile_enable(1) makes the instrumented entry points (sort, query, emit,

@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_DIR = os.path.join(_HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libminuet_hip.so")
-SOURCES = ["runtime.hip", "sort.hip", "unique.hip", "query.hip", "conv.hip", "implicit.hip"]
+SOURCES = ["runtime.hip", "sort.hip", "unique.hip", "query.hip", "conv.hip", "implicit.hip", "lookahead.hip"]
 ARCH = "gfx950"
 FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC",

@@ -1,6 +1,7 @@
 // Library plumbing: last-error slot, per-stream scratch arena, buffer knobs.
 #include <atomic>
 #include <chrono>
+#include <thread>
 #include <map>
 #include <mutex>
 
@@ -190,8 +191,12 @@ static std::vector<std::pair<const char *, hipEvent_t>> g_marks;
 static std::vector<hipEvent_t> g_event_pool;
 static constexpr size_t kMaxMarks = 4096;
 
+static std::thread::id g_profile_thread;
+
 void profile_mark(const char *label, hipStream_t stream) {
-  if (!g_profile_on || g_marks.size() >= kMaxMarks) return;
+  // marks are kept for the thread that turned profiling on: the look-ahead
+  // worker runs the same entry points on another stream at the same time
+  if (!g_profile_on || std::this_thread::get_id() != g_profile_thread || g_marks.size() >= kMaxMarks) return;
   hipEvent_t event;
   if (!g_event_pool.empty()) {
     event = g_event_pool.back();
@@ -249,6 +254,7 @@ size_t mnt_buffer_used_size(void *stream) {
 int mnt_profile_enable(int on) {
   return guarded([&] {
     profile_clear();
+    g_profile_thread = std::this_thread::get_id();
     g_profile_on = on != 0;
   });
 }
@@ -292,6 +298,7 @@ int mnt_host_wait_stats(int64_t *waits_out, int64_t *nanoseconds_out, int reset)
 
 int mnt_device_reset(void) {
   return guarded([&] {
+    if (mnt_lookahead_finish(nullptr) != 0) throw Error{mnt_last_error()};
     MNT_HIP(hipDeviceSynchronize());
     Arena::reset_device();
     (void)hipGetLastError();

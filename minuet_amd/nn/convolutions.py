@@ -43,7 +43,7 @@ class KernelMapCache(object):
     when a layer asks for them."""
 
     def __init__(self, ndim: int, dtype: torch.dtype, device: Union[str, torch.device],
-                 layout: str = "minuet", disable_reordering: bool = False):
+                 layout: str = "minuet", disable_reordering: bool = False, lookahead: bool = False):
         self._ndim = ndim
         self._dtype = dtype
         self._device = device
@@ -58,6 +58,16 @@ class KernelMapCache(object):
         self._bounds_cache = dict()
         self.num_map_builds = 0
         self.num_coordinate_builds = 0
+        # look-ahead: the requests of the last pass that built something, and the
+        # session that builds them for the current cloud on the library's worker thread
+        self._lookahead = lookahead
+        self._recording = []
+        self._recipe = None
+        self._recipe_rest = None      # the recipe without a first entry that this thread builds itself
+        self._ahead = None
+        self._ahead_layout = None
+        self._ahead_tried = False
+        self.num_ahead_hits = 0
 
     @functools.lru_cache(maxsize=None)
     def _kernel_offsets(self, source_stride, kernel_size, kernel_dilation) -> np.ndarray:
@@ -67,12 +77,64 @@ class KernelMapCache(object):
                                     layout=self._layout), dtype=np.int64)
 
     def reset(self):
+        if self._ahead is not None:
+            # the worker may still write buffers of maps nobody asked for
+            self._ahead.finish()
+            self._ahead = None
+        if self._recording:
+            recipe = tuple(self._recording)
+            if recipe != self._recipe:
+                self._recipe = recipe
+                # The first request of a pass is needed at once: when it is a dense
+                # map that no later entry builds on, the asking thread makes it
+                # itself while the worker starts on the rest.
+                first = recipe[0]
+                alone = first[0] == "dense" and not any(
+                    entry[0] in ("tables", "invert") and entry[1] == first[1] for entry in recipe[1:])
+                self._recipe_rest = recipe[1:] if alone and len(recipe) > 1 else None
+            self._recording = []
+        self._ahead_tried = False
         self._coordinates_cache.clear()
         self._kernel_maps_cache.clear()
         self._swapped_maps_cache.clear()
         self._dense_maps_cache.clear()
         self._inverse_maps_cache.clear()
         self._bounds_cache.clear()
+
+    def _from_ahead(self, tag, record, coordinates, stride, batch_dims):
+        """Notes the request ``record`` for the next pass's recipe and, with the
+        look-ahead on, returns what the worker built for ``tag`` (None when it
+        was not given that request, or failed at it).  The first request of a
+        pass starts the worker on the recipe of the last one, from the cloud
+        ``coordinates`` of stride ``stride``."""
+        if not self._lookahead:
+            return None
+        self._recording.extend(record)
+        if self._ahead is None:
+            if self._ahead_tried or self._recipe is None or coordinates is None:
+                return None
+            self._ahead_tried = True
+            from minuet_amd.nn.lookahead import AheadSession
+            recipe = self._recipe
+            if self._recipe_rest is not None and record and record[0] == recipe[0]:
+                recipe = self._recipe_rest
+            try:
+                self._ahead = AheadSession(recipe, self._kernel_offsets, coordinates, tuple(stride),
+                                           batch_dims, self._known_bounds(coordinates),
+                                           layout=self._ahead_layout)
+            except (ValueError, RuntimeError):
+                _C.cuda_reset_error()
+                return None
+            self._ahead_layout = self._ahead.layout
+        if tag not in self._ahead.index:
+            return None
+        try:
+            result = self._ahead.take(tag)
+        except RuntimeError:
+            _C.cuda_reset_error()
+            return None
+        self.num_ahead_hits += 1
+        return result
 
     def _known_bounds(self, coordinates: torch.Tensor):
         """Host copy of the per-dimension min / max of a coordinate tensor seen
@@ -104,9 +166,14 @@ class KernelMapCache(object):
         if transposed:
             raise RuntimeError(_TRANSPOSED_FIRST)
         known = self._known_bounds(source_coordinates)
-        coords, batch_dims = _C.target_coordinates(source_coordinates.contiguous(),
-                                                   source_batch_dims, target_stride,
-                                                   source_bounds=known)
+        ahead = self._from_ahead(("coords", target_stride), [("coords", source_stride, target_stride)],
+                                 source_coordinates, source_stride, source_batch_dims)
+        if ahead is not None:
+            coords, batch_dims = ahead
+        else:
+            coords, batch_dims = _C.target_coordinates(source_coordinates.contiguous(),
+                                                       source_batch_dims, target_stride,
+                                                       source_bounds=known)
         self.num_coordinate_builds += 1
         if known is not None and source_coordinates.shape[0] > 0:
             # floor(c / s) * s is monotone, so the extremes map to the extremes
@@ -172,14 +239,17 @@ class KernelMapCache(object):
             offsets = self._kernel_offsets(source_stride, kernel_size, kernel_dilation)
             source_coordinates = source_coordinates.contiguous()
             target_coordinates = target_coordinates.contiguous()
-            dense, bounds = _C.kernel_map_dense(
-                source_coordinates, target_coordinates, offsets, source_batch_dims, target_batch_dims,
-                source_bounds=self._known_bounds(source_coordinates),
-                target_bounds=self._known_bounds(target_coordinates))
+            dense = self._from_ahead(("dense", key), [("dense", key)], source_coordinates, source_stride,
+                                     source_batch_dims)
+            if dense is None:
+                dense, bounds = _C.kernel_map_dense(
+                    source_coordinates, target_coordinates, offsets, source_batch_dims, target_batch_dims,
+                    source_bounds=self._known_bounds(source_coordinates),
+                    target_bounds=self._known_bounds(target_coordinates))
+                if source_coordinates.shape[0] > 0 and target_coordinates.shape[0] > 0:
+                    self._remember_bounds(source_coordinates, bounds[:8])
+                    self._remember_bounds(target_coordinates, bounds[8:])
             self.num_map_builds += 1
-            if source_coordinates.shape[0] > 0 and target_coordinates.shape[0] > 0:
-                self._remember_bounds(source_coordinates, bounds[:8])
-                self._remember_bounds(target_coordinates, bounds[8:])
             entry = (dense, source_coordinates.shape[0])
             self._dense_maps_cache[key] = entry
         if not transposed:
@@ -191,7 +261,9 @@ class KernelMapCache(object):
         inverse = self._inverse_maps_cache.get(key)
         if inverse is None:
             dense, num_sources = self._dense_maps_cache[key]
-            inverse = _C.kernel_map_invert(dense, num_sources)
+            inverse = self._from_ahead(("invert", key), [("invert", key)], None, None, None)
+            if inverse is None:
+                inverse = _C.kernel_map_invert(dense, num_sources)
             self._inverse_maps_cache[key] = inverse
         return inverse
 
@@ -232,11 +304,25 @@ class KernelMapCache(object):
         round, but then the dense map exists and they are not used.)"""
         reorder = not self._disable_reordering and not disable_reordering
         entry = self._dense_maps_cache.get(key)
+        if entry is None and self._lookahead:
+            # the worker builds the two halves as two items: take the dense map first
+            dense = self._from_ahead(("dense", key), [("dense", key)], source_coordinates, source_stride,
+                                     source_batch_dims)
+            if dense is not None:
+                self.num_map_builds += 1
+                entry = self._dense_maps_cache[key] = (dense, source_coordinates.shape[0])
+            else:
+                del self._recording[-1]           # the all-at-once build below notes its own requests
         if entry is not None:
             # the query ran earlier for a layer that needed the dense map only
             dense, num_sources = entry
-            built = _C.kernel_map_tables(dense, num_sources, reorder=reorder, want_lists=True)
+            built = self._from_ahead(("tables", key), [("tables", key, reorder)], source_coordinates,
+                                     source_stride, source_batch_dims)
+            if built is None:
+                built = _C.kernel_map_tables(dense, num_sources, reorder=reorder, want_lists=True)
         else:
+            if self._lookahead:
+                self._recording.extend([("dense", key), ("tables", key, reorder)])
             offsets = self._kernel_offsets(source_stride, kernel_size, kernel_dilation)
             source_coordinates = source_coordinates.contiguous()
             target_coordinates = target_coordinates.contiguous()

@@ -44,6 +44,10 @@ SIGNATURES = {
     "mnt_reset_error": (_int, []),
     "mnt_device_reset": (_int, []),
     "mnt_host_wait_stats": (_int, [_pi64, _pi64, _int]),
+    "mnt_lookahead_start": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _pi64, _vp, _int, _int, _pi64,
+                                   _vp, _vp]),
+    "mnt_lookahead_wait": (_int, [_int, _vp, _pi64]),
+    "mnt_lookahead_finish": (_int, [_vp]),
     "mnt_arg_sort_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _vp, _pi64, _vp]),
     "mnt_unique_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _pi64, _vp]),
     "mnt_fill_unique_coordinates": (_int, [_vp, _i64, _int, _int, _vp, _int, _vp, _vp]),
@@ -1258,6 +1262,54 @@ def host_wait_stats(reset: bool = False):
     waits, ns = ctypes.c_int64(0), ctypes.c_int64(0)
     _check(load_library().mnt_host_wait_stats(ctypes.byref(waits), ctypes.byref(ns), 1 if reset else 0))
     return waits.value, ns.value * 1e-9
+
+
+AHEAD_COORDS, AHEAD_DENSE, AHEAD_TABLES, AHEAD_INVERT = 0, 1, 2, 3
+
+
+class LookaheadItem(ctypes.Structure):
+    """``mnt_lookahead_item`` of include/minuet_hip.h."""
+    _fields_ = [("kind", ctypes.c_int32), ("source_level", ctypes.c_int32),
+                ("target_level", ctypes.c_int32), ("dense_item", ctypes.c_int32),
+                ("reorder", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("stride", ctypes.c_int64 * 4), ("offsets", ctypes.c_void_p),
+                ("num_offsets", ctypes.c_int64), ("capacity", ctypes.c_int64),
+                ("out0", ctypes.c_void_p), ("out1", ctypes.c_void_p), ("out2", ctypes.c_void_p),
+                ("out3", ctypes.c_void_p), ("out4", ctypes.c_void_p), ("out5", ctypes.c_void_p),
+                ("host0", ctypes.c_void_p), ("host1", ctypes.c_void_p)]
+
+
+def lookahead_start(coordinates: torch.Tensor, batch_dims: Optional[torch.Tensor], bounds,
+                    items, num_levels: int):
+    """Hands ``items`` (a ctypes array of :class:`LookaheadItem`) to the
+    library's worker thread, which builds them for the sorted cloud
+    ``coordinates`` on a stream of its own; returns at once."""
+    device = coordinates.device
+    n, ndim = coordinates.shape
+    known = None if bounds is None else np.ascontiguousarray(bounds, dtype=np.int64)
+    with _on(device):
+        _check(load_library().mnt_lookahead_start(
+            coordinates.data_ptr(), n, ndim, _INT[coordinates.dtype], _ptr(batch_dims),
+            batch_dims.numel() - 1 if batch_dims is not None else 1,
+            _INT[batch_dims.dtype] if batch_dims is not None else 0,
+            None if known is None else known.ctypes.data_as(_pi64), ctypes.addressof(items),
+            len(items), num_levels, None, None, _stream(device)))
+
+
+def lookahead_wait(item: int, device: torch.device) -> int:
+    """Blocks until ``item`` is built, orders the current stream after the
+    kernels that wrote it and returns its size."""
+    size = ctypes.c_int64(0)
+    with _on(device):
+        _check(load_library().mnt_lookahead_wait(item, _stream(device), ctypes.byref(size)))
+    return size.value
+
+
+def lookahead_finish(device: torch.device):
+    """Waits for the worker to go idle and orders the current stream after all
+    it enqueued; a no-op without a session."""
+    with _on(device):
+        _check(load_library().mnt_lookahead_finish(_stream(device)))
 
 
 def profile_enable(on: bool):

@@ -168,3 +168,37 @@ def test_auto_dataflow_rule():
     assert not prefers(27, 256, 64, half)                 # 512-byte rows
     assert not prefers(27, 30, 32, half)                  # rows not a multiple of 16 bytes
     assert prefers(8, 32, 32, single) and not prefers(27, 32, 32, single) and not prefers(8, 64, 64, single)
+
+
+def test_lookahead_layout_places_every_output():
+    """The plan of a look-ahead session (no GPU needed): every output of every
+    recipe entry gets a 256-byte aligned place of its own inside one allocation,
+    entries that need a level or map nobody builds are refused."""
+    import torch
+    from minuet_amd.nn.functional import _C
+    from minuet_amd.nn.lookahead import AheadLayout
+    cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cpu")
+    one, two = (1, 1, 1), (2, 2, 2)
+    sub = (one, one, (3, 3, 3), one)
+    down = (one, two, (2, 2, 2), one)
+    recipe = (("dense", sub), ("coords", one, two), ("dense", down), ("tables", down, True), ("invert", down))
+    layout = AheadLayout(recipe, cache._kernel_offsets, one, 1 << 14, 3, torch.int32, torch.int32, 2)
+    assert layout.num_levels == 2 and len(layout.items) == 5
+    assert [item.kind for item in layout.items] == [_C.AHEAD_DENSE, _C.AHEAD_COORDS, _C.AHEAD_DENSE,
+                                                    _C.AHEAD_TABLES, _C.AHEAD_INVERT]
+    assert layout.items[3].dense_item == 2 and layout.items[4].dense_item == 2 and layout.items[3].reorder == 1
+    assert layout.items[0].num_offsets == 27 and layout.items[2].num_offsets == 8
+    spans = []
+    for places, (_, _, _, sizes) in zip(layout.places, layout.plan):
+        for place, size in zip(places, sizes):
+            if size:
+                assert place % 256 == 0
+                spans.append((place, place + size))
+    spans.sort()
+    assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:])) and spans[-1][1] <= layout.total
+    layout.bind(1 << 20)
+    assert layout.items[0].out0 == (1 << 20) + layout.places[0][0]
+    assert layout.items[1].out1 == (1 << 20) + layout.places[1][1]          # batch boundaries of the new level
+    for bad in ((("tables", sub, True),), (("coords", two, (4, 4, 4)),), (("dense", down),), ()):
+        with pytest.raises(ValueError):
+            AheadLayout(bad, cache._kernel_offsets, one, 1 << 14, 3, torch.int32, None, 1)
