@@ -1027,6 +1027,71 @@ def cuda_sparse_convolution_forward(gather_tile_size: int, scatter_tile_size: in
     return out
 
 
+def sparse_convolution_forward_map(sources: torch.Tensor, weights: torch.Tensor, kernel_map,
+                                   gather_tile_size: int = 0, scatter_tile_size: int = 0,
+                                   allow_shortcut_matmul: bool = False, parallel: int = 4,
+                                   threshold: Optional[float] = 0, epilogue: Optional["Epilogue"] = None,
+                                   packed_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """:func:`cuda_sparse_convolution_forward` for a
+    :class:`~minuet_amd.nn.KernelMap` that carries host sizes and pair lists:
+    the same library call, with everything that depends on the map alone
+    (shapes, dtypes, devices, pointers) checked and worked out once per map
+    instead of once per forward."""
+    prepared = kernel_map.prepared
+    if prepared is None:
+        source_masks, target_masks, order, sizes = kernel_map
+        _conv_shapes(torch.empty((sizes.shape[0], 1, 1), device="meta"), source_masks, target_masks, sizes)
+        tensors = [source_masks, target_masks, sizes] + ([order] if order is not None else [])
+        device = _common_device(tensors + [kernel_map.in_idx])
+        icode = _int_code(_common_dtype(tensors), "index", "CUDASparseConvolutionForward")
+        O = target_masks.size(0)
+        if order is not None:
+            _ensure_dim("kernel_map_order", order, 0, O)
+        if kernel_map.in_idx.dtype != torch.int32 or kernel_map.in_idx.numel() != int(np.sum(kernel_map.sizes_host)):
+            _fail("gather_index needs the host sizes and one entry per kernel map hit")
+        keep = [t.contiguous() for t in (source_masks, target_masks, sizes, kernel_map.in_idx)]
+        keep_order = None if order is None else order.contiguous()
+        sizes_host, sizes_ptr = _host_sizes_arg(kernel_map.sizes_host, O)
+        order_host, order_ptr = ((None, None) if kernel_map.order_host is None
+                                 else _host_sizes_arg(kernel_map.order_host, O))
+        if order is not None and order_host is None:
+            _fail("packed weights need the host copy of kernel_map_order")
+        prepared = kernel_map.prepared = (
+            source_masks.size(1), target_masks.size(1), O, icode, device, _ptr(keep[0]), _ptr(keep[1]),
+            _ptr(keep_order), _ptr(keep[2]), sizes_ptr, order_ptr, _ptr(keep[3]),
+            (keep, keep_order, sizes_host, order_host))
+    S, T, O, icode, device, p_sm, p_tm, p_order, p_sizes, sizes_ptr, order_ptr, p_gather, _ = prepared
+    dtype = weights.dtype
+    if not (sources.dim() == 2 and weights.dim() == 3 and sources.shape[0] == S and weights.shape[0] == O
+            and sources.shape[1] == weights.shape[1] and sources.dtype == dtype and sources.device == device
+            and weights.device == device and dtype in _FLOAT):
+        source_masks, target_masks, order, sizes = kernel_map           # the checks one by one, for the message
+        return cuda_sparse_convolution_forward(
+            gather_tile_size, scatter_tile_size, allow_shortcut_matmul, parallel, threshold, sources, weights,
+            source_masks, target_masks, order, sizes, kernel_map_sizes_host=kernel_map.sizes_host,
+            gather_index=kernel_map.in_idx, epilogue=epilogue, packed_weights=packed_weights,
+            kernel_map_order_host=kernel_map.order_host)
+    K, N = weights.shape[1], weights.shape[2]
+    if not sources.is_contiguous():
+        sources = sources.contiguous()
+    if not weights.is_contiguous():
+        weights = weights.contiguous()
+    out = torch.empty((T, N), dtype=dtype, device=device)
+    ep = Epilogue() if epilogue is None else epilogue.checked(T, N, dtype, device)
+    if packed_weights is not None:
+        _check_packed(packed_weights, weights)
+    with _on(device):
+        _check(load_library().mnt_sparse_convolution_forward_fused(
+            int(gather_tile_size), int(scatter_tile_size), 1 if allow_shortcut_matmul else 0,
+            int(parallel), 0 if threshold is None else 1,
+            0.0 if threshold is None else float(threshold), _ptr(sources), _ptr(weights), p_sm, p_tm, p_order,
+            p_sizes, sizes_ptr, S, T, O, K, N, icode, _FLOAT[dtype], p_gather, _ptr(ep.scale), _ptr(ep.shift),
+            _ptr(ep.residual), ACTIVATION_CODES[ep.activation], float(ep.negative_slope),
+            _ptr(packed_weights), order_ptr if packed_weights is not None else None, _ptr(out),
+            _stream(device)))
+    return out
+
+
 def sparse_convolution_forward_rows(sources: torch.Tensor, weights: torch.Tensor, sizes_host, order_host,
                                     in_idx: torch.Tensor, out_pos: torch.Tensor, row_ptr: torch.Tensor,
                                     scatter_tile_size: int = 0, epilogue: Optional["Epilogue"] = None,

@@ -155,6 +155,11 @@ def sparse_convolution_forward(sources: torch.Tensor, weights: torch.Tensor,
         raise ValueError("the Gather-GEMM-Scatter dataflow needs the rank tables and sizes of the kernel map")
     if parallel is None:
         parallel = GEMM_PARALLEL_LEVEL
+    if gather_index is not None and (kernel_map_order is None or host_order is not None):
+        # the map brings host sizes and pair lists: what depends on it alone is checked once per map
+        return _C.sparse_convolution_forward_map(
+            sources, weights, kernel_map, gather_tile_size, scatter_tile_size, allow_shortcut_matmul,
+            parallel, threshold, epilogue=epilogue, packed_weights=packed_weights)
     if kernel_map_order is not None:
         if host_order is None:
             packed_weights = None

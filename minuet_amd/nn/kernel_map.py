@@ -53,6 +53,7 @@ class KernelMap(tuple):
                            else dense.shape[1] if dense is not None else None)
         self.num_sources, self.num_targets = num_sources, num_targets
         self.inverse_dense = None           # dense map of the transposed direction, made on first use
+        self.prepared = None                # the forward call's view of this map, worked out on first use
         return self
 
     source_masks = property(lambda self: self[0])

@@ -601,13 +601,19 @@ def test_kernel_map_object_is_the_fast_path(monkeypatch):
     assert kernel_map.nnz == int(host(sizes).sum()) and kernel_map.num_offsets == 27
     assert kernel_map.in_idx.numel() == kernel_map.nnz and kernel_map.dense.shape == (27, src.shape[0])
     seen = []
-    real = _C.cuda_sparse_convolution_forward
+    real, real_map = _C.cuda_sparse_convolution_forward, _C.sparse_convolution_forward_map
 
     def spy(*args, **kwargs):
         seen.append((kwargs.get("kernel_map_sizes_host") is not None, kwargs.get("gather_index") is not None))
         return real(*args, **kwargs)
 
+    def spy_map(sources, weights, kernel_map, *args, **kwargs):
+        # the KernelMap's own entry: host sizes and pair lists come with the map
+        seen.append((kernel_map.sizes_host is not None, kernel_map.in_idx is not None))
+        return real_map(sources, weights, kernel_map, *args, **kwargs)
+
     monkeypatch.setattr(_C, "cuda_sparse_convolution_forward", spy)
+    monkeypatch.setattr(_C, "sparse_convolution_forward_map", spy_map)
     f, w = dev(feats).float(), dev(weights).float()
     common = dict(gather_tile_size=0, scatter_tile_size=0, allow_shortcut_matmul=True, threshold=-1,
                   dataflow="gather_gemm_scatter")
