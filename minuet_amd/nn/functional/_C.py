@@ -124,6 +124,10 @@ def load_library():
         fn.restype = restype
         fn.argtypes = argtypes
     _lib = lib
+    # a look-ahead session still running when the interpreter goes down would have
+    # the library's worker thread inside the GPU runtime while that is torn down
+    import atexit
+    atexit.register(lambda: lib.mnt_lookahead_finish(None))
     return lib
 
 

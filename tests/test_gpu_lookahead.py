@@ -107,3 +107,46 @@ def test_session_errors_are_reported_and_leave_the_library_usable():
     torch.cuda.synchronize()
     assert torch.equal(dense, want)
     assert torch.equal(inverse, _C.kernel_map_invert(want, coords.shape[0]))
+
+
+@pytest.mark.parametrize("coord_dtype,batched,wide", [(torch.int64, False, False), (torch.int32, False, True),
+                                                       (torch.int64, True, True)])
+def test_down_sub_up_chain_through_every_item_kind(coord_dtype, batched, wide):
+    """Coordinates, dense maps, rank tables and inverse maps from the worker for
+    int64 coordinates, single clouds and layers that run as Gather-GEMM-Scatter
+    (fp32 features with 27 offsets do)."""
+    torch.manual_seed(2)
+    dtype = torch.float32 if wide else torch.float16
+    width = 16
+    first = minuet.nn.SparseConv3d(8, width, 3, dtype=dtype, device="cuda")
+    down = minuet.nn.SparseConv3d(width, width, 2, stride=2, dtype=dtype, device="cuda")
+    sub = minuet.nn.SparseConv3d(width, width, 3, dtype=dtype, device="cuda")
+    up = minuet.nn.SparseConv(3, width, 8, 2, stride=2, transposed=True, dtype=dtype, device="cuda")
+    layers = (first, down, sub, up)
+
+    def forward(cache, coords, bd, feats):
+        cache.reset()
+        for layer in layers:
+            layer.set_kernel_map_cache(cache)
+        x = minuet.SparseTensor(feats, coords, batch_dims=bd)
+        with torch.no_grad():
+            for layer in layers:
+                x = layer(x)
+        return x
+
+    plain = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+    ahead = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda", lookahead=True)
+    for step, (scale, shift) in enumerate([(0.03, 0), (0.04, 7), (0.02, -3)]):
+        coords, bd = _cloud(scale, shift)
+        if not batched:
+            coords, bd = _C.sort_coordinates(coords)[1], None
+        coords = coords.to(coord_dtype)
+        feats = torch.randn(coords.shape[0], 8, device="cuda").to(dtype)
+        want = forward(plain, coords, bd, feats)
+        before = ahead.num_ahead_hits
+        got = forward(ahead, coords, bd, feats)
+        torch.cuda.synchronize()
+        assert torch.equal(got.C, want.C) and torch.equal(got.F, want.F), f"pass {step}"
+        if step > 0:
+            assert ahead.num_ahead_hits - before >= 4
+    ahead.reset()
