@@ -422,6 +422,34 @@ def test_module_down_sub_up(kind, batched, dataflow):
     assert_features_close(y3.F, r3, kind)
 
 
+@pytest.mark.parametrize("dataflow", ["gather_gemm_scatter", "implicit", "list_driven"])
+@pytest.mark.parametrize("kernel_size,dilation,stride,source_stride", [
+    (3, 2, 1, 1), ((3, 1, 2), (2, 1, 3), 1, 1), ((1, 3, 3), 1, (1, 2, 2), 1), (3, (1, 2, 1), 1, (2, 2, 1)),
+    ((2, 3, 1), 1, (2, 1, 1), (1, 2, 2)),
+])
+def test_module_dilated_and_anisotropic_kernels(kernel_size, dilation, stride, source_stride, dataflow):
+    """Dilation, per-dimension kernel sizes and strides, and inputs that already
+    carry a tensor stride (the offsets scale with it, helpers.py:165-212),
+    through every dataflow against the oracle's layer."""
+    rng = np.random.default_rng(6)
+    ss = np.asarray(orc.as_tuple(source_stride, 3))
+    c, _ = sorted_unique(random_cloud(6000, 14, seed=9, lo=-7) * ss)
+    feats = quantise(rng.normal(size=(c.shape[0], 16)), "fp16")
+    conv = minuet.nn.SparseConv3d(16, 24, kernel_size, stride=stride, dilation=dilation, dtype=torch.float16,
+                                  device="cuda")
+    cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+    conv.set_kernel_map_cache(cache)
+    conv.tunable_config["dataflow"] = dataflow
+    x = minuet.SparseTensor(dev(feats).half(), dev(c), stride=orc.as_tuple(source_stride, 3))
+    with torch.no_grad():
+        y = conv(x)
+    ref, rc, _, rs = orc.conv_layer(c, None, feats, host(conv.kernel.detach().float()).astype(np.float64),
+                                    kernel_size, stride=stride, dilation=dilation, source_stride=source_stride)
+    np.testing.assert_array_equal(host(y.C), rc)
+    assert tuple(y.stride) == tuple(rs)
+    assert_features_close(y.F, ref, "fp16")
+
+
 def test_module_errors_and_trivial():
     cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
     c, _ = sorted_unique(random_cloud(500, 8, seed=1))
