@@ -450,6 +450,43 @@ def test_module_dilated_and_anisotropic_kernels(kernel_size, dilation, stride, s
     assert_features_close(y.F, ref, "fp16")
 
 
+@pytest.mark.parametrize("dataflow", ["gather_gemm_scatter", "implicit"])
+@pytest.mark.parametrize("ndim,kernel_size,extent", [(1, 5, 3000), (2, 3, 90), (4, 3, 9), (4, 2, 9)])
+def test_module_other_dimensionalities(ndim, kernel_size, extent, dataflow):
+    """1-D, 2-D and 4-D layers (csrc/minuet/enabled_arguments.h:3-22 enables
+    ndim 1..4): a submanifold layer, a strided one and its transposed twin
+    against the oracle's layers."""
+    rng = np.random.default_rng(10 + ndim)
+    cloud = rng.integers(-extent // 2, extent // 2, size=(4000, ndim)).astype(np.int32)
+    c, _ = sorted_unique(cloud)
+    feats = quantise(rng.normal(size=(c.shape[0], 8)), "fp16")
+    factory = dict(dtype=torch.float16, device="cuda")
+    sub = minuet.nn.SparseConv(ndim, 8, 16, kernel_size, **factory)
+    down = minuet.nn.SparseConv(ndim, 16, 16, 2, stride=2, **factory)
+    up = minuet.nn.SparseConv(ndim, 16, 8, 2, stride=2, transposed=True, **factory)
+    cache = minuet.nn.KernelMapCache(ndim=ndim, dtype=torch.int32, device="cuda")
+    for conv in (sub, down, up):
+        conv.set_kernel_map_cache(cache)
+        conv.tunable_config["dataflow"] = dataflow
+    with torch.no_grad():
+        y1 = sub(minuet.SparseTensor(dev(feats).half(), dev(c)))
+        y2 = down(y1)
+        y3 = up(y2)
+    w = lambda conv: host(conv.kernel.detach().float()).astype(np.float64)
+    r1, c1, _, s1 = orc.conv_layer(c, None, feats, w(sub), kernel_size)
+    np.testing.assert_array_equal(host(y1.C), c1)
+    assert_features_close(y1.F, r1, "fp16")
+    q1 = quantise(host(y1.F.float()).astype(np.float64), "fp16")
+    r2, c2, _, s2 = orc.conv_layer(c1, None, q1, w(down), 2, stride=2)
+    np.testing.assert_array_equal(host(y2.C), c2)
+    assert tuple(y2.stride) == (2,) * ndim == tuple(s2)
+    assert_features_close(y2.F, r2, "fp16")
+    q2 = quantise(host(y2.F.float()).astype(np.float64), "fp16")
+    r3, c3, _, _ = orc.conv_layer(c2, None, q2, w(up), 2, stride=2, source_stride=2, transposed_from=(c, None, 1))
+    np.testing.assert_array_equal(host(y3.C), c)
+    assert_features_close(y3.F, r3, "fp16")
+
+
 def test_module_errors_and_trivial():
     cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
     c, _ = sorted_unique(random_cloud(500, 8, seed=1))
