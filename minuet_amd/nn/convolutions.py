@@ -9,6 +9,7 @@ size with a STABLE sort (the reference's device sort is unstable, so its tie
 order is not reproducible)."""
 import contextlib
 import functools
+import os
 import operator
 from typing import Any, Dict, Optional, Union
 
@@ -60,7 +61,7 @@ class KernelMapCache(object):
         self.num_coordinate_builds = 0
         # look-ahead: the requests of the last pass that built something, and the
         # session that builds them for the current cloud on the library's worker thread
-        self._lookahead = lookahead
+        self._lookahead = lookahead or os.environ.get("MINUET_LOOKAHEAD", "") == "1"
         self._recording = []
         self._recipe = None
         self._recipe_rest = None      # the recipe without a first entry that this thread builds itself

@@ -93,6 +93,7 @@ def test_config3_down_up_fp16_full_size():
 def test_config5_large_kernel_bf16_properties():
     """5x5x5, 125 offsets, bf16, ~1M voxels: kernel-map invariants and linearity at
     full size, oracle parity on a 5 % sample of the same generator."""
+    torch.manual_seed(5)
     for scale, check_oracle in ((0.05, True), (1.0, False)):
         coords = make_cloud(5, scale)["coords"]
         assert coords.min() >= 0 and coords[:, :2].max() < 2048

@@ -205,6 +205,7 @@ def test_unet_fp16_matches_layerwise_oracle():
 def test_unet_full_size_properties():
     """Configuration-4 size (2 x ~100k voxels, fp16): structural checks that do not
     need the oracle at this size."""
+    torch.manual_seed(4)
     coords, bd = build_input(1.0)
     net = SparseUNet(4, 32, dtype=torch.float16, device="cuda").eval()
     cache = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
