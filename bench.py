@@ -187,6 +187,20 @@ def layer_stages(device, config, channels, kernel_size, dtype_name, tune=False):
             if flow == "implicit" and not _C.implicit_forward_supported(channels, channels, dtype):
                 continue
             conv.tunable_config["dataflow"] = flow
+            if flow == "list_driven":
+                # its Scatter alone, from the library's stage marks: target-major row lists,
+                # every hit's product row read once (the centre offset's too), no rank table
+                for _ in range(5):
+                    conv(x)
+                _C.profile_enable(True)
+                marks = []
+                for _ in range(15):
+                    conv(x)
+                    marks += [ms for name, ms in _C.profile_read() if name == "scatter"]
+                _C.profile_enable(False)
+                if marks:
+                    rows_bytes = nnz * channels * esize + voxels * channels * esize + 4 * (voxels + 1)
+                    out["scatter_rows_kernel"] = hbm(rows_bytes, float(np.median(marks)))
             stats = _time_stats(lambda: conv(x), 10, 50)
             stats["mvoxels_per_s"] = round(voxels / stats["ms_mean"] / 1e3, 1)
             stats["achieved_TFLOPs"] = round(flops / (stats["ms_mean"] * 1e-3) / 1e12, 1)
