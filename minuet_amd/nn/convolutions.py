@@ -41,7 +41,17 @@ class KernelMapCache(object):
     A map exists in up to two forms: the dense map (``get_dense_kernel_map``,
     the query alone, no wait on the device) and the rank tables with sizes and
     order (``get_kernel_map``, the reference's tuple), made from the dense map
-    when a layer asks for them."""
+    when a layer asks for them.
+
+    ``lookahead=True`` (or ``MINUET_LOOKAHEAD=1`` in the environment) makes the
+    cache remember what a pass built and hand that list, at the first request
+    after the next ``reset()``, to a worker thread of the library, which builds
+    the levels and maps of the new cloud on a stream of its own while the
+    calling thread enqueues layers (:mod:`minuet_amd.nn.lookahead`).  Results
+    are the same; the price is one worst-case allocation per pass (no level has
+    more rows than the input cloud) and one such session per process at a time
+    (a second cache builds the ordinary way meanwhile).  ``num_ahead_hits``
+    counts the requests served that way."""
 
     def __init__(self, ndim: int, dtype: torch.dtype, device: Union[str, torch.device],
                  layout: str = "minuet", disable_reordering: bool = False, lookahead: bool = False):
