@@ -1647,7 +1647,7 @@ extern "C" int mnt_sorted_kernel_map_lists(const void *coords, int64_t n, int nd
       buf.counters = scope.alloc<unsigned>(buf.counter_words);
       buf.info = scope.alloc<unsigned>(4);
       buf.status = scope.alloc<unsigned>(4);
-      buf.chunks = scope.alloc<uint2>(chain_sort_max_pairs(n));
+      buf.chunks = scope.alloc<uint4>(chain_sort_max_pairs(n));
       buf.words = scope.alloc<unsigned long long>(n);
       buf.plan = scope.alloc<DevicePlan>(1);
       unsigned *row_totals = buf.counters + 2 * buckets;

@@ -50,7 +50,7 @@ struct ChainSortBuffers {
   unsigned *info;                // [4]
   unsigned *status;              // [4]: [0] set by the dealing kernel (non-zero: the sort declined),
                                  // [2] number of (bucket, chunk) pairs of the ranking launch
-  uint2 *chunks;                 // [chain_sort_max_pairs(n)]
+  uint4 *chunks;                 // [chain_sort_max_pairs(n)]
   unsigned long long *words;     // [n]
   DevicePlan *plan;              // query plan written by the ranking launch (nullable)
 };

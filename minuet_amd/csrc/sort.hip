@@ -295,6 +295,30 @@ struct FinalSink {
   }
 };
 
+// Output of the bucket sort's ranking step.  A one-round key spells its row
+// out (every field is c[k] - lo[k], nothing is dropped), so the sorted
+// coordinates are unpacked from the key instead of being fetched through the
+// permutation: that fetch is a 64-byte sector per 12-byte row at a random
+// place of the input.
+template <typename CT, typename IT>
+struct KeySink {
+  SortSpec spec;
+  IT *indices;
+  CT *sorted;
+  __device__ __forceinline__ void store(unsigned pos, unsigned long long key, unsigned val) const {
+    if (indices) indices[pos] = static_cast<IT>(val);
+    if (sorted) {
+#pragma unroll
+      for (int k = 0; k < MNT_MAX_NDIM; ++k) {
+        if (k < spec.ndim) {
+          sorted[static_cast<long long>(pos) * spec.ndim + k] =
+              static_cast<CT>(((key >> spec.shift[k]) & spec.mask[k]) + spec.lo[k]);
+        }
+      }
+    }
+  }
+};
+
 // ------------------------------------------------------------ radix sort ----
 
 constexpr int kMaxRadixBits = 11;
@@ -612,8 +636,10 @@ __host__ __device__ inline int single_round_spec(const long long *bounds, int nd
       const unsigned long long range = static_cast<unsigned long long>(bounds[MNT_MAX_NDIM + k]) -
                                        static_cast<unsigned long long>(bounds[k]);
       const int w = range == 0 ? 0 : 64 - __builtin_clzll(range);
+      // also for a dimension of one value, which takes no key bits: a key is
+      // turned back into its row by adding lo to every field
+      spec.lo[k] = static_cast<unsigned long long>(bounds[k]);
       if (w > 0) {
-        spec.lo[k] = static_cast<unsigned long long>(bounds[k]);
         spec.mask[k] = w >= 64 ? ~0ull : ((1ull << w) - 1ull);
         spec.shift[k] = bits & 63;
         bits += w;
@@ -762,10 +788,10 @@ __device__ __forceinline__ unsigned bucket_pieces(unsigned m) {
 // largest bucket (all ones when the layout does not hold)
 // and the number of pairs.
 // chunks[i] = {first row of the bucket, rows of the bucket | mode << 13 |
-// chunk << 16}.
+// chunk << 16, the bucket (the top bits of its rows' keys), 0}.
 __global__ __launch_bounds__(1024) void bucket_scan_kernel(
     const unsigned *__restrict__ totals, int buckets, unsigned *__restrict__ info,
-    unsigned *__restrict__ starts, unsigned *__restrict__ cursors, uint2 *__restrict__ chunks,
+    unsigned *__restrict__ starts, unsigned *__restrict__ cursors, uint4 *__restrict__ chunks,
     const long long *__restrict__ folded, long long *host_bounds,
     unsigned *host_out, unsigned long long *flag, unsigned long long sequence) {
   constexpr int kPer = kBucketMax / 1024;
@@ -837,8 +863,10 @@ __global__ __launch_bounds__(1024) void bucket_scan_kernel(
       if (v[j] <= kBucketCap) {
         const unsigned mine = bucket_pieces(v[j]);
         const unsigned head = v[j] | (bucket_mode(v[j]) << 13);
-        if (mine == 1) chunks[single_at++] = make_uint2(run, head);
-        for (unsigned c = 0; mine > 1 && c < mine; ++c) chunks[shared_at++] = make_uint2(run, head | (c << 16));
+        if (mine == 1) chunks[single_at++] = make_uint4(run, head, d, 0u);
+        for (unsigned c = 0; mine > 1 && c < mine; ++c) {
+          chunks[shared_at++] = make_uint4(run, head | (c << 16), d, 0u);
+        }
       }
     }
     run += v[j];
@@ -947,8 +975,8 @@ struct RankShared {
 
 template <typename CT, typename IT>
 __device__ __forceinline__ void rank_bucket_chunk(
-    const unsigned long long *__restrict__ words, const uint2 entry, int idx_bits, int word_bits,
-    const FinalSink<CT, IT> &sink, unsigned long long *s_words, RankShared &sh) {
+    const unsigned long long *__restrict__ words, const uint4 entry, int idx_bits, int word_bits,
+    const KeySink<CT, IT> &sink, unsigned long long *s_words, RankShared &sh) {
   unsigned (&part_cursor)[kSortBlock] = sh.part_cursor;
   unsigned (&part_start)[kSortBlock + 1] = sh.part_start;
   unsigned (&wave_sums)[kSortWaves] = sh.wave_sums;
@@ -958,6 +986,9 @@ __device__ __forceinline__ void rank_bucket_chunk(
   const unsigned mode = (entry.y >> 13) & 7u;
   const unsigned chunk = entry.y >> 16;
   const unsigned long long idx_mask = (1ull << idx_bits) - 1ull;
+  // key of a row = its bucket above the rest of the key that its word carries
+  const int rest_bits = word_bits - idx_bits;
+  const unsigned long long key_top = rest_bits >= 64 ? 0ull : static_cast<unsigned long long>(entry.z) << rest_bits;
 
   if (mode != kBucketSplit) {
     // words are read four at a time by each of the 1 << mode sharers
@@ -975,7 +1006,9 @@ __device__ __forceinline__ void rank_bucket_chunk(
     }
     // the sharers of a row sit in neighbouring lanes
     for (unsigned off = 1; off < (1u << mode); off <<= 1) rank += __shfl_xor(rank, off);
-    if (e < m && part == 0) sink.store(start + rank, 0ull, static_cast<unsigned>(mine & idx_mask));
+    if (e < m && part == 0) {
+      sink.store(start + rank, key_top | (mine >> idx_bits), static_cast<unsigned>(mine & idx_mask));
+    }
     return;
   }
 
@@ -1040,14 +1073,14 @@ __device__ __forceinline__ void rank_bucket_chunk(
       for (int u = 0; u < 8; ++u) rank += x[u] < mine ? 1u : 0u;
     }
     for (; j < hi; ++j) rank += s_words[j] < mine ? 1u : 0u;
-    sink.store(start + rank, 0ull, static_cast<unsigned>(mine & idx_mask));
+    sink.store(start + rank, key_top | (mine >> idx_bits), static_cast<unsigned>(mine & idx_mask));
   }
 }
 
 template <typename CT, typename IT>
 __global__ __launch_bounds__(kSortBlock) void bucket_rank_kernel(
-    const unsigned long long *__restrict__ words, const uint2 *__restrict__ chunks, int idx_bits,
-    int word_bits, FinalSink<CT, IT> sink) {
+    const unsigned long long *__restrict__ words, const uint4 *__restrict__ chunks, int idx_bits,
+    int word_bits, KeySink<CT, IT> sink) {
   extern __shared__ __align__(16) unsigned long long s_words[];
   __shared__ RankShared sh;
   rank_bucket_chunk<CT, IT>(words, chunks[blockIdx.x], idx_bits, word_bits, sink, s_words, sh);
@@ -1109,7 +1142,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_deal_scan_kernel(
     const CT *__restrict__ coords, int ndim, long long n, const long long *__restrict__ folded,
     int msd_cap, int idx_bits_, const unsigned *__restrict__ info,
     const unsigned *__restrict__ totals, unsigned *__restrict__ cursors,
-    uint2 *__restrict__ chunks_out, unsigned *__restrict__ status,
+    uint4 *__restrict__ chunks_out, unsigned *__restrict__ status,
     unsigned long long *__restrict__ words) {
   extern __shared__ __align__(16) unsigned s_deal[];
   __shared__ unsigned long long s_wave[kSortWaves];
@@ -1201,8 +1234,10 @@ __global__ __launch_bounds__(kSortBlock) void bucket_deal_scan_kernel(
         if (blockIdx.x == 0) {
           const unsigned pieces = bucket_pieces(v[j]);
           const unsigned head = v[j] | (bucket_mode(v[j]) << 13);
-          if (pieces == 1) chunks_out[single_at++] = make_uint2(run, head);
-          for (unsigned c = 0; pieces > 1 && c < pieces; ++c) chunks_out[shared_at++] = make_uint2(run, head | (c << 16));
+          if (pieces == 1) chunks_out[single_at++] = make_uint4(run, head, d, 0u);
+          for (unsigned c = 0; pieces > 1 && c < pieces; ++c) {
+            chunks_out[shared_at++] = make_uint4(run, head | (c << 16), d, 0u);
+          }
         }
       }
       run += v[j];
@@ -1258,7 +1293,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_deal_scan_kernel(
 // query plan of the launches that follow.
 template <typename CT, typename IT>
 __global__ __launch_bounds__(kSortBlock) void bucket_rank_chain_kernel(
-    const unsigned long long *__restrict__ words, const uint2 *__restrict__ chunks,
+    const unsigned long long *__restrict__ words, const uint4 *__restrict__ chunks,
     const unsigned *__restrict__ pair_count, int max_pairs, const long long *__restrict__ folded,
     int ndim, int msd_cap, int idx_bits, const unsigned *__restrict__ status, FinalSink<CT, IT> sink,
     OffsetTable offsets, int num_offsets, DevicePlan *__restrict__ plan_out) {
@@ -1276,7 +1311,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_rank_chain_kernel(
   }
   const unsigned pair = blockIdx.x - 1;
   const unsigned pairs = pair_count[0];
-  const uint2 entry = chunks[pair];                    // the list has room for max_pairs entries
+  const uint4 entry = chunks[pair];                    // the list has room for max_pairs entries
   long long bounds[2 * MNT_MAX_NDIM];
 #pragma unroll
   for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) bounds[slot] = folded[slot];
@@ -1284,7 +1319,8 @@ __global__ __launch_bounds__(kSortBlock) void bucket_rank_chain_kernel(
   SortSpec spec;
   const int key_bits = single_round_spec(bounds, ndim, 1, spec);
   const BucketLayout lay = bucket_layout(key_bits, msd_cap, idx_bits);
-  rank_bucket_chunk<CT, IT>(words, entry, idx_bits, lay.shift + idx_bits, sink, s_words, sh);
+  const KeySink<CT, IT> key_sink{spec, sink.indices, sink.sorted};
+  rank_bucket_chunk<CT, IT>(words, entry, idx_bits, lay.shift + idx_bits, key_sink, s_words, sh);
 }
 
 bool chain_sort_takes(int64_t n, int64_t num_batches, int num_offsets) {
@@ -1370,7 +1406,7 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
   const int idx_bits = bit_width(static_cast<unsigned long long>(n - 1));
   const int msd_cap = std::max(1, std::min(kBucketMaxBits, bit_width(static_cast<unsigned long long>(n / kBucketRows))));
   unsigned *bucket_starts = nullptr;
-  uint2 *bucket_chunks = nullptr;
+  uint4 *bucket_chunks = nullptr;
   unsigned long long *bucket_words = nullptr;
   if (try_buckets) {
     Arena &arena = scope.arena();
@@ -1379,7 +1415,7 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
     bucket_starts = scope.alloc<unsigned>(kBucketMax + 1);
     unsigned *cursors = scope.alloc<unsigned>(kBucketMax);
     // a bucket of m rows makes at most m / 256 + 1 pairs
-    bucket_chunks = scope.alloc<uint2>(kBucketMax + static_cast<size_t>(n / kSortBlock) + 1);
+    bucket_chunks = scope.alloc<uint4>(kBucketMax + static_cast<size_t>(n / kSortBlock) + 1);
     bucket_words = scope.alloc<unsigned long long>(n);
     const int num_partials = static_cast<int>(std::min<int64_t>(div_ceil(n, kBoundsBlock * 4), kBucketBoundsBlocks));
     long long *partial = scope.alloc<long long>(static_cast<size_t>(num_partials) * 8);
@@ -1492,7 +1528,7 @@ static void arg_sort_typed(const CT *coords, int64_t n, int ndim, const IT *batc
         const size_t lds = (static_cast<size_t>(biggest) + 128) * sizeof(unsigned long long);
         bucket_rank_kernel<CT, IT><<<pairs, kSortBlock, lds, stream>>>(
             words, bucket_chunks, lay.idx_bits, lay.shift + lay.idx_bits,
-            FinalSink<CT, IT>{coords, ndim, indices_out, sorted_out});
+            KeySink<CT, IT>{src.spec, indices_out, sorted_out});
         check_launch("bucket_rank_kernel");
         profile_mark("sort_rank", stream);
         return;
