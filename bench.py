@@ -41,11 +41,11 @@ def measured_traffic(kernel):
     return json.loads(match.group(1)).get(kernel)
 
 
-def map_step(_C, coords_dev, offsets):
+def map_step(_C, coords_dev, offsets, want_coordinates=False):
     """One Map step: unsorted voxels -> sorted voxels -> per-offset pair lists in
     the order KernelMapCache keeps them (rows by ascending size), one library call."""
-    _, sorted_dev, built = _C.sorted_kernel_map_lists(coords_dev, offsets, reorder=True)
-    return sorted_dev, built
+    built = _C.sorted_kernel_map_lists(coords_dev, offsets, reorder=True, result_only=True)
+    return built["coordinates"] if want_coordinates else None, built
 
 
 def cpu_model():
@@ -390,7 +390,7 @@ def main():
     while time.perf_counter() < spin_until:
         map_step(_C, coords_dev, offsets)
     for _ in range(max(1, args.warmup)):
-        sorted_dev, built = map_step(_C, coords_dev, offsets)
+        sorted_dev, built = map_step(_C, coords_dev, offsets, want_coordinates=True)
     torch.cuda.synchronize()
     nnz = int(built["sizes_host"].sum())
 

@@ -669,14 +669,17 @@ class SortedMapLists:
                        "order_host", "bounds", "source_masks", "target_masks")
 
 
-def sorted_kernel_map_lists(coordinates: torch.Tensor, offsets_host: np.ndarray, reorder: bool = True):
+def sorted_kernel_map_lists(coordinates: torch.Tensor, offsets_host: np.ndarray, reorder: bool = True,
+                            result_only: bool = False):
     """The Map step of a stride-1 layer on an unsorted cloud (one batch) in one
     library call: ``sort_coordinates`` then the lists-only ``kernel_map_build``
     of the sorted cloud onto itself.  Returns ``(indices int32 [n], sorted
     coordinates, built)`` with ``built`` a :class:`SortedMapLists` that reads
     like the dict :func:`kernel_map_build` returns for ``want_masks=False,
     want_lists=True`` (``bounds`` holds the 8 bounds of the cloud twice:
-    sources, then targets)."""
+    sources, then targets) and also holds ``"indices"`` and ``"coordinates"``;
+    ``result_only=True`` returns ``built`` alone, whose tensors are views made
+    when first asked for."""
     if coordinates.dim() != 2:
         _ensure_ndim("coordinates", coordinates, 2)
     device = coordinates.device
@@ -695,8 +698,11 @@ def sorted_kernel_map_lists(coordinates: torch.Tensor, offsets_host: np.ndarray,
     num_offsets = offs.shape[0]
     if n == 0 or num_offsets == 0:
         indices, out = sort_coordinates(coordinates)
-        return indices, out, kernel_map_build(out, out, offs, None, None, reorder, want_masks=False,
-                                              want_lists=True)
+        built = kernel_map_build(out, out, offs, None, None, reorder, want_masks=False, want_lists=True)
+        if result_only:
+            built = dict(built, indices=indices, coordinates=out)
+            return built
+        return indices, out, built
     if not coordinates.is_contiguous():
         coordinates = coordinates.contiguous()
     capacity = num_offsets * n
@@ -717,6 +723,8 @@ def sorted_kernel_map_lists(coordinates: torch.Tensor, offsets_host: np.ndarray,
     if status != 0:
         _check(status)
     built = SortedMapLists(store, coords_out, host, n, ndim, num_offsets)
+    if result_only:
+        return built
     return built["indices"], built["coordinates"], built
 
 

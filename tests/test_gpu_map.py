@@ -520,6 +520,14 @@ def _check_sorted_lists(cloud, off, reorder=True):
     ein, eout, _ = orc.kernel_map_pair_lists(em)
     np.testing.assert_array_equal(host(built["in_idx"]), ein)
     np.testing.assert_array_equal(host(built["out_idx"]), eout)
+    # the result object alone: the same tensors, made when asked for
+    alone = _C.sorted_kernel_map_lists(dev(cloud), off.astype(np.int64), reorder=reorder, result_only=True)
+    for key in ("indices", "coordinates", "in_idx", "out_idx", "sizes", "order"):
+        assert key in alone
+        np.testing.assert_array_equal(host(alone[key]), host(indices if key == "indices" else
+                                                             sorted_dev if key == "coordinates" else built[key]))
+    np.testing.assert_array_equal(alone["sizes_host"], built["sizes_host"])
+    np.testing.assert_array_equal(alone["order_host"], built["order_host"])
 
 
 @pytest.mark.parametrize("reorder", [True, False])
@@ -553,6 +561,17 @@ def test_sorted_kernel_map_lists_lidar_and_clustered():
     order = orc.arg_sort_coordinates(dup)
     np.testing.assert_array_equal(host(indices).astype(np.int64), order)
     np.testing.assert_array_equal(host(sorted_dev), dup[order])
+
+
+def test_sorted_kernel_map_lists_empty_cloud():
+    off = orc.generate_kernel_offsets(3, 3, 1, 1).astype(np.int64)
+    empty = np.zeros((0, 3), dtype=np.int32)
+    indices, sorted_dev, built = _C.sorted_kernel_map_lists(dev(empty), off)
+    assert indices.numel() == 0 and tuple(sorted_dev.shape) == (0, 3)
+    assert built["in_idx"].numel() == 0 and int(np.asarray(built["sizes_host"]).sum()) == 0
+    alone = _C.sorted_kernel_map_lists(dev(empty), off, result_only=True)
+    assert alone["indices"].numel() == 0 and tuple(alone["coordinates"].shape) == (0, 3)
+    assert alone["out_idx"].numel() == 0
 
 
 def test_sorted_kernel_map_lists_2d_and_4d():
