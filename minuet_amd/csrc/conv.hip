@@ -11,6 +11,7 @@
 // are multiplied in ONE grouped launch whose tiles never cross an offset, so
 // padded rows are never computed.
 #include <algorithm>
+#include <atomic>
 #include <cstring>
 
 #include "conv_device.h"
@@ -527,10 +528,20 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
   const int at_prefix = 1, at_start = at_prefix + G + 1, at_rows = at_start + G + 1, at_weight = at_rows + G,
             at_list = at_weight + G;
 
-  const int tid = threadIdx.x;
+  const int n0 = blockIdx.y * TN;
+  // A workgroup walks the tiles blockIdx.x, blockIdx.x + gridDim.x, ...: the
+  // grid is what the compute units hold at once, since workgroups that live for
+  // a few microseconds are launched more slowly than they finish.
+  const int num_tiles = entry(at_prefix + G);
+  for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
+  // (the thread's number is made opaque per tile: what is derived from it is
+  // worked out again for every tile instead of being kept in registers)
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
   const int lane = tid & 63;
   const int wv = tid >> 6;
-  const int tile = blockIdx.x;
+  const int r = lane & 31;
+  const int h = lane >> 5;
   int g_prefix, g_rows, g_start, g_weight, g_list;
   if (G <= kWave) {
     // One trip to memory instead of a search of dependent reads: lane i
@@ -564,12 +575,9 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
   const int r0 = (tile - g_prefix) * kGemmRows;
   const int valid = min(kGemmRows, g_rows - r0);
   const long long row_base = static_cast<long long>(g_start) + r0;
-  const int n0 = blockIdx.y * TN;
   const T *w_base = wt + (static_cast<long long>(g_weight) * Np + n0) * Kp;
   const int list_at = g_list;
 
-  const int r = lane & 31;
-  const int h = lane >> 5;
   const int row = wv * 32 + r;
   const bool row_ok = row < valid;
   long long a_index = row_base + row;
@@ -761,10 +769,12 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
       }
     }
   }
+  __syncthreads();                      // the next tile's weights go where this one's were (and its turned blocks)
+  }
 }
 
 template <typename T, typename TC, int NB, bool VEC, int CH>
-__global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
+__global__ __launch_bounds__(kGemmBlock, 3) void grouped_gemm_kernel(
     const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt,
     const int *__restrict__ meta, int K, int N, int Kp, int Np,
     const int *__restrict__ gather_index, const int *__restrict__ out_pos) {
@@ -773,7 +783,7 @@ __global__ __launch_bounds__(kGemmBlock) void grouped_gemm_kernel(
 
 // The same with the tables as a by-value argument.
 template <typename T, typename TC, int NB, bool VEC, int CH>
-__global__ __launch_bounds__(kGemmBlock) void grouped_gemm_riding_kernel(
+__global__ __launch_bounds__(kGemmBlock, 3) void grouped_gemm_riding_kernel(
     const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt, int K, int N, int Kp, int Np,
     const int *__restrict__ gather_index, PlanChunk table, int table_count, int meta_at,
     int *__restrict__ table_out, const int *__restrict__ out_pos) {
@@ -924,11 +934,31 @@ struct RidingTable {
   int *out = nullptr;
 };
 
+// Compute units of the current device (asked for once per device).
+static int compute_units() {
+  static std::atomic<int> known[64];
+  int device = 0;
+  MNT_HIP(hipGetDevice(&device));
+  const int slot = device & 63;
+  int units = known[slot].load(std::memory_order_relaxed);
+  if (units == 0) {
+    MNT_HIP(hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device));
+    units = units > 0 ? units : 256;
+    known[slot].store(units, std::memory_order_relaxed);
+  }
+  return units;
+}
+
 template <typename T, typename TC, int NB>
 static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int num_tiles, int K, int N,
                            int Kp, int Np, bool vec, const int *gather_index, const RidingTable &riding,
                            hipStream_t stream, const int *out_pos) {
-  dim3 grid(num_tiles, static_cast<unsigned>(div_ceil(Np, NB * 32)));
+  // as many workgroups as the compute units hold at once (by registers); each
+  // walks its share of the tiles
+  const int slices = static_cast<int>(div_ceil(Np, NB * 32));
+  const int resident = compute_units() * (NB >= 3 ? 3 : NB == 2 ? 4 : 6);
+  dim3 grid(static_cast<unsigned>(std::min(num_tiles, std::max(1, resident / slices))),
+            static_cast<unsigned>(slices));
   // rows of one or two chunks are loaded whole, ahead of the first product
   const int chunks = Kp / (kChunkBytes / static_cast<int>(sizeof(T)));
   const int held = vec && chunks <= 2 ? chunks : 0;
