@@ -132,6 +132,53 @@ __device__ __forceinline__ void finish_piece(float (&v)[E], const Epilogue &ep, 
   *reinterpret_cast<uint4 *>(out + (t * N + ch) * static_cast<long long>(sizeof(T))) = raw;
 }
 
+// Epilogue and store of one 32 x 32 block of fp32 sums as the matrix
+// instructions leave it (lane (r, h) holds channels q * 8 + h * 4 .. + 3 of
+// target block_t0 + r in acc[q * 4 .. + 3]), for output rows that are whole
+// 16-byte pieces: the wavefront turns the block around in its own `turn` area
+// of LDS (kTurnBytes), so that one store instruction covers rows in contiguous
+// pieces of 64 bytes (128 in fp32), and the residual is read the same way.
+constexpr int kTurnRow = 32 * 4 + 16;
+constexpr int kTurnBytes = 32 * kTurnRow;
+
+template <typename T>
+__device__ __forceinline__ void store_turned_block(const floatx16 &acc, unsigned char *turn, int lane, int r,
+                                                   int h, long long block_t0, long long num_targets, int ch0,
+                                                   int N, const Epilogue &ep, unsigned char *__restrict__ out) {
+  constexpr int EPV = 16 / static_cast<int>(sizeof(T));
+  constexpr int kOutPieces = 32 / EPV;                          // 16-byte pieces of a block's output row
+  constexpr int kPieces = 32 * kOutPieces / 64;                 // per lane
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    *reinterpret_cast<float4 *>(turn + r * kTurnRow + (q * 8 + h * 4) * 4) =
+        make_float4(acc[q * 4], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int i = 0; i < kPieces; ++i) {
+    const int piece = lane + i * 64;
+    const int pr = piece / kOutPieces, part = piece % kOutPieces;
+    const int ch = ch0 + part * EPV;
+    float v[EPV];
+#pragma unroll
+    for (int x = 0; x < EPV; x += 4) {
+      const float4 f = *reinterpret_cast<const float4 *>(turn + pr * kTurnRow + (part * EPV + x) * 4);
+      v[x] = f.x;
+      v[x + 1] = f.y;
+      v[x + 2] = f.z;
+      v[x + 3] = f.w;
+    }
+    if (block_t0 + pr < num_targets && ch < N) {                // N % EPV == 0: a piece is all in or all out
+      finish_piece<T, EPV>(v, ep, block_t0 + pr, ch, N, out);
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // KS: 32-byte steps of K per pipeline stage.  A source row takes `chunks`
 // stages of KS * 32 bytes (Kp * sizeof(T) must be a multiple of that when
 // chunks > 1).  packed_row = Kp, packed_rows = rows of one offset in wt.
@@ -157,8 +204,6 @@ __device__ __forceinline__ void implicit_forward_body(
   constexpr int kLdsRow = kStageBytes + 16;
   constexpr int kBufferBytes = Np * kLdsRow;
   // the output pass turns one 32 x 32 block of fp32 sums per wavefront around in the same memory
-  constexpr int kTurnRow = 32 * 4 + 16;
-  constexpr int kTurnBytes = 32 * kTurnRow;
   constexpr int kLdsBytes = 2 * kBufferBytes > 4 * kTurnBytes ? 2 * kBufferBytes : 4 * kTurnBytes;
   __shared__ __align__(16) unsigned char w_lds[kLdsBytes];
   const int num_stages = num_offsets * chunks;
@@ -367,9 +412,6 @@ __device__ __forceinline__ void implicit_forward_body(
   // covers rows in contiguous pieces of 64 bytes (128 in fp32), and the
   // residual is read the same way.
   if ((static_cast<long long>(N) * sizeof(T)) % 16 == 0) {
-    constexpr int EPV = 16 / static_cast<int>(sizeof(T));
-    constexpr int kOutPieces = 32 / EPV;                          // 16-byte pieces of a block's output row
-    constexpr int kPieces = 32 * kOutPieces / 64;                 // per lane and block
     unsigned char *turn = w_lds + wv * kTurnBytes;
 #pragma unroll
     for (int m = 0; m < MW; ++m) {
@@ -378,35 +420,7 @@ __device__ __forceinline__ void implicit_forward_body(
 #pragma unroll
       for (int b = 0; b < NB; ++b) {
         if (first_channel + b * 32 >= N) break;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          *reinterpret_cast<float4 *>(turn + r * kTurnRow + (q * 8 + h * 4) * 4) =
-              make_float4(acc[m][b][q * 4], acc[m][b][q * 4 + 1], acc[m][b][q * 4 + 2], acc[m][b][q * 4 + 3]);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-        for (int i = 0; i < kPieces; ++i) {
-          const int piece = lane + i * 64;
-          const int pr = piece / kOutPieces, part = piece % kOutPieces;
-          const int ch = first_channel + b * 32 + part * EPV;
-          float v[EPV];
-#pragma unroll
-          for (int x = 0; x < EPV; x += 4) {
-            const float4 f = *reinterpret_cast<const float4 *>(turn + pr * kTurnRow + (part * EPV + x) * 4);
-            v[x] = f.x;
-            v[x + 1] = f.y;
-            v[x + 2] = f.z;
-            v[x + 3] = f.w;
-          }
-          if (block_t0 + pr < num_targets && ch < N) {            // N % EPV == 0: a piece is all in or all out
-            finish_piece<T, EPV>(v, ep, block_t0 + pr, ch, N, out);
-          }
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        store_turned_block<T>(acc[m][b], turn, lane, r, h, block_t0, num_targets, first_channel + b * 32, N, ep, out);
       }
     }
     return;
@@ -438,6 +452,137 @@ __global__ __launch_bounds__(kImplicitBlock) void implicit_forward_kernel(
                                        chunks, packed_row, packed_rows, out, ep);
 }
 
+// Forward of a layer whose source rows are 4, 8 or 16 bytes of a 16-bit type
+// (a stem: 2, 4 or 8 input channels).  A pipeline stage per offset would be
+// all overhead for rows that short, so the offsets lie side by side along K
+// instead: K' = O * K, 16 elements per matrix instruction, and a lane's
+// 16-byte operand piece is 4, 2 or 1 whole source rows of consecutive offsets.
+// The weights [O][K][N], read as [O * K][N], are already the matrix to
+// multiply by: a workgroup puts them into LDS once, in operand order (piece
+// (step, channel block, lane) = 8 elements of K' for one output channel), and
+// each wavefront takes its blocks of 32 targets from there.  Nothing is
+// pipelined by hand: the kernel is short on registers, and the wavefronts a
+// SIMD holds cover each other's trips to memory.
+// Dynamic LDS: steps * NB KiB of weight pieces + 4 turn areas.
+constexpr int kNarrowBlock = 256;
+constexpr int kNarrowBlocksPerWave = 2;    // 32-target blocks a wavefront takes
+constexpr int kNarrowSteps = 8;            // steps of K' whose rows are in flight together
+constexpr int kNarrowMaxLds = 64 * 1024;
+
+// Whether narrow_forward_kernel takes the layer: 16-bit rows of 4, 8 or 16
+// bytes, at most 128 output channels, weights given as they are, and all of
+// them in LDS at once.
+static bool narrow_fits(int64_t O, int64_t K, int64_t N, int esize, bool has_weights) {
+  const int64_t row_bytes = K * esize;
+  if (esize != 2 || (row_bytes != 4 && row_bytes != 8 && row_bytes != 16) || !has_weights ||
+      N > 32 * kImplicitMaxBlocks) {
+    return false;
+  }
+  const int64_t lds = div_ceil(O * K, 16) * div_ceil(N, 32) * 1024 + (kNarrowBlock / 64) * kTurnBytes;
+  return lds <= kNarrowMaxLds;
+}
+
+template <typename T, int NB, int RB>
+__global__ __launch_bounds__(kNarrowBlock, NB == 1 ? 4 : 2) void narrow_forward_kernel(
+    const unsigned char *__restrict__ sources, const T *__restrict__ weights,
+    const int *__restrict__ kernel_map, long long num_targets, int num_offsets, int N, int steps,
+    unsigned char *__restrict__ out, Epilogue ep) {
+  constexpr int SL = 16 / RB;                                   // source rows per operand piece
+  constexpr int KR = RB / static_cast<int>(sizeof(T));          // input channels
+  typedef typename VecOf<RB>::type RowVec;
+  extern __shared__ __align__(16) unsigned char narrow_lds[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wv = tid >> 6;
+  const int r = lane & 31;
+  const int h = lane >> 5;
+  {
+    // a thread gathers whole pieces: eight loads in flight, then one LDS store
+    const int total_k = num_offsets * KR;
+    const int count = steps * NB * 64;
+    for (int p = tid; p < count; p += kNarrowBlock) {
+      const int ln = p & 63, sb = p >> 6;
+      const int b = sb % NB, s = sb / NB;
+      const int k0 = 16 * s + 8 * (ln >> 5);
+      const int n = b * 32 + (ln & 31);
+      T e[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        e[i] = (k0 + i < total_k && n < N) ? weights[static_cast<long long>(k0 + i) * N + n] : static_cast<T>(0.0f);
+      }
+      reinterpret_cast<uint4 *>(narrow_lds)[p] = *reinterpret_cast<const uint4 *>(e);
+    }
+  }
+  __syncthreads();
+  const uint4 *w_pieces = reinterpret_cast<const uint4 *>(narrow_lds) + lane;
+  unsigned char *turn = narrow_lds + static_cast<size_t>(steps) * NB * 1024 + wv * kTurnBytes;
+  const bool turned = (static_cast<long long>(N) * sizeof(T)) % 16 == 0;
+  for (int j = 0; j < kNarrowBlocksPerWave; ++j) {
+    const long long block_t0 =
+        ((static_cast<long long>(blockIdx.x) * kNarrowBlocksPerWave + j) * (kNarrowBlock / 64) + wv) * 32;
+    if (block_t0 >= num_targets) break;
+    const long long t = block_t0 + r;
+    const bool t_ok = t < num_targets;
+    const int *column = kernel_map + (t_ok ? t : num_targets - 1);
+    floatx16 acc[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+#pragma unroll
+      for (int x = 0; x < 16; ++x) acc[b][x] = 0.0f;
+    }
+    for (int s0 = 0; s0 < steps; s0 += kNarrowSteps) {
+      int index[kNarrowSteps][SL];
+#pragma unroll
+      for (int g = 0; g < kNarrowSteps; ++g) {
+#pragma unroll
+        for (int q = 0; q < SL; ++q) {
+          const int o = (2 * (s0 + g) + h) * SL + q;
+          index[g][q] = (t_ok && o < num_offsets) ? column[static_cast<long long>(o) * num_targets] : -1;
+        }
+      }
+      uint4 piece[kNarrowSteps];
+#pragma unroll
+      for (int g = 0; g < kNarrowSteps; ++g) {
+        RowVec rows[SL];
+#pragma unroll
+        for (int q = 0; q < SL; ++q) {
+          rows[q] = RowVec{};
+          if (index[g][q] >= 0) {
+            rows[q] = *reinterpret_cast<const RowVec *>(sources + static_cast<long long>(index[g][q]) * RB);
+          }
+        }
+        piece[g] = *reinterpret_cast<const uint4 *>(rows);
+      }
+#pragma unroll
+      for (int g = 0; g < kNarrowSteps; ++g) {
+        if (s0 + g < steps) {
+#pragma unroll
+          for (int b = 0; b < NB; ++b) {
+            acc[b] = Mfma<T>::run(w_pieces[((s0 + g) * NB + b) * 64], piece[g], acc[b]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      if (b * 32 >= N) break;
+      if (turned) {
+        store_turned_block<T>(acc[b], turn, lane, r, h, block_t0, num_targets, b * 32, N, ep, out);
+      } else if (t_ok) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int ch = b * 32 + q * 8 + h * 4;
+          if (ch >= N) continue;               // N % 4 == 0: a group of four is all in or all out
+          float v[4];
+#pragma unroll
+          for (int x = 0; x < 4; ++x) v[x] = acc[b][q * 4 + x];
+          finish_four<T>(v, ep, t, ch, N, out);
+        }
+      }
+    }
+  }
+}
+
 // inverse[o][m] = t for every hit kernel_map[o][t] = m (at most one t per
 // (o, m): the targets of one offset are distinct translates of their sources).
 __global__ __launch_bounds__(256) void invert_map_kernel(const int *__restrict__ kernel_map,
@@ -466,10 +611,45 @@ static void implicit_typed(const T *sources, const T *weights, const T *packed, 
                            int64_t S, int64_t Tn, int64_t O, int64_t K, int64_t N, const Epilogue &ep,
                            T *out, hipStream_t stream) {
   Scope scope(stream);
+  profile_mark("enter:implicit", stream);
+  if constexpr (sizeof(T) == 2) {
+    if (narrow_fits(O, K, N, sizeof(T), weights != nullptr)) {
+      {
+        const int64_t narrow_bytes = K * static_cast<int64_t>(sizeof(T));
+        const int steps = static_cast<int>(div_ceil(O * K, 16));
+        const int blocks = static_cast<int>(div_ceil(N, 32));
+        const size_t lds = static_cast<size_t>(steps) * blocks * 1024 + (kNarrowBlock / 64) * kTurnBytes;
+        const unsigned grid = static_cast<unsigned>(
+            div_ceil(Tn, int64_t{32} * (kNarrowBlock / 64) * kNarrowBlocksPerWave));
+#define MNT_NARROW(NB, RB)                                                                              \
+  narrow_forward_kernel<T, NB, RB><<<grid, kNarrowBlock, lds, stream>>>(                                \
+      reinterpret_cast<const unsigned char *>(sources), weights, kernel_map, Tn, static_cast<int>(O),   \
+      static_cast<int>(N), steps, reinterpret_cast<unsigned char *>(out), ep)
+#define MNT_NARROW_RB(NB)            \
+  if (narrow_bytes == 4) {           \
+    MNT_NARROW(NB, 4);               \
+  } else if (narrow_bytes == 8) {    \
+    MNT_NARROW(NB, 8);               \
+  } else {                           \
+    MNT_NARROW(NB, 16);              \
+  }
+        switch (blocks) {
+          case 1: MNT_NARROW_RB(1); break;
+          case 2: MNT_NARROW_RB(2); break;
+          case 3: MNT_NARROW_RB(3); break;
+          default: MNT_NARROW_RB(4); break;
+        }
+#undef MNT_NARROW_RB
+#undef MNT_NARROW
+        check_launch("narrow_forward_kernel");
+        profile_mark("implicit", stream);
+        return;
+      }
+    }
+  }
   const int kc = kChunkBytes / static_cast<int>(sizeof(T));
   const int Kp = static_cast<int>(div_ceil(K, kc) * kc);
   const int Np = static_cast<int>(div_ceil(N, 32) * 32);
-  profile_mark("enter:implicit", stream);
   const T *wt = packed;
   if (packed == nullptr) {
     T *fresh = scope.alloc<T>(static_cast<size_t>(O) * Np * Kp);
@@ -553,10 +733,12 @@ extern "C" int mnt_sparse_convolution_forward_implicit(
     MNT_CHECK(S * K * esize < static_cast<int64_t>(kMaxSourceBytes),
               "source features of %lld bytes exceed the 4 GiB a buffer resource addresses",
               (long long)(S * K * esize));
-    MNT_CHECK((K * esize) % 16 == 0 && K * esize <= kImplicitMaxRowBytes && N % 4 == 0 &&
+    const bool narrow = narrow_fits(O, K, N, esize, weights != nullptr);
+    MNT_CHECK(((K * esize) % 16 == 0 || narrow) && K * esize <= kImplicitMaxRowBytes && N % 4 == 0 &&
                   N <= 32 * kImplicitMaxBlocks * kImplicitMaxGroups,
               "Unsupported channel counts for the implicit forward: Cin = %lld (rows must be a multiple "
-              "of 16 bytes, at most %d), Cout = %lld (a multiple of 4, at most %d)",
+              "of 16 bytes, at most %d; 16-bit rows of 4 or 8 bytes are taken too where weights are given "
+              "unpacked, Cout is at most 128 and the kernel is small), Cout = %lld (a multiple of 4, at most %d)",
               (long long)K, kImplicitMaxRowBytes, (long long)N, 32 * kImplicitMaxBlocks * kImplicitMaxGroups);
     MNT_CHECK(activation >= MNT_ACT_NONE && activation <= MNT_ACT_RELU6, "unknown activation code %d",
               activation);

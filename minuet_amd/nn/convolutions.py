@@ -615,17 +615,20 @@ class SparseConv(Module):
         return self._packed[1], self._packed[2]
 
     def _row_padding(self, features: torch.Tensor) -> int:
-        """Zero input channels to append so that feature rows become a multiple
-        of 16 bytes, when that lets a 16-bit layer (a stem with 3 or 4 input
-        channels, say) take the single-kernel dataflow; else 0."""
-        per_piece = 16 // features.element_size()
-        pad = -self.in_channels % per_piece
-        if (pad == 0 or features.dtype == torch.float32 or not features.is_cuda
-                or self._tunable_config.get("dataflow", "auto") in ("gather_gemm_scatter", "list_driven")
-                or not _C.implicit_forward_supported(self.in_channels + pad, self.out_channels,
-                                                     features.dtype)):
+        """Zero input channels to append so that the feature rows of a 16-bit
+        layer become ones the single-kernel dataflow takes (4 or 8 bytes under
+        a small kernel, else a multiple of 16 bytes); 0 where they already are,
+        or where that dataflow is not an option."""
+        if (features.dtype == torch.float32 or not features.is_cuda
+                or self._tunable_config.get("dataflow", "auto") in ("gather_gemm_scatter", "list_driven")):
             return 0
-        return pad
+        esize = features.element_size()
+        row_bytes = self.in_channels * esize
+        widths = [b // esize for b in (4, 8) if row_bytes <= b] + [-(-row_bytes // 16) * 16 // esize]
+        for width in widths:
+            if _C.implicit_forward_supported(width, self.out_channels, features.dtype, self.kernel.shape[0]):
+                return width - self.in_channels
+        return 0
 
     def _takes_implicit(self, features: torch.Tensor, pad: int) -> bool:
         """Whether this call runs the single-kernel dataflow: forced by the

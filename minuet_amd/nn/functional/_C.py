@@ -1193,13 +1193,27 @@ IMPLICIT_MAX_TARGET_FEATURES = 512
 IMPLICIT_MAX_SOURCE_ROW_BYTES = 2048
 
 
+IMPLICIT_NARROW_LDS_BYTES = 64 * 1024
+_IMPLICIT_TURN_BYTES = 4 * 32 * (32 * 4 + 16)
+
+
 def implicit_forward_supported(num_source_features: int, num_target_features: int,
-                               dtype: torch.dtype) -> bool:
-    """Shapes ``sparse_convolution_forward_implicit`` accepts."""
+                               dtype: torch.dtype, num_offsets: Optional[int] = None) -> bool:
+    """Shapes ``sparse_convolution_forward_implicit`` accepts: source rows of a
+    multiple of 16 bytes, or, for 16-bit features, rows of 4 or 8 bytes (a
+    stem's 2 or 4 input channels) under a kernel of ``num_offsets`` offsets
+    small enough for its weights to sit in LDS as a whole."""
     row_bytes = num_source_features * dtype.itemsize
-    return (row_bytes % 16 == 0 and row_bytes <= IMPLICIT_MAX_SOURCE_ROW_BYTES
-            and num_target_features % 4 == 0
-            and num_target_features <= IMPLICIT_MAX_TARGET_FEATURES)
+    if (num_target_features % 4 != 0 or num_target_features > IMPLICIT_MAX_TARGET_FEATURES
+            or row_bytes > IMPLICIT_MAX_SOURCE_ROW_BYTES):
+        return False
+    if row_bytes % 16 == 0:
+        return row_bytes > 0
+    if dtype.itemsize != 2 or row_bytes not in (4, 8) or num_offsets is None or num_target_features > 128:
+        return False
+    steps = -(-num_offsets * num_source_features // 16)
+    blocks = -(-num_target_features // 32)
+    return steps * blocks * 1024 + _IMPLICIT_TURN_BYTES <= IMPLICIT_NARROW_LDS_BYTES
 
 
 def sparse_convolution_forward_implicit(sources: torch.Tensor, weights: torch.Tensor,

@@ -38,7 +38,7 @@ def prefers_implicit(num_offsets: int, num_source_features: int, num_target_feat
     saves).  fp32 matrix work is 16x dearer, so there it only pays where most
     (offset, target) pairs are hits, i.e. for small layers with strided 2^D
     kernels."""
-    if not _C.implicit_forward_supported(num_source_features, num_target_features, dtype):
+    if not _C.implicit_forward_supported(num_source_features, num_target_features, dtype, num_offsets):
         return False
     if dtype != torch.float32:
         row_bytes = num_source_features * dtype.itemsize

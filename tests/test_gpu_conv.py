@@ -176,8 +176,50 @@ def test_forward_implicit(kind, kernel, stride, cin, cout, n, extent):
     assert_features_close(out, ref, kind)
 
 
+@pytest.mark.parametrize("kind", ["fp16", "bf16"])
+@pytest.mark.parametrize("kernel,stride,cin,cout,n,extent", [
+    (3, 1, 4, 32, 20000, 60), (3, 1, 2, 32, 5000, 20), (3, 1, 8, 32, 6000, 25), (3, 1, 4, 16, 3000, 16),
+    (3, 1, 4, 64, 4000, 20), (3, 1, 4, 100, 2000, 12), (2, 2, 4, 128, 6000, 30), (5, 1, 4, 32, 3000, 16),
+    (5, 1, 2, 48, 2500, 14), (1, 1, 4, 12, 999, 12), ((3, 1, 2), 1, 8, 24, 3000, 16), (3, 1, 4, 32, 31, 4),
+])
+def test_forward_implicit_narrow_rows(kind, kernel, stride, cin, cout, n, extent):
+    """Source rows of 4, 8 or 16 bytes (the offsets side by side along K, the
+    weights in LDS as they are) against the float64 oracle."""
+    dtype = TORCH[kind]
+    src, sbd, tgt, tbd, off, feats, weights = make_layer_case(6, n, extent, kernel, cin, cout, kind, stride)
+    assert _C.implicit_forward_supported(cin, cout, dtype, off.shape[0])
+    kmap = orc.query_sorted_index_with_offsets(src, tgt, off, sbd, tbd)
+    esm, etm, eorder, esizes, _ = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=True)
+    conv = orc.sparse_convolution_forward(feats, weights, esm, etm, eorder, esizes)
+    _C.profile_enable(True)
+    out = _C.sparse_convolution_forward_implicit(dev(feats).to(dtype), dev(weights).to(dtype), dev(kmap))
+    stages = [name for name, _ in _C.profile_read()]
+    _C.profile_enable(False)
+    assert "pack_weights" not in stages               # the short-row kernel reads the weights as they are
+    assert out.dtype == dtype and out.shape == (tgt.shape[0], cout)
+    assert_features_close(out, conv, kind)
+    rng = np.random.default_rng(5)
+    scale = rng.uniform(0.5, 1.5, size=cout).astype(np.float32)
+    shift = rng.uniform(-0.5, 0.5, size=cout).astype(np.float32)
+    residual = quantise(rng.normal(size=conv.shape), kind)
+    ref = conv * scale.astype(np.float64) + shift.astype(np.float64) + residual
+    # (no ReLU for bf16: it halves the RMS the bound is taken from, and rounding
+    # an output of five times that RMS to 8 bits then exceeds the bound by itself)
+    activation = "relu" if kind == "fp16" else None
+    if activation == "relu":
+        ref = np.maximum(ref, 0.0)
+    out = _C.sparse_convolution_forward_implicit(
+        dev(feats).to(dtype), dev(weights).to(dtype), dev(kmap),
+        epilogue=F.Epilogue(dev(scale), dev(shift), dev(residual).to(dtype), activation))
+    assert_features_close(out, ref, kind)
+
+
 def test_forward_implicit_rejects_unsupported_shapes():
-    assert not _C.implicit_forward_supported(4, 32, torch.float16)       # 8-byte rows
+    assert not _C.implicit_forward_supported(4, 32, torch.float16)       # 8-byte rows, kernel unknown
+    assert _C.implicit_forward_supported(4, 32, torch.float16, 27)
+    assert not _C.implicit_forward_supported(4, 128, torch.float16, 125)  # weights beyond LDS
+    assert not _C.implicit_forward_supported(3, 32, torch.float16, 27)    # 6-byte rows
+    assert not _C.implicit_forward_supported(1, 32, torch.float32, 27)
     assert not _C.implicit_forward_supported(32, 30, torch.float16)
     assert not _C.implicit_forward_supported(32, 516, torch.float16)
     assert not _C.implicit_forward_supported(1032, 32, torch.float16)    # rows beyond 2048 bytes
@@ -186,7 +228,11 @@ def test_forward_implicit_rejects_unsupported_shapes():
     kmap = torch.full((27, 10), -1, dtype=torch.int32, device="cuda")
     with pytest.raises(RuntimeError, match="Unsupported channel counts"):
         _C.sparse_convolution_forward_implicit(torch.zeros(10, 4, device="cuda").half(),
-                                               torch.zeros(27, 4, 32, device="cuda").half(), kmap)
+                                               torch.zeros(125, 4, 128, device="cuda").half(),
+                                               torch.full((125, 10), -1, dtype=torch.int32, device="cuda"))
+    with pytest.raises(RuntimeError, match="Unsupported channel counts"):
+        _C.sparse_convolution_forward_implicit(torch.zeros(10, 3, device="cuda").half(),
+                                               torch.zeros(27, 3, 32, device="cuda").half(), kmap)
     out = _C.sparse_convolution_forward_implicit(torch.ones(10, 8, device="cuda").half(),
                                                  torch.ones(27, 8, 32, device="cuda").half(), kmap)
     assert torch.count_nonzero(out).item() == 0                        # no hits: all zero
@@ -217,10 +263,11 @@ def test_packed_weights_follow_the_parameter():
                 torch.zeros(3, device="cuda").half(), conv.kernel)
 
 
-@pytest.mark.parametrize("cin", [3, 4, 12])
+@pytest.mark.parametrize("cin", [1, 3, 4, 5, 12])
 def test_narrow_rows_are_padded_for_the_single_kernel_form(cin):
     """16-bit layers whose rows are not a multiple of 16 bytes (stems) still
-    take the implicit dataflow, through zero channels appended on the fly."""
+    take the implicit dataflow: rows of 4 or 8 bytes as they are, others
+    through zero channels appended on the fly."""
     src, sbd, tgt, tbd, off, feats, weights = make_layer_case(13, 4000, 18, 3, cin, 32, "fp16")
     esm, etm, eorder, esizes, _ = orc.build_kernel_map(src, sbd, tgt, tbd, off, reorder=True)
     ref = orc.sparse_convolution_forward(feats, weights, esm, etm, eorder, esizes)
