@@ -170,6 +170,9 @@ void profile_mark(const char *label, hipStream_t stream);
 
 // ---------------------------------------------------------------- launch ----
 
+// Compute units of the current device (asked for once per device).
+int compute_units();
+
 inline int64_t div_ceil(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 inline unsigned grid_for(int64_t items, int block, int64_t cap = (int64_t(1) << 20)) {

@@ -11,7 +11,6 @@
 // are multiplied in ONE grouped launch whose tiles never cross an offset, so
 // padded rows are never computed.
 #include <algorithm>
-#include <atomic>
 #include <cstring>
 
 #include "conv_device.h"
@@ -933,21 +932,6 @@ struct RidingTable {
   int meta_at = 0;
   int *out = nullptr;
 };
-
-// Compute units of the current device (asked for once per device).
-static int compute_units() {
-  static std::atomic<int> known[64];
-  int device = 0;
-  MNT_HIP(hipGetDevice(&device));
-  const int slot = device & 63;
-  int units = known[slot].load(std::memory_order_relaxed);
-  if (units == 0) {
-    MNT_HIP(hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device));
-    units = units > 0 ? units : 256;
-    known[slot].store(units, std::memory_order_relaxed);
-  }
-  return units;
-}
 
 template <typename T, typename TC, int NB>
 static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int num_tiles, int K, int N,

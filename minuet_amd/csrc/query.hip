@@ -421,7 +421,18 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
   __shared__ long long s_bounds[2];
   // dynamic LDS: [group table: 4 words each][member table: 2 words each][hit counts]
   // [row directory: dir_rows 16-bit entries]
-  const int4 *s_groups = reinterpret_cast<const int4 *>(s_dynamic);
+  // With gridDim.y > 1 the offset groups are dealt over the y index: every
+  // workgroup of a tile finds and stages the same window and resolves its
+  // share of the groups (a cloud of a few tiles fills the chip that way).
+  int my_first_group = 0, my_groups = num_groups;
+  if (gridDim.y > 1) {
+    const int share = (num_groups + static_cast<int>(gridDim.y) - 1) / static_cast<int>(gridDim.y);
+    my_first_group = static_cast<int>(blockIdx.y) * share;
+    my_groups = min(num_groups, my_first_group + share) - my_first_group;
+    if (my_groups <= 0) return;
+  }
+  const int4 *s_all_groups = reinterpret_cast<const int4 *>(s_dynamic);
+  const int4 *s_groups = s_all_groups + my_first_group;
   const int2 *s_members = reinterpret_cast<const int2 *>(s_dynamic + 4 * num_groups);
   unsigned *s_counts = s_dynamic + 4 * num_groups + 2 * num_offsets;
   unsigned *s_dir_words = s_counts + num_offsets;
@@ -522,17 +533,17 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
       resolve_chunk_rows<OT, WHOLE, kLists>(reinterpret_cast<const unsigned *>(win), s_dir, len,   \
                                             zbits, static_cast<unsigned>(num_rows), base, c0, key, \
                                             valid, answers_from, answers_to, s_groups, s_members,  \
-                                            num_groups, s_counts, counting, t, num_targets,        \
+                                            my_groups, s_counts, counting, t, num_targets,        \
                                             kernel_map, sink);                                     \
     } else if (narrow) {                                                                           \
       resolve_chunk<unsigned, OT, WHOLE, kLists>(reinterpret_cast<const unsigned *>(win), top,     \
                                                  base, c0, key, valid, answers_from, answers_to,   \
-                                                 s_groups, s_members, num_groups, s_counts,        \
+                                                 s_groups, s_members, my_groups, s_counts,        \
                                                  counting, t, num_targets, kernel_map, sink);      \
     } else {                                                                                       \
       resolve_chunk<unsigned long long, OT, WHOLE, kLists>(win, top, 0ull, c0, key, valid,         \
                                                            answers_from, answers_to, s_groups,     \
-                                                           s_members, num_groups, s_counts,        \
+                                                           s_members, my_groups, s_counts,        \
                                                            counting, t, num_targets, kernel_map,   \
                                                            sink);                                  \
     }
@@ -545,7 +556,10 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
   }
   if (tile_counts != nullptr) {
     __syncthreads();
-    for (int o = tid; o < num_offsets; o += kQueryThreads) {
+    // the offsets of this workgroup's groups: a run of the member table
+    const int4 last_group = s_groups[my_groups - 1];
+    for (int m = s_groups[0].z + tid; m < last_group.z + last_group.w; m += kQueryThreads) {
+      const int o = s_members[m].y;
       const unsigned hits = s_counts[o];
       tile_counts[static_cast<long long>(o) * num_tiles + blockIdx.x] = hits;
       if (kLists && hits != 0) atomicAdd(&sink.row_totals[o], hits);
@@ -1115,7 +1129,16 @@ static void launch_query(const QueryArgs &a, const QueryPlan &plan, const int *d
   CarriedTables carried;
   memset(&carried, 0, sizeof(carried));
   if (d_tables == nullptr) memcpy(carried.v, plan.tables.data(), sizeof(int) * plan.tables.size());
-  query_kernel<CT, BT, OT, kLists><<<num_tiles, kQueryThreads, dyn, stream>>>(
+  // a cloud of fewer tiles than compute units: the offset groups of a tile go
+  // to several workgroups (not under kLists, whose staging is per tile)
+  int split = 1;
+  if (!kLists && plan.num_groups > 1 && num_tiles > 0) {
+    const int wanted = std::min(plan.num_groups, std::max(1, compute_units() / num_tiles));
+    const int share = static_cast<int>(div_ceil(plan.num_groups, wanted));
+    split = static_cast<int>(div_ceil(plan.num_groups, share));
+  }
+  const dim3 grid(static_cast<unsigned>(num_tiles), static_cast<unsigned>(split));
+  query_kernel<CT, BT, OT, kLists><<<grid, kQueryThreads, dyn, stream>>>(
       src, tgt, plan.frame, d_tables, carried, plan.num_groups, num_offsets, plan.delta_min,
       plan.delta_max, kernel_map, tile_counts, num_tiles, dir_rows, sink, nullptr);
   check_launch("query_kernel");

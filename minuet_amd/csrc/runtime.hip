@@ -193,6 +193,20 @@ static constexpr size_t kMaxMarks = 4096;
 
 static std::thread::id g_profile_thread;
 
+int compute_units() {
+  static std::atomic<int> known[64];
+  int device = 0;
+  MNT_HIP(hipGetDevice(&device));
+  const int slot = device & 63;
+  int units = known[slot].load(std::memory_order_relaxed);
+  if (units == 0) {
+    MNT_HIP(hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device));
+    units = units > 0 ? units : 256;
+    known[slot].store(units, std::memory_order_relaxed);
+  }
+  return units;
+}
+
 void profile_mark(const char *label, hipStream_t stream) {
   // marks are kept for the thread that turned profiling on: the look-ahead
   // worker runs the same entry points on another stream at the same time
