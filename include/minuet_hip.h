@@ -490,7 +490,12 @@ int mnt_time_gemm(int allow_shortcut_matmul, int64_t parallel, int has_threshold
  * [O, Cin, Cout] in the same offset order.  No gather or GEMM-output buffer is
  * written: each wavefront keeps 32 output rows in its matrix accumulators and
  * walks the offsets.  Requires Cin * sizeof(element) to be a multiple of 16
- * and at most 2048, Cout % 4 == 0 and Cout <= 512.  Rows beyond 128 bytes are
+ * and at most 2048, Cout % 4 == 0 and Cout <= 512.  16-bit rows of 4 or 8
+ * bytes (2 or 4 input channels) are taken as well when `weights` is given,
+ * Cout <= 128 and ceil(O * Cin / 16) * ceil(Cout / 32) KiB + 18 KiB of LDS
+ * stay within 64 KiB: such layers, and 16-byte rows under the same
+ * conditions, run a kernel that lays the offsets side by side along K and
+ * reads `weights` as they are (packed_weights is not used).  Rows beyond 128 bytes are
  * walked in chunks and more than 128 output channels in groups of 128; the
  * form pays for rows of up to 128 bytes and up to 128 output channels, where
  * the three-kernel form is bound by its buffer traffic, and loses beyond
