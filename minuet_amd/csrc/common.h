@@ -121,6 +121,12 @@ class Arena {
     alignas(8) unsigned char blob[256] = {0};
   } pending;
 
+  // The target bitmap in persistent block 0 is left all zero by the kernel
+  // that walks it: the words from the block's start on that are known to be
+  // zero (0 after anything else has written there, or after the block moved).
+  long long zero_bitmap_words = 0;
+  long long zero_bitmap_words_after = 0;   // what the count becomes once the walk of the build under way is launched
+
   // State handed from mnt_kernel_map_query to mnt_kernel_map_emit.
   bool map_state_valid = false;
   alignas(8) unsigned char map_state[64] = {0};

@@ -180,6 +180,7 @@ void *Arena::persistent(int slot, size_t bytes) {
     }
     persistent_size_[slot] = align_up(bytes + bytes / 4, 1 << 20);
     MNT_HIP(hipMalloc(&persistent_[slot], persistent_size_[slot]));
+    if (slot == 0) zero_bitmap_words = 0;
   }
   return persistent_[slot];
 }

@@ -5,6 +5,8 @@
 // FillUniqueCoordinates (csrc/minuet/cuda/functions/unique_coordinates.cu:10-102,
 // csrc/minuet/cuda/kernels/fill_unique_coordinate.cuh:8-22) and
 // KernelMapCache.get_target_coordinates (minuet/nn/convolutions.py:84-99).
+#include <algorithm>
+
 #include "device_utils.h"
 #include "sort.h"
 
@@ -254,6 +256,10 @@ static int bit_width64(unsigned long long range) {
 constexpr int kBitmapMaxBits = 28;                   // 32 MiB of bits
 constexpr int kBitmapWords = 8;                      // 32-bit words per thread
 constexpr int kBitmapTile = kScanBlock * kBitmapWords;
+// persistent block 0 in the bitmap form: the tile bases of the largest bitmap
+// first, so that the bitmap itself always starts at the same place
+constexpr size_t kBitmapBasesBytes =
+    ((((size_t{1} << (kBitmapMaxBits - 5)) / kBitmapTile + 1) * 4 + 255) / 256) * 256;
 
 template <typename CT, typename IT>
 __device__ __forceinline__ unsigned long long target_key(const CT *__restrict__ coords, long long i,
@@ -279,11 +285,25 @@ __global__ __launch_bounds__(256) void mark_targets_kernel(const CT *__restrict_
                                                            TargetSpec spec,
                                                            const IT *__restrict__ batch_dims,
                                                            unsigned *__restrict__ bitmap) {
+  // Rows that follow each other in a sorted cloud fall into the same word of
+  // the bitmap more often than not (their cells differ in the last coordinate
+  // only): a run of neighbouring lanes with one word ORs its bits into the
+  // run's first lane, which issues the run's only atomic.
   const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
-  for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
-       i += stride) {
-    const unsigned long long key = target_key<CT, IT>(coords, i, spec, batch_dims);
-    atomicOr(&bitmap[key >> 5], 1u << (key & 31u));
+  const int lane = static_cast<int>(lane_id());
+  for (long long first = static_cast<long long>(blockIdx.x) * blockDim.x; first < n; first += stride) {
+    const long long i = first + threadIdx.x;
+    const bool valid = i < n;
+    const unsigned long long key = valid ? target_key<CT, IT>(coords, i, spec, batch_dims) : 0ull;
+    const unsigned word = valid ? static_cast<unsigned>(key >> 5) : 0xffffffffu;   // no word has this index
+    unsigned bits = valid ? 1u << (key & 31u) : 0u;
+    for (int off = 1; off < kWave; off <<= 1) {
+      const unsigned next_word = __shfl_down(word, off);
+      const unsigned next_bits = __shfl_down(bits, off);
+      if (lane + off < kWave && next_word == word) bits |= next_bits;
+    }
+    const unsigned word_before = __shfl_up(word, 1);
+    if (valid && (lane == 0 || word_before != word)) atomicOr(&bitmap[word], bits);
   }
 }
 
@@ -307,29 +327,37 @@ __global__ __launch_bounds__(1024) void bitmap_scan_kernel(unsigned *__restrict_
                                                            unsigned *host_count,
                                                            unsigned long long *flag,
                                                            unsigned long long sequence) {
-  __shared__ unsigned partial[1024];
+  __shared__ unsigned wave_sums[1024 / kWave];
   const int t = threadIdx.x;
   const int chunk = (tiles + 1023) / 1024;
   const int lo = t * chunk;
   const int hi = min(tiles, lo + chunk);
   unsigned sum = 0;
   for (int i = lo; i < hi; ++i) sum += tile_sums[i];
-  partial[t] = sum;
-  __syncthreads();
-  for (int off = 1; off < 1024; off <<= 1) {
-    const unsigned v = t >= off ? partial[t - off] : 0;
-    __syncthreads();
-    partial[t] += v;
-    __syncthreads();
+  // scan of the 1 024 per-thread sums: inside each wavefront by shuffles, then
+  // every thread adds the wavefronts before its own
+  unsigned inclusive = sum;
+  for (int off = 1; off < kWave; off <<= 1) {
+    const unsigned v = __shfl_up(inclusive, off);
+    if (static_cast<int>(lane_id()) >= off) inclusive += v;
   }
-  unsigned run = partial[t] - sum;
+  const int w = t >> 6;
+  if (lane_id() == kWave - 1) wave_sums[w] = inclusive;
+  __syncthreads();
+  unsigned before = 0, all = 0;
+  for (int ww = 0; ww < 1024 / kWave; ++ww) {
+    const unsigned v = wave_sums[ww];
+    before += ww < w ? v : 0u;
+    all += v;
+  }
+  unsigned run = before + inclusive - sum;
   for (int i = lo; i < hi; ++i) {
     const unsigned v = tile_sums[i];
     tile_sums[i] = run;
     run += v;
   }
   if (t == 1023) {
-    const unsigned total = partial[1023];
+    const unsigned total = all;
     tile_sums[tiles] = total;
     *host_count = total;
     __threadfence_system();
@@ -339,7 +367,7 @@ __global__ __launch_bounds__(1024) void bitmap_scan_kernel(unsigned *__restrict_
 
 template <typename CT, typename IT>
 __global__ __launch_bounds__(kScanBlock) void bitmap_emit_kernel(
-    const unsigned *__restrict__ bitmap, long long words, const unsigned *__restrict__ tile_bases,
+    unsigned *__restrict__ bitmap, long long words, const unsigned *__restrict__ tile_bases,
     int tiles, TargetSpec spec, CT *__restrict__ out, IT *__restrict__ batch_dims_out) {
   const long long base = static_cast<long long>(blockIdx.x) * kBitmapTile + threadIdx.x * kBitmapWords;
   // a tile without a set bit has nothing to write, unless a batch boundary
@@ -352,8 +380,19 @@ __global__ __launch_bounds__(kScanBlock) void bitmap_emit_kernel(
     word[r] = base + r < words ? bitmap[base + r] : 0u;
     count += __popc(word[r]);
   }
+  // Set bits cluster (cells that differ in the last coordinate share a word):
+  // a thread that walked its own 8 words would hold up its wavefront for up to
+  // 256 rows while others have none.  The tile's non-empty words, with the rank
+  // of their first row, are therefore listed in LDS and dealt round-robin.
+  __shared__ unsigned s_word[kBitmapTile], s_rank[kBitmapTile];
+  __shared__ unsigned short s_at[kBitmapTile];
   unsigned total;
   unsigned run = block_exclusive_scan(count, &total) + tile_bases[blockIdx.x];
+  unsigned filled = 0;
+#pragma unroll
+  for (int r = 0; r < kBitmapWords; ++r) filled += word[r] != 0u ? 1u : 0u;
+  unsigned listed;
+  unsigned slot = block_exclusive_scan(filled, &listed);
 #pragma unroll
   for (int r = 0; r < kBitmapWords; ++r) {
     const unsigned long long first_key = static_cast<unsigned long long>(base + r) << 5;
@@ -367,19 +406,38 @@ __global__ __launch_bounds__(kScanBlock) void bitmap_emit_kernel(
         batch_dims_out[g] = static_cast<IT>(run + __popc(word[r] & ((1u << bit) - 1u)));
       }
     }
-    unsigned bits = word[r];
+    if (word[r] != 0u) {
+      bitmap[base + r] = 0u;                     // the bitmap goes back all zero: the next build clears nothing
+      s_word[slot] = word[r];
+      s_rank[slot] = run;
+      s_at[slot] = static_cast<unsigned short>(threadIdx.x * kBitmapWords + r);
+      ++slot;
+      run += __popc(word[r]);
+    }
+  }
+  __syncthreads();
+  // Keys of the bitmap form have at most 28 bits, and (field + base) * stride
+  // worked out in CT wraps exactly as the wide product cut to CT does: the
+  // loop stays in 32-bit arithmetic for 32-bit coordinates.
+  const unsigned tile_key = static_cast<unsigned>(static_cast<unsigned long long>(blockIdx.x) * kBitmapTile << 5);
+  for (unsigned i = threadIdx.x; i < listed; i += kScanBlock) {
+    unsigned bits = s_word[i];
+    unsigned at = s_rank[i];
+    const unsigned first_key = tile_key + (static_cast<unsigned>(s_at[i]) << 5);
     while (bits != 0u) {
       const unsigned bit = __ffs(bits) - 1;
       bits &= bits - 1u;
-      const unsigned long long key = first_key | bit;
+      const unsigned key = first_key | bit;
+      CT *row = out + static_cast<long long>(at) * spec.ndim;
 #pragma unroll
       for (int k = 0; k < MNT_MAX_NDIM; ++k) {
         if (k < spec.ndim) {
-          const long long cell = static_cast<long long>((key >> spec.shift[k]) & spec.mask[k]) + spec.base[k];
-          out[static_cast<long long>(run) * spec.ndim + k] = static_cast<CT>(cell * spec.stride[k]);
+          const CT cell = static_cast<CT>((key >> spec.shift[k]) & static_cast<unsigned>(spec.mask[k])) +
+                          static_cast<CT>(spec.base[k]);
+          row[k] = cell * static_cast<CT>(spec.stride[k]);
         }
       }
-      ++run;
+      ++at;
     }
   }
   if (batch_dims_out != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
@@ -444,12 +502,16 @@ static void target_count_typed(const CT *coords, int64_t n, int ndim, const int6
     if (bits <= kBitmapMaxBits) {
       const long long words = bits <= 5 ? 1 : (1ll << (bits - 5));
       const int tiles = static_cast<int>(div_ceil(words, kBitmapTile));
-      // persistent block: bitmap [words] then tile bases [tiles + 1]
-      const size_t map_bytes = (static_cast<size_t>(words) * 4 + 255) / 256 * 256;
-      char *keep = static_cast<char *>(arena.persistent(0, map_bytes + (static_cast<size_t>(tiles) + 1) * 4));
-      unsigned *bitmap = reinterpret_cast<unsigned *>(keep);
-      unsigned *tile_bases = reinterpret_cast<unsigned *>(keep + map_bytes);
-      MNT_HIP(hipMemsetAsync(bitmap, 0, static_cast<size_t>(words) * 4, stream));
+      // persistent block: tile bases [tiles + 1] in a fixed-size head, then bitmap [words]
+      char *keep = static_cast<char *>(arena.persistent(0, kBitmapBasesBytes + static_cast<size_t>(words) * 4));
+      unsigned *tile_bases = reinterpret_cast<unsigned *>(keep);
+      unsigned *bitmap = reinterpret_cast<unsigned *>(keep + kBitmapBasesBytes);
+      // (the walk of the last build left its words zero; anything else that
+      // wrote here, or a build whose walk never ran, has reset the count)
+      const long long zero_words = arena.zero_bitmap_words;
+      if (zero_words < words) MNT_HIP(hipMemsetAsync(bitmap, 0, static_cast<size_t>(words) * 4, stream));
+      arena.zero_bitmap_words = 0;
+      arena.zero_bitmap_words_after = std::max(zero_words, words);
       mark_targets_kernel<CT, IT><<<grid_for(n, 256, 4096), 256, 0, stream>>>(coords, n, spec, batch_dims, bitmap);
       check_launch("mark_targets_kernel");
       bitmap_tile_sums_kernel<<<tiles, kScanBlock, 0, stream>>>(bitmap, words, tile_bases);
@@ -463,6 +525,7 @@ static void target_count_typed(const CT *coords, int64_t n, int ndim, const int6
         bitmap_emit_kernel<CT, IT><<<tiles, kScanBlock, 0, stream>>>(
             bitmap, words, tile_bases, tiles, spec, early_out, batched ? early_dims_out : nullptr);
         check_launch("bitmap_emit_kernel");
+        arena.zero_bitmap_words = arena.zero_bitmap_words_after;
       }
       arena.wait_flag(2, sequence);
       *count_out = static_cast<int64_t>(*h);
@@ -490,6 +553,7 @@ static void target_count_typed(const CT *coords, int64_t n, int ndim, const int6
     // persistent block: sorted keys [n] then ranks [n+1]
     size_t key_bytes = (static_cast<size_t>(n) * 8 + 255) / 256 * 256;
     char *keep = static_cast<char *>(arena.persistent(0, key_bytes + (static_cast<size_t>(n) + 1) * 4));
+    arena.zero_bitmap_words = 0;                 // the sorted keys go where the bitmap form keeps its bitmap
     // the sort ping-pongs between two buffers: start in the one that makes it
     // end in the persistent block
     unsigned long long *kept_keys = reinterpret_cast<unsigned long long *>(keep);
@@ -550,14 +614,14 @@ static void target_fill_typed(CT *out, IT *batch_dims_out, hipStream_t stream) {
   const TargetSpec spec = state.spec;
   const int64_t n = p.n;
   if (state.bitmap) {
-    const size_t map_bytes = (static_cast<size_t>(state.words) * 4 + 255) / 256 * 256;
     char *keep = static_cast<char *>(arena.persistent(0, 0));
-    const unsigned *bitmap = reinterpret_cast<const unsigned *>(keep);
-    const unsigned *tile_bases = reinterpret_cast<const unsigned *>(keep + map_bytes);
+    const unsigned *tile_bases = reinterpret_cast<const unsigned *>(keep);
+    unsigned *bitmap = reinterpret_cast<unsigned *>(keep + kBitmapBasesBytes);
     bitmap_emit_kernel<CT, IT><<<state.tiles, kScanBlock, 0, stream>>>(
         bitmap, state.words, tile_bases, state.tiles, spec, out,
         p.num_batches > 0 ? batch_dims_out : nullptr);
     check_launch("bitmap_emit_kernel");
+    arena.zero_bitmap_words = arena.zero_bitmap_words_after;
     p.valid = false;
     return;
   }

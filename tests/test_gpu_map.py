@@ -218,6 +218,52 @@ def test_target_coordinates_one_call_equals_two_calls(extent, batches):
         np.testing.assert_array_equal(host(one_bd), exp_bd)
 
 
+def test_target_coordinates_builds_in_a_row():
+    """The bitmap of one build is left zero for the next (no clearing launch):
+    large, small, large again, the sorted-key form in between (it writes where
+    the bitmap lives), a count whose fill never comes, clustered and spread
+    clouds -- every build must equal the oracle."""
+    import ctypes
+    rng = np.random.default_rng(91)
+
+    def cloud(n, extent, batches):
+        c = rng.integers(-extent, extent, size=(n, 3)).astype(np.int32)
+        bd = None
+        if batches > 1:
+            bd = np.concatenate([[0], np.sort(rng.integers(0, n, size=batches - 1)), [n]]).astype(np.int32)
+        return sorted_unique(c, bd)
+
+    def dense_slab(n_side):
+        g = np.stack(np.meshgrid(np.arange(n_side), np.arange(n_side), np.arange(6), indexing="ij"), -1)
+        return sorted_unique(g.reshape(-1, 3).astype(np.int32), None)
+
+    def abandoned_count(c, bd, stride):
+        lib = _C.load_library()
+        count = ctypes.c_int64(0)
+        c_dev, bd_dev = dev(c), dev(bd)
+        with _C._on(c_dev.device):
+            _C._check(lib.mnt_target_coordinates_count(
+                _C._ptr(c_dev), c.shape[0], 3, 0, (ctypes.c_int64 * 3)(*stride), _C._ptr(bd_dev),
+                bd.size - 1 if bd is not None else 1, 0, None, ctypes.byref(count), _C._stream(c_dev.device)))
+        return count.value
+
+    builds = [cloud(30000, 300, 1), cloud(2000, 20, 3), cloud(30000, 300, 2), cloud(4000, 1 << 20, 2),
+              cloud(25000, 250, 1), dense_slab(60), cloud(500, 6, 1), cloud(30000, 400, 4), dense_slab(90)]
+    for round_ in range(2):
+        for i, (c, bd) in enumerate(builds):
+            for stride in ((2, 2, 2), (4, 4, 2)):
+                if round_ == 1 and i % 3 == 0:
+                    assert abandoned_count(c, bd, stride) == orc.target_coordinates(c, bd, stride)[0].shape[0]
+                exp, exp_bd = orc.target_coordinates(c, bd, stride)
+                if (i + round_) % 2 == 0:
+                    got, got_bd = _C.target_coordinates(dev(c), dev(bd), stride)
+                else:
+                    got, got_bd = _target_coordinates_two_calls(dev(c), dev(bd), stride)
+                np.testing.assert_array_equal(host(got), exp)
+                if bd is not None:
+                    np.testing.assert_array_equal(host(got_bd), exp_bd)
+
+
 def test_target_coordinates_one_call_rejects_short_room():
     import ctypes
     c = dev(sorted_unique(random_cloud(300, 12, seed=3), None)[0])
