@@ -88,6 +88,7 @@ void Arena::free_all(bool synchronise) {
   }
   pending.valid = false;
   map_state_valid = false;
+  zero_bitmap_words = 0;
 }
 
 void Arena::reset_device() {

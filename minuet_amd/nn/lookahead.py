@@ -12,6 +12,7 @@ those of the same library calls, only made earlier and elsewhere.
 
 Outputs live in one allocation sized for the worst case (no level has more
 rows than the input cloud); the tensors handed out are views of it."""
+import weakref
 from typing import Dict, Optional
 
 import numpy as np
@@ -19,7 +20,20 @@ import torch
 
 from minuet_amd.nn.functional import _C
 
-__all__ = ["AheadLayout", "AheadSession"]
+__all__ = ["AheadLayout", "AheadSession", "end_running_session"]
+
+# The session the library's worker is running for (a weak reference): a session
+# object that is no longer this one neither takes items nor ends anything.
+_running = None
+
+
+def end_running_session(device: torch.device):
+    """Ends whatever session the worker is running; the cache that started it
+    builds the rest of its pass the ordinary way."""
+    global _running
+    _running = None
+    _C.lookahead_finish(device)
+
 
 _ALIGN = 256
 _ROW_STEP = 1 << 14          # layouts are made for row counts rounded up to this
@@ -179,6 +193,8 @@ class AheadSession:
         self._rows = {0: n}               # level -> number of rows, as items are taken
         _C.lookahead_start(coordinates, batch_dims, bounds, layout.items, layout.num_levels)
         self._open = True                  # only a session that started may finish the worker's
+        global _running
+        _running = weakref.ref(self)
         self._inputs = (coordinates, batch_dims)       # alive while the worker may read them
 
     def _ints(self, item: int, slot: int, rows: int, columns: int) -> torch.Tensor:
@@ -198,6 +214,8 @@ class AheadSession:
         """What the worker built for ``tag``, the current stream ordered after
         it: ``(coordinates, batch_dims)``, the dense map, the dict
         ``kernel_map_tables`` returns, or the inverse map."""
+        if not self._is_running():
+            raise RuntimeError("this look-ahead session is over")
         item = self.index.pop(tag)
         size = _C.lookahead_wait(item, self.device)
         layout = self.layout
@@ -228,12 +246,19 @@ class AheadSession:
                     target_masks=self._ints(item, 1, num_offsets, num_targets),
                     in_idx=self._ints(item, 2, size, 0), out_idx=self._ints(item, 3, size, 0))
 
+    def _is_running(self) -> bool:
+        return self._open and _running is not None and _running() is self
+
     def finish(self):
         """Waits for the worker to go idle and orders the current stream after
         everything it enqueued; the buffers may be released afterwards."""
+        global _running
         if self._open:
+            running = self._is_running()
             self._open = False
-            _C.lookahead_finish(self.device)
+            if running:
+                _running = None
+                _C.lookahead_finish(self.device)
             self._inputs = None
 
     def __del__(self):
