@@ -25,20 +25,57 @@ HBM_PEAK_GBS = 8000.0
 MAP_PROFILE = os.path.join(ROOT, "profiles", "map_step_config2_200k_voxels.md")
 
 
+def kernel_sources_digest():
+    """Digest of the HIP sources the library is built from: a profile summary
+    records the one it was taken with, so a reader can tell whether counters
+    quoted from it belong to the code that is running."""
+    import glob
+    import hashlib
+    digest = hashlib.sha256()
+    for path in sorted(glob.glob(os.path.join(ROOT, "minuet_amd", "csrc", "*"))):
+        digest.update(os.path.basename(path).encode())
+        digest.update(open(path, "rb").read())
+    return digest.hexdigest()[:16]
+
+
 def measured_traffic(kernel):
     """HBM bytes per launch of `kernel` on this workload at scale 1, from the
     committed rocprofv3 summary (FETCH_SIZE + WRITE_SIZE, each scaled by what
-    the counter reads for a plain device copy of known size); None when the
-    summary does not list the kernel."""
+    the counter reads for a plain device copy of known size), and where the
+    figure comes from: the counters need a profiler run of their own, so they
+    are those of the summary's run, with its date and the digest of the kernel
+    sources it profiled beside the digest of the sources at hand.  (None, ...)
+    when the summary does not list the kernel."""
     import re
+    source = {"file": os.path.relpath(MAP_PROFILE, ROOT), "sources_now": kernel_sources_digest()}
     try:
         text = open(MAP_PROFILE).read()
     except OSError:
-        return None
+        return None, source
+    for key in ("date", "sources"):
+        found = re.search(rf"^{key}:\s*(\S+)", text, flags=re.M)
+        source[f"profile_{key}"] = found.group(1) if found else None
+    source["same_sources"] = source.get("profile_sources") == source["sources_now"]
     match = re.search(r"traffic_bytes:\s*(\{.*?\})", text)
     if not match:
-        return None
-    return json.loads(match.group(1)).get(kernel)
+        return None, source
+    return json.loads(match.group(1)).get(kernel), source
+
+
+def device_record(_C):
+    """What the box is: compute units and clocks as the runtime reports them, and
+    the memory ceilings measured here and now with one plain streaming kernel
+    each over 512 MiB (copy = bytes read + bytes written per second)."""
+    facts = _C.device_facts()
+    nbytes = 512 << 20
+    ceilings = {}
+    for kind, moved in (("copy", 2 * nbytes), ("read", nbytes), ("write", nbytes)):
+        ms = min(_C.time_memory(kind, nbytes, repeats=10) for _ in range(3))
+        ceilings[kind + "_GBs"] = round(moved / (ms * 1e-3) / 1e9, 1)
+    facts["measured_hbm_ceiling"] = dict(ceilings, bytes_per_pass=nbytes,
+                                         note="plain 16-byte streaming kernels, 10 back-to-back passes, best of 3")
+    facts["vendor_hbm_peak_GBs"] = HBM_PEAK_GBS
+    return facts
 
 
 def map_step(_C, coords_dev, offsets, want_coordinates=False):
@@ -46,6 +83,21 @@ def map_step(_C, coords_dev, offsets, want_coordinates=False):
     the order KernelMapCache keeps them (rows by ascending size), one library call."""
     built = _C.sorted_kernel_map_lists(coords_dev, offsets, reorder=True, result_only=True)
     return built["coordinates"] if want_coordinates else None, built
+
+
+def check_parity(coords, offsets, sorted_dev, built):
+    """The timed call's results against the CPU restatement of the reference
+    algorithm, bit for bit (sorted voxels, both pair lists).  The only place of
+    the measured path that touches the oracle: as the checker."""
+    import c_oracle
+    import minuet_oracle as orc
+    order = orc.arg_sort_coordinates(coords)
+    ref_sorted = coords[order]
+    assert np.array_equal(sorted_dev.cpu().numpy(), ref_sorted)
+    ref_map = c_oracle.query(ref_sorted, ref_sorted, offsets.astype(np.int32))
+    ein, eout, _ = orc.kernel_map_pair_lists(ref_map[orc.stable_size_order(orc.compute_kernel_map_sizes(ref_map))])
+    assert np.array_equal(built["in_idx"].cpu().numpy(), ein)
+    assert np.array_equal(built["out_idx"].cpu().numpy(), eout)
 
 
 def cpu_model():
@@ -165,21 +217,39 @@ def layer_stages(device, config, channels, kernel_size, dtype_name, tune=False):
         gather_ms = med(F.cuda_time_gather, tile_size=0)
         scatter_ms = med(F.cuda_time_scatter, tile_size=0)
         gemm_ms = med(F.cuda_time_gemm)
+        # second clock: 20 launches back to back between the two events, time of
+        # one (no launch gap inside the interval: what a kernel trace shows per launch)
+        _C.timer_repeats(20)
+        try:
+            gather_b2b = med(F.cuda_time_gather, tile_size=0)
+            scatter_b2b = med(F.cuda_time_scatter, tile_size=0)
+            gemm_b2b = med(F.cuda_time_gemm)
+        finally:
+            _C.timer_repeats(1)
         bytes_gather = voxels * channels * esize + moved * channels * esize + 4 * moved
         bytes_scatter = moved * channels * esize + voxels * channels * esize + 4 * moved
         flops = 2.0 * nnz * channels * channels
         out = {"voxels": voxels, "nnz": nnz, "channels": channels, "dtype": dtype_name,
                "offsets": int(host_sizes.shape[0])}
 
-        def hbm(nbytes, ms):
+        def hbm(nbytes, ms, ms_b2b=None):
             gbs = nbytes / (ms * 1e-3) / 1e9
-            return {"ms": round(ms, 4), "algorithmic_bytes": int(nbytes), "achieved_GBs": round(gbs, 1),
-                    "frac_of_8TBs": round(gbs / HBM_PEAK_GBS, 4)}
-        out["gather_kernel"] = hbm(bytes_gather, gather_ms)
-        out["scatter_kernel"] = hbm(bytes_scatter, scatter_ms)
+            rec = {"ms": round(ms, 4), "algorithmic_bytes": int(nbytes), "achieved_GBs": round(gbs, 1),
+                   "frac_of_8TBs": round(gbs / HBM_PEAK_GBS, 4)}
+            if ms_b2b is not None:
+                rec.update(ms_back_to_back=round(ms_b2b, 4),
+                           frac_of_8TBs_back_to_back=round(nbytes / (ms_b2b * 1e-3) / 1e9 / HBM_PEAK_GBS, 4))
+            return rec
+        out["clocks"] = ("ms: one launch between two stream events (the reference's cuda_time_* protocol, "
+                         "launch gap included); ms_back_to_back: 20 launches between the events, time of one")
+        out["gather_kernel"] = hbm(bytes_gather, gather_ms, gather_b2b)
+        out["scatter_kernel"] = hbm(bytes_scatter, scatter_ms, scatter_b2b)
         tflops = flops / (gemm_ms * 1e-3) / 1e12
-        out["grouped_gemm_kernel"] = {"ms": round(gemm_ms, 4), "flops": flops, "achieved_TFLOPs": round(tflops, 1),
+        out["grouped_gemm_kernel"] = {"ms": round(gemm_ms, 4), "ms_back_to_back": round(gemm_b2b, 4),
+                                      "flops": flops, "achieved_TFLOPs": round(tflops, 1),
                                       "frac_of_mfma_peak": round(tflops / MFMA_PEAK_TFLOPS[dtype_name], 4),
+                                      "frac_of_mfma_peak_back_to_back": round(
+                                          flops / (gemm_b2b * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS[dtype_name], 4),
                                       # rows in and out of the buffers: what bounds it at small widths
                                       **{"hbm_" + k: v for k, v in hbm(2 * nnz * channels * esize, gemm_ms).items()
                                          if k != "ms"}}
@@ -248,6 +318,29 @@ def extras(device, with_config5, section="all"):
     if section == "config5":
         return {"config5_layer_bf16_c64_k5": layer_stages(device, 5, 64, 5, "bf16", tune=True)}
     with torch.no_grad():
+        # The configuration-2 cloud through the cache a NETWORK uses: what a layer pays
+        # for its map on an unsorted cloud.  A single-kernel layer asks for the dense
+        # map [27, N] alone; a Gather-GEMM-Scatter layer for dense map, both rank
+        # tables, sizes, order and the pair lists.  (The headline times the lists-only
+        # build, which is the output configuration 2 names.)
+        c2 = torch.from_numpy(make_cloud(2)["coords"]).to(device)
+        cache2 = minuet.nn.KernelMapCache(3, torch.int32, device)
+
+        def through_cache(tables):
+            def run():
+                cache2.reset()
+                _, s2 = _C.sort_coordinates(c2)
+                if tables:
+                    cache2.get_kernel_map(s2, 1, None, s2, 1, None, 3, 1)
+                else:
+                    cache2.get_dense_kernel_map(s2, 1, None, s2, 1, None, 3, 1)
+            return run
+        out["config2_map_through_kernel_map_cache"] = {
+            "voxels": int(c2.shape[0]),
+            "sort+dense_map (single-kernel layers)": _time_stats(through_cache(False), 10, 100),
+            "sort+dense_map+rank_tables+lists (gather-GEMM-scatter layers)": _time_stats(through_cache(True), 10, 100)}
+        cache2.reset()
+        del c2, cache2
         # configuration 1: submanifold 3x3x3, 32 -> 32, fp32
         c1 = torch.from_numpy(make_cloud(1)["coords"]).to(device)
         _, s1 = _C.sort_coordinates(c1)
@@ -362,9 +455,9 @@ def main():
         sys.exit(2)
 
     import torch
-    import minuet_oracle as orc
     from minuet_amd.nn.functional import _C
     from minuet_amd.synthetic import make_cloud
+    from minuet_amd.utils.helpers import generate_kernel_offsets
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -372,8 +465,7 @@ def main():
     device = torch.device("cuda:0")
     cloud = make_cloud(2, scale=args.scale)
     coords = cloud["coords"]
-    offsets = orc.generate_kernel_offsets(3, 3, 1, 1)
-    offsets32 = offsets.astype(np.int32)
+    offsets = np.ascontiguousarray(generate_kernel_offsets(3, 3, 1, 1), dtype=np.int64)
     coords_dev = torch.from_numpy(coords).to(device)
     n = coords.shape[0]
 
@@ -385,25 +477,22 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # bring the GPU out of its idle power state before anything is measured
+    # parity of what is being timed (bit-exact against the CPU restatement), once,
+    # BEFORE the timed region: the check keeps the host busy for a while, and the
+    # warm-up has to come right before the steps that are timed
+    sorted_dev, built = map_step(_C, coords_dev, offsets, want_coordinates=True)
+    torch.cuda.synchronize()
+    nnz = int(built["sizes_host"].sum())
+    check_parity(coords, offsets, sorted_dev, built)
+    device_facts = device_record(_C)
+
+    # bring the GPU out of its idle power state, then the W untimed steps, then
+    # exactly K timed steps between two device-wide waits
     spin_until = time.perf_counter() + 1.5
     while time.perf_counter() < spin_until:
         map_step(_C, coords_dev, offsets)
     for _ in range(max(1, args.warmup)):
-        sorted_dev, built = map_step(_C, coords_dev, offsets, want_coordinates=True)
-    torch.cuda.synchronize()
-    nnz = int(built["sizes_host"].sum())
-
-    # parity of what is being timed (bit-exact), once
-    order = orc.arg_sort_coordinates(coords)
-    ref_sorted = coords[order]
-    assert np.array_equal(sorted_dev.cpu().numpy(), ref_sorted)
-    import c_oracle
-    ref_map = c_oracle.query(ref_sorted, ref_sorted, offsets32)
-    ein, eout, _ = orc.kernel_map_pair_lists(ref_map[orc.stable_size_order(orc.compute_kernel_map_sizes(ref_map))])
-    assert np.array_equal(built["in_idx"].cpu().numpy(), ein)
-    assert np.array_equal(built["out_idx"].cpu().numpy(), eout)
-
+        map_step(_C, coords_dev, offsets)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
@@ -436,6 +525,8 @@ def main():
     bytes_query = 12 * n + 8 * nnz
     query_ms = stage_ms.get("query", float("nan"))
     achieved = bytes_query / (query_ms * 1e-3) / 1e9 if query_ms == query_ms and query_ms > 0 else None
+    traffic, traffic_source = measured_traffic("query_kernel") if args.scale == 1.0 else (None, None)
+    copy_ceiling = device_facts["measured_hbm_ceiling"]["copy_GBs"]
     result = {
         "metric": "Map-step ms + SC layer Mvoxels/s + sparse UNet fwd latency (1 GPU)",
         "value": round(wall_ms, 4),
@@ -460,7 +551,8 @@ def main():
                      "achieved": None if achieved is None else round(achieved, 2),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": None if achieved is None else round(achieved / HBM_PEAK_GBS, 5),
-                     "traffic": measured_traffic("query_kernel") if args.scale == 1.0 else None,
+                     "traffic": traffic, "traffic_source": traffic_source,
+                     "frac_of_measured_copy_ceiling": None if achieved is None else round(achieved / copy_ceiling, 5),
                      "algorithmic_bytes": bytes_query,
                      "avg_launch_ms": None if achieved is None else round(query_ms, 5),
                      "map_step": {"algorithmic_bytes": bytes_map,
@@ -469,10 +561,11 @@ def main():
                                   "frac": round(bytes_map / (wall_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 5),
                                   "stage_ms": {k: round(v, 5) for k, v in stage_ms.items()}}},
     }
+    result["device"] = device_facts
     if not args.no_extras:
         result["extra"] = extras(device, not args.no_config5, args.section)
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(coords, offsets32)
+        result["cpu_baseline"] = cpu_baseline(coords, offsets.astype(np.int32))
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result))

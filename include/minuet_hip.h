@@ -68,6 +68,22 @@ int mnt_reset_error(void);                                /* cuda_reset_error */
  * are forgotten. */
 int mnt_device_reset(void);
 
+/* Threading.  The library keeps state per (device, stream): the scratch arena,
+ * what the two-phase entry points hand from their first call to their second,
+ * a pinned staging block.  None of it is locked, so the contract is ONE CALLER
+ * THREAD PER STREAM AT A TIME.  It is enforced: a call takes the state of every
+ * stream it touches for the calling thread until it returns, and a thread
+ * that enters on a stream another thread is inside of fails with a message
+ * instead of racing.  Threads on different streams run side by side.
+ * mnt_stream_acquire keeps a stream for the calling thread ACROSS calls (every
+ * other thread's calls on it fail until mnt_stream_release); a caller that
+ * hands a stream from thread to thread brackets its use with the pair.
+ * The reference is called with the interpreter lock held for the whole of
+ * every _C function (csrc/minuet/torch/common.h:17-21), which serialises
+ * everything; a ctypes binding releases that lock, hence the rule here. */
+int mnt_stream_acquire(void *stream);
+int mnt_stream_release(void *stream);
+
 /* How often, and for how long in total, library calls of this process have
  * made the host wait for a result of the device (every such wait is the poll
  * of one completion flag in pinned memory) since the last reset of the tally.
@@ -583,6 +599,25 @@ int mnt_lookahead_wait(int item, void *stream, int64_t *size_out);
 int mnt_lookahead_finish(void *stream);
 
 /* ---- stage timing -------------------------------------------------------- */
+
+/* Streams `bytes` of device memory through one plain kernel (kind 0: copy a -> b,
+ * `bytes` read and `bytes` written; 1: read only; 2: write only), `repeats`
+ * times back to back between two stream events, and returns the milliseconds
+ * of ONE pass: the memory ceilings of the machine at hand, which a benchmark
+ * quotes beside the vendor's peak.  The buffers come from the stream's scratch
+ * arena.  No counterpart in the reference. */
+int mnt_time_memory(int kind, size_t bytes, int repeats, float *ms_out, void *stream);
+
+/* Facts of the current device for a benchmark's record, facts_out[0..5]:
+ * compute units, engine clock (kHz), memory clock (kHz), memory bus width
+ * (bits), L2 bytes, device memory bytes.  No counterpart in the reference. */
+int mnt_device_facts(int64_t *facts_out, int capacity);
+
+/* Launches per timing run of mnt_time_gather / _scatter / _gemm (default 1, the
+ * reference's protocol: one launch between two events, which also times the
+ * launch gap).  With more, the launches go back to back between the events and
+ * the time of one is returned: the sustained rate of the kernel alone. */
+int mnt_timer_repeats(int repeats);
 
 /* mnt_profile_enable(1) makes the instrumented entry points (sort, query, emit,
  * forward) record a timestamp event on their stream after every stage; (0)

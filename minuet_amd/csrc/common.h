@@ -47,9 +47,26 @@ void set_last_error(const std::string &message);
       MNT_FAIL("%s failed: %s", #expr, hipGetErrorString(status_));            \
   } while (0)
 
+// One caller thread per stream at a time: the scratch arena of a stream, the
+// state its two-phase entry points hand from call to call and its pinned
+// block have no locks of their own.  A library call takes the arena of every
+// stream it touches for the calling thread until it returns (calls nest: an
+// entry point may go through others); a thread that enters the library on a
+// stream another thread is inside of gets an error instead of a data race.
+// (The reference is called with the interpreter lock held,
+// csrc/minuet/torch/common.h:17-21; a ctypes call releases that lock.)
+void enter_call();
+void leave_call();
+
+struct CallDepth {
+  CallDepth() { enter_call(); }
+  ~CallDepth() { leave_call(); }
+};
+
 // Wraps the body of every extern "C" entry point.
 template <typename Fn>
 inline int guarded(Fn &&fn) {
+  CallDepth depth;
   try {
     fn();
     return 0;
@@ -69,7 +86,14 @@ inline int guarded(Fn &&fn) {
 // the same stream, which is ordered after the earlier work.
 class Arena {
  public:
+  // The arena of `stream` on the current device, taken for the calling thread
+  // until its outermost library call returns (see enter_call); fails when
+  // another thread holds it.
   static Arena &of(hipStream_t stream);
+  // Keeps / gives up the arena for the calling thread across calls
+  // (mnt_stream_acquire / mnt_stream_release).
+  static void pin(hipStream_t stream);
+  static void unpin(hipStream_t stream);
   // Gives back everything the library holds on the current device: the arenas
   // of all its streams (pages, persistent blocks, pinned staging blocks).
   static void reset_device();
@@ -139,6 +163,7 @@ class Arena {
   };
   explicit Arena(hipStream_t s) : stream_(s) {}
   void add_page(size_t bytes);
+  friend void leave_call();
 
   hipStream_t stream_;
   std::vector<Page> pages_;
@@ -150,6 +175,9 @@ class Arena {
   unsigned long long sequence_ = 0;
   void *persistent_[2] = {nullptr, nullptr};
   size_t persistent_size_[2] = {0, 0};
+  // guarded by the registry's mutex
+  bool held_ = false, pinned_by_thread_ = false;
+  unsigned long long holder_ = 0;            // token of the thread inside a call / that pinned it
 };
 
 class Scope {

@@ -1518,6 +1518,8 @@ extern "C" int mnt_pack_weights(const void *weights, int64_t O, int64_t K, int64
 
 namespace mnt {
 
+static int g_timer_repeats = 1;            // launches between the two events of a stage timer
+
 struct TimerScope {
   hipEvent_t start, stop;
   hipStream_t stream;
@@ -1535,7 +1537,7 @@ struct TimerScope {
     MNT_HIP(hipEventSynchronize(stop));
     float ms = 0.0f;
     MNT_HIP(hipEventElapsedTime(&ms, start, stop));
-    return ms;
+    return ms / static_cast<float>(g_timer_repeats);
   }
 };
 
@@ -1551,8 +1553,10 @@ static float time_gather_typed(int64_t tile, const ForwardPlan &plan, const IT *
   const LaneShape sh = lane_shape(tile, K, sizeof(T), sources, abuf, "num_source_features");
   TimerScope timer(stream);
   timer.begin();
-  launch_gather<IT>(sh, sources, abuf, source_masks, d_row_start, S, static_cast<int>(plan.active_offsets),
-                    static_cast<int>(K * sizeof(T)), stream);
+  for (int r = 0; r < g_timer_repeats; ++r) {
+    launch_gather<IT>(sh, sources, abuf, source_masks, d_row_start, S, static_cast<int>(plan.active_offsets),
+                      static_cast<int>(K * sizeof(T)), stream);
+  }
   return timer.end();
 }
 
@@ -1569,9 +1573,11 @@ static float time_scatter_typed(int64_t tile, const ForwardPlan &plan, const IT 
   const LaneShape sh = lane_shape(tile, N, sizeof(T), cbuf, out, "num_target_features");
   TimerScope timer(stream);
   timer.begin();
-  launch_scatter<TB, T, IT>(sh, cbuf, out, target_masks, d_row_start, Tn,
-                            static_cast<int>(plan.active_offsets), static_cast<int>(N),
-                            plan.shortcut ? cbuf + rows * N : nullptr, Epilogue{}, stream);
+  for (int r = 0; r < g_timer_repeats; ++r) {
+    launch_scatter<TB, T, IT>(sh, cbuf, out, target_masks, d_row_start, Tn,
+                              static_cast<int>(plan.active_offsets), static_cast<int>(N),
+                              plan.shortcut ? cbuf + rows * N : nullptr, Epilogue{}, stream);
+  }
   return timer.end();
 }
 
@@ -1610,11 +1616,13 @@ static float time_gemm_typed(const ForwardPlan &plan, const T *weights, int64_t 
   upload_ints(plan.meta, d_meta, stream);
   TimerScope timer(stream);
   timer.begin();
-  launch_gemm<T, TB>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np,
-                     nullptr, stream);
-  if (plan.shortcut) {
-    launch_gemm<T, TB>(direct_a, direct_c, wt, d_direct, dmeta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np,
+  for (int r = 0; r < g_timer_repeats; ++r) {
+    launch_gemm<T, TB>(abuf, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np,
                        nullptr, stream);
+    if (plan.shortcut) {
+      launch_gemm<T, TB>(direct_a, direct_c, wt, d_direct, dmeta[2], static_cast<int>(K), static_cast<int>(N), Kp,
+                         Np, nullptr, stream);
+    }
   }
   return timer.end();
 }
@@ -1628,6 +1636,13 @@ static ForwardPlan timer_plan(const void *sizes_dev, int index_dtype, int64_t S,
 }
 
 }  // namespace mnt
+
+extern "C" int mnt_timer_repeats(int repeats) {
+  return guarded([&] {
+    MNT_CHECK(repeats >= 1 && repeats <= 1000, "repeats must be in [1, 1000], found %d", repeats);
+    g_timer_repeats = repeats;
+  });
+}
 
 extern "C" int mnt_time_gather(int64_t tile, int allow_shortcut_matmul, int has_threshold,
                                double threshold, const void *source_masks,

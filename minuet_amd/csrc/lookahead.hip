@@ -38,6 +38,8 @@ struct Session {
   int64_t *bounds_out = nullptr;
   int32_t *bounds_known_out = nullptr;
   hipEvent_t inputs_ready = nullptr;       // recorded on the caller's stream at the start
+  hipEvent_t session_end = nullptr;        // recorded on the worker's stream behind the last item, built or failed
+  bool end_recorded = false;
 };
 
 // The worker outlives main(): what it waits on is never destroyed.
@@ -227,6 +229,13 @@ void run_session(Session &s) {
     }
     g_progress.notify_all();
   }
+  // Whatever the items enqueued, failed ones included, lies before this event:
+  // an item that fails half-way records no event of its own, yet its kernels
+  // may still be writing the session's buffers.
+  if (usable && hipEventRecord(s.session_end, stream) == hipSuccess) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    s.end_recorded = true;
+  }
   if (s.bounds_out != nullptr && s.bounds_known_out != nullptr) {
     for (size_t l = 0; l < s.levels.size(); ++l) {
       memcpy(s.bounds_out + 8 * l, s.levels[l].bounds, 8 * sizeof(int64_t));
@@ -301,6 +310,8 @@ extern "C" int mnt_lookahead_start(const void *coords, int64_t n, int ndim, int 
     s.bounds_out = bounds_out;
     s.bounds_known_out = bounds_known_out;
     if (s.inputs_ready == nullptr) s.inputs_ready = take_event();
+    if (s.session_end == nullptr) s.session_end = take_event();
+    s.end_recorded = false;
     MNT_HIP(hipEventRecord(s.inputs_ready, stream));
     if (!g_worker_started) {
       std::thread(worker_main).detach();
@@ -337,11 +348,9 @@ extern "C" int mnt_lookahead_finish(void *stream_) {
     if (!g_active) return;
     g_progress.wait(lock, [] { return !g_job_posted && !g_busy; });
     Session &s = g_session;
-    // the caller's stream waits for the last kernels the worker enqueued
-    hipEvent_t last = nullptr;
-    for (size_t i = 0; i < s.items.size(); ++i) {
-      if (s.status[i] == 0) last = s.built[i];
-    }
+    // the caller's stream waits for everything the worker enqueued, the
+    // kernels of items that failed after their first launch included
+    hipEvent_t last = s.end_recorded ? s.session_end : nullptr;
     g_active = false;
     lock.unlock();
     if (last != nullptr) MNT_HIP(hipStreamWaitEvent(stream, last, 0));

@@ -568,6 +568,75 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
   if (kLists && tid == 0) sink.tile_mode[blockIdx.x] = num_chunks == 1 ? 0u : 1u;
 }
 
+// The query for frames too wide for a packed key (more than 63 bits of
+// coordinate ranges, kernel reach and batch id): the reference's own way,
+// a binary search per (offset, target) pair that compares whole coordinate
+// tuples (csrc/minuet/common/functions.h:94-105,
+// csrc/minuet/cuda/kernels/query_sorted_index_with_offsets.cuh:36-77), inside
+// the target's batch.  Slow next to query_kernel (no shared window, log2 S
+// dependent reads per pair) and only taken when that one cannot run.
+// offsets: [O, ndim] as (low, high) halves of 64-bit values.
+template <typename CT, typename BT, typename OT>
+__global__ __launch_bounds__(kQueryBlock) void query_tuples_kernel(
+    const CT *__restrict__ sources, long long num_sources, const CT *__restrict__ targets,
+    long long num_targets, const int *__restrict__ offsets, int ndim,
+    const BT *__restrict__ source_batch_dims, const BT *__restrict__ target_batch_dims,
+    int num_batches, OT *__restrict__ kernel_map) {
+  const long long t = static_cast<long long>(blockIdx.x) * kQueryBlock + threadIdx.x;
+  const int o = blockIdx.y;
+  if (t >= num_targets) return;
+  long long q[MNT_MAX_NDIM];
+  load_row<CT>(targets + t * ndim, ndim, q);
+  bool representable = true;
+#pragma unroll
+  for (int k = 0; k < MNT_MAX_NDIM; ++k) {
+    if (k < ndim) {
+      const unsigned lo = static_cast<unsigned>(offsets[(o * ndim + k) * 2 + 0]);
+      const unsigned hi = static_cast<unsigned>(offsets[(o * ndim + k) * 2 + 1]);
+      const long long d = static_cast<long long>((static_cast<unsigned long long>(hi) << 32) | lo);
+      long long sum;
+      // a shifted coordinate beyond the coordinate type equals no source
+      representable = representable && !__builtin_add_overflow(q[k], d, &sum) &&
+                      sum == static_cast<long long>(static_cast<CT>(sum));
+      q[k] = sum;
+    }
+  }
+  long long lo = 0, hi = num_sources;
+  if (source_batch_dims != nullptr) {
+    const int b = batch_of<BT>(t, target_batch_dims, num_batches);
+    lo = static_cast<long long>(source_batch_dims[b]);
+    hi = static_cast<long long>(source_batch_dims[b + 1]);
+  }
+  const long long end = hi;
+  // first source row of the batch that is not below q (lexicographic, dimension 0 first)
+  while (representable && lo < hi) {
+    const long long mid = lo + ((hi - lo) >> 1);
+    long long c[MNT_MAX_NDIM];
+    load_row<CT>(sources + mid * ndim, ndim, c);
+    bool below = false, decided = false;
+#pragma unroll
+    for (int k = 0; k < MNT_MAX_NDIM; ++k) {
+      if (k < ndim && !decided && c[k] != q[k]) {
+        below = c[k] < q[k];
+        decided = true;
+      }
+    }
+    if (below) {
+      lo = mid + 1;
+    } else {
+      hi = mid;
+    }
+  }
+  bool found = representable && lo < end;
+  if (found) {
+    long long c[MNT_MAX_NDIM];
+    load_row<CT>(sources + lo * ndim, ndim, c);
+#pragma unroll
+    for (int k = 0; k < MNT_MAX_NDIM; ++k) found = found && (k >= ndim || c[k] == q[k]);
+  }
+  kernel_map[static_cast<long long>(o) * num_targets + t] = found ? static_cast<OT>(lo) : static_cast<OT>(-1);
+}
+
 // Hit counts of every (row, tile of 512 targets) of an existing dense map.
 template <typename IT>
 __global__ __launch_bounds__(kQueryBlock) void count_tiles_kernel(
@@ -996,6 +1065,7 @@ struct QueryPlan {
   int num_groups;
   long long delta_min, delta_max;
   bool groups_in_rows;                   // the offsets of every group differ in the last coordinate only
+  bool fits;                             // the frame packs into one 64-bit key; otherwise nothing else is filled in
 };
 
 // Builds the packing frame from the coordinate bounds of sources and targets
@@ -1005,6 +1075,10 @@ static QueryPlan make_plan(const long long *src_bounds, const long long *tgt_bou
                            int64_t num_batches) {
   QueryPlan plan;
   memset(&plan.frame, 0, sizeof(Frame));
+  plan.fits = true;
+  plan.num_groups = 0;
+  plan.delta_min = plan.delta_max = 0;
+  plan.groups_in_rows = false;
   Frame &f = plan.frame;
   f.ndim = ndim;
   int bits = 0;
@@ -1020,9 +1094,10 @@ static QueryPlan make_plan(const long long *src_bounds, const long long *tgt_bou
     if (src_bounds[k] < lo) lo = src_bounds[k];
     if (src_bounds[MNT_MAX_NDIM + k] > hi) hi = src_bounds[MNT_MAX_NDIM + k];
     __int128 range = hi - lo;
-    MNT_CHECK(range >= 0 && range < (static_cast<__int128>(1) << 63) &&
-                  lo >= INT64_MIN && lo <= INT64_MAX,
-              "coordinate range of dimension %d is too large to pack into a voxel key", k);
+    if (!(range >= 0 && range < (static_cast<__int128>(1) << 63) && lo >= INT64_MIN && lo <= INT64_MAX)) {
+      plan.fits = false;
+      return plan;
+    }
     f.lo[k] = static_cast<long long>(lo);
     f.width[k] = width_of(static_cast<unsigned long long>(range));
     f.shift[k] = bits < 63 ? bits : 63;
@@ -1032,10 +1107,12 @@ static QueryPlan make_plan(const long long *src_bounds, const long long *tgt_bou
   f.batch_shift = bits < 63 ? bits : 63;
   bits += f.batch_width;
   f.total_bits = bits;
-  MNT_CHECK(bits <= 63,
-            "voxel keys need %d bits (coordinate ranges plus kernel reach plus batch id); at most "
-            "63 are supported",
-            bits);
+  // coordinate ranges plus kernel reach plus batch id beyond 63 bits: the caller
+  // takes the tuple-comparing query instead
+  if (bits > 63) {
+    plan.fits = false;
+    return plan;
+  }
   std::vector<std::pair<long long, int>> keyed(num_offsets);
   for (int64_t o = 0; o < num_offsets; ++o) {
     long long d = 0;
@@ -1050,7 +1127,10 @@ static QueryPlan make_plan(const long long *src_bounds, const long long *tgt_bou
                    });
   std::vector<int> group_start;
   for (int64_t i = 0; i < num_offsets; ++i) {
-    if (i == 0 || keyed[i].first - keyed[group_start.back()].first > kGroupSpan) {
+    // a group spans at most kGroupSpan in key and holds at most kGroupSpan + 1
+    // members (repeated offsets would otherwise overfill it)
+    if (i == 0 || keyed[i].first - keyed[group_start.back()].first > kGroupSpan ||
+        i - group_start.back() > kGroupSpan) {
       group_start.push_back(static_cast<int>(i));
     }
   }
@@ -1163,11 +1243,55 @@ static void resolve_bounds(const QueryArgs &a, const int64_t *source_bounds, con
   if (bounds_out != nullptr) memcpy(bounds_out, bounds, sizeof(long long) * 16);
 }
 
+static void enqueue_count_tiles(const void *kernel_map, int index_dtype, int64_t num_offsets,
+                                int64_t num_targets, unsigned *tile_counts, int num_tiles,
+                                hipStream_t stream);
+
+// The query of a frame that does not fit a packed key: tuple comparisons
+// (query_tuples_kernel), then the per-tile hit counts from the map it wrote.
+static void run_wide_query(const QueryArgs &a, const int64_t *offsets_host, int64_t num_offsets,
+                           bool batched, void *kernel_map, int out_dtype, unsigned *tile_counts,
+                           int num_tiles, Scope &scope, hipStream_t stream) {
+  std::vector<int> halves(static_cast<size_t>(num_offsets) * a.ndim * 2);
+  for (size_t i = 0; i < halves.size() / 2; ++i) {
+    const unsigned long long v = static_cast<unsigned long long>(offsets_host[i]);
+    halves[2 * i + 0] = static_cast<int>(static_cast<unsigned>(v & 0xffffffffull));
+    halves[2 * i + 1] = static_cast<int>(static_cast<unsigned>(v >> 32));
+  }
+  int *d_offsets = scope.alloc<int>(halves.size());
+  upload_ints(halves, d_offsets, stream);
+  const dim3 grid(static_cast<unsigned>(div_ceil(a.num_targets, kQueryBlock)), static_cast<unsigned>(num_offsets));
+  const int nb = static_cast<int>(a.num_batches);
+#define MNT_QT(CT, BT, OT)                                                                         \
+  query_tuples_kernel<CT, BT, OT><<<grid, kQueryBlock, 0, stream>>>(                               \
+      static_cast<const CT *>(a.sources), a.num_sources, static_cast<const CT *>(a.targets),       \
+      a.num_targets, d_offsets, a.ndim, batched ? static_cast<const BT *>(a.source_batch_dims) : nullptr, \
+      batched ? static_cast<const BT *>(a.target_batch_dims) : nullptr, nb, static_cast<OT *>(kernel_map))
+  const bool c32 = a.coord_dtype == MNT_INT32;
+  const bool b32 = !batched || a.batch_dtype == MNT_INT32;
+  const bool o32 = out_dtype == MNT_INT32;
+  if (c32 && b32 && o32) MNT_QT(int32_t, int32_t, int32_t);
+  else if (c32 && b32) MNT_QT(int32_t, int32_t, int64_t);
+  else if (c32 && o32) MNT_QT(int32_t, int64_t, int32_t);
+  else if (c32) MNT_QT(int32_t, int64_t, int64_t);
+  else if (b32 && o32) MNT_QT(int64_t, int32_t, int32_t);
+  else if (b32) MNT_QT(int64_t, int32_t, int64_t);
+  else if (o32) MNT_QT(int64_t, int64_t, int32_t);
+  else MNT_QT(int64_t, int64_t, int64_t);
+#undef MNT_QT
+  check_launch("query_tuples_kernel");
+  if (tile_counts != nullptr) {
+    enqueue_count_tiles(kernel_map, out_dtype, num_offsets, a.num_targets, tile_counts, num_tiles, stream);
+  }
+}
+
 // Runs the query into kernel_map (element type out_dtype) and, when tile_counts
 // is given, the per-(offset, tile) hit counts.  offsets_host: int64 [O, ndim].
 // With a sink the hits are staged for the pair lists instead and kernel_map
-// is not touched (tile_counts is needed then).
-static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t num_offsets,
+// is not touched (tile_counts is needed then).  Returns false, with nothing
+// launched, when a sink was given but the frame is too wide for packed keys:
+// the staged form needs them, the caller goes through a dense map instead.
+static bool run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t num_offsets,
                       const int64_t *source_bounds, const int64_t *target_bounds,
                       int64_t *bounds_out, void *kernel_map, int out_dtype, unsigned *tile_counts,
                       Scope &scope, hipStream_t stream, const HitSink *sink = nullptr) {
@@ -1179,6 +1303,13 @@ static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t n
   profile_mark("query_bounds+sync", stream);
   QueryPlan plan = make_plan(bounds, bounds + 8, offsets_host, num_offsets, a.ndim,
                              batched ? a.num_batches : 1);
+  if (!plan.fits) {
+    if (sink != nullptr) return false;
+    run_wide_query(a, offsets_host, num_offsets, batched, kernel_map, out_dtype, tile_counts, num_tiles,
+                   scope, stream);
+    profile_mark("query", stream);
+    return true;
+  }
   // Large tables are uploaded as kernel arguments of a tiny copy kernel: nothing
   // to keep alive on the host and no staging buffer another call could overwrite.
   const int no = static_cast<int>(num_offsets);
@@ -1208,7 +1339,7 @@ static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t n
     else MNT_QL(int64_t, int64_t);
 #undef MNT_QL
     profile_mark("query", stream);
-    return;
+    return true;
   }
   const HitSink none{nullptr, nullptr, nullptr, nullptr, 0, 0};
 #define MNT_Q(CT, BT, OT)                                                                        \
@@ -1224,6 +1355,7 @@ static void run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t n
   else MNT_Q(int64_t, int64_t, int64_t);
 #undef MNT_Q
   profile_mark("query", stream);
+  return true;
 }
 
 template <typename T>
@@ -1585,8 +1717,26 @@ extern "C" int mnt_kernel_map_lists(const void *sources, int64_t num_sources, co
     unsigned *plan = scope.alloc<unsigned>(4 * num_offsets + 1);
     enqueue_fill<unsigned>(row_totals, num_offsets, 0u, stream);
     const HitSink sink{stage, masks, row_totals, tile_mode, num_wave_tiles, no};
-    run_query(a, offsets_host, num_offsets, source_bounds_host, target_bounds_host, bounds_host_out,
-              nullptr, MNT_INT32, tile_counts, scope, stream, &sink);
+    if (!run_query(a, offsets_host, num_offsets, source_bounds_host, target_bounds_host, bounds_host_out,
+                   nullptr, MNT_INT32, tile_counts, scope, stream, &sink)) {
+      // a frame too wide for packed keys: dense map by tuple comparisons (the
+      // staging block has the right size for it), then the lists from that map
+      int64_t known[16];
+      if (bounds_host_out != nullptr) memcpy(known, bounds_host_out, sizeof(known));
+      const int64_t *src_known = bounds_host_out != nullptr ? known : source_bounds_host;
+      const int64_t *tgt_known = bounds_host_out != nullptr ? known + 8 : target_bounds_host;
+      run_query(a, offsets_host, num_offsets, src_known, tgt_known, nullptr, stage, MNT_INT32, tile_counts,
+                scope, stream);
+      unsigned *row_sizes = scope.alloc<unsigned>(num_offsets);
+      const MapState state{num_sources, num_targets, num_offsets, num_tiles, reorder, stage};
+      const unsigned long long sequence = enqueue_sizes(arena, state, tile_counts, row_sizes, plan, stream);
+      enqueue_emit<int32_t>(stage, num_sources, num_targets, no, tile_counts, num_tiles, plan + no, plan + 3 * no,
+                            nullptr, nullptr, in_idx_out, out_idx_out, stream, plan, sizes_dev_out,
+                            order_dev_out);
+      collect_sizes(arena, sequence, num_offsets, sizes_host_out, order_host_out);
+      profile_mark("map_sizes_order+emit+sync", stream);
+      return;
+    }
     unsigned *d_plan_host = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned_device()) + Arena::kPlanOffset);
     const unsigned long long sequence = arena.next_sequence();
     dim3 grid(static_cast<unsigned>(div_ceil(num_tiles, kPlaceTiles)), static_cast<unsigned>(num_offsets));

@@ -115,12 +115,14 @@ __device__ __forceinline__ void make_plan_on_device(const long long *__restrict_
   int lead[MNT_MAX_NDIM];
 #pragma unroll
   for (int k = 0; k < MNT_MAX_NDIM; ++k) lead[k] = __shfl(d[k], origin);
-  // first place whose delta lies beyond this one's group span (num_offsets if none)
+  // first place whose delta lies beyond this one's group span (num_offsets if
+  // none), and never more than kPlanGroupSpan + 1 members (repeated offsets)
   int next = num_offsets;
   for (int p = num_offsets - 1; p >= 0; --p) {
     const long long other = __shfl(mine, p);
     next = p > lane && other - mine > kPlanGroupSpan ? p : next;
   }
+  next = next < lane + kPlanGroupSpan + 1 ? next : lane + kPlanGroupSpan + 1;
   // the greedy grouping follows those links from place 0
   unsigned long long starts = 0;
   int num_groups = 0;

@@ -16,14 +16,70 @@ void set_last_error(const std::string &message) { g_last_error = message; }
 static std::mutex g_arena_mutex;
 static std::map<std::pair<int, hipStream_t>, Arena *> g_arenas;
 
-Arena &Arena::of(hipStream_t stream) {
+// ---- one caller thread per stream ------------------------------------------
+
+static std::atomic<unsigned long long> g_next_thread_token{1};
+static thread_local unsigned long long t_token = 0;
+static thread_local int t_depth = 0;
+static thread_local std::vector<Arena *> t_taken;      // arenas this thread took during the call under way
+
+static unsigned long long thread_token() {
+  if (t_token == 0) t_token = g_next_thread_token.fetch_add(1, std::memory_order_relaxed);
+  return t_token;
+}
+
+void enter_call() { ++t_depth; }
+
+// Current device, or -1 on a machine without one (the registry and its
+// ownership rules work there too; anything that allocates fails later).
+static int registry_device() {
   int device = 0;
-  MNT_HIP(hipGetDevice(&device));
+  if (hipGetDevice(&device) != hipSuccess) {
+    (void)hipGetLastError();
+    device = -1;
+  }
+  return device;
+}
+
+Arena &Arena::of(hipStream_t stream) {
+  const int device = registry_device();
+  const unsigned long long me = thread_token();
   std::lock_guard<std::mutex> lock(g_arena_mutex);
   auto key = std::make_pair(device, stream);
   auto it = g_arenas.find(key);
   if (it == g_arenas.end()) it = g_arenas.emplace(key, new Arena(stream)).first;
-  return *it->second;
+  Arena &arena = *it->second;
+  if ((arena.held_ || arena.pinned_by_thread_) && arena.holder_ != me) {
+    MNT_FAIL("stream %p is in use by another thread: the library keeps per-stream state (scratch arena, "
+             "two-phase build state) and takes one caller thread per stream at a time",
+             static_cast<void *>(stream));
+  }
+  if (t_depth > 0 && !arena.held_) {
+    arena.held_ = true;
+    arena.holder_ = me;
+    t_taken.push_back(&arena);
+  }
+  return arena;
+}
+
+void leave_call() {
+  if (--t_depth > 0 || t_taken.empty()) return;
+  std::lock_guard<std::mutex> lock(g_arena_mutex);
+  for (Arena *arena : t_taken) arena->held_ = false;
+  t_taken.clear();
+}
+
+void Arena::pin(hipStream_t stream) {
+  Arena &arena = Arena::of(stream);              // fails when another thread is inside or has pinned it
+  std::lock_guard<std::mutex> lock(g_arena_mutex);
+  arena.pinned_by_thread_ = true;
+  arena.holder_ = thread_token();
+}
+
+void Arena::unpin(hipStream_t stream) {
+  Arena &arena = Arena::of(stream);
+  std::lock_guard<std::mutex> lock(g_arena_mutex);
+  arena.pinned_by_thread_ = false;
 }
 
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -94,7 +150,16 @@ void Arena::free_all(bool synchronise) {
 void Arena::reset_device() {
   int device = 0;
   MNT_HIP(hipGetDevice(&device));
+  const unsigned long long me = thread_token();
   std::lock_guard<std::mutex> lock(g_arena_mutex);
+  for (const auto &entry : g_arenas) {
+    const Arena *arena = entry.second;
+    MNT_CHECK(entry.first.first != device || !(arena->held_ || arena->pinned_by_thread_) || arena->holder_ == me,
+              "another thread is inside the library on stream %p of this device: no reset while it is",
+              static_cast<void *>(entry.first.second));
+  }
+  for (Arena *arena : t_taken) arena->held_ = false;     // this thread's own: they are about to go
+  t_taken.clear();
   for (auto it = g_arenas.begin(); it != g_arenas.end();) {
     if (it->first.first != device) {
       ++it;
@@ -224,6 +289,55 @@ void profile_mark(const char *label, hipStream_t stream) {
   g_marks.emplace_back(label, event);
 }
 
+// ---- plain streaming kernels: the memory ceilings a benchmark quotes -------
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+constexpr int kStreamBlock = 256;
+constexpr int kStreamUnroll = 4;            // 16-byte vectors in flight per lane
+
+__global__ __launch_bounds__(kStreamBlock) void stream_copy_kernel(const u32x4 *__restrict__ src,
+                                                                  u32x4 *__restrict__ dst, long long vectors) {
+  const long long stride = static_cast<long long>(gridDim.x) * kStreamBlock;
+  long long i = static_cast<long long>(blockIdx.x) * kStreamBlock + threadIdx.x;
+  for (; i + (kStreamUnroll - 1) * stride < vectors; i += kStreamUnroll * stride) {
+    u32x4 v[kStreamUnroll];
+#pragma unroll
+    for (int u = 0; u < kStreamUnroll; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < kStreamUnroll; ++u) __builtin_nontemporal_store(v[u], dst + i + u * stride);
+  }
+  for (; i < vectors; i += stride) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
+__global__ __launch_bounds__(kStreamBlock) void stream_read_kernel(const u32x4 *__restrict__ src,
+                                                                  long long vectors, unsigned *__restrict__ sink) {
+  const long long stride = static_cast<long long>(gridDim.x) * kStreamBlock;
+  long long i = static_cast<long long>(blockIdx.x) * kStreamBlock + threadIdx.x;
+  unsigned acc = 0;
+  for (; i + (kStreamUnroll - 1) * stride < vectors; i += kStreamUnroll * stride) {
+    u32x4 v[kStreamUnroll];
+#pragma unroll
+    for (int u = 0; u < kStreamUnroll; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < kStreamUnroll; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+  for (; i < vectors; i += stride) {
+    const u32x4 v = __builtin_nontemporal_load(src + i);
+    acc ^= v.x ^ v.y ^ v.z ^ v.w;
+  }
+  // the data is all zero, so nothing is ever stored; the test keeps the loads alive
+  if (acc == 0x9e3779b9u) sink[0] = acc;
+}
+
+__global__ __launch_bounds__(kStreamBlock) void stream_write_kernel(u32x4 *__restrict__ dst, long long vectors,
+                                                                   unsigned value) {
+  const long long stride = static_cast<long long>(gridDim.x) * kStreamBlock;
+  const u32x4 v = {value, value, value, value};
+  for (long long i = static_cast<long long>(blockIdx.x) * kStreamBlock + threadIdx.x; i < vectors; i += stride) {
+    __builtin_nontemporal_store(v, dst + i);
+  }
+}
+
 static void profile_clear() {
   for (auto &m : g_marks) g_event_pool.push_back(m.second);
   g_marks.clear();
@@ -265,6 +379,72 @@ size_t mnt_buffer_used_size(void *stream) {
   size_t value = 0;
   guarded([&] { value = Arena::of(static_cast<hipStream_t>(stream)).used(); });
   return value;
+}
+
+int mnt_stream_acquire(void *stream) {
+  return guarded([&] { Arena::pin(static_cast<hipStream_t>(stream)); });
+}
+
+int mnt_stream_release(void *stream) {
+  return guarded([&] { Arena::unpin(static_cast<hipStream_t>(stream)); });
+}
+
+int mnt_time_memory(int kind, size_t bytes, int repeats, float *ms_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MNT_CHECK(kind >= 0 && kind <= 2, "kind must be 0 (copy), 1 (read) or 2 (write), found %d", kind);
+    MNT_CHECK(bytes >= 4096 && bytes % 16 == 0 && bytes <= (size_t(64) << 30), "bytes = %zu out of range", bytes);
+    MNT_CHECK(repeats >= 1 && repeats <= 1000 && ms_out != nullptr, "bad argument");
+    Scope scope(stream);
+    const long long vectors = static_cast<long long>(bytes / 16);
+    u32x4 *a = scope.alloc<u32x4>(vectors);
+    u32x4 *b = kind == 0 ? scope.alloc<u32x4>(vectors) : nullptr;
+    unsigned *sink = scope.alloc<unsigned>(4);
+    // enough workgroups to keep every compute unit's load queues full, few
+    // enough that each lane streams a long run
+    const unsigned grid = static_cast<unsigned>(compute_units()) * 16u;
+    stream_write_kernel<<<grid, kStreamBlock, 0, stream>>>(a, vectors, 0u);          // also faults the pages in
+    if (b != nullptr) stream_write_kernel<<<grid, kStreamBlock, 0, stream>>>(b, vectors, 0u);
+    auto once = [&] {
+      if (kind == 0) stream_copy_kernel<<<grid, kStreamBlock, 0, stream>>>(a, b, vectors);
+      else if (kind == 1) stream_read_kernel<<<grid, kStreamBlock, 0, stream>>>(a, vectors, sink);
+      else stream_write_kernel<<<grid, kStreamBlock, 0, stream>>>(a, vectors, 1u);
+    };
+    once();
+    check_launch("stream kernel");
+    hipEvent_t start, stop;
+    MNT_HIP(hipEventCreate(&start));
+    MNT_HIP(hipEventCreate(&stop));
+    MNT_HIP(hipEventRecord(start, stream));
+    for (int r = 0; r < repeats; ++r) once();
+    MNT_HIP(hipEventRecord(stop, stream));
+    hipError_t status = hipEventSynchronize(stop);
+    float ms = 0.0f;
+    if (status == hipSuccess) status = hipEventElapsedTime(&ms, start, stop);
+    (void)hipEventDestroy(start);
+    (void)hipEventDestroy(stop);
+    MNT_HIP(status);
+    *ms_out = ms / static_cast<float>(repeats);
+  });
+}
+
+int mnt_device_facts(int64_t *facts_out, int capacity) {
+  return guarded([&] {
+    MNT_CHECK(facts_out != nullptr && capacity >= 6, "facts_out needs room for 6 values");
+    int device = 0;
+    MNT_HIP(hipGetDevice(&device));
+    const hipDeviceAttribute_t wanted[5] = {hipDeviceAttributeMultiprocessorCount, hipDeviceAttributeClockRate,
+                                            hipDeviceAttributeMemoryClockRate, hipDeviceAttributeMemoryBusWidth,
+                                            hipDeviceAttributeL2CacheSize};
+    for (int i = 0; i < 5; ++i) {
+      int value = 0;
+      MNT_HIP(hipDeviceGetAttribute(&value, wanted[i], device));
+      facts_out[i] = value;
+    }
+    size_t free_bytes = 0, total_bytes = 0;
+    MNT_HIP(hipMemGetInfo(&free_bytes, &total_bytes));
+    facts_out[5] = static_cast<int64_t>(total_bytes);
+  });
 }
 
 int mnt_profile_enable(int on) {

@@ -43,6 +43,8 @@ SIGNATURES = {
     "mnt_buffer_used_size": (_sz, [_vp]),
     "mnt_reset_error": (_int, []),
     "mnt_device_reset": (_int, []),
+    "mnt_stream_acquire": (_int, [_vp]),
+    "mnt_stream_release": (_int, [_vp]),
     "mnt_host_wait_stats": (_int, [_pi64, _pi64, _int]),
     "mnt_lookahead_start": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _pi64, _vp, _int, _int, _pi64,
                                    _vp, _vp]),
@@ -101,6 +103,9 @@ SIGNATURES = {
                                 _int, _pf, _vp]),
     "mnt_time_gemm": (_int, [_int, _i64, _int, _dbl, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int,
                              _int, _pf, _vp]),
+    "mnt_time_memory": (_int, [_int, _sz, _int, _pf, _vp]),
+    "mnt_device_facts": (_int, [_pi64, _int]),
+    "mnt_timer_repeats": (_int, [_int]),
     "mnt_profile_enable": (_int, [_int]),
     "mnt_profile_read": (_int, [_int, _pf, _c.c_char_p, _int, _c.POINTER(_c.c_int)]),
 }
@@ -1339,11 +1344,38 @@ def cuda_reset_error():
     load_library().mnt_reset_error()
 
 
+_device_resets = 0
+
+
+def device_reset_count() -> int:
+    """How often :func:`cuda_device_reset` has run in this process (what holds
+    addresses of the library's scratch memory checks it before using them)."""
+    return _device_resets
+
+
 def cuda_device_reset():
     """csrc/minuet/torch/cuda_memory_buffer.cu:38,47.  Frees everything the library
     holds on the current device (every stream's arena); unlike the reference's
-    cudaDeviceReset() it leaves the context, and with it every torch tensor, alone."""
+    cudaDeviceReset() it leaves the context, and with it every torch tensor, alone.
+    Passes captured with ``minuet.capture_forward`` before the reset refuse to
+    replay after it (their kernels point into the freed scratch memory)."""
+    global _device_resets
+    _device_resets += 1
     _check(load_library().mnt_device_reset())
+
+
+def stream_acquire(stream=None):
+    """Keeps the library's state of ``stream`` (a raw handle; None = the null
+    stream) for the calling thread until :func:`stream_release`: calls of other
+    threads on that stream fail meanwhile.  One caller thread per stream at a
+    time is the library's threading contract (ctypes releases the interpreter
+    lock during a call, so two Python threads can be inside the library at once;
+    the reference's pybind module holds the lock, csrc/minuet/torch/common.h:17-21)."""
+    _check(load_library().mnt_stream_acquire(stream))
+
+
+def stream_release(stream=None):
+    _check(load_library().mnt_stream_release(stream))
 
 
 def host_wait_stats(reset: bool = False):
@@ -1401,6 +1433,32 @@ def lookahead_finish(device: torch.device):
     it enqueued; a no-op without a session."""
     with _on(device):
         _check(load_library().mnt_lookahead_finish(_stream(device)))
+
+
+def time_memory(kind: str, nbytes: int, repeats: int = 10, device=None) -> float:
+    """Milliseconds one plain streaming kernel takes for ``nbytes`` of device
+    memory: ``kind`` "copy" (reads and writes that many bytes), "read" or "write"."""
+    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    ms = ctypes.c_float(0.0)
+    with _on(device):
+        _check(load_library().mnt_time_memory({"copy": 0, "read": 1, "write": 2}[kind], nbytes, repeats,
+                                              ctypes.byref(ms), _stream(device)))
+    return float(ms.value)
+
+
+def device_facts():
+    """Compute units, clocks, bus width, L2 and memory size of the current device."""
+    facts = (ctypes.c_int64 * 6)()
+    _check(load_library().mnt_device_facts(facts, 6))
+    return {"compute_units": int(facts[0]), "engine_clock_mhz": facts[1] / 1e3,
+            "memory_clock_mhz": facts[2] / 1e3, "memory_bus_bits": int(facts[3]),
+            "l2_bytes": int(facts[4]), "memory_bytes": int(facts[5])}
+
+
+def timer_repeats(repeats: int):
+    """Launches per run of the ``cuda_time_*`` stage timers (1 = the reference's
+    protocol; more = back-to-back launches, time of one)."""
+    _check(load_library().mnt_timer_repeats(int(repeats)))
 
 
 def profile_enable(on: bool):

@@ -22,11 +22,19 @@ class GraphedForward:
     coordinates must not change), replay, and read ``output``."""
 
     def __init__(self, graph: "torch.cuda.CUDAGraph", output, stream: "torch.cuda.Stream"):
+        from minuet_amd.nn.functional import _C
         self.graph = graph
         self.output = output
         self.stream = stream
+        self._reset_count = _C.device_reset_count()
 
     def replay(self):
+        """Raises after ``cuda_device_reset()``: the reset gave back the scratch
+        memory whose addresses the captured kernels hold."""
+        from minuet_amd.nn.functional import _C
+        if _C.device_reset_count() != self._reset_count:
+            raise RuntimeError("[Minuet] this captured pass is no longer valid: cuda_device_reset() freed the "
+                               "scratch memory its kernels point into; capture the pass again")
         self.graph.replay()
         return self.output
 
@@ -44,15 +52,24 @@ def capture_forward(forward: Callable[[], object], warmup: int = 3) -> GraphedFo
     graph's kernels use scratch pointers of that stream's arena, which
     therefore must not be freed (``cuda_free_buffers`` acts on the arena of
     the stream that is current, never this one) nor used by other work.  Replays
-    of one ``GraphedForward`` must not overlap (they share that scratch)."""
+    of one ``GraphedForward`` must not overlap (they share that scratch).
+    ``cuda_device_reset()`` does free that arena: a ``GraphedForward`` captured
+    before it refuses to replay afterwards.
+
+    A look-ahead session of a ``KernelMapCache(lookahead=True)`` that is still
+    running is ended before the capture starts: its worker thread allocates and
+    launches on its own, which would invalidate a capture under way on this
+    thread."""
     if not torch.cuda.is_available():
         raise RuntimeError("[Minuet] graph capture needs a GPU")
+    from minuet_amd.nn.lookahead import end_running_session
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.no_grad(), torch.cuda.stream(side):
         for _ in range(max(1, warmup)):
             forward()
     torch.cuda.current_stream().wait_stream(side)
+    end_running_session(torch.device("cuda", torch.cuda.current_device()))
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.no_grad(), torch.cuda.graph(graph, stream=side):

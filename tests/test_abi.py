@@ -87,3 +87,44 @@ def test_padding_plan_rejects_bad_boundaries():
     assert _C.load_library().mnt_last_error().startswith(b"[Minuet]")
     _C.cuda_reset_error()
     assert _C.load_library().mnt_last_error() == b""
+
+
+def test_one_caller_thread_per_stream():
+    """A second thread that enters the library on a stream another thread holds
+    fails with a message instead of racing; after the release it gets through."""
+    import threading
+    lib = _C.load_library()
+    results = {}
+
+    def other(tag):
+        status = lib.mnt_buffer_set_growth(None, ctypes.c_float(1.0))
+        results[tag] = (status, lib.mnt_last_error().decode())
+
+    _C.stream_acquire(None)
+    try:
+        assert lib.mnt_buffer_set_growth(None, ctypes.c_float(1.0)) == 0      # the holder itself gets through
+        worker = threading.Thread(target=other, args=("held",))
+        worker.start()
+        worker.join()
+    finally:
+        _C.stream_release(None)
+    worker = threading.Thread(target=other, args=("free",))
+    worker.start()
+    worker.join()
+    status, message = results["held"]
+    assert status != 0 and "in use by another thread" in message and message.startswith("[Minuet]")
+    assert results["free"][0] == 0
+    # a stream nobody holds is unaffected by the hold on another one
+    _C.stream_acquire(None)
+    try:
+        side = ctypes.c_void_p(0x1000)          # never dereferenced: only names the registry entry
+        done = {}
+
+        def elsewhere():
+            done["status"] = lib.mnt_buffer_set_growth(side, ctypes.c_float(1.0))
+        worker = threading.Thread(target=elsewhere)
+        worker.start()
+        worker.join()
+        assert done["status"] == 0
+    finally:
+        _C.stream_release(None)

@@ -45,6 +45,35 @@ def test_config2_map_step_full_size_bit_exact():
     np.testing.assert_array_equal(host(built["out_idx"]), eout)
 
 
+@pytest.mark.parametrize("reorder", [True, False])
+def test_config2_map_step_one_call_full_size_bit_exact(reorder):
+    """The entry point bench.py times (mnt_sorted_kernel_map_lists: unsorted
+    voxels -> sorted voxels -> per-offset pair lists in one call) at the full
+    200 000 voxels of configuration 2, rows in size order and in offset order
+    (reference flow: minuet/nn/convolutions.py:147-170)."""
+    coords = make_cloud(2)["coords"]
+    offsets = orc.generate_kernel_offsets(3, 3)
+    built = _C.sorted_kernel_map_lists(dev(coords), offsets, reorder=reorder, result_only=True)
+    ref_index, ref_sorted = c_oracle.arg_sort(coords)
+    np.testing.assert_array_equal(host(built["indices"]).astype(np.int64), ref_index)
+    np.testing.assert_array_equal(host(built["coordinates"]), ref_sorted)
+    np.testing.assert_array_equal(built["bounds"][:3], coords.min(0))
+    np.testing.assert_array_equal(built["bounds"][4:7], coords.max(0))
+    ref_map = c_oracle.query(ref_sorted, ref_sorted, offsets.astype(np.int32))
+    sizes = c_oracle.sizes(ref_map)
+    order = orc.stable_size_order(sizes) if reorder else np.arange(offsets.shape[0])
+    np.testing.assert_array_equal(built["order_host"], order)
+    np.testing.assert_array_equal(built["sizes_host"], sizes[order])
+    np.testing.assert_array_equal(host(built["order"]), order)
+    np.testing.assert_array_equal(host(built["sizes"]), sizes[order])
+    ein, eout = c_oracle.pair_lists(np.ascontiguousarray(ref_map[order]))
+    np.testing.assert_array_equal(host(built["in_idx"]), ein)
+    np.testing.assert_array_equal(host(built["out_idx"]), eout)
+    # what the timed loop does: the same call again and again on the same stream
+    again = _C.sorted_kernel_map_lists(dev(coords), offsets, reorder=reorder, result_only=True)
+    assert torch.equal(again["in_idx"], built["in_idx"]) and torch.equal(again["out_idx"], built["out_idx"])
+
+
 def test_config1_layer_fp32_full_size():
     coords = make_cloud(1)["coords"]
     rng = np.random.default_rng(1001)

@@ -56,3 +56,20 @@ def test_capture_after_cache_reset_warms_up_first():
     graphed = minuet.capture_forward(lambda: net(x), warmup=1)
     with torch.no_grad():
         assert torch.equal(graphed.replay().F, net(x).F)
+
+
+def test_replay_is_refused_after_a_device_reset():
+    """cuda_device_reset() frees the capture stream's scratch arena, whose
+    addresses the captured kernels hold: the captured pass must not run again."""
+    net, x, _ = _unet_and_input(torch.float16)
+    graphed = minuet.capture_forward(lambda: net(x), warmup=1)
+    with torch.no_grad():
+        assert torch.equal(graphed.replay().F, net(x).F)
+    torch.cuda.synchronize()
+    _C.cuda_device_reset()
+    with pytest.raises(RuntimeError, match="no longer valid"):
+        graphed.replay()
+    # the library itself goes on working, and a new capture is fine
+    again = minuet.capture_forward(lambda: net(x), warmup=1)
+    with torch.no_grad():
+        assert torch.equal(again.replay().F, net(x).F)

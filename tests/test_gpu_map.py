@@ -547,6 +547,89 @@ def test_kernel_map_lists_only_many_chunks_and_int64():
     assert built["in_idx"].numel() == 0
 
 
+def test_repeated_offsets_fill_their_own_rows():
+    """An offset table that names the same offset several times: every copy
+    gets its own row of the map, sizes and lists (the reference resolves each
+    row of the table on its own, query_sorted_index_with_offsets.cuh:36-77);
+    seven copies of one offset overfill a group of the query's plan."""
+    src, _, _, _, base = _query_case(37, 30000, 45, -10, 3)
+    off = np.concatenate([base[:5], np.repeat(base[13:14], 7, axis=0), base[20:], base[4:6]]).astype(np.int32)
+    dense = orc.query_sorted_index_with_offsets(src, src, off, dtype=np.int32)
+    got = F.query_sorted_index_with_offsets(dev(src), dev(src), dev(off))
+    np.testing.assert_array_equal(host(got), dense)
+    for reorder in (True, False):
+        _check_lists_only(src, None, src, None, off, reorder)
+    cloud = src[np.random.default_rng(2).permutation(src.shape[0])]
+    _check_sorted_lists(cloud, off.astype(np.int64))
+
+
+def _wide_cloud(ndim, span_bits, dtype, clusters=60, per_cluster=60, seed=23):
+    """Clusters of neighbouring voxels scattered over a range of 2^span_bits per
+    dimension: neighbours exist, and a packed key of the frame would need
+    ndim * span_bits bits."""
+    rng = np.random.default_rng(seed)
+    half = 1 << (span_bits - 1)
+    centres = rng.integers(-half, half, size=(clusters, ndim))
+    centres[0], centres[1] = -half, half - 4                    # the corners of the range
+    rows = (centres[:, None, :] + rng.integers(0, 4, size=(clusters, per_cluster, ndim))).reshape(-1, ndim)
+    return rows.astype(dtype)
+
+
+def _brute_force_map(src, sbd, tgt, tbd, off):
+    """Dict look-up of every shifted target, batch by batch."""
+    nb = 1 if sbd is None else len(sbd) - 1
+    sb = [0, src.shape[0]] if sbd is None else [int(v) for v in sbd]
+    tb = [0, tgt.shape[0]] if tbd is None else [int(v) for v in tbd]
+    out = np.full((off.shape[0], tgt.shape[0]), -1, dtype=np.int64)
+    for b in range(nb):
+        where = {tuple(int(v) for v in src[j]): j for j in range(sb[b], sb[b + 1])}
+        for t in range(tb[b], tb[b + 1]):
+            row = [int(v) for v in tgt[t]]
+            for o in range(off.shape[0]):
+                out[o, t] = where.get(tuple(c + int(d) for c, d in zip(row, off[o])), -1)
+    return out
+
+
+@pytest.mark.parametrize("ndim,span_bits,cdtype,batched", [
+    (4, 40, np.int64, False), (4, 40, np.int64, True), (3, 30, np.int64, False),
+    (4, 20, np.int32, False), (3, 31, np.int32, True), (4, 62, np.int64, False),
+])
+def test_query_on_frames_wider_than_a_packed_key(ndim, span_bits, cdtype, batched):
+    """Coordinate ranges whose packed key would need more than 63 bits: the
+    reference compares whole tuples (csrc/minuet/common/functions.h:94-105), so
+    any range works there; here such frames take the tuple-comparing query.
+    Dense map, sizes, rank tables, pair lists and the one-call Map step."""
+    cloud = _wide_cloud(ndim, span_bits, cdtype)
+    bd = np.array([0, cloud.shape[0] // 3, cloud.shape[0]], dtype=np.int32) if batched else None
+    src, sbd = sorted_unique(cloud, bd)
+    kernel = 3 if ndim == 3 else 2
+    off = orc.generate_kernel_offsets(ndim, kernel, 1, 1).astype(cdtype)
+    expect = _brute_force_map(src, sbd, src, sbd, off)
+    assert (expect >= 0).sum() > 2 * src.shape[0]                 # neighbours were found
+    np.testing.assert_array_equal(orc.query_sorted_index_with_offsets(src, src, off, sbd, sbd), expect)
+    got = F.query_sorted_index_with_offsets(dev(src), dev(src), dev(off), dev(sbd), dev(sbd))
+    np.testing.assert_array_equal(host(got), expect)
+    for reorder in (True, False):
+        built = _C.kernel_map_build(dev(src), dev(src), off.astype(np.int64), dev(sbd), dev(sbd),
+                                    reorder=reorder, want_masks=True, want_lists=True, want_dense=True)
+        esm, etm, eorder, esizes, em = orc.build_kernel_map(src, sbd, src, sbd, off, reorder=reorder)
+        np.testing.assert_array_equal(host(built["kernel_map"]), expect)
+        np.testing.assert_array_equal(built["sizes_host"], esizes.astype(np.int64))
+        np.testing.assert_array_equal(host(built["source_masks"]), esm)
+        np.testing.assert_array_equal(host(built["target_masks"]), etm)
+        ein, eout, _ = orc.kernel_map_pair_lists(em)
+        np.testing.assert_array_equal(host(built["in_idx"]), ein)
+        np.testing.assert_array_equal(host(built["out_idx"]), eout)
+        _check_lists_only(src, sbd, src, sbd, off, reorder)
+    if not batched:
+        shuffled = src[np.random.default_rng(1).permutation(src.shape[0])]
+        _check_sorted_lists(shuffled, off.astype(np.int64))
+        # ... and through a layer's cache
+        cache = minuet.nn.KernelMapCache(ndim=ndim, dtype=torch.int32, device="cuda")
+        dense = cache.get_dense_kernel_map(dev(src), 1, None, dev(src), 1, None, kernel, 1)
+        np.testing.assert_array_equal(host(dense), expect)
+
+
 def _check_sorted_lists(cloud, off, reorder=True):
     """mnt_sorted_kernel_map_lists against the oracle's sort and kernel map."""
     indices, sorted_dev, built = _C.sorted_kernel_map_lists(dev(cloud), off.astype(np.int64), reorder=reorder)

@@ -67,6 +67,30 @@ def test_unet_passes_match_the_ordinary_cache():
     assert FORCED_FOR_ALL or (hits[0] == 0 and all(h >= 13 for h in hits[1:])), hits
 
 
+def test_config4_full_size_cold_passes_bit_equal_to_the_plain_cache():
+    """The UNet of configuration 4 at its full size (2 x 100 000 voxels, widths
+    32 ... 256): cold passes with the look-ahead against cold passes of the
+    ordinary cache, bit for bit, coordinates and features."""
+    torch.manual_seed(4)
+    net = SparseUNet(4, 32, dtype=torch.float16, device="cuda").eval()
+    plain = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda")
+    ahead = minuet.nn.KernelMapCache(ndim=3, dtype=torch.int32, device="cuda", lookahead=True)
+    coords, bd = _cloud(1.0, 0)
+    feats = torch.randn(coords.shape[0], 4, device="cuda").half()
+    minuet.set_kernel_map_cache(net, plain)
+    want = _run(net, plain, coords, bd, feats)
+    minuet.set_kernel_map_cache(net, ahead)
+    hits = []
+    for step in range(3):
+        before = ahead.num_ahead_hits
+        got = _run(net, ahead, coords, bd, feats)
+        torch.cuda.synchronize()
+        assert torch.equal(got.C, want.C) and torch.equal(got.F, want.F), f"pass {step}"
+        hits.append(ahead.num_ahead_hits - before)
+    ahead.reset()
+    assert FORCED_FOR_ALL or (hits[0] == 0 and all(h >= 13 for h in hits[1:])), hits
+
+
 def test_changed_requests_fall_back_to_ordinary_builds():
     """A pass that asks for other maps than the recipe holds builds them itself;
     what the worker built for nobody is dropped at reset()."""
