@@ -92,10 +92,14 @@ __device__ __forceinline__ long long wave_lower_bound(const KeyReader<CT, BT> &s
 struct HitSink {
   int *stage;                      // [O, T]
   unsigned long long *masks;       // [O, ceil(T / 64)]
-  unsigned *row_totals;            // [O], zero before the launch; hits are added with atomics
+  unsigned *row_totals;            // [total_copies][total_stride], zero before the launch; a tile adds its hits
+                                   // to copy (tile % total_copies) with atomics: one copy of a few dozen words
+                                   // is two cache lines that every tile's atomics would queue up behind
   unsigned *tile_mode;             // [tiles]: 0 = compacted, 1 = a slot per target
   long long num_wave_tiles;        // ceil(T / 64)
   int num_offsets;
+  unsigned *repeats;               // raised when two rows of a cloud mapped onto itself are equal (nullable)
+  int total_copies, total_stride;
 };
 
 // Settles the queries of one group against the candidates cand[0 .. span]
@@ -395,6 +399,11 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     OT *__restrict__ kernel_map, unsigned *__restrict__ tile_counts, int num_tiles, int dir_rows,
     HitSink sink, const DevicePlan *__restrict__ device_plan) {
   extern __shared__ __align__(16) unsigned s_dynamic[];
+  // Only half of the offsets are looked up (a cloud mapped onto itself under
+  // offsets that come in pairs d / -d; see DevicePlan): the totals of the other
+  // half are kept here as well, and equal rows, which break the symmetry, are
+  // reported.
+  bool halves = false;
   if (device_plan != nullptr) {
     // a launch inside a chain that never went back to the host: the verdict of
     // the launches before it and the plan come from device memory.  The values
@@ -414,11 +423,13 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     delta_min = uniform64(device_plan->delta_min);
     delta_max = uniform64(device_plan->delta_max);
     const int in_rows = __builtin_amdgcn_readfirstlane(device_plan->groups_in_rows);
+    halves = __builtin_amdgcn_readfirstlane(device_plan->halves) != 0;
     if (__builtin_amdgcn_readfirstlane(verdict) != 0) return;
     dir_rows = in_rows != 0 && last_width(frame) >= 3 ? dir_rows : 0;
   }
   __shared__ unsigned long long win[kWindowChunk + kWindowPad];
   __shared__ long long s_bounds[2];
+  __shared__ unsigned long long s_wave_first[kQueryThreads / kWave + 1];
   // dynamic LDS: [group table: 4 words each][member table: 2 words each][hit counts]
   // [row directory: dir_rows 16-bit entries]
   // With gridDim.y > 1 the offset groups are dealt over the y index: every
@@ -463,6 +474,17 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     }
   }
   for (int o = tid; o < num_offsets; o += kQueryThreads) s_counts[o] = 0;
+  // where the totals of the offsets that are not looked up go: read now, used by the
+  // last lines of the kernel, which would otherwise wait for a trip to memory
+  __shared__ short s_mirror[kPlanMaxOffsets];
+  __shared__ int s_zero_offset;
+  if (halves && w == 2) {                      // one wavefront, a lane per offset (at most 64 of them in a chain)
+    const int o = lane_id();
+    const bool named = o < num_offsets && o < kPlanMaxOffsets;
+    if (named) s_mirror[o] = static_cast<short>(device_plan->mirror[o]);
+    const unsigned long long zero = __ballot(named && device_plan->kind[o] == 2);
+    if (o == 0) s_zero_offset = zero != 0ull ? __builtin_ctzll(zero) : -1;
+  }
 
   // ---- window of sources that can match any (offset, target) pair of the tile:
   // wavefront 0 finds its lower end, wavefront 1 its upper end
@@ -476,7 +498,18 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     const long long pos = wave_lower_bound<CT, BT>(src, frame, edge, 0, num_sources);
     if (lane_id() == 0) s_bounds[w] = pos;
   }
+  if (halves) {
+    if (lane_id() == 0) s_wave_first[w] = key;
+    if (tid == kQueryThreads - 1) s_wave_first[kQueryThreads / kWave] = t_end < num_targets ? tgt(t_end, frame) : ~0ull;
+  }
   __syncthreads();
+  if (halves) {
+    // a row equal to the row behind it (the rows are sorted): no symmetry to rely on
+    const unsigned long long down = __shfl_down(key, 1);
+    const unsigned long long next_key = t + 1 >= t_end ? s_wave_first[kQueryThreads / kWave]
+                                        : lane_id() == kWave - 1 ? s_wave_first[w + 1] : down;
+    if (__ballot(valid && next_key == key) != 0ull && lane_id() == 0) sink.repeats[0] = 1u;
+  }
   const long long w_lo = s_bounds[0];
   const long long w_hi = s_bounds[1] > w_lo ? s_bounds[1] : w_lo;
   const long long span = w_hi - w_lo;
@@ -562,7 +595,16 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
       const int o = s_members[m].y;
       const unsigned hits = s_counts[o];
       tile_counts[static_cast<long long>(o) * num_tiles + blockIdx.x] = hits;
-      if (kLists && hits != 0) atomicAdd(&sink.row_totals[o], hits);
+      if (kLists && hits != 0) {
+        unsigned *totals = sink.row_totals + static_cast<int>(blockIdx.x % sink.total_copies) * sink.total_stride;
+        atomicAdd(&totals[o], hits);
+        if (halves) atomicAdd(&totals[s_mirror[o]], hits);               // the mirror image has the same hits
+      }
+    }
+    // the zero offset: every target of the tile is its own hit
+    if (kLists && halves && tid == 0 && s_zero_offset >= 0) {
+      unsigned *totals = sink.row_totals + static_cast<int>(blockIdx.x % sink.total_copies) * sink.total_stride;
+      atomicAdd(&totals[s_zero_offset], static_cast<unsigned>(t_end - t0));
     }
   }
   if (kLists && tid == 0) sink.tile_mode[blockIdx.x] = num_chunks == 1 ? 0u : 1u;
@@ -832,25 +874,41 @@ __global__ __launch_bounds__(kQueryBlock) void emit_kernel(
 constexpr int kPlaceTiles = 4;
 constexpr int kPlaceBlock = 256;
 
+constexpr int kMaxTotalCopies = 16;          // copies of the per-offset totals a chain's query launch adds to
+
+template <bool kChain>
 __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
     const int *__restrict__ stage, const unsigned long long *__restrict__ masks,
-    const unsigned *__restrict__ tile_counts, const unsigned *__restrict__ row_totals,
+    const unsigned *__restrict__ tile_counts, const unsigned *row_totals,
     const unsigned *__restrict__ tile_mode, long long num_targets, int num_offsets, int num_tiles,
     long long num_wave_tiles, int reorder, int *__restrict__ in_idx, int *__restrict__ out_idx,
     unsigned *__restrict__ plan, unsigned *__restrict__ plan_host, unsigned long long *flag,
     unsigned long long sequence, int *__restrict__ sizes_out, int *__restrict__ order_out,
     const DevicePlan *__restrict__ chain_plan, const long long *__restrict__ folded_bounds,
-    long long *chain_host) {
+    long long *chain_host, const unsigned *__restrict__ repeats, int total_copies, int total_stride) {
   __shared__ unsigned s_partial[kPlaceBlock / kWave];
+  __shared__ unsigned s_partial_mirror[kPlaceBlock / kWave];
+  __shared__ unsigned s_totals[kPlanMaxOffsets];
   const int tid = threadIdx.x;
   const int lane = lane_id();
   const int w = tid >> 6;
-  const int o = blockIdx.y;
+  // Half of the offsets looked up (see DevicePlan): the workgroups of a
+  // looked-up offset write the rows of its mirror image as well, those of the
+  // zero offset write the identity, and mirror images have no workgroups.
+  int o = blockIdx.y, kind = 0, twin = -1;
+  if (kChain) {
+    const int packed = __builtin_amdgcn_readfirstlane(chain_plan->rows[blockIdx.y]);
+    o = packed & 0xff;
+    kind = (packed >> 8) & 0xff;
+    twin = ((packed >> 16) & 0xff) - 1;
+  }
   const int tile0 = blockIdx.x * kPlaceTiles;
-  if (chain_plan != nullptr) {
+  if (kChain) {
     // end of a chain of launches: the host learns the chain's verdict and the
     // coordinate bounds together with the sizes
-    const int verdict = chain_plan->verdict;
+    int verdict = chain_plan->verdict;
+    // equal rows were found: the halves do not mirror each other, the caller starts over
+    if (repeats != nullptr && repeats[0] != 0 && verdict == 0) verdict = 3;
     if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) {
 #pragma unroll
       for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) chain_host[slot] = folded_bounds[slot];
@@ -862,6 +920,20 @@ __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
     }
     if (verdict != 0) return;
   }
+  // the hits per offset: the query launch of a chain kept several copies (their
+  // loads are all in flight together), at most kPlanMaxOffsets offsets then
+  if (total_copies > 1) {
+    if (tid < num_offsets) {
+      unsigned part[kMaxTotalCopies], sum = 0;
+#pragma unroll
+      for (int c = 0; c < kMaxTotalCopies; ++c) part[c] = c < total_copies ? row_totals[c * total_stride + tid] : 0u;
+#pragma unroll
+      for (int c = 0; c < kMaxTotalCopies; ++c) sum += part[c];
+      s_totals[tid] = sum;
+    }
+    __syncthreads();
+    row_totals = s_totals;
+  }
   if (blockIdx.x == 0 && blockIdx.y == 0) {
     plan_from_sizes(row_totals, num_offsets, reorder, plan, plan_host, flag, sequence);
     for (int j = tid; j < num_offsets; j += kPlaceBlock) {
@@ -869,22 +941,55 @@ __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
       if (sizes_out) sizes_out[j] = static_cast<int>(plan[2 * num_offsets + j]);
     }
   }
-  // list position of the first hit of (o, tile0): rows before row o, tiles before tile0
+  if (kind == 1) return;                       // written by the workgroups of its mirror image
+  // list position of the first hit of (o, tile0): rows before row o (and before
+  // the mirror image's row), tiles before tile0
   const unsigned mine = row_totals[o];
-  unsigned before = 0;
+  unsigned before = 0, before_twin = 0;
   for (int p = tid; p < num_offsets; p += kPlaceBlock) {
     const unsigned other = row_totals[p];
     const bool first = reorder ? (other < mine || (other == mine && p < o)) : p < o;
     before += first ? other : 0u;
+    const bool first_twin = reorder ? (other < mine || (other == mine && p < twin)) : p < twin;
+    before_twin += twin >= 0 && first_twin ? other : 0u;
+  }
+  if (kind == 2) {
+    // the zero offset: hit number t of the row is target t with source t
+    for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off);
+    if (lane == 0) s_partial[w] = before;
+    __syncthreads();
+    unsigned row_start = 0;
+#pragma unroll
+    for (int ww = 0; ww < kPlaceBlock / kWave; ++ww) row_start += s_partial[ww];
+    const long long first = static_cast<long long>(tile0) * kTargetsPerTile;
+    for (long long t = first + tid; t < first + kPlaceTiles * kTargetsPerTile && t < num_targets; t += kPlaceBlock) {
+      in_idx[row_start + t] = static_cast<int>(t);
+      out_idx[row_start + t] = static_cast<int>(t);
+    }
+    return;
   }
   const unsigned *counts = tile_counts + static_cast<long long>(o) * num_tiles;
-  for (int i = tid; i < tile0; i += kPlaceBlock) before += counts[i];
-  for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off);
-  if (lane == 0) s_partial[w] = before;
+  unsigned tiles_before = 0;
+  for (int i = tid; i < tile0; i += kPlaceBlock) tiles_before += counts[i];
+  before += tiles_before;
+  before_twin += tiles_before;
+  for (int off = 32; off > 0; off >>= 1) {
+    before += __shfl_xor(before, off);
+    before_twin += __shfl_xor(before_twin, off);
+  }
+  if (lane == 0) {
+    s_partial[w] = before;
+    s_partial_mirror[w] = before_twin;
+  }
   __syncthreads();
-  unsigned base = 0;
+  unsigned base = 0, base_twin = 0;
 #pragma unroll
-  for (int ww = 0; ww < kPlaceBlock / kWave; ++ww) base += s_partial[ww];
+  for (int ww = 0; ww < kPlaceBlock / kWave; ++ww) {
+    base += s_partial[ww];
+    base_twin += s_partial_mirror[ww];
+  }
+  // entry number e of row o is entry number e of the mirror image's row with source and target exchanged
+  const unsigned to_twin = base_twin - base;
   // tiles of this workgroup: exclusive prefix of their counts
   const int my_tile = tile0 + lane;
   const unsigned count = lane < kPlaceTiles && my_tile < num_tiles ? counts[my_tile] : 0u;
@@ -931,8 +1036,13 @@ __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
 #pragma unroll
       for (int s = 0; s < kSegments; ++s) {
         if (hit[s]) {
+          const int target = static_cast<int>(t_tile + s * kWave + lane);
           in_idx[rank[s]] = found[s];
-          out_idx[rank[s]] = static_cast<int>(t_tile + s * kWave + lane);
+          out_idx[rank[s]] = target;
+          if (twin >= 0) {
+            in_idx[rank[s] + to_twin] = target;
+            out_idx[rank[s] + to_twin] = found[s];
+          }
         }
       }
     } else {
@@ -948,8 +1058,13 @@ __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
         const unsigned long long mask = __ballot(hit);
         if (hit) {
           const unsigned r = at + __popcll(mask & below);
+          const int target = static_cast<int>(t_tile + s * kWave + lane);
           in_idx[r] = found[s];
-          out_idx[r] = static_cast<int>(t_tile + s * kWave + lane);
+          out_idx[r] = target;
+          if (twin >= 0) {
+            in_idx[r + to_twin] = target;
+            out_idx[r + to_twin] = found[s];
+          }
         }
         at += __popcll(mask);
       }
@@ -1341,7 +1456,7 @@ static bool run_query(const QueryArgs &a, const int64_t *offsets_host, int64_t n
     profile_mark("query", stream);
     return true;
   }
-  const HitSink none{nullptr, nullptr, nullptr, nullptr, 0, 0};
+  const HitSink none{nullptr, nullptr, nullptr, nullptr, 0, 0, nullptr, 1, 0};
 #define MNT_Q(CT, BT, OT)                                                                        \
   launch_query<CT, BT, OT, false>(b, plan, d_tables, no, static_cast<OT *>(kernel_map), tile_counts, \
                                   num_tiles, none, stream)
@@ -1716,7 +1831,7 @@ extern "C" int mnt_kernel_map_lists(const void *sources, int64_t num_sources, co
     unsigned *row_totals = scope.alloc<unsigned>(num_offsets);
     unsigned *plan = scope.alloc<unsigned>(4 * num_offsets + 1);
     enqueue_fill<unsigned>(row_totals, num_offsets, 0u, stream);
-    const HitSink sink{stage, masks, row_totals, tile_mode, num_wave_tiles, no};
+    const HitSink sink{stage, masks, row_totals, tile_mode, num_wave_tiles, no, nullptr, 1, no};
     if (!run_query(a, offsets_host, num_offsets, source_bounds_host, target_bounds_host, bounds_host_out,
                    nullptr, MNT_INT32, tile_counts, scope, stream, &sink)) {
       // a frame too wide for packed keys: dense map by tuple comparisons (the
@@ -1740,11 +1855,11 @@ extern "C" int mnt_kernel_map_lists(const void *sources, int64_t num_sources, co
     unsigned *d_plan_host = reinterpret_cast<unsigned *>(static_cast<char *>(arena.pinned_device()) + Arena::kPlanOffset);
     const unsigned long long sequence = arena.next_sequence();
     dim3 grid(static_cast<unsigned>(div_ceil(num_tiles, kPlaceTiles)), static_cast<unsigned>(num_offsets));
-    place_kernel<<<grid, kPlaceBlock, 0, stream>>>(stage, masks, tile_counts, row_totals, tile_mode,
+    place_kernel<false><<<grid, kPlaceBlock, 0, stream>>>(stage, masks, tile_counts, row_totals, tile_mode,
                                                    num_targets, no, num_tiles, num_wave_tiles, reorder,
                                                    in_idx_out, out_idx_out, plan, d_plan_host,
                                                    arena.flag_device(1), sequence, sizes_dev_out,
-                                                   order_dev_out, nullptr, nullptr, nullptr);
+                                                   order_dev_out, nullptr, nullptr, nullptr, nullptr, 1, no);
     check_launch("place_kernel");
     collect_sizes(arena, sequence, num_offsets, sizes_host_out, order_host_out);
     profile_mark("map_place+sync", stream);
@@ -1754,6 +1869,24 @@ extern "C" int mnt_kernel_map_lists(const void *sources, int64_t num_sources, co
 // ---- sort -> query -> pair lists as one chain of six launches and one wait ----
 
 namespace mnt {
+
+static int total_copies() {
+  static const int value = [] {
+    const char *text = getenv("MINUET_TOTAL_COPIES");
+    const int v = text != nullptr && *text != 0 ? atoi(text) : 4;
+    return v < 1 ? 1 : v > kMaxTotalCopies ? kMaxTotalCopies : v;
+  }();
+  return value;
+}
+
+// MINUET_MAP_HALVES=0 looks every offset up (for comparisons).
+static bool map_halves_enabled() {
+  static const bool value = [] {
+    const char *text = getenv("MINUET_MAP_HALVES");
+    return text == nullptr || *text == 0 || atoi(text) != 0;
+  }();
+  return value;
+}
 
 constexpr size_t kChainHostOffset = 128;      // pinned block: bounds (8 words), then the chain's verdict
 
@@ -1816,7 +1949,8 @@ extern "C" int mnt_sorted_kernel_map_lists(const void *coords, int64_t n, int nd
       ChainSortBuffers buf;
       buf.partial = scope.alloc<long long>(128 * 8);
       buf.folded = scope.alloc<long long>(2 * MNT_MAX_NDIM);
-      buf.counter_words = 2 * buckets + no;
+      // bucket totals, cursors, the copies of the hits per offset, the equal-rows flag
+      buf.counter_words = 2 * buckets + kMaxTotalCopies * kPlanMaxOffsets + 1;
       buf.counters = scope.alloc<unsigned>(buf.counter_words);
       buf.info = scope.alloc<unsigned>(4);
       buf.status = scope.alloc<unsigned>(4);
@@ -1834,8 +1968,14 @@ extern "C" int mnt_sorted_kernel_map_lists(const void *coords, int64_t n, int nd
       for (int o = 0; o < no; ++o) {
         for (int k = 0; k < ndim; ++k) table.v[o][k] = static_cast<int>(offsets_host[o * ndim + k]);
       }
+      // the cloud is mapped onto itself: offsets that come in pairs d / -d need one look-up per pair
+      classify_offset_pairs(table, no, ndim, map_halves_enabled());
+      int num_rows = 0;                            // offsets with rows of their own to write (DevicePlan::rows)
+      for (int o = 0; o < no; ++o) num_rows += table.kind[o] != 1 ? 1 : 0;
       enqueue_chain_sort(coords, n, ndim, coord_dtype, indices_out, sorted_coords_out, buf, table, no, stream);
-      const HitSink sink{stage, masks, row_totals, tile_mode, num_wave_tiles, no};
+      unsigned *repeats = row_totals + kMaxTotalCopies * kPlanMaxOffsets;
+      const HitSink sink{stage, masks, row_totals, tile_mode, num_wave_tiles, no, repeats, total_copies(),
+                         kPlanMaxOffsets};
       if (coord_dtype == MNT_INT32) {
         launch_query_chain<int32_t>(static_cast<const int32_t *>(sorted_coords_out), n, ndim, no, tile_counts,
                                     num_tiles, sink, buf.plan, stream);
@@ -1848,12 +1988,13 @@ extern "C" int mnt_sorted_kernel_map_lists(const void *coords, int64_t n, int nd
       unsigned *d_plan_host = reinterpret_cast<unsigned *>(pinned_device + Arena::kPlanOffset);
       long long *d_chain_host = reinterpret_cast<long long *>(pinned_device + kChainHostOffset);
       const unsigned long long sequence = arena.next_sequence();
-      dim3 grid(static_cast<unsigned>(div_ceil(num_tiles, kPlaceTiles)), static_cast<unsigned>(num_offsets));
-      place_kernel<<<grid, kPlaceBlock, 0, stream>>>(stage, masks, tile_counts, row_totals, tile_mode, n, no,
+      // a workgroup per four tiles and per offset that is looked up (or is the zero offset)
+      dim3 grid(static_cast<unsigned>(div_ceil(num_tiles, kPlaceTiles)), static_cast<unsigned>(num_rows));
+      place_kernel<true><<<grid, kPlaceBlock, 0, stream>>>(stage, masks, tile_counts, row_totals, tile_mode, n, no,
                                                      num_tiles, num_wave_tiles, reorder, in_idx_out,
                                                      out_idx_out, plan, d_plan_host, arena.flag_device(1),
                                                      sequence, sizes_dev_out, order_dev_out, buf.plan,
-                                                     buf.folded, d_chain_host);
+                                                     buf.folded, d_chain_host, repeats, total_copies(), kPlanMaxOffsets);
       check_launch("place_kernel");
       arena.wait_flag(1, sequence);
       const long long *h_chain = reinterpret_cast<const long long *>(static_cast<char *>(arena.pinned()) + kChainHostOffset);

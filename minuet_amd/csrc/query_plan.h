@@ -14,10 +14,56 @@ constexpr int kPlanGroupSpan = 4;                // key span of one offset group
 constexpr int kPlanMaxOffsets = 64;              // one lane per offset
 constexpr int kPlanInts = 6 * kPlanMaxOffsets;   // 4 words per group + 2 per member
 
-// Kernel offsets as launch arguments (rows past the count are ignored).
+// Kernel offsets as launch arguments (rows past the count are ignored), and
+// what the host worked out about them for a cloud that is mapped onto itself:
+// halves != 0 when the offsets come in pairs d / -d (no offset named twice, at
+// least one pair); kind[o] is then 0 for the offset of a pair that is looked
+// up (the one whose first non-zero coordinate is positive, i.e. whose key delta
+// is), 1 for its mirror image, 2 for the zero offset, and mirror[o] the index
+// of the offset's mirror image.
 struct OffsetTable {
   int v[kPlanMaxOffsets][MNT_MAX_NDIM];
+  int halves;
+  signed char kind[kPlanMaxOffsets];
+  signed char mirror[kPlanMaxOffsets];
 };
+
+// Fills halves / kind / mirror of `table` from its first num_offsets rows.
+inline void classify_offset_pairs(OffsetTable &table, int num_offsets, int ndim, bool allow) {
+  table.halves = 0;
+  for (int o = 0; o < kPlanMaxOffsets; ++o) {
+    table.kind[o] = 0;
+    table.mirror[o] = -1;
+  }
+  if (!allow || num_offsets > kPlanMaxOffsets) return;
+  bool paired = true, any_positive = false;
+  for (int o = 0; o < num_offsets && paired; ++o) {
+    int sign = 0;
+    for (int k = 0; k < ndim && sign == 0; ++k) sign = table.v[o][k] > 0 ? 1 : table.v[o][k] < 0 ? -1 : 0;
+    int mirror = -1;
+    for (int p = 0; p < num_offsets; ++p) {
+      bool negated = true, same = true;
+      for (int k = 0; k < ndim; ++k) {
+        negated = negated && table.v[p][k] == -table.v[o][k];
+        same = same && table.v[p][k] == table.v[o][k];
+      }
+      if (negated && mirror < 0) mirror = p;
+      if (same && p != o) paired = false;                     // an offset named twice
+    }
+    paired = paired && mirror >= 0;
+    table.kind[o] = static_cast<signed char>(sign > 0 ? 0 : sign == 0 ? 2 : 1);
+    table.mirror[o] = static_cast<signed char>(mirror);
+    any_positive = any_positive || sign > 0;
+  }
+  if (paired && any_positive) {
+    table.halves = 1;
+    return;
+  }
+  for (int o = 0; o < kPlanMaxOffsets; ++o) {
+    table.kind[o] = 0;
+    table.mirror[o] = -1;
+  }
+}
 
 struct DevicePlan {
   Frame frame;
@@ -27,6 +73,18 @@ struct DevicePlan {
   int verdict;              // 0: go; otherwise the chain stops (sort declined, or keys beyond 63 bits)
   int num_offsets;
   int tables[kPlanInts];    // groups (first delta low / high, first member, members), then members (step, offset)
+  // A cloud mapped onto itself under offsets that come in pairs d / -d: the
+  // hits of -d are those of d with source and target exchanged, in the same
+  // order (source positions rise with target positions), so only the offsets
+  // of positive key delta are looked up.  halves != 0: kind[o] says what
+  // offset o is (0 looked up, 1 the mirror image of offset mirror[o], 2 the
+  // zero offset: every voxel is its own hit).
+  int halves;
+  int kind[kPlanMaxOffsets];
+  int mirror[kPlanMaxOffsets];
+  // the offsets that have rows of their own to write (all but the mirror
+  // images), in offset order: offset | kind << 8 | (mirror + 1) << 16
+  int rows[kPlanMaxOffsets];
 };
 
 struct PlanScratch {        // LDS of the wavefront that builds the plan
@@ -99,26 +157,39 @@ __device__ __forceinline__ void make_plan_on_device(const long long *__restrict_
       delta += static_cast<long long>(static_cast<unsigned long long>(static_cast<long long>(d[k])) << f.shift[k]);
     }
   }
-  // place among the offsets in ascending delta order (ties keep offset order)
+  // what the host found out about the offsets: lane o takes entry o
+  const bool halves = offsets.halves != 0;
+  int kind = 0, mirror = -1;
+#pragma unroll
+  for (int l = 0; l < kPlanMaxOffsets; ++l) {
+    kind = lane == l ? offsets.kind[l] : kind;
+    mirror = lane == l ? offsets.mirror[l] : mirror;
+  }
+  // the offsets that are looked up: all of them, or those of positive key delta
+  const bool kept = live && (!halves || kind == 0);
+  const int num_kept = __popcll(__ballot(kept));
+  // place among the kept offsets in ascending delta order (ties keep offset order)
   int place = 0;
   for (int p = 0; p < num_offsets; ++p) {
     const long long other = __shfl(delta, p);
-    place += (other < delta || (other == delta && p < lane)) ? 1 : 0;
+    const bool other_kept = __shfl(kept ? 1 : 0, p) != 0;
+    place += other_kept && (other < delta || (other == delta && p < lane)) ? 1 : 0;
   }
   // lane i takes over the offset of place i; from here on lanes are places
-  if (live) lds.inverse[place] = lane;
+  if (kept) lds.inverse[place] = lane;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-  const int origin = live ? lds.inverse[lane] : lane;
+  const bool placed = lane < num_kept;
+  const int origin = placed ? lds.inverse[lane] : lane;
   const long long mine = __shfl(delta, origin);
   int lead[MNT_MAX_NDIM];
 #pragma unroll
   for (int k = 0; k < MNT_MAX_NDIM; ++k) lead[k] = __shfl(d[k], origin);
-  // first place whose delta lies beyond this one's group span (num_offsets if
+  // first place whose delta lies beyond this one's group span (num_kept if
   // none), and never more than kPlanGroupSpan + 1 members (repeated offsets)
-  int next = num_offsets;
-  for (int p = num_offsets - 1; p >= 0; --p) {
+  int next = num_kept;
+  for (int p = num_kept - 1; p >= 0; --p) {
     const long long other = __shfl(mine, p);
     next = p > lane && other - mine > kPlanGroupSpan ? p : next;
   }
@@ -126,13 +197,13 @@ __device__ __forceinline__ void make_plan_on_device(const long long *__restrict_
   // the greedy grouping follows those links from place 0
   unsigned long long starts = 0;
   int num_groups = 0;
-  for (int cur = 0; cur < num_offsets; cur = __shfl(next, cur)) {
+  for (int cur = 0; cur < num_kept; cur = __shfl(next, cur)) {
     starts |= 1ull << cur;
     ++num_groups;
   }
   const unsigned long long upto = starts & ((2ull << lane) - 1ull);
   const int group = __popcll(upto) - 1;
-  const int first_place = live ? 63 - __builtin_clzll(upto) : 0;
+  const int first_place = placed ? 63 - __builtin_clzll(upto) : 0;
   const long long first_delta = __shfl(mine, first_place);
   bool same_row = true;
 #pragma unroll
@@ -140,8 +211,8 @@ __device__ __forceinline__ void make_plan_on_device(const long long *__restrict_
     const int other = __shfl(lead[k], first_place);
     same_row = same_row && (k + 1 >= ndim || other == lead[k]);
   }
-  const bool in_rows = __ballot(live && !same_row) == 0ull;
-  if (live) {
+  const bool in_rows = __ballot(placed && !same_row) == 0ull;
+  if (placed) {
     out->tables[4 * num_groups + 2 * lane + 0] = static_cast<int>(mine - first_delta);
     out->tables[4 * num_groups + 2 * lane + 1] = origin;
     if ((starts >> lane) & 1ull) {
@@ -152,15 +223,29 @@ __device__ __forceinline__ void make_plan_on_device(const long long *__restrict_
       out->tables[4 * group + 3] = next - lane;
     }
   }
+  if (live) {
+    out->kind[lane] = halves ? kind : 0;
+    out->mirror[lane] = halves ? mirror : -1;
+    const bool writes = !halves || kind != 1;
+    const unsigned long long writers = __ballot(writes);
+    if (writes) {
+      const int y = __popcll(writers & ((1ull << lane) - 1ull));
+      out->rows[y] = lane | ((halves ? kind : 0) << 8) | ((halves ? mirror + 1 : 0) << 16);
+    }
+  }
+  // an offset that is looked up must have a positive key delta, which is what
+  // the host's reading of its coordinates says; anything else stops the chain
+  const bool consistent = !halves || __ballot(kept && delta <= 0) == 0ull;
   const long long delta_min = __shfl(mine, 0);
-  const long long delta_max = __shfl(mine, num_offsets > 0 ? num_offsets - 1 : 0);
+  const long long delta_max = __shfl(mine, num_kept > 0 ? num_kept - 1 : 0);
   if (lane == 0) {
     out->frame = f;
-    out->delta_min = num_offsets > 0 ? delta_min : 0;
-    out->delta_max = num_offsets > 0 ? delta_max : 0;
+    out->delta_min = num_kept > 0 ? delta_min : 0;
+    out->delta_max = num_kept > 0 ? delta_max : 0;
+    out->halves = halves ? 1 : 0;
     out->num_groups = num_groups;
     out->groups_in_rows = in_rows ? 1 : 0;
-    out->verdict = declined != 0 ? static_cast<int>(declined) : (fits ? 0 : 2);
+    out->verdict = declined != 0 ? static_cast<int>(declined) : (fits && consistent ? 0 : 2);
     out->num_offsets = num_offsets;
   }
 }
