@@ -24,6 +24,14 @@ __device__ __forceinline__ long long uniform64(long long v) {
   return static_cast<long long>((static_cast<unsigned long long>(hi) << 32) | lo);
 }
 
+// A load that goes through to the memory every compute die sees (device-scope
+// atomic load): what device-scope atomics of other workgroups, possibly on
+// another die, have left there, not what this die's caches hold.
+template <typename T>
+__device__ __forceinline__ T load_through(const T *p) {
+  return __hip_atomic_load(const_cast<T *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // Batch of row i: the g with dims[g] <= i < dims[g+1] (dims has num_batches+1
 // entries).  Rows at or past dims[num_batches] land in the last batch.
 template <typename IT>

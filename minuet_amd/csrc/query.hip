@@ -102,6 +102,23 @@ struct HitSink {
   int total_copies, total_stride;
 };
 
+// What the last tile of a chain's query launch needs to tell the host the
+// result's sizes (all null / zero outside a chain).  The tiles count themselves
+// off on `done` as they finish; the one that finds all others counted ranks the
+// offsets by their totals and raises the host's flag, so that the host goes on
+// while the placing launch still runs.
+struct ChainFinish {
+  unsigned *done;                  // zero before the launch
+  unsigned *plan;                  // order | position_of | sorted sizes | prefix (plan_from_sizes)
+  unsigned *plan_host;             // pinned host mirror of the first three blocks
+  unsigned long long *flag;
+  unsigned long long sequence;
+  long long *chain_host;           // pinned: coordinate bounds (8 words), then the chain's verdict
+  const long long *folded_bounds;
+  int *sizes_out, *order_out;      // device copies of sizes / order in row order (nullable)
+  int reorder;
+};
+
 // Settles the queries of one group against the candidates cand[0 .. span]
 // read from window position p on: writes the map entries this workgroup's
 // chunk is responsible for and counts the hits per offset.  The group and
@@ -387,6 +404,12 @@ __device__ __forceinline__ void resolve_chunk_rows(
 // tables == nullptr), which saves the launch that would upload them; the last
 // wavefront copies them into LDS with uniform (scalar) reads while the first
 // two look for the window.
+__device__ __forceinline__ void plan_from_sizes(const unsigned *row_sizes, int num_offsets, int reorder,
+                                                unsigned *__restrict__ plan,
+                                                unsigned *__restrict__ plan_host,
+                                                unsigned long long *flag,
+                                                unsigned long long sequence);
+constexpr int kMaxTotalCopies = 16;          // copies of the per-offset totals a chain's query launch adds to
 constexpr int kCarriedInts = 160;
 struct CarriedTables {
   int v[kCarriedInts];
@@ -397,7 +420,7 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     KeyReader<CT, BT> src, KeyReader<CT, BT> tgt, Frame frame, const int *__restrict__ tables,
     CarriedTables carried, int num_groups, int num_offsets, long long delta_min, long long delta_max,
     OT *__restrict__ kernel_map, unsigned *__restrict__ tile_counts, int num_tiles, int dir_rows,
-    HitSink sink, const DevicePlan *__restrict__ device_plan) {
+    HitSink sink, const DevicePlan *__restrict__ device_plan, ChainFinish finish) {
   extern __shared__ __align__(16) unsigned s_dynamic[];
   // Only half of the offsets are looked up (a cloud mapped onto itself under
   // offsets that come in pairs d / -d; see DevicePlan): the totals of the other
@@ -608,6 +631,46 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     }
   }
   if (kLists && tid == 0) sink.tile_mode[blockIdx.x] = num_chunks == 1 ? 0u : 1u;
+  if (kLists && finish.done != nullptr) {
+    // the totals this tile added (device-scope atomics) have been performed once
+    // their acknowledgements are in; only then is the tile counted off
+    __shared__ int s_last;
+    __shared__ unsigned s_totals[kPlanMaxOffsets];
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) s_last = atomicAdd(finish.done, 1u) == gridDim.x - 1 ? 1 : 0;
+    __syncthreads();
+    if (s_last != 0) {
+      // every tile's totals are in: loads that go through to where the atomics were performed
+      if (tid < num_offsets && tid < kPlanMaxOffsets) {
+        unsigned part[kMaxTotalCopies], sum = 0;
+#pragma unroll
+        for (int c = 0; c < kMaxTotalCopies; ++c) {
+          part[c] = c < sink.total_copies ? load_through(sink.row_totals + c * sink.total_stride + tid) : 0u;
+        }
+#pragma unroll
+        for (int c = 0; c < kMaxTotalCopies; ++c) sum += part[c];
+        s_totals[tid] = sum;
+      }
+      const unsigned repeated = sink.repeats != nullptr ? load_through(sink.repeats) : 0u;
+      if (tid == 0) {
+#pragma unroll
+        for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) finish.chain_host[slot] = finish.folded_bounds[slot];
+        finish.chain_host[2 * MNT_MAX_NDIM] = repeated != 0 ? 3 : 0;
+      }
+      __syncthreads();
+      if (repeated == 0) {
+        // thread 0 wrote the bounds and the verdict; it also raises the flag, behind a system-scope fence
+        plan_from_sizes(s_totals, num_offsets, finish.reorder, finish.plan, finish.plan_host, finish.flag,
+                        finish.sequence);
+        for (int j = tid; j < num_offsets; j += kQueryThreads) {
+          if (finish.order_out) finish.order_out[j] = static_cast<int>(finish.plan[j]);
+          if (finish.sizes_out) finish.sizes_out[j] = static_cast<int>(finish.plan[2 * num_offsets + j]);
+        }
+      }
+      // (equal rows: the placing launch reports the verdict and raises the flag)
+    }
+  }
 }
 
 // The query for frames too wide for a packed key (more than 63 bits of
@@ -874,8 +937,6 @@ __global__ __launch_bounds__(kQueryBlock) void emit_kernel(
 constexpr int kPlaceTiles = 4;
 constexpr int kPlaceBlock = 256;
 
-constexpr int kMaxTotalCopies = 16;          // copies of the per-offset totals a chain's query launch adds to
-
 template <bool kChain>
 __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
     const int *__restrict__ stage, const unsigned long long *__restrict__ masks,
@@ -885,56 +946,102 @@ __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
     unsigned *__restrict__ plan, unsigned *__restrict__ plan_host, unsigned long long *flag,
     unsigned long long sequence, int *__restrict__ sizes_out, int *__restrict__ order_out,
     const DevicePlan *__restrict__ chain_plan, const long long *__restrict__ folded_bounds,
-    long long *chain_host, const unsigned *__restrict__ repeats, int total_copies, int total_stride) {
+    long long *chain_host, const unsigned *__restrict__ repeats, int total_copies, int total_stride,
+    int told_by_query) {
   __shared__ unsigned s_partial[kPlaceBlock / kWave];
   __shared__ unsigned s_partial_mirror[kPlaceBlock / kWave];
   __shared__ unsigned s_totals[kPlanMaxOffsets];
+  static_assert(kPlaceTiles == kPlaceBlock / kWave, "one tile per wavefront");
   const int tid = threadIdx.x;
   const int lane = lane_id();
   const int w = tid >> 6;
+  const int tile0 = blockIdx.x * kPlaceTiles;
+  const int tile = tile0 + w;
+  constexpr int kSegments = kTargetsPerTile / kWave;
+
+  // ---- Everything the workgroup reads from memory is asked for here, and
+  // waited for ONCE: a trip to memory takes about two microseconds, and seven of
+  // them one after the other (verdict, totals, tile counts, ballots, staged hits
+  // ...) were most of this kernel's time.  What does not depend on the row this
+  // workgroup writes comes first; the row's offset itself is read from the
+  // chain's plan.  The staged hits are read as whole segments, lane l slot l,
+  // instead of the slot a hit's rank names once the ballots are in.  After a
+  // chain that declined the scratch arrays hold whatever was there: reading
+  // that is harmless (every index is in range), nothing is written then.
+  int verdict = 0, packed = blockIdx.y;
+  unsigned repeated = 0;
+  if (kChain) {
+    verdict = chain_plan->verdict;
+    packed = chain_plan->rows[blockIdx.y];
+    repeated = repeats != nullptr ? repeats[0] : 0u;
+  }
+  unsigned total_mine = 0;                       // hits of offset tid (tid < num_offsets <= 64 when there are copies)
+  if (total_copies > 1) {
+    unsigned part[kMaxTotalCopies];
+#pragma unroll
+    for (int c = 0; c < kMaxTotalCopies; ++c) {
+      part[c] = c < total_copies && tid < num_offsets ? row_totals[c * total_stride + tid] : 0u;
+    }
+#pragma unroll
+    for (int c = 0; c < kMaxTotalCopies; ++c) total_mine += part[c];
+  }
+  const unsigned mode = tile < num_tiles ? tile_mode[tile] : 0u;
   // Half of the offsets looked up (see DevicePlan): the workgroups of a
   // looked-up offset write the rows of its mirror image as well, those of the
   // zero offset write the identity, and mirror images have no workgroups.
-  int o = blockIdx.y, kind = 0, twin = -1;
-  if (kChain) {
-    const int packed = __builtin_amdgcn_readfirstlane(chain_plan->rows[blockIdx.y]);
-    o = packed & 0xff;
-    kind = (packed >> 8) & 0xff;
-    twin = ((packed >> 16) & 0xff) - 1;
+  packed = __builtin_amdgcn_readfirstlane(packed);
+  const int o = kChain ? packed & 0xff : packed;
+  const int kind = kChain ? (packed >> 8) & 0xff : 0;
+  const int twin = kChain ? ((packed >> 16) & 0xff) - 1 : -1;
+  const bool live = tile < num_tiles && kind == 0;                    // uniform per wavefront
+  const long long t_tile = static_cast<long long>(tile) * kTargetsPerTile;
+  const long long row = static_cast<long long>(o) * num_targets;
+  int entry[kSegments];
+#pragma unroll
+  for (int s = 0; s < kSegments; ++s) {
+    const long long t = t_tile + s * kWave + lane;
+    entry[s] = live && t < num_targets ? stage[row + t] : -1;
   }
-  const int tile0 = blockIdx.x * kPlaceTiles;
-  if (kChain) {
+  const long long wave_tile = (t_tile >> 6) + lane;
+  const unsigned long long my_mask =
+      live && lane < kSegments && wave_tile < num_wave_tiles
+          ? masks[static_cast<long long>(o) * num_wave_tiles + wave_tile] : 0ull;
+  const unsigned *counts = tile_counts + static_cast<long long>(o) * num_tiles;
+  const int my_tile = tile0 + lane;
+  const unsigned count = kind == 0 && lane < kPlaceTiles && my_tile < num_tiles ? counts[my_tile] : 0u;
+  unsigned tiles_before = 0;
+  if (kind == 0) {
+    for (int i = tid; i < tile0; i += kPlaceBlock) tiles_before += counts[i];
+  }
+  // the one wait: everything above has been asked for by now
+  {
+    unsigned lo = static_cast<unsigned>(my_mask), hi = static_cast<unsigned>(my_mask >> 32);
+    asm volatile("" : "+v"(entry[0]), "+v"(entry[1]), "+v"(entry[2]), "+v"(entry[3]), "+v"(entry[4]),
+                 "+v"(entry[5]), "+v"(entry[6]), "+v"(entry[7]), "+v"(lo), "+v"(hi));
+  }
+  if (repeated != 0 && verdict == 0) verdict = 3;       // equal rows: the halves do not mirror each other
+  // told_by_query: the query launch's last tile has told the host the sizes of a
+  // chain that went through; this launch only speaks up when it did not
+  const bool silent = told_by_query != 0 && verdict == 0;
+  if (kChain && !silent && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) {
     // end of a chain of launches: the host learns the chain's verdict and the
     // coordinate bounds together with the sizes
-    int verdict = chain_plan->verdict;
-    // equal rows were found: the halves do not mirror each other, the caller starts over
-    if (repeats != nullptr && repeats[0] != 0 && verdict == 0) verdict = 3;
-    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) {
 #pragma unroll
-      for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) chain_host[slot] = folded_bounds[slot];
-      chain_host[2 * MNT_MAX_NDIM] = static_cast<long long>(verdict);
-      if (verdict != 0) {
-        __threadfence_system();
-        __hip_atomic_store(flag, sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-      }
+    for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) chain_host[slot] = folded_bounds[slot];
+    chain_host[2 * MNT_MAX_NDIM] = static_cast<long long>(verdict);
+    if (verdict != 0) {
+      __threadfence_system();
+      __hip_atomic_store(flag, sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
-    if (verdict != 0) return;
   }
-  // the hits per offset: the query launch of a chain kept several copies (their
-  // loads are all in flight together), at most kPlanMaxOffsets offsets then
+  if (verdict != 0) return;
   if (total_copies > 1) {
-    if (tid < num_offsets) {
-      unsigned part[kMaxTotalCopies], sum = 0;
-#pragma unroll
-      for (int c = 0; c < kMaxTotalCopies; ++c) part[c] = c < total_copies ? row_totals[c * total_stride + tid] : 0u;
-#pragma unroll
-      for (int c = 0; c < kMaxTotalCopies; ++c) sum += part[c];
-      s_totals[tid] = sum;
-    }
+    if (tid < num_offsets) s_totals[tid] = total_mine;
     __syncthreads();
     row_totals = s_totals;
   }
-  if (blockIdx.x == 0 && blockIdx.y == 0) {
+  if (blockIdx.x == 0 && blockIdx.y == 0 && !silent) {
+    // sizes, order and the flag for the host; device copies of sizes and order
     plan_from_sizes(row_totals, num_offsets, reorder, plan, plan_host, flag, sequence);
     for (int j = tid; j < num_offsets; j += kPlaceBlock) {
       if (order_out) order_out[j] = static_cast<int>(plan[j]);
@@ -942,8 +1049,7 @@ __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
     }
   }
   if (kind == 1) return;                       // written by the workgroups of its mirror image
-  // list position of the first hit of (o, tile0): rows before row o (and before
-  // the mirror image's row), tiles before tile0
+  // rows before row o and before the mirror image's row
   const unsigned mine = row_totals[o];
   unsigned before = 0, before_twin = 0;
   for (int p = tid; p < num_offsets; p += kPlaceBlock) {
@@ -968,9 +1074,7 @@ __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
     }
     return;
   }
-  const unsigned *counts = tile_counts + static_cast<long long>(o) * num_tiles;
-  unsigned tiles_before = 0;
-  for (int i = tid; i < tile0; i += kPlaceBlock) tiles_before += counts[i];
+  // list position of the first hit of (o, tile0): rows before, tiles before tile0
   before += tiles_before;
   before_twin += tiles_before;
   for (int off = 32; off > 0; off >>= 1) {
@@ -991,83 +1095,58 @@ __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
   // entry number e of row o is entry number e of the mirror image's row with source and target exchanged
   const unsigned to_twin = base_twin - base;
   // tiles of this workgroup: exclusive prefix of their counts
-  const int my_tile = tile0 + lane;
-  const unsigned count = lane < kPlaceTiles && my_tile < num_tiles ? counts[my_tile] : 0u;
   unsigned inclusive = count;
   for (int off = 1; off < kPlaceTiles; off <<= 1) {
     const unsigned u = __shfl_up(inclusive, off);
     if (lane >= off) inclusive += u;
   }
   const unsigned exclusive = inclusive - count;
-  const long long row = static_cast<long long>(o) * num_targets;
   const unsigned long long below = lanes_below();
-  for (int j = w; j < kPlaceTiles; j += kPlaceBlock / kWave) {
-    const int tile = tile0 + j;
-    if (tile >= num_tiles) break;                                   // uniform per wavefront
-    const unsigned tile_hits = __shfl(count, j);
-    if (tile_hits == 0) continue;
-    unsigned at = base + __shfl(exclusive, j);
-    const long long t_tile = static_cast<long long>(tile) * kTargetsPerTile;
-    constexpr int kSegments = kTargetsPerTile / kWave;
-    if (tile_mode[tile] == 0) {
-      // lane s holds the ballot of segment s and the hits before it
-      const long long wave_tile = (t_tile >> 6) + lane;
-      const unsigned long long my_mask =
-          lane < kSegments && wave_tile < num_wave_tiles
-              ? masks[static_cast<long long>(o) * num_wave_tiles + wave_tile] : 0ull;
-      const unsigned my_hits = __popcll(my_mask);
-      unsigned seg_inclusive = my_hits;
-      for (int off = 1; off < kSegments; off <<= 1) {
-        const unsigned u = __shfl_up(seg_inclusive, off);
-        if (lane >= off) seg_inclusive += u;
-      }
-      const unsigned seg_exclusive = seg_inclusive - my_hits;
-      int found[kSegments];
-      unsigned rank[kSegments];
-      bool hit[kSegments];
+  if (tile >= num_tiles || __shfl(count, w) == 0) return;              // uniform per wavefront
+  unsigned at = base + __shfl(exclusive, w);
+  if (mode == 0) {
+    // lane s holds the ballot of segment s and the hits before it
+    const unsigned my_hits = __popcll(my_mask);
+    unsigned seg_inclusive = my_hits;
+    for (int off = 1; off < kSegments; off <<= 1) {
+      const unsigned u = __shfl_up(seg_inclusive, off);
+      if (lane >= off) seg_inclusive += u;
+    }
+    const unsigned seg_exclusive = seg_inclusive - my_hits;
 #pragma unroll
-      for (int s = 0; s < kSegments; ++s) {
-        const unsigned long long mask = __shfl(my_mask, s);
-        hit[s] = (mask >> lane) & 1ull;
-        const unsigned r = __popcll(mask & below);
-        rank[s] = at + __shfl(seg_exclusive, s) + r;
-        found[s] = hit[s] ? stage[row + t_tile + s * kWave + r] : -1;
-      }
-#pragma unroll
-      for (int s = 0; s < kSegments; ++s) {
-        if (hit[s]) {
-          const int target = static_cast<int>(t_tile + s * kWave + lane);
-          in_idx[rank[s]] = found[s];
-          out_idx[rank[s]] = target;
-          if (twin >= 0) {
-            in_idx[rank[s] + to_twin] = target;
-            out_idx[rank[s] + to_twin] = found[s];
-          }
+    for (int s = 0; s < kSegments; ++s) {
+      const unsigned long long mask = __shfl(my_mask, s);
+      const bool hit = (mask >> lane) & 1ull;
+      const unsigned r = __popcll(mask & below);
+      // the hit of this lane's target is the r-th staged entry of the segment, which lane r read
+      const int found = __shfl(entry[s], static_cast<int>(r));
+      const unsigned rank = at + __shfl(seg_exclusive, s) + r;
+      if (hit) {
+        const int target = static_cast<int>(t_tile + s * kWave + lane);
+        in_idx[rank] = found;
+        out_idx[rank] = target;
+        if (twin >= 0) {
+          in_idx[rank + to_twin] = target;
+          out_idx[rank + to_twin] = found;
         }
       }
-    } else {
-      int found[kSegments];
+    }
+  } else {
 #pragma unroll
-      for (int s = 0; s < kSegments; ++s) {
-        const long long t = t_tile + s * kWave + lane;
-        found[s] = t < num_targets ? stage[row + t] : -1;
-      }
-#pragma unroll
-      for (int s = 0; s < kSegments; ++s) {
-        const bool hit = found[s] != -1;
-        const unsigned long long mask = __ballot(hit);
-        if (hit) {
-          const unsigned r = at + __popcll(mask & below);
-          const int target = static_cast<int>(t_tile + s * kWave + lane);
-          in_idx[r] = found[s];
-          out_idx[r] = target;
-          if (twin >= 0) {
-            in_idx[r + to_twin] = target;
-            out_idx[r + to_twin] = found[s];
-          }
+    for (int s = 0; s < kSegments; ++s) {
+      const bool hit = entry[s] != -1;
+      const unsigned long long mask = __ballot(hit);
+      if (hit) {
+        const unsigned r = at + __popcll(mask & below);
+        const int target = static_cast<int>(t_tile + s * kWave + lane);
+        in_idx[r] = entry[s];
+        out_idx[r] = target;
+        if (twin >= 0) {
+          in_idx[r + to_twin] = target;
+          out_idx[r + to_twin] = entry[s];
         }
-        at += __popcll(mask);
       }
+      at += __popcll(mask);
     }
   }
 }
@@ -1335,7 +1414,7 @@ static void launch_query(const QueryArgs &a, const QueryPlan &plan, const int *d
   const dim3 grid(static_cast<unsigned>(num_tiles), static_cast<unsigned>(split));
   query_kernel<CT, BT, OT, kLists><<<grid, kQueryThreads, dyn, stream>>>(
       src, tgt, plan.frame, d_tables, carried, plan.num_groups, num_offsets, plan.delta_min,
-      plan.delta_max, kernel_map, tile_counts, num_tiles, dir_rows, sink, nullptr);
+      plan.delta_max, kernel_map, tile_counts, num_tiles, dir_rows, sink, nullptr, ChainFinish{});
   check_launch("query_kernel");
 }
 
@@ -1859,7 +1938,7 @@ extern "C" int mnt_kernel_map_lists(const void *sources, int64_t num_sources, co
                                                    num_targets, no, num_tiles, num_wave_tiles, reorder,
                                                    in_idx_out, out_idx_out, plan, d_plan_host,
                                                    arena.flag_device(1), sequence, sizes_dev_out,
-                                                   order_dev_out, nullptr, nullptr, nullptr, nullptr, 1, no);
+                                                   order_dev_out, nullptr, nullptr, nullptr, nullptr, 1, no, 0);
     check_launch("place_kernel");
     collect_sizes(arena, sequence, num_offsets, sizes_host_out, order_host_out);
     profile_mark("map_place+sync", stream);
@@ -1893,7 +1972,7 @@ constexpr size_t kChainHostOffset = 128;      // pinned block: bounds (8 words),
 template <typename CT>
 static void launch_query_chain(const CT *sorted, int64_t n, int ndim, int num_offsets,
                                unsigned *tile_counts, int num_tiles, const HitSink &sink,
-                               const DevicePlan *plan, hipStream_t stream) {
+                               const DevicePlan *plan, const ChainFinish &finish, hipStream_t stream) {
   KeyReader<CT, int32_t> rows{sorted, nullptr, 1, n};
   Frame frame;
   memset(&frame, 0, sizeof(frame));
@@ -1905,7 +1984,7 @@ static void launch_query_chain(const CT *sorted, int64_t n, int ndim, int num_of
                      sizeof(unsigned short) * static_cast<size_t>(kDirectoryRows);
   query_kernel<CT, int32_t, int32_t, true><<<num_tiles, kQueryThreads, dyn, stream>>>(
       rows, rows, frame, nullptr, carried, 0, num_offsets, 0, 0, nullptr, tile_counts, num_tiles,
-      kDirectoryRows, sink, plan);
+      kDirectoryRows, sink, plan, finish);
   check_launch("query_kernel");
 }
 
@@ -1950,7 +2029,8 @@ extern "C" int mnt_sorted_kernel_map_lists(const void *coords, int64_t n, int nd
       buf.partial = scope.alloc<long long>(128 * 8);
       buf.folded = scope.alloc<long long>(2 * MNT_MAX_NDIM);
       // bucket totals, cursors, the copies of the hits per offset, the equal-rows flag
-      buf.counter_words = 2 * buckets + kMaxTotalCopies * kPlanMaxOffsets + 1;
+      // ..., the count of finished query tiles
+      buf.counter_words = 2 * buckets + kMaxTotalCopies * kPlanMaxOffsets + 2;
       buf.counters = scope.alloc<unsigned>(buf.counter_words);
       buf.info = scope.alloc<unsigned>(4);
       buf.status = scope.alloc<unsigned>(4);
@@ -1976,25 +2056,28 @@ extern "C" int mnt_sorted_kernel_map_lists(const void *coords, int64_t n, int nd
       unsigned *repeats = row_totals + kMaxTotalCopies * kPlanMaxOffsets;
       const HitSink sink{stage, masks, row_totals, tile_mode, num_wave_tiles, no, repeats, total_copies(),
                          kPlanMaxOffsets};
-      if (coord_dtype == MNT_INT32) {
-        launch_query_chain<int32_t>(static_cast<const int32_t *>(sorted_coords_out), n, ndim, no, tile_counts,
-                                    num_tiles, sink, buf.plan, stream);
-      } else {
-        launch_query_chain<int64_t>(static_cast<const int64_t *>(sorted_coords_out), n, ndim, no, tile_counts,
-                                    num_tiles, sink, buf.plan, stream);
-      }
-      profile_mark("query", stream);
       char *pinned_device = static_cast<char *>(arena.pinned_device());
       unsigned *d_plan_host = reinterpret_cast<unsigned *>(pinned_device + Arena::kPlanOffset);
       long long *d_chain_host = reinterpret_cast<long long *>(pinned_device + kChainHostOffset);
       const unsigned long long sequence = arena.next_sequence();
+      // the query launch's last tile tells the host the sizes: the host goes on while the lists are being placed
+      const ChainFinish finish{repeats + 1, plan, d_plan_host, arena.flag_device(1), sequence, d_chain_host,
+                               buf.folded, sizes_dev_out, order_dev_out, reorder};
+      if (coord_dtype == MNT_INT32) {
+        launch_query_chain<int32_t>(static_cast<const int32_t *>(sorted_coords_out), n, ndim, no, tile_counts,
+                                    num_tiles, sink, buf.plan, finish, stream);
+      } else {
+        launch_query_chain<int64_t>(static_cast<const int64_t *>(sorted_coords_out), n, ndim, no, tile_counts,
+                                    num_tiles, sink, buf.plan, finish, stream);
+      }
+      profile_mark("query", stream);
       // a workgroup per four tiles and per offset that is looked up (or is the zero offset)
       dim3 grid(static_cast<unsigned>(div_ceil(num_tiles, kPlaceTiles)), static_cast<unsigned>(num_rows));
       place_kernel<true><<<grid, kPlaceBlock, 0, stream>>>(stage, masks, tile_counts, row_totals, tile_mode, n, no,
                                                      num_tiles, num_wave_tiles, reorder, in_idx_out,
                                                      out_idx_out, plan, d_plan_host, arena.flag_device(1),
                                                      sequence, sizes_dev_out, order_dev_out, buf.plan,
-                                                     buf.folded, d_chain_host, repeats, total_copies(), kPlanMaxOffsets);
+                                                     buf.folded, d_chain_host, repeats, total_copies(), kPlanMaxOffsets, 1);
       check_launch("place_kernel");
       arena.wait_flag(1, sequence);
       const long long *h_chain = reinterpret_cast<const long long *>(static_cast<char *>(arena.pinned()) + kChainHostOffset);

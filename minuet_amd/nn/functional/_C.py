@@ -619,12 +619,21 @@ class SortedMapLists:
     ``sizes``, ``order``) are views of it, made when first asked for.  Reads like
     the dict of :func:`kernel_map_build` (``built["in_idx"]``, ``"sizes_host"``,
     ``"order_host"``, ``"bounds"`` ...)."""
-    __slots__ = ("_store", "_coords", "_host", "_n", "_ndim", "_num_offsets", "_views")
+    __slots__ = ("_store", "_coords", "_raw_host", "_n", "_ndim", "_num_offsets", "_views")
 
     def __init__(self, store, coords, host, n, ndim, num_offsets):
-        self._store, self._coords, self._host = store, coords, host
+        # host: a ctypes int64 array (bounds [8], sizes [O], order [O]) that the
+        # library filled; its NumPy view is made when first asked for
+        self._store, self._coords, self._raw_host = store, coords, host
         self._n, self._ndim, self._num_offsets = n, ndim, num_offsets
         self._views = {}
+
+    @property
+    def _host(self):
+        host = self._views.get("_host")
+        if host is None:
+            host = self._views["_host"] = np.frombuffer(self._raw_host, dtype=np.int64)
+        return host
 
     @property
     def sizes_host(self):
@@ -674,6 +683,22 @@ class SortedMapLists:
                        "order_host", "bounds", "source_masks", "target_masks")
 
 
+_ADDRESSES = {}
+
+
+def _host_address(array: np.ndarray) -> int:
+    """Address of a NumPy array's data, remembered per array object (asking
+    NumPy for it costs a microsecond, which a call on a hot path feels)."""
+    hit = _ADDRESSES.get(id(array))
+    if hit is not None and hit[0] is array:
+        return hit[1]
+    if len(_ADDRESSES) > 64:
+        _ADDRESSES.clear()
+    address = array.ctypes.data
+    _ADDRESSES[id(array)] = (array, address)
+    return address
+
+
 def sorted_kernel_map_lists(coordinates: torch.Tensor, offsets_host: np.ndarray, reorder: bool = True,
                             result_only: bool = False):
     """The Map step of a stride-1 layer on an unsorted cloud (one batch) in one
@@ -715,12 +740,12 @@ def sorted_kernel_map_lists(coordinates: torch.Tensor, offsets_host: np.ndarray,
     lists = n * (1 + ndim) if narrow else n
     store = torch.empty((lists + 2 * capacity + 2 * num_offsets,), dtype=torch.int32, device=device)
     coords_out = None if narrow else torch.empty_like(coordinates)
-    host = np.empty(8 + 2 * num_offsets, dtype=np.int64)
+    host = (ctypes.c_int64 * (8 + 2 * num_offsets))()
     base = store.data_ptr()
-    hbase = host.ctypes.data
+    hbase = ctypes.addressof(host)
     with _on(device):
         status = load_library().mnt_sorted_kernel_map_lists(
-            coordinates.data_ptr(), n, ndim, ccode, offs.ctypes.data, num_offsets,
+            coordinates.data_ptr(), n, ndim, ccode, _host_address(offs), num_offsets,
             1 if reorder else 0, base, base + 4 * n if narrow else coords_out.data_ptr(),
             base + 4 * lists, base + 4 * (lists + capacity), capacity,
             base + 4 * (lists + 2 * capacity), base + 4 * (lists + 2 * capacity + num_offsets),
