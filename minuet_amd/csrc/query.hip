@@ -102,23 +102,6 @@ struct HitSink {
   int total_copies, total_stride;
 };
 
-// What the last tile of a chain's query launch needs to tell the host the
-// result's sizes (all null / zero outside a chain).  The tiles count themselves
-// off on `done` as they finish; the one that finds all others counted ranks the
-// offsets by their totals and raises the host's flag, so that the host goes on
-// while the placing launch still runs.
-struct ChainFinish {
-  unsigned *done;                  // zero before the launch
-  unsigned *plan;                  // order | position_of | sorted sizes | prefix (plan_from_sizes)
-  unsigned *plan_host;             // pinned host mirror of the first three blocks
-  unsigned long long *flag;
-  unsigned long long sequence;
-  long long *chain_host;           // pinned: coordinate bounds (8 words), then the chain's verdict
-  const long long *folded_bounds;
-  int *sizes_out, *order_out;      // device copies of sizes / order in row order (nullable)
-  int reorder;
-};
-
 // Settles the queries of one group against the candidates cand[0 .. span]
 // read from window position p on: writes the map entries this workgroup's
 // chunk is responsible for and counts the hits per offset.  The group and
@@ -420,7 +403,7 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     KeyReader<CT, BT> src, KeyReader<CT, BT> tgt, Frame frame, const int *__restrict__ tables,
     CarriedTables carried, int num_groups, int num_offsets, long long delta_min, long long delta_max,
     OT *__restrict__ kernel_map, unsigned *__restrict__ tile_counts, int num_tiles, int dir_rows,
-    HitSink sink, const DevicePlan *__restrict__ device_plan, ChainFinish finish) {
+    HitSink sink, const DevicePlan *__restrict__ device_plan) {
   extern __shared__ __align__(16) unsigned s_dynamic[];
   // Only half of the offsets are looked up (a cloud mapped onto itself under
   // offsets that come in pairs d / -d; see DevicePlan): the totals of the other
@@ -631,46 +614,6 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     }
   }
   if (kLists && tid == 0) sink.tile_mode[blockIdx.x] = num_chunks == 1 ? 0u : 1u;
-  if (kLists && finish.done != nullptr) {
-    // the totals this tile added (device-scope atomics) have been performed once
-    // their acknowledgements are in; only then is the tile counted off
-    __shared__ int s_last;
-    __shared__ unsigned s_totals[kPlanMaxOffsets];
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (tid == 0) s_last = atomicAdd(finish.done, 1u) == gridDim.x - 1 ? 1 : 0;
-    __syncthreads();
-    if (s_last != 0) {
-      // every tile's totals are in: loads that go through to where the atomics were performed
-      if (tid < num_offsets && tid < kPlanMaxOffsets) {
-        unsigned part[kMaxTotalCopies], sum = 0;
-#pragma unroll
-        for (int c = 0; c < kMaxTotalCopies; ++c) {
-          part[c] = c < sink.total_copies ? load_through(sink.row_totals + c * sink.total_stride + tid) : 0u;
-        }
-#pragma unroll
-        for (int c = 0; c < kMaxTotalCopies; ++c) sum += part[c];
-        s_totals[tid] = sum;
-      }
-      const unsigned repeated = sink.repeats != nullptr ? load_through(sink.repeats) : 0u;
-      if (tid == 0) {
-#pragma unroll
-        for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) finish.chain_host[slot] = finish.folded_bounds[slot];
-        finish.chain_host[2 * MNT_MAX_NDIM] = repeated != 0 ? 3 : 0;
-      }
-      __syncthreads();
-      if (repeated == 0) {
-        // thread 0 wrote the bounds and the verdict; it also raises the flag, behind a system-scope fence
-        plan_from_sizes(s_totals, num_offsets, finish.reorder, finish.plan, finish.plan_host, finish.flag,
-                        finish.sequence);
-        for (int j = tid; j < num_offsets; j += kQueryThreads) {
-          if (finish.order_out) finish.order_out[j] = static_cast<int>(finish.plan[j]);
-          if (finish.sizes_out) finish.sizes_out[j] = static_cast<int>(finish.plan[2 * num_offsets + j]);
-        }
-      }
-      // (equal rows: the placing launch reports the verdict and raises the flag)
-    }
-  }
 }
 
 // The query for frames too wide for a packed key (more than 63 bits of
@@ -946,8 +889,7 @@ __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
     unsigned *__restrict__ plan, unsigned *__restrict__ plan_host, unsigned long long *flag,
     unsigned long long sequence, int *__restrict__ sizes_out, int *__restrict__ order_out,
     const DevicePlan *__restrict__ chain_plan, const long long *__restrict__ folded_bounds,
-    long long *chain_host, const unsigned *__restrict__ repeats, int total_copies, int total_stride,
-    int told_by_query) {
+    long long *chain_host, const unsigned *__restrict__ repeats, int total_copies, int total_stride) {
   __shared__ unsigned s_partial[kPlaceBlock / kWave];
   __shared__ unsigned s_partial_mirror[kPlaceBlock / kWave];
   __shared__ unsigned s_totals[kPlanMaxOffsets];
@@ -955,6 +897,45 @@ __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
   const int tid = threadIdx.x;
   const int lane = lane_id();
   const int w = tid >> 6;
+  if (kChain && blockIdx.y == 0) {
+    // Row 0 of a chain's grid places nothing: its first workgroup tells the
+    // host how the chain went (verdict, coordinate bounds, sizes, order) and
+    // leaves the device copies of sizes and order.  It reads three things in
+    // one trip to memory and is among the first workgroups to start, so the
+    // host hears of the sizes while the lists are still being placed.
+    if (blockIdx.x != 0) return;
+    int verdict = chain_plan->verdict;
+    const unsigned repeated = repeats != nullptr ? repeats[0] : 0u;
+    unsigned total = 0;
+    {
+      unsigned part[kMaxTotalCopies];
+#pragma unroll
+      for (int c = 0; c < kMaxTotalCopies; ++c) {
+        part[c] = c < total_copies && tid < num_offsets ? row_totals[c * total_stride + tid] : 0u;
+      }
+#pragma unroll
+      for (int c = 0; c < kMaxTotalCopies; ++c) total += part[c];
+    }
+    if (repeated != 0 && verdict == 0) verdict = 3;     // equal rows: the halves do not mirror each other
+    if (tid == 0) {
+#pragma unroll
+      for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) chain_host[slot] = folded_bounds[slot];
+      chain_host[2 * MNT_MAX_NDIM] = static_cast<long long>(verdict);
+      if (verdict != 0) {
+        __threadfence_system();
+        __hip_atomic_store(flag, sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
+    }
+    if (verdict != 0) return;
+    if (tid < num_offsets && tid < kPlanMaxOffsets) s_totals[tid] = total;
+    __syncthreads();
+    plan_from_sizes(s_totals, num_offsets, reorder, plan, plan_host, flag, sequence);
+    for (int j = tid; j < num_offsets; j += kPlaceBlock) {
+      if (order_out) order_out[j] = static_cast<int>(plan[j]);
+      if (sizes_out) sizes_out[j] = static_cast<int>(plan[2 * num_offsets + j]);
+    }
+    return;
+  }
   const int tile0 = blockIdx.x * kPlaceTiles;
   const int tile = tile0 + w;
   constexpr int kSegments = kTargetsPerTile / kWave;
@@ -972,7 +953,7 @@ __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
   unsigned repeated = 0;
   if (kChain) {
     verdict = chain_plan->verdict;
-    packed = chain_plan->rows[blockIdx.y];
+    packed = chain_plan->rows[blockIdx.y - 1];                       // row 0 of the grid is the teller above
     repeated = repeats != nullptr ? repeats[0] : 0u;
   }
   unsigned total_mine = 0;                       // hits of offset tid (tid < num_offsets <= 64 when there are copies)
@@ -1020,27 +1001,13 @@ __global__ __launch_bounds__(kPlaceBlock) void place_kernel(
                  "+v"(entry[5]), "+v"(entry[6]), "+v"(entry[7]), "+v"(lo), "+v"(hi));
   }
   if (repeated != 0 && verdict == 0) verdict = 3;       // equal rows: the halves do not mirror each other
-  // told_by_query: the query launch's last tile has told the host the sizes of a
-  // chain that went through; this launch only speaks up when it did not
-  const bool silent = told_by_query != 0 && verdict == 0;
-  if (kChain && !silent && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) {
-    // end of a chain of launches: the host learns the chain's verdict and the
-    // coordinate bounds together with the sizes
-#pragma unroll
-    for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) chain_host[slot] = folded_bounds[slot];
-    chain_host[2 * MNT_MAX_NDIM] = static_cast<long long>(verdict);
-    if (verdict != 0) {
-      __threadfence_system();
-      __hip_atomic_store(flag, sequence, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
-    }
-  }
   if (verdict != 0) return;
   if (total_copies > 1) {
     if (tid < num_offsets) s_totals[tid] = total_mine;
     __syncthreads();
     row_totals = s_totals;
   }
-  if (blockIdx.x == 0 && blockIdx.y == 0 && !silent) {
+  if (!kChain && blockIdx.x == 0 && blockIdx.y == 0) {
     // sizes, order and the flag for the host; device copies of sizes and order
     plan_from_sizes(row_totals, num_offsets, reorder, plan, plan_host, flag, sequence);
     for (int j = tid; j < num_offsets; j += kPlaceBlock) {
@@ -1414,7 +1381,7 @@ static void launch_query(const QueryArgs &a, const QueryPlan &plan, const int *d
   const dim3 grid(static_cast<unsigned>(num_tiles), static_cast<unsigned>(split));
   query_kernel<CT, BT, OT, kLists><<<grid, kQueryThreads, dyn, stream>>>(
       src, tgt, plan.frame, d_tables, carried, plan.num_groups, num_offsets, plan.delta_min,
-      plan.delta_max, kernel_map, tile_counts, num_tiles, dir_rows, sink, nullptr, ChainFinish{});
+      plan.delta_max, kernel_map, tile_counts, num_tiles, dir_rows, sink, nullptr);
   check_launch("query_kernel");
 }
 
@@ -1938,7 +1905,7 @@ extern "C" int mnt_kernel_map_lists(const void *sources, int64_t num_sources, co
                                                    num_targets, no, num_tiles, num_wave_tiles, reorder,
                                                    in_idx_out, out_idx_out, plan, d_plan_host,
                                                    arena.flag_device(1), sequence, sizes_dev_out,
-                                                   order_dev_out, nullptr, nullptr, nullptr, nullptr, 1, no, 0);
+                                                   order_dev_out, nullptr, nullptr, nullptr, nullptr, 1, no);
     check_launch("place_kernel");
     collect_sizes(arena, sequence, num_offsets, sizes_host_out, order_host_out);
     profile_mark("map_place+sync", stream);
@@ -1972,7 +1939,7 @@ constexpr size_t kChainHostOffset = 128;      // pinned block: bounds (8 words),
 template <typename CT>
 static void launch_query_chain(const CT *sorted, int64_t n, int ndim, int num_offsets,
                                unsigned *tile_counts, int num_tiles, const HitSink &sink,
-                               const DevicePlan *plan, const ChainFinish &finish, hipStream_t stream) {
+                               const DevicePlan *plan, hipStream_t stream) {
   KeyReader<CT, int32_t> rows{sorted, nullptr, 1, n};
   Frame frame;
   memset(&frame, 0, sizeof(frame));
@@ -1984,7 +1951,7 @@ static void launch_query_chain(const CT *sorted, int64_t n, int ndim, int num_of
                      sizeof(unsigned short) * static_cast<size_t>(kDirectoryRows);
   query_kernel<CT, int32_t, int32_t, true><<<num_tiles, kQueryThreads, dyn, stream>>>(
       rows, rows, frame, nullptr, carried, 0, num_offsets, 0, 0, nullptr, tile_counts, num_tiles,
-      kDirectoryRows, sink, plan, finish);
+      kDirectoryRows, sink, plan);
   check_launch("query_kernel");
 }
 
@@ -2029,8 +1996,7 @@ extern "C" int mnt_sorted_kernel_map_lists(const void *coords, int64_t n, int nd
       buf.partial = scope.alloc<long long>(128 * 8);
       buf.folded = scope.alloc<long long>(2 * MNT_MAX_NDIM);
       // bucket totals, cursors, the copies of the hits per offset, the equal-rows flag
-      // ..., the count of finished query tiles
-      buf.counter_words = 2 * buckets + kMaxTotalCopies * kPlanMaxOffsets + 2;
+      buf.counter_words = 2 * buckets + kMaxTotalCopies * kPlanMaxOffsets + 1;
       buf.counters = scope.alloc<unsigned>(buf.counter_words);
       buf.info = scope.alloc<unsigned>(4);
       buf.status = scope.alloc<unsigned>(4);
@@ -2060,24 +2026,21 @@ extern "C" int mnt_sorted_kernel_map_lists(const void *coords, int64_t n, int nd
       unsigned *d_plan_host = reinterpret_cast<unsigned *>(pinned_device + Arena::kPlanOffset);
       long long *d_chain_host = reinterpret_cast<long long *>(pinned_device + kChainHostOffset);
       const unsigned long long sequence = arena.next_sequence();
-      // the query launch's last tile tells the host the sizes: the host goes on while the lists are being placed
-      const ChainFinish finish{repeats + 1, plan, d_plan_host, arena.flag_device(1), sequence, d_chain_host,
-                               buf.folded, sizes_dev_out, order_dev_out, reorder};
       if (coord_dtype == MNT_INT32) {
         launch_query_chain<int32_t>(static_cast<const int32_t *>(sorted_coords_out), n, ndim, no, tile_counts,
-                                    num_tiles, sink, buf.plan, finish, stream);
+                                    num_tiles, sink, buf.plan, stream);
       } else {
         launch_query_chain<int64_t>(static_cast<const int64_t *>(sorted_coords_out), n, ndim, no, tile_counts,
-                                    num_tiles, sink, buf.plan, finish, stream);
+                                    num_tiles, sink, buf.plan, stream);
       }
       profile_mark("query", stream);
-      // a workgroup per four tiles and per offset that is looked up (or is the zero offset)
-      dim3 grid(static_cast<unsigned>(div_ceil(num_tiles, kPlaceTiles)), static_cast<unsigned>(num_rows));
+      // a workgroup per four tiles and per offset that is looked up (or is the zero offset); row 0 tells the host
+      dim3 grid(static_cast<unsigned>(div_ceil(num_tiles, kPlaceTiles)), static_cast<unsigned>(num_rows + 1));
       place_kernel<true><<<grid, kPlaceBlock, 0, stream>>>(stage, masks, tile_counts, row_totals, tile_mode, n, no,
                                                      num_tiles, num_wave_tiles, reorder, in_idx_out,
                                                      out_idx_out, plan, d_plan_host, arena.flag_device(1),
                                                      sequence, sizes_dev_out, order_dev_out, buf.plan,
-                                                     buf.folded, d_chain_host, repeats, total_copies(), kPlanMaxOffsets, 1);
+                                                     buf.folded, d_chain_host, repeats, total_copies(), kPlanMaxOffsets);
       check_launch("place_kernel");
       arena.wait_flag(1, sequence);
       const long long *h_chain = reinterpret_cast<const long long *>(static_cast<char *>(arena.pinned()) + kChainHostOffset);
