@@ -297,9 +297,12 @@ int mnt_kernel_map_lists(const void *sources, int64_t num_sources,
  * a chain of six launches (bounds, bucket histogram, dealing, ranking, query,
  * list placing) that never returns to the host in between: key layouts, bucket
  * starts and the query plan are worked out on the device, and the host waits
- * once, for the sizes.  A cloud the chain declines (a bucket beyond 4 096
- * rows, keys that do not fit a word) and every other shape go through the two
- * separate entry points inside this call; the results are the same.
+ * once, for the sizes.  Offsets that come in pairs d / -d are looked up once
+ * per pair there: a cloud mapped onto itself has the pair list of -d equal to
+ * the pair list of d with the two indices exchanged, in the same order.  A
+ * cloud the chain declines (a bucket beyond 4 096 rows, keys that do not fit
+ * a word, equal rows under paired offsets) and every other shape go through
+ * the two separate entry points inside this call; the results are the same.
  * Replaces F.arg_sort_coordinates (minuet/nn/functional/indexing.py:14-56)
  * followed by the miss path of KernelMapCache.get_kernel_map
  * (minuet/nn/convolutions.py:147-170). */
