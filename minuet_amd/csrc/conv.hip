@@ -102,11 +102,15 @@ __global__ __launch_bounds__(256) void gather_kernel(const unsigned char *__rest
 template <typename T, typename V, int E, int NV>
 __device__ __forceinline__ void finish_row(float (&acc)[NV][E], const Epilogue &ep, long long t,
                                            int channels, int lr, int lanes_per_row,
-                                           unsigned char *__restrict__ dst) {
+                                           unsigned char *__restrict__ dst, float unscale = 1.0f) {
   constexpr int VB = E * static_cast<int>(sizeof(T));
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int piece = lr + i * lanes_per_row;
+    if (ep.range != nullptr) {
+#pragma unroll
+      for (int k = 0; k < E; ++k) acc[i][k] *= unscale;
+    }
     if (ep.scale != nullptr) {
 #pragma unroll
       for (int k = 0; k < E; ++k) acc[i][k] *= ep.scale[piece * E + k];
@@ -157,6 +161,7 @@ __global__ __launch_bounds__(256) void scatter_wide_kernel(const TB *__restrict_
                                                       int channels, int lanes_per_row,
                                                       const TB *__restrict__ direct, Epilogue ep) {
   typedef typename VecOf<VB>::type V;
+  const float unscale = 1.0f / range_scale(ep.range);            // every lane is still here
   constexpr int E = VB / static_cast<int>(sizeof(T));
   constexpr int BB = E * static_cast<int>(sizeof(TB));          // buffer bytes per vector
   typedef typename VecOf<(BB > 16 ? 16 : BB)>::type BV;
@@ -225,7 +230,7 @@ __global__ __launch_bounds__(256) void scatter_wide_kernel(const TB *__restrict_
       }
     }
   }
-  finish_row<T, V, E, NV>(acc, ep, t, channels, lr, lanes_per_row, dst);
+  finish_row<T, V, E, NV>(acc, ep, t, channels, lr, lanes_per_row, dst, unscale);
 }
 
 // Scatter in two phases per workgroup of `tile_targets` (a power of two)
@@ -251,6 +256,7 @@ __global__ __launch_bounds__(kScatterBlock) void scatter_kernel(
     int num_offsets, int channels, int lanes_per_row, const TB *__restrict__ direct,
     int tile_shift, Epilogue ep) {
   typedef typename VecOf<VB>::type V;
+  const float unscale = 1.0f / range_scale(ep.range);            // every lane is still here
   constexpr int E = VB / static_cast<int>(sizeof(T));
   constexpr int BB = E * static_cast<int>(sizeof(TB));          // buffer bytes per vector
   typedef typename VecOf<(BB > 16 ? 16 : BB)>::type BV;
@@ -379,7 +385,7 @@ __global__ __launch_bounds__(kScatterBlock) void scatter_kernel(
       }
     }
     unsigned char *dst = targets + t * channels * static_cast<long long>(sizeof(T));
-    finish_row<T, V, E, NV>(acc, ep, t, channels, lr, lanes_per_row, dst);
+    finish_row<T, V, E, NV>(acc, ep, t, channels, lr, lanes_per_row, dst, unscale);
   }
 }
 
@@ -395,6 +401,7 @@ __global__ __launch_bounds__(kScatterBlock) void scatter_rows_kernel(
     const TB *__restrict__ buffer, unsigned char *__restrict__ targets, const int *__restrict__ row_ptr,
     long long num_targets, int channels, int lanes_per_row, int tile, Epilogue ep) {
   typedef typename VecOf<VB>::type V;
+  const float unscale = 1.0f / range_scale(ep.range);            // every lane is still here
   constexpr int E = VB / static_cast<int>(sizeof(T));
   constexpr int BB = E * static_cast<int>(sizeof(TB));          // buffer bytes per vector
   typedef typename VecOf<(BB > 16 ? 16 : BB)>::type BV;
@@ -443,17 +450,22 @@ __global__ __launch_bounds__(kScatterBlock) void scatter_rows_kernel(
       }
     }
     unsigned char *dst = targets + t * channels * static_cast<long long>(sizeof(T));
-    finish_row<T, V, E, NV>(acc, ep, t, channels, lr, lanes_per_row, dst);
+    finish_row<T, V, E, NV>(acc, ep, t, channels, lr, lanes_per_row, dst, unscale);
   }
 }
 
 // Element type of the GEMM-output / scatter-input buffer for feature type T.
 // bfloat16 keeps only 8 significant bits, so rounding every partial product
-// to it would cost more accuracy than the output rounding itself.
+// to it would cost more accuracy than the output rounding itself: its rows are
+// IEEE half words under the per-pass power-of-two scale of range_kernel.
 template <typename T>
 struct BufferOf { typedef T type; };
 template <>
-struct BufferOf<bf16_t> { typedef float type; };
+struct BufferOf<bf16_t> { typedef half_t type; };
+template <typename T>
+struct ScaledBuffer { static constexpr bool value = false; };
+template <>
+struct ScaledBuffer<bf16_t> { static constexpr bool value = true; };
 
 // ------------------------------------------------------------ grouped GEMM ----
 
@@ -511,7 +523,10 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
                                                   const T *__restrict__ wt, const Meta &entry, int K,
                                                   int N, int Kp, int Np,
                                                   const int *__restrict__ gather_index,
-                                                  const int *__restrict__ out_pos) {
+                                                  const int *__restrict__ out_pos,
+                                                  const float *__restrict__ range) {
+  // product rows of a scaled buffer leave as acc * scale (a power of two)
+  const float scale = ScaledBuffer<T>::value ? range_scale(range) : 1.0f;
   constexpr int EPC = 16 / static_cast<int>(sizeof(T));        // elements per 16-byte piece
   constexpr int KC = kChunkBytes / static_cast<int>(sizeof(T));
   constexpr int TN = NB * 32;
@@ -718,7 +733,7 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
       for (int q = 0; q < 4; ++q) {
         TC four[4];
 #pragma unroll
-        for (int x = 0; x < 4; ++x) four[x] = static_cast<TC>(acc[b][q * 4 + x]);
+        for (int x = 0; x < 4; ++x) four[x] = static_cast<TC>(ScaledBuffer<T>::value ? acc[b][q * 4 + x] * scale : acc[b][q * 4 + x]);
         unsigned char *at = turn + r * kTurnRow + (q * 8 + h * 4) * static_cast<int>(sizeof(TC));
         if (sizeof(TC) == 2) {
           *reinterpret_cast<uint2 *>(at) = *reinterpret_cast<const uint2 *>(four);
@@ -753,7 +768,7 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
         if (VEC && ch + 4 <= N) {
           TC out[4];
 #pragma unroll
-          for (int x = 0; x < 4; ++x) out[x] = static_cast<TC>(acc[b][q * 4 + x]);
+          for (int x = 0; x < 4; ++x) out[x] = static_cast<TC>(ScaledBuffer<T>::value ? acc[b][q * 4 + x] * scale : acc[b][q * 4 + x]);
           if (sizeof(TC) == 2) {
             *reinterpret_cast<uint2 *>(dst + ch) = *reinterpret_cast<const uint2 *>(out);
           } else {
@@ -762,7 +777,7 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
         } else {
 #pragma unroll
           for (int x = 0; x < 4; ++x) {
-            if (ch + x < N) dst[ch + x] = static_cast<TC>(acc[b][q * 4 + x]);
+            if (ch + x < N) dst[ch + x] = static_cast<TC>(ScaledBuffer<T>::value ? acc[b][q * 4 + x] * scale : acc[b][q * 4 + x]);
           }
         }
       }
@@ -776,8 +791,8 @@ template <typename T, typename TC, int NB, bool VEC, int CH>
 __global__ __launch_bounds__(kGemmBlock, 3) void grouped_gemm_kernel(
     const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt,
     const int *__restrict__ meta, int K, int N, int Kp, int Np,
-    const int *__restrict__ gather_index, const int *__restrict__ out_pos) {
-  grouped_gemm_body<T, TC, NB, VEC, CH>(a, c, wt, MetaInMemory{meta}, K, N, Kp, Np, gather_index, out_pos);
+    const int *__restrict__ gather_index, const int *__restrict__ out_pos, const float *__restrict__ range) {
+  grouped_gemm_body<T, TC, NB, VEC, CH>(a, c, wt, MetaInMemory{meta}, K, N, Kp, Np, gather_index, out_pos, range);
 }
 
 // The same with the tables as a by-value argument.
@@ -785,12 +800,12 @@ template <typename T, typename TC, int NB, bool VEC, int CH>
 __global__ __launch_bounds__(kGemmBlock, 3) void grouped_gemm_riding_kernel(
     const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt, int K, int N, int Kp, int Np,
     const int *__restrict__ gather_index, PlanChunk table, int table_count, int meta_at,
-    int *__restrict__ table_out, const int *__restrict__ out_pos) {
+    int *__restrict__ table_out, const int *__restrict__ out_pos, const float *__restrict__ range) {
   if (blockIdx.x == 0 && blockIdx.y == 0) {
     for (int i = threadIdx.x; i < table_count; i += kGemmBlock) table_out[i] = table.v[i];
   }
   grouped_gemm_body<T, TC, NB, VEC, CH>(a, c, wt, MetaInArguments{&table, meta_at}, K, N, Kp, Np,
-                                        gather_index, out_pos);
+                                        gather_index, out_pos, range);
 }
 
 // ---------------------------------------------------------- host launchers ----
@@ -936,7 +951,7 @@ struct RidingTable {
 template <typename T, typename TC, int NB>
 static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int num_tiles, int K, int N,
                            int Kp, int Np, bool vec, const int *gather_index, const RidingTable &riding,
-                           hipStream_t stream, const int *out_pos) {
+                           hipStream_t stream, const int *out_pos, const float *range) {
   // as many workgroups as the compute units hold at once (by registers); each
   // walks its share of the tiles
   const int slices = static_cast<int>(div_ceil(Np, NB * 32));
@@ -952,7 +967,7 @@ static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int 
     std::memcpy(chunk.v, riding.ints->data(), count * sizeof(int));
 #define MNT_RIDING(VEC, CH)                                                                 \
   grouped_gemm_riding_kernel<T, TC, NB, VEC, CH><<<grid, kGemmBlock, 0, stream>>>(          \
-      a, c, wt, K, N, Kp, Np, gather_index, chunk, count, riding.meta_at, riding.out, out_pos)
+      a, c, wt, K, N, Kp, Np, gather_index, chunk, count, riding.meta_at, riding.out, out_pos, range)
     if (held == 1) {
       MNT_RIDING(true, 1);
     } else if (held == 2) {
@@ -966,7 +981,7 @@ static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int 
   } else {
 #define MNT_PLAIN(VEC, CH)                                                                  \
   grouped_gemm_kernel<T, TC, NB, VEC, CH><<<grid, kGemmBlock, 0, stream>>>(a, c, wt, meta, K, N, Kp, Np, \
-                                                                           gather_index, out_pos)
+                                                                           gather_index, out_pos, range)
     if (held == 1) {
       MNT_PLAIN(true, 1);
     } else if (held == 2) {
@@ -983,7 +998,8 @@ static void launch_gemm_nb(const T *a, TC *c, const T *wt, const int *meta, int 
 template <typename T, typename TC>
 static void launch_gemm(const T *a, TC *c, const T *wt, const int *meta, int num_tiles, int K, int N,
                         int Kp, int Np, const int *gather_index, hipStream_t stream,
-                        const RidingTable &riding = RidingTable(), const int *out_pos = nullptr) {
+                        const RidingTable &riding = RidingTable(), const int *out_pos = nullptr,
+                        const float *range = nullptr) {
   if (num_tiles == 0) return;
   const bool vec = (static_cast<int64_t>(K) * sizeof(T)) % 16 == 0 &&
                    reinterpret_cast<uintptr_t>(a) % 16 == 0 && N % 4 == 0 &&
@@ -995,10 +1011,10 @@ static void launch_gemm(const T *a, TC *c, const T *wt, const int *meta, int num
   const int blocks = Np / 32;
   const int slices = static_cast<int>(div_ceil(blocks, kMaxChannelBlocks));
   switch (static_cast<int>(div_ceil(blocks, slices))) {
-    case 1: launch_gemm_nb<T, TC, 1>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream, out_pos); break;
-    case 2: launch_gemm_nb<T, TC, 2>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream, out_pos); break;
-    case 3: launch_gemm_nb<T, TC, 3>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream, out_pos); break;
-    default: launch_gemm_nb<T, TC, 4>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream, out_pos); break;
+    case 1: launch_gemm_nb<T, TC, 1>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream, out_pos, range); break;
+    case 2: launch_gemm_nb<T, TC, 2>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream, out_pos, range); break;
+    case 3: launch_gemm_nb<T, TC, 3>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream, out_pos, range); break;
+    default: launch_gemm_nb<T, TC, 4>(a, c, wt, meta, num_tiles, K, N, Kp, Np, vec, gather_index, riding, stream, out_pos, range); break;
   }
   check_launch("grouped_gemm_kernel");
 }
@@ -1080,6 +1096,21 @@ static void read_sizes(const void *sizes_dev, int index_dtype, int64_t num_offse
     out[j] = isz == 4 ? static_cast<int64_t>(reinterpret_cast<int32_t *>(raw.data())[j])
                       : reinterpret_cast<int64_t *>(raw.data())[j];
   }
+}
+
+
+// Range of the pass's product rows (see range_kernel): null unless the
+// buffer of feature type T is a scaled one.
+template <typename T>
+static float *measure_range(Scope &scope, const T *features, int64_t count, const T *wt, int64_t columns,
+                            int Kp, hipStream_t stream) {
+  if (!ScaledBuffer<T>::value) return nullptr;
+  float *range = scope.alloc<float>(kRangeParts);
+  range_kernel<T><<<kRangeParts, 256, 0, stream>>>(features, static_cast<long long>(count), wt,
+                                                   static_cast<long long>(columns), Kp, range);
+  check_launch("range_kernel");
+  profile_mark("range", stream);
+  return range;
 }
 
 template <typename T, typename IT>
@@ -1186,10 +1217,13 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
   // with the shortcut the centre offset's product takes one extra buffer row per target
   TB *cbuf = scope.alloc<TB>((rows + (plan.shortcut ? static_cast<size_t>(Tn) : 0)) * N);
   TB *direct = plan.shortcut ? cbuf + rows * N : nullptr;
+  const float *range = measure_range<T>(scope, sources, S * K, wt, O * Np, Kp, stream);
+  Epilogue finish = epilogue;
+  finish.range = range;
 
   if (folded) {
     launch_gemm<T, TB>(sources, cbuf, wt, d_meta, num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np,
-                       gather_index, stream, riding);
+                       gather_index, stream, riding, nullptr, range);
   } else {
     T *abuf = scope.alloc<T>(rows * K);
     const LaneShape gsh = lane_shape(gather_tile, K, sizeof(T), sources, abuf, "num_source_features");
@@ -1197,17 +1231,17 @@ static void forward_typed(int64_t gather_tile, int64_t scatter_tile, const Forwa
                       static_cast<int>(K * sizeof(T)), stream);
     profile_mark("gather", stream);
     launch_gemm<T, TB>(abuf, cbuf, wt, d_meta, num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np,
-                       nullptr, stream);
+                       nullptr, stream, RidingTable(), nullptr, range);
   }
   if (plan.shortcut && !merged) {
     launch_gemm<T, TB>(sources, direct, wt, d_direct, dmeta[2], static_cast<int>(K), static_cast<int>(N), Kp, Np,
-                       nullptr, stream);
+                       nullptr, stream, RidingTable(), nullptr, range);
   }
   profile_mark("gemm", stream);
 
   const LaneShape ssh = lane_shape(scatter_tile, N, sizeof(T), cbuf, out, "num_target_features");
   launch_scatter<TB, T, IT>(ssh, cbuf, out, target_masks, d_row_start, Tn, active,
-                            static_cast<int>(N), direct, epilogue, stream);
+                            static_cast<int>(N), direct, finish, stream);
   profile_mark("scatter", stream);
 }
 
@@ -1309,11 +1343,14 @@ static void forward_rows_typed(int64_t scatter_tile, const ForwardPlan &plan, co
   typedef typename BufferOf<T>::type TB;
   const size_t rows = static_cast<size_t>(plan.total_rows > 0 ? plan.total_rows : 1);
   TB *cbuf = scope.alloc<TB>(rows * N);
+  const float *range = measure_range<T>(scope, sources, S * K, wt, O * Np, Kp, stream);
+  Epilogue finish = epilogue;
+  finish.range = range;
   launch_gemm<T, TB>(sources, cbuf, wt, d_meta, plan.num_tiles, static_cast<int>(K), static_cast<int>(N), Kp, Np,
-                     in_idx, stream, riding, out_pos);
+                     in_idx, stream, riding, out_pos, range);
   profile_mark("gemm", stream);
   const LaneShape ssh = lane_shape(scatter_tile, N, sizeof(T), cbuf, out, "num_target_features");
-  launch_scatter_rows<TB, T>(ssh, cbuf, out, row_ptr, Tn, static_cast<int>(N), epilogue, stream);
+  launch_scatter_rows<TB, T>(ssh, cbuf, out, row_ptr, Tn, static_cast<int>(N), finish, stream);
   profile_mark("scatter", stream);
 }
 

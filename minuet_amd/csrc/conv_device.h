@@ -45,6 +45,7 @@ struct Epilogue {
   const void *residual;
   int activation;      // MNT_ACT_*
   float slope;         // LeakyReLU negative slope
+  const float *range;  // see range_kernel: the buffer rows are scaled (null: they are not)
 };
 
 
@@ -118,5 +119,89 @@ __global__ __launch_bounds__(256) void pack_weights_kernel(const T *__restrict__
   }
 }
 
+// ------------------------------------------------- range of the product rows ----
+
+// Product rows of bfloat16 layers travel from the GEMM to Scatter as IEEE half
+// words (11 significant bits against bfloat16's 8, so rounding the partial
+// products costs less than rounding the output does) times a power of two
+// chosen per pass so that no product can leave half's range: every entry of a
+// product row is bounded by max|x| * max over (offset, channel) of
+// sum_k |w[k][channel]|.  range_kernel leaves the two maxima as kRangeParts
+// partial maxima (blocks [0, kRangeFeatureParts): features; the rest: weight
+// column sums over the packed weights wt[O][Np][Kp]); range_scale folds them
+// (every workgroup of the GEMM and of Scatter does so for itself: 1 KB from
+// the L2) into the scale 2^(15 - e), where bound < 2^e.  Non-finite features
+// are left out of the maximum (their products are non-finite under any scale).
+constexpr int kRangeFeatureParts = 192;
+constexpr int kRangeParts = 256;
+
+template <typename T>
+__global__ __launch_bounds__(256) void range_kernel(const T *__restrict__ features, long long count,
+                                                    const T *__restrict__ wt, long long columns, int Kp,
+                                                    float *__restrict__ range) {
+  __shared__ float s_part[4];
+  float best = 0.0f;
+  if (blockIdx.x < kRangeFeatureParts) {
+    constexpr int E = 16 / static_cast<int>(sizeof(T));
+    const long long stride = static_cast<long long>(kRangeFeatureParts) * 256;
+    const long long first = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+    if (reinterpret_cast<uintptr_t>(features) % 16 == 0) {
+      const long long pieces = count / E;
+      for (long long i = first; i < pieces; i += stride) {
+        const uint4 raw = reinterpret_cast<const uint4 *>(features)[i];
+        const T *e = reinterpret_cast<const T *>(&raw);
+#pragma unroll
+        for (int k = 0; k < E; ++k) {
+          const float v = fabsf(to_float(e[k]));
+          best = v <= 3.0e38f ? fmaxf(best, v) : best;
+        }
+      }
+      for (long long i = pieces * E + first; i < count; i += stride) {
+        const float v = fabsf(to_float(features[i]));
+        best = v <= 3.0e38f ? fmaxf(best, v) : best;
+      }
+    } else {
+      for (long long i = first; i < count; i += stride) {
+        const float v = fabsf(to_float(features[i]));
+        best = v <= 3.0e38f ? fmaxf(best, v) : best;
+      }
+    }
+  } else {
+    // a thread per (offset, channel) row of the packed weights
+    const long long stride = static_cast<long long>(kRangeParts - kRangeFeatureParts) * 256;
+    for (long long c = static_cast<long long>(blockIdx.x - kRangeFeatureParts) * 256 + threadIdx.x; c < columns;
+         c += stride) {
+      float sum = 0.0f;
+      for (int k = 0; k < Kp; ++k) sum += fabsf(to_float(wt[c * Kp + k]));
+      best = fmaxf(best, sum);
+    }
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) best = fmaxf(best, __shfl_xor(best, d));
+  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = best;
+  __syncthreads();
+  if (threadIdx.x == 0) range[blockIdx.x] = fmaxf(fmaxf(s_part[0], s_part[1]), fmaxf(s_part[2], s_part[3]));
+}
+
+// The scale of the pass (a power of two; 1 without a range or when the bound
+// is zero or not finite).  The same in every lane of every workgroup.
+__device__ __forceinline__ float range_scale(const float *__restrict__ range) {
+  if (range == nullptr) return 1.0f;
+  const int lane = threadIdx.x & 63;
+  float fx = fmaxf(fmaxf(range[lane], range[lane + 64]), range[lane + 128]);
+  float fw = range[kRangeFeatureParts + lane];
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) {
+    fx = fmaxf(fx, __shfl_xor(fx, d));
+    fw = fmaxf(fw, __shfl_xor(fw, d));
+  }
+  const float bound = fx * fw;
+  if (!(bound > 0.0f) || !(bound <= 3.0e38f)) return 1.0f;
+  int e;
+  frexpf(bound, &e);                                  // bound = m * 2^e, m in [0.5, 1)
+  int shift = 15 - e;
+  shift = shift > 120 ? 120 : shift < -120 ? -120 : shift;
+  return ldexpf(1.0f, shift);
+}
 
 }  // namespace mnt
