@@ -471,6 +471,49 @@ int mnt_sparse_convolution_forward_rows(int64_t scatter_tile, const void *source
                                         const void *residual, int activation, float negative_slope,
                                         const void *packed_weights, void *out, void *stream);
 
+/* Offset groups of a 3 x 3 x 3 layer, from its dense int32 map
+ * kernel_map[27, T] (original offset order).  Along each of the three axes the
+ * 27 offsets fall into 9 groups of 3 that differ along that axis only;
+ * group_offsets_host int32 [3][9][3] lists them (offset index of member m of
+ * group j along axis a; every axis lists each of the 27 offsets once).  A
+ * target belongs to a group when any of the group's offsets reaches a source.
+ * The axis with the fewest (group, target) rows is chosen ON THE DEVICE and
+ * written to head_out[0]; head_out[1 + j] = rows of group j (head_out: 16 x
+ * int32); rank_out int32 [9, T] = rank of target t among the rows of group j
+ * (-1: not in the group); src_out int32 [9 * T, 4] = the three source rows (-1:
+ * none) of row i of group j at [j * T + i] (fourth word unused; 16-byte
+ * aligned).  Three launches, nothing is read back.  Feeds
+ * mnt_sparse_convolution_forward_groups.  No counterpart in the reference,
+ * whose kernel map has one row per offset
+ * (minuet/nn/convolutions.py:147-170). */
+int mnt_kernel_map_offset_groups(const int32_t *kernel_map, int64_t num_targets,
+                                 const int32_t *group_offsets_host, int32_t *rank_out,
+                                 int32_t *src_out, int32_t *head_out, void *stream);
+
+/* The convolution of mnt_sparse_convolution_forward over the offset groups of
+ * mnt_kernel_map_offset_groups (rank, src, head, group_offsets_host as there):
+ * the three offsets of a group are multiplied in one product whose K dimension
+ * is their three weight matrices one after the other, the data row of a target
+ * being its three source rows end to end (zeros where an offset has none), so
+ * a group writes one buffer row per target it reaches instead of one per
+ * (offset, target) pair; Scatter then sums at most 9 rows per target.  For
+ * clouds that are dense along the chosen axis this halves the buffer traffic
+ * that bounds wide layers, at 1.3 x the multiplications.  16-bit features
+ * whose rows are whole 128-byte chunks, Cout a multiple of 8, 27 offsets;
+ * packed_weights = mnt_pack_weights of the weights in the layer's own offset
+ * order.  Sums differ from the other forms' in order only.  Epilogue arguments
+ * as in mnt_sparse_convolution_forward_fused.  Same reference code
+ * (csrc/minuet/cuda/functions/sparse_convolution.cu:504-661). */
+int mnt_sparse_convolution_forward_groups(const void *sources, const void *packed_weights,
+                                          const int32_t *rank, const int32_t *src,
+                                          const int32_t *head, const int32_t *group_offsets_host,
+                                          int64_t num_sources, int64_t num_targets,
+                                          int64_t num_source_features, int64_t num_target_features,
+                                          int float_dtype, const float *channel_scale,
+                                          const float *channel_shift, const void *residual,
+                                          int activation, float negative_slope, void *out,
+                                          void *stream);
+
 /* Weights [O, Cin, Cout] -> the layout the matrix kernels stage:
  * packed[O][Np][Kp] = W^T per offset, K-contiguous, zero-padded to
  * Np = ceil(Cout / 32) * 32 rows of Kp = ceil(Cin * e / 128) * 128 / e elements

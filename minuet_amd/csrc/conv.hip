@@ -518,13 +518,36 @@ struct MetaInArguments {
   __device__ __forceinline__ int operator()(int i) const { return table->v[meta_at + i]; }
 };
 
-template <typename T, typename TC, int NB, bool VEC, int CH, typename Meta>
+// Offset groups (GM > 0): the GM offsets of a group are multiplied in ONE
+// product whose K dimension is their GM weight matrices one after the other.
+// A data row then stands for a target that ANY offset of its group reaches,
+// and holds that target's GM source rows end to end (zeros where an offset has
+// no source), so a group needs as many buffer rows as it has such targets
+// instead of one per (offset, target) pair: offsets that differ along an axis
+// in which the cloud is dense share most of their targets.  The tables come
+// from group_emit_kernel: head[0] is the axis the groups lie along (chosen on
+// the device), head[1 + j] the rows of group j; src[j * stride + i] holds the
+// source rows (x, y, z; -1: none) of data row i of group j, which is also its
+// buffer row; offset_of[axis][j][m] is the offset (weight matrix) of member m.
+// Needs K * sizeof(T) to be whole 128-byte chunks.
+constexpr int kGroupCount = 9;
+constexpr int kGroupMembers = 3;
+struct GroupView {
+  const int *head;
+  const int4 *src;
+  long long stride;
+  int tiles_per_group;
+  int offset_of[3 * kGroupCount * kGroupMembers];
+};
+
+template <typename T, typename TC, int NB, bool VEC, int CH, typename Meta, int GM = 0>
 __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *__restrict__ c,
                                                   const T *__restrict__ wt, const Meta &entry, int K,
                                                   int N, int Kp, int Np,
                                                   const int *__restrict__ gather_index,
                                                   const int *__restrict__ out_pos,
-                                                  const float *__restrict__ range) {
+                                                  const float *__restrict__ range,
+                                                  const GroupView *__restrict__ groups = nullptr) {
   // product rows of a scaled buffer leave as acc * scale (a power of two)
   const float scale = ScaledBuffer<T>::value ? range_scale(range) : 1.0f;
   constexpr int EPC = 16 / static_cast<int>(sizeof(T));        // elements per 16-byte piece
@@ -538,7 +561,7 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
   constexpr int kLdsBytes = kWeightBytes > 4 * kTurnBytes ? kWeightBytes : 4 * kTurnBytes;
   __shared__ __align__(16) unsigned char b_lds[kLdsBytes];
 
-  const int G = entry(0);
+  const int G = GM > 0 ? kGroupCount : entry(0);
   const int at_prefix = 1, at_start = at_prefix + G + 1, at_rows = at_start + G + 1, at_weight = at_rows + G,
             at_list = at_weight + G;
 
@@ -546,8 +569,97 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
   // A workgroup walks the tiles blockIdx.x, blockIdx.x + gridDim.x, ...: the
   // grid is what the compute units hold at once, since workgroups that live for
   // a few microseconds are launched more slowly than they finish.
-  const int num_tiles = entry(at_prefix + G);
-  for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
+  const int num_tiles = GM > 0 ? kGroupCount * groups->tiles_per_group : entry(at_prefix + G);
+
+  // What a tile is made of is worked out from tables that do not depend on the
+  // tile: they are fetched once per workgroup (lane i keeps the entries of
+  // group i), and finding a tile's group is a ballot.  The one thing a tile
+  // still has to fetch before its operands, the source row(s) of each data
+  // row, is asked for one tile ahead, while the tile before it is multiplied:
+  // a tile then waits for ONE trip to memory (its operands) instead of three.
+  struct TileAt {
+    bool ok;
+    int prefix, rows, start, weight, list, group;
+  };
+  const int lane0 = threadIdx.x & 63;
+  int m_prefix = 0, m_rows = 0, m_start = 0, m_weight = 0, m_list = 0, m_total = 0, axis = 0;
+  if constexpr (GM > 0) {
+    // tiles are numbered over the rows the groups really have (the grid only
+    // knows the worst case): a scan over the nine lanes that hold the groups'
+    // row counts gives every group's first tile
+    m_rows = groups->head[1 + min(lane0, kGroupCount - 1)];
+    axis = groups->head[0];
+    const int tiles = (m_rows + kGemmRows - 1) / kGemmRows;
+    int upto = tiles;
+#pragma unroll
+    for (int d = 1; d < 16; d <<= 1) {
+      const int below = __shfl_up(upto, d);
+      if (lane0 >= d) upto += below;
+    }
+    m_total = __builtin_amdgcn_readlane(upto, kGroupCount - 1);
+    m_prefix = upto - tiles;
+  } else {
+    m_total = num_tiles;
+    if (G <= kWave) {
+      const int i = min(lane0, G - 1);
+      m_prefix = entry(at_prefix + i);
+      m_rows = entry(at_rows + i);
+      m_start = entry(at_start + i);
+      m_weight = entry(at_weight + i);
+      m_list = entry(at_list + i);
+    }
+  }
+  auto tile_at = [&](int tile) {
+    TileAt t = {tile < m_total, 0, 0, 0, 0, 0, 0};
+    if (!t.ok) return t;
+    if (GM > 0 || G <= kWave) {
+      const int g = __popcll(__ballot(lane0 < G && m_prefix <= tile)) - 1;
+      t.group = g;
+      t.prefix = __builtin_amdgcn_readlane(m_prefix, g);
+      t.rows = __builtin_amdgcn_readlane(m_rows, g);
+      t.start = __builtin_amdgcn_readlane(m_start, g);
+      t.weight = __builtin_amdgcn_readlane(m_weight, g);
+      t.list = __builtin_amdgcn_readlane(m_list, g);
+    } else {
+      int lo = 0, hi = G - 1;
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (entry(at_prefix + mid) <= tile) {
+          lo = mid;
+        } else {
+          hi = mid - 1;
+        }
+      }
+      t.prefix = entry(at_prefix + lo);
+      t.rows = entry(at_rows + lo);
+      t.start = entry(at_start + lo);
+      t.weight = entry(at_weight + lo);
+      t.list = entry(at_list + lo);
+    }
+    return t;
+  };
+  // the source row (plain) or the member source rows (groups) of this lane's data row of a tile
+  auto rows_of = [&](const TileAt &t, int tile) {
+    int4 v = make_int4(-1, -1, -1, 0);
+    if (!t.ok) return v;
+    const int row = (threadIdx.x >> 6) * 32 + (threadIdx.x & 31);
+    const int r0 = (tile - t.prefix) * kGemmRows;
+    const bool row_ok = row < t.rows - r0;
+    if constexpr (GM > 0) {
+      if (row_ok) v = groups->src[t.group * groups->stride + r0 + row];
+    } else {
+      if (gather_index != nullptr && t.list >= 0 && row_ok) {
+        v.x = gather_index[static_cast<long long>(t.list) + r0 + row];
+      }
+    }
+    return v;
+  };
+
+  int tile = blockIdx.x;
+  TileAt here = tile_at(tile);
+  if (!here.ok) return;                              // the same for the whole workgroup
+  int4 here_rows = rows_of(here, tile);
+  for (;;) {
   // (the thread's number is made opaque per tile: what is derived from it is
   // worked out again for every tile instead of being kept in registers)
   int tid = threadIdx.x;
@@ -556,39 +668,14 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
   const int wv = tid >> 6;
   const int r = lane & 31;
   const int h = lane >> 5;
-  int g_prefix, g_rows, g_start, g_weight, g_list;
-  if (G <= kWave) {
-    // One trip to memory instead of a search of dependent reads: lane i
-    // fetches the entries of group i, a ballot over the tile prefix finds the
-    // group of this tile, and its lane hands the entries to everyone.
-    const int i = min(lane, G - 1);
-    const int prefix = entry(at_prefix + i), rows = entry(at_rows + i), start = entry(at_start + i),
-              weight = entry(at_weight + i), list = entry(at_list + i);
-    const int g = __popcll(__ballot(lane < G && prefix <= tile)) - 1;
-    g_prefix = __builtin_amdgcn_readlane(prefix, g);
-    g_rows = __builtin_amdgcn_readlane(rows, g);
-    g_start = __builtin_amdgcn_readlane(start, g);
-    g_weight = __builtin_amdgcn_readlane(weight, g);
-    g_list = __builtin_amdgcn_readlane(list, g);
-  } else {
-    int lo = 0, hi = G - 1;
-    while (lo < hi) {
-      const int mid = (lo + hi + 1) >> 1;
-      if (entry(at_prefix + mid) <= tile) {
-        lo = mid;
-      } else {
-        hi = mid - 1;
-      }
-    }
-    g_prefix = entry(at_prefix + lo);
-    g_rows = entry(at_rows + lo);
-    g_start = entry(at_start + lo);
-    g_weight = entry(at_weight + lo);
-    g_list = entry(at_list + lo);
-  }
+  const int g_prefix = here.prefix, g_rows = here.rows, g_start = here.start, g_weight = here.weight,
+            g_list = here.list, group = here.group;
+  const int next_tile = tile + gridDim.x;
+  const TileAt next = tile_at(next_tile);
+  int4 next_rows = make_int4(-1, -1, -1, 0);
   const int r0 = (tile - g_prefix) * kGemmRows;
   const int valid = min(kGemmRows, g_rows - r0);
-  const long long row_base = static_cast<long long>(g_start) + r0;
+  const long long row_base = (GM > 0 ? group * groups->stride : static_cast<long long>(g_start)) + r0;
   const T *w_base = wt + (static_cast<long long>(g_weight) * Np + n0) * Kp;
   const int list_at = g_list;
 
@@ -596,10 +683,10 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
   const bool row_ok = row < valid;
   long long a_index = row_base + row;
   if (gather_index != nullptr) {
-    a_index = list_at < 0 ? r0 + row
-                          : (row_ok ? gather_index[static_cast<long long>(list_at) + r0 + row] : 0);
+    a_index = list_at < 0 ? r0 + row : (row_ok ? here_rows.x : 0);
   }
   const T *a_row = a + a_index * K;
+  const int4 member_rows = here_rows;
   // where this tile's rows go, for the lists of the output pass (null: buffer order)
   const int *pos_list = out_pos != nullptr ? out_pos + (static_cast<long long>(list_at) + r0) : nullptr;
 
@@ -671,7 +758,68 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
     }
   };
 
-  if constexpr (CH > 0) {
+  if constexpr (GM > 0) {
+    // The concatenated K is walked in stages of SC chunks (SC = CH here: 2 where
+    // a member's row is an even number of chunks, else 1).  A stage lies inside
+    // one member: its A pieces come from that member's source row, its W^T
+    // pieces from that member's weight matrix.  All loads of a stage are issued
+    // together; the W^T pieces of the next stage are asked for as soon as this
+    // stage's are in LDS (their registers are free then), the A pieces after
+    // the products that still read the present ones.
+    constexpr int SC = CH;
+    const int per_member = Kp / KC;
+    const int stages = GM * per_member / SC;
+    auto load_a_of = [&](int st, uint4 (&dst)[SC][kSteps]) {
+      const int chunk = st * SC;
+      const int m = chunk / per_member;
+      const int s = m == 0 ? member_rows.x : m == 1 ? member_rows.y : member_rows.z;
+      const T *from = a + static_cast<long long>(s < 0 ? 0 : s) * K + (chunk - m * per_member) * KC + h * EPC;
+#pragma unroll
+      for (int c2 = 0; c2 < SC; ++c2) {
+#pragma unroll
+        for (int kk = 0; kk < kSteps; ++kk) {
+          uint4 v = make_uint4(0u, 0u, 0u, 0u);
+          if (s >= 0) v = *reinterpret_cast<const uint4 *>(from + c2 * KC + kk * 2 * EPC);
+          dst[c2][kk] = v;
+        }
+      }
+    };
+    auto load_w_of = [&](int st, uint4 (&wpiece)[SC][kWPieces]) {
+      const int chunk = st * SC;
+      const int m = chunk / per_member;
+      const int offset = groups->offset_of[(axis * kGroupCount + group) * kGroupMembers + m];
+      const T *from = wt + (static_cast<long long>(offset) * Np + n0) * Kp + (chunk - m * per_member) * KC;
+#pragma unroll
+      for (int c2 = 0; c2 < SC; ++c2) {
+#pragma unroll
+        for (int p = 0; p < kWPieces; ++p) {
+          const int piece = tid + p * kGemmBlock;
+          uint4 v = make_uint4(0u, 0u, 0u, 0u);
+          if (piece < TN * 8 && n0 + (piece >> 3) < Np) {
+            v = *reinterpret_cast<const uint4 *>(from + c2 * KC + static_cast<long long>(piece >> 3) * Kp +
+                                                 (piece & 7) * EPC);
+          }
+          wpiece[c2][p] = v;
+        }
+      }
+    };
+    uint4 frag[SC][kSteps];
+    uint4 wpiece[SC][kWPieces];
+    load_w_of(0, wpiece);
+    load_a_of(0, frag);
+    next_rows = rows_of(next, next_tile);
+    for (int st = 0; st < stages; ++st) {
+      if (st > 0) __syncthreads();                   // previous stage of W^T fully consumed
+#pragma unroll
+      for (int c2 = 0; c2 < SC; ++c2) store_w(c2, wpiece[c2]);
+      __syncthreads();
+      const bool more = st + 1 < stages;
+      if (more) load_w_of(st + 1, wpiece);
+#pragma unroll
+      for (int c2 = 0; c2 < SC; ++c2) multiply(c2, frag[c2]);
+      if (more) load_a_of(st + 1, frag);
+    }
+  } else if constexpr (CH > 0) {
     // K of CH chunks (Kp == CH * KC): every load of the tile is issued at
     // once, so the tile pays for one trip to memory instead of one per chunk.
     uint4 frags[CH][kSteps];
@@ -680,6 +828,7 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
     for (int c = 0; c < CH; ++c) load_w(c * KC, wpieces[c]);
 #pragma unroll
     for (int c = 0; c < CH; ++c) load_a(c * KC, frags[c]);
+    next_rows = rows_of(next, next_tile);
 #pragma unroll
     for (int c = 0; c < CH; ++c) store_w(c, wpieces[c]);
     __syncthreads();
@@ -690,6 +839,7 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
     uint4 wpiece[kWPieces];
     load_a(0, frag);
     load_w(0, wpiece);
+    next_rows = rows_of(next, next_tile);
     for (int k0 = 0; k0 < Kp; k0 += KC) {
       if (k0 > 0) __syncthreads();                   // previous chunk of W^T fully consumed
       store_w(0, wpiece);
@@ -783,7 +933,11 @@ __device__ __forceinline__ void grouped_gemm_body(const T *__restrict__ a, TC *_
       }
     }
   }
+  if (!next.ok) break;                  // the same for the whole workgroup
   __syncthreads();                      // the next tile's weights go where this one's were (and its turned blocks)
+  tile = next_tile;
+  here = next;
+  here_rows = next_rows;
   }
 }
 
@@ -806,6 +960,151 @@ __global__ __launch_bounds__(kGemmBlock, 3) void grouped_gemm_riding_kernel(
   }
   grouped_gemm_body<T, TC, NB, VEC, CH>(a, c, wt, MetaInArguments{&table, meta_at}, K, N, Kp, Np,
                                         gather_index, out_pos, range);
+}
+
+// The grouped GEMM over offset groups (see GroupView).  Workgroup (0, 0) also
+// leaves the buffer row at which every group starts, for the Scatter that
+// follows in the stream.
+template <typename T, typename TC, int NB, int SC>
+__global__ __launch_bounds__(kGemmBlock, 3) void group_gemm_kernel(
+    const T *__restrict__ a, TC *__restrict__ c, const T *__restrict__ wt, int K, int N, int Kp, int Np,
+    GroupView groups, int *__restrict__ row_start_out, const float *__restrict__ range) {
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x <= kGroupCount) {
+    row_start_out[threadIdx.x] = static_cast<int>(threadIdx.x * groups.stride);
+  }
+  grouped_gemm_body<T, TC, NB, true, SC, MetaInMemory, kGroupMembers>(a, c, wt, MetaInMemory{nullptr}, K, N, Kp, Np,
+                                                                      nullptr, nullptr, range, &groups);
+}
+
+// ---------------------------------------------------- offset-group tables ----
+//
+// From the dense kernel map M [27, T] of a 3 x 3 x 3 layer: for each of the
+// three axes the 27 offsets fall into 9 groups of 3 that differ along that
+// axis only.  A target belongs to a group when any of the group's offsets
+// reaches a source.  Three launches, no wait on the host:
+//   group_count_kernel   targets per (axis, group, tile of 256 targets);
+//   group_scan_kernel    one workgroup: totals per axis, the axis with the
+//                        fewest rows wins (the lowest on a tie), its tile counts
+//                        become exclusive prefixes, head = [axis, rows of the
+//                        9 groups];
+//   group_emit_kernel    rank of every target inside its groups (-1: none) and
+//                        the member source rows of every data row.
+struct GroupOffsets {
+  int o[3 * kGroupCount * kGroupMembers];     // offset of member m of group j along axis a: [a][j][m]
+};
+constexpr int kGroupTile = 256;
+
+__device__ __forceinline__ bool group_reaches(const int *__restrict__ dense, long long num_targets,
+                                              const GroupOffsets &tab, int slot, long long t, int (&row)[3]) {
+  bool any = false;
+#pragma unroll
+  for (int m = 0; m < kGroupMembers; ++m) {
+    row[m] = dense[static_cast<long long>(tab.o[slot * kGroupMembers + m]) * num_targets + t];
+    any |= row[m] >= 0;
+  }
+  return any;
+}
+
+__global__ __launch_bounds__(kGroupTile) void group_count_kernel(const int *__restrict__ dense,
+                                                                  long long num_targets, GroupOffsets tab,
+                                                                  int tiles, int *__restrict__ tile_counts) {
+  __shared__ int s_count[kGroupTile / kWave];
+  const int slot = blockIdx.y;                                   // axis * 9 + group
+  const long long t = static_cast<long long>(blockIdx.x) * kGroupTile + threadIdx.x;
+  int row[3];
+  const bool any = t < num_targets && group_reaches(dense, num_targets, tab, slot, t, row);
+  const int count = __popcll(__ballot(any));
+  if ((threadIdx.x & (kWave - 1)) == 0) s_count[threadIdx.x / kWave] = count;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int sum = 0;
+#pragma unroll
+    for (int w = 0; w < kGroupTile / kWave; ++w) sum += s_count[w];
+    tile_counts[slot * tiles + blockIdx.x] = sum;
+  }
+}
+
+__global__ __launch_bounds__(1024) void group_scan_kernel(int *__restrict__ tile_counts, int tiles,
+                                                           int *__restrict__ head) {
+  __shared__ int s_part[1024 / kWave];
+  __shared__ int s_axis_total[3];
+  __shared__ int s_carry;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  auto block_sum = [&](int v) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
+    __syncthreads();
+    if (lane == 0) s_part[wave] = v;
+    __syncthreads();
+    int sum = 0;
+    for (int w = 0; w < 1024 / kWave; ++w) sum += s_part[w];
+    return sum;
+  };
+  for (int axis = 0; axis < 3; ++axis) {
+    int mine = 0;
+    for (int i = tid; i < kGroupCount * tiles; i += 1024) mine += tile_counts[axis * kGroupCount * tiles + i];
+    const int total = block_sum(mine);
+    if (tid == 0) s_axis_total[axis] = total;
+  }
+  __syncthreads();
+  int axis = 0;
+  if (s_axis_total[1] < s_axis_total[axis]) axis = 1;
+  if (s_axis_total[2] < s_axis_total[axis]) axis = 2;
+  if (tid == 0) head[0] = axis;
+  // exclusive prefixes of the winning axis' tile counts, group by group
+  int *counts = tile_counts + axis * kGroupCount * tiles;
+  for (int j = 0; j < kGroupCount; ++j) {
+    if (tid == 0) s_carry = 0;
+    __syncthreads();
+    for (int base = 0; base < tiles; base += 1024) {
+      const int i = base + tid;
+      const int v = i < tiles ? counts[j * tiles + i] : 0;
+      int scan = v;                                              // inclusive scan inside the wavefront
+#pragma unroll
+      for (int d = 1; d < kWave; d <<= 1) {
+        const int up = __shfl_up(scan, d);
+        if (lane >= d) scan += up;
+      }
+      __syncthreads();
+      if (lane == kWave - 1) s_part[wave] = scan;
+      __syncthreads();
+      int before = s_carry;
+      for (int w = 0; w < wave; ++w) before += s_part[w];
+      if (i < tiles) counts[j * tiles + i] = before + scan - v;
+      __syncthreads();
+      if (tid == 1023) s_carry = before + scan;
+      __syncthreads();
+    }
+    if (tid == 0) head[1 + j] = s_carry;
+    __syncthreads();
+  }
+}
+
+__global__ __launch_bounds__(kGroupTile) void group_emit_kernel(const int *__restrict__ dense,
+                                                                 long long num_targets, GroupOffsets tab,
+                                                                 int tiles, const int *__restrict__ tile_counts,
+                                                                 const int *__restrict__ head,
+                                                                 int *__restrict__ rank_out,
+                                                                 int4 *__restrict__ src_out) {
+  __shared__ int s_count[kGroupTile / kWave];
+  const int axis = head[0];
+  const int group = blockIdx.y;
+  const int slot = axis * kGroupCount + group;
+  const int base = tile_counts[slot * tiles + blockIdx.x];
+  const long long t = static_cast<long long>(blockIdx.x) * kGroupTile + threadIdx.x;
+  int row[3] = {-1, -1, -1};
+  const bool any = t < num_targets && group_reaches(dense, num_targets, tab, slot, t, row);
+  const unsigned long long ballot = __ballot(any);
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  if (lane == 0) s_count[wave] = __popcll(ballot);
+  __syncthreads();
+  int before = base;
+  for (int w = 0; w < wave; ++w) before += s_count[w];
+  const int rank = before + __popcll(ballot & ((1ull << lane) - 1ull));
+  if (t < num_targets) {
+    rank_out[static_cast<long long>(group) * num_targets + t] = any ? rank : -1;
+    if (any) src_out[static_cast<long long>(group) * num_targets + rank] = make_int4(row[0], row[1], row[2], 0);
+  }
 }
 
 // ---------------------------------------------------------- host launchers ----
@@ -1519,6 +1818,146 @@ extern "C" int mnt_sparse_convolution_forward_rows(
       MNT_ROWS(bf16_t);
     }
 #undef MNT_ROWS
+  });
+}
+
+// Forward pass over offset groups: the grouped GEMM with K-concatenated members,
+// then the ordinary Scatter with the groups' rank table in place of the
+// offsets' (9 rows instead of 27).
+template <typename T>
+static void forward_groups_typed(const T *sources, const T *packed, const int *rank, const int4 *src,
+                                 const int *head, const int32_t *offsets_host, int64_t S, int64_t Tn, int64_t K,
+                                 int64_t N, const Epilogue &epilogue, T *out, hipStream_t stream) {
+  Scope scope(stream);
+  const int kc = kChunkBytes / static_cast<int>(sizeof(T));
+  const int Kp = static_cast<int>(div_ceil(K, kc) * kc);
+  const int Np = static_cast<int>(div_ceil(N, 32) * 32);
+  profile_mark("enter:forward", stream);
+  typedef typename BufferOf<T>::type TB;
+  // room for the worst case (every target in every group); a group's rows start at a multiple of T
+  TB *cbuf = scope.alloc<TB>(static_cast<size_t>(kGroupCount) * Tn * N);
+  int *d_row_start = scope.alloc<int>(kGroupCount + 1);
+  const float *range = measure_range<T>(scope, sources, S * K, packed, int64_t{27} * Np, Kp, stream);
+  Epilogue finish = epilogue;
+  finish.range = range;
+  GroupView view;
+  view.head = head;
+  view.src = src;
+  view.stride = Tn;
+  view.tiles_per_group = static_cast<int>(div_ceil(Tn, kGemmRows));
+  for (int i = 0; i < 3 * kGroupCount * kGroupMembers; ++i) view.offset_of[i] = offsets_host[i];
+  const int blocks = Np / 32;
+  const int slices = static_cast<int>(div_ceil(blocks, kMaxChannelBlocks));
+  const int nb = static_cast<int>(div_ceil(blocks, slices));
+  const int num_tiles = kGroupCount * view.tiles_per_group;
+  const int resident = compute_units() * (nb >= 3 ? 3 : nb == 2 ? 4 : 6);
+  dim3 grid(static_cast<unsigned>(std::min(num_tiles, std::max(1, resident / slices))), static_cast<unsigned>(slices));
+  const bool pairs = (Kp / kc) % 2 == 0;            // stages of two chunks where a member's row divides so
+#define MNT_GG(NB)                                                                                              \
+  if (pairs) {                                                                                                  \
+    group_gemm_kernel<T, TB, NB, 2><<<grid, kGemmBlock, 0, stream>>>(sources, cbuf, packed, static_cast<int>(K), \
+                                                                     static_cast<int>(N), Kp, Np, view,         \
+                                                                     d_row_start, range);                       \
+  } else {                                                                                                      \
+    group_gemm_kernel<T, TB, NB, 1><<<grid, kGemmBlock, 0, stream>>>(sources, cbuf, packed, static_cast<int>(K), \
+                                                                     static_cast<int>(N), Kp, Np, view,         \
+                                                                     d_row_start, range);                       \
+  }
+  switch (nb) {
+    case 1: MNT_GG(1); break;
+    case 2: MNT_GG(2); break;
+    case 3: MNT_GG(3); break;
+    default: MNT_GG(4); break;
+  }
+#undef MNT_GG
+  check_launch("group_gemm_kernel");
+  profile_mark("gemm", stream);
+  const LaneShape ssh = lane_shape(0, N, sizeof(T), cbuf, out, "num_target_features");
+  launch_scatter<TB, T, int32_t>(ssh, cbuf, out, rank, d_row_start, Tn, kGroupCount, static_cast<int>(N), nullptr,
+                                 finish, stream);
+  profile_mark("scatter", stream);
+}
+
+static void check_group_offsets(const int32_t *offsets_host) {
+  MNT_CHECK(offsets_host != nullptr, "group_offsets_host is null");
+  for (int axis = 0; axis < 3; ++axis) {
+    bool seen[27] = {};
+    for (int i = 0; i < kGroupCount * kGroupMembers; ++i) {
+      const int o = offsets_host[axis * kGroupCount * kGroupMembers + i];
+      MNT_CHECK(o >= 0 && o < 27 && !seen[o], "group_offsets_host[%d] does not list each of the 27 offsets once",
+                axis);
+      seen[o] = true;
+    }
+  }
+}
+
+extern "C" int mnt_kernel_map_offset_groups(const int32_t *kernel_map, int64_t T,
+                                            const int32_t *group_offsets_host, int32_t *rank_out,
+                                            int32_t *src_out, int32_t *head_out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MNT_CHECK(T >= 0 && T * kGroupCount <= INT32_MAX, "bad number of targets %lld", (long long)T);
+    check_group_offsets(group_offsets_host);
+    MNT_CHECK(head_out != nullptr, "head_out is null");
+    MNT_CHECK(reinterpret_cast<uintptr_t>(src_out) % 16 == 0, "src_out is not 16-byte aligned");
+    Scope scope(stream);
+    GroupOffsets tab;
+    for (int i = 0; i < 3 * kGroupCount * kGroupMembers; ++i) tab.o[i] = group_offsets_host[i];
+    const int tiles = static_cast<int>(std::max<int64_t>(1, div_ceil(T, kGroupTile)));
+    int *tile_counts = scope.alloc<int>(static_cast<size_t>(3) * kGroupCount * tiles);
+    if (T > 0) MNT_CHECK(kernel_map != nullptr && rank_out != nullptr && src_out != nullptr, "null argument");
+    group_count_kernel<<<dim3(tiles, 3 * kGroupCount), kGroupTile, 0, stream>>>(kernel_map, T, tab, tiles,
+                                                                                 tile_counts);
+    check_launch("group_count_kernel");
+    group_scan_kernel<<<1, 1024, 0, stream>>>(tile_counts, tiles, head_out);
+    check_launch("group_scan_kernel");
+    group_emit_kernel<<<dim3(tiles, kGroupCount), kGroupTile, 0, stream>>>(
+        kernel_map, T, tab, tiles, tile_counts, head_out, rank_out, reinterpret_cast<int4 *>(src_out));
+    check_launch("group_emit_kernel");
+    profile_mark("offset_groups", stream);
+  });
+}
+
+extern "C" int mnt_sparse_convolution_forward_groups(
+    const void *sources, const void *packed_weights, const int32_t *rank, const int32_t *src,
+    const int32_t *head, const int32_t *group_offsets_host, int64_t S, int64_t T, int64_t K, int64_t N,
+    int float_dtype, const float *channel_scale, const float *channel_shift, const void *residual,
+    int activation, float negative_slope, void *out, void *stream_) {
+  return guarded([&] {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int esize = float_size(float_dtype);
+    MNT_CHECK(float_dtype != MNT_FLOAT32, "the offset-group forward takes 16-bit features");
+    MNT_CHECK(S >= 0 && T >= 0 && K >= 1 && N >= 1 && S <= INT32_MAX && T * kGroupCount <= INT32_MAX &&
+                  K <= 65536 && N <= 65536,
+              "bad shape S=%lld T=%lld Cin=%lld Cout=%lld", (long long)S, (long long)T, (long long)K, (long long)N);
+    MNT_CHECK((K * esize) % kChunkBytes == 0, "source rows of %lld bytes are not whole 128-byte chunks",
+              (long long)(K * esize));
+    MNT_CHECK(N % 8 == 0, "num_target_features = %lld is not a multiple of 8", (long long)N);
+    MNT_CHECK(activation >= MNT_ACT_NONE && activation <= MNT_ACT_RELU6, "unknown activation code %d",
+              activation);
+    MNT_CHECK(reinterpret_cast<uintptr_t>(residual) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(channel_scale) % 4 == 0 &&
+                  reinterpret_cast<uintptr_t>(channel_shift) % 4 == 0,
+              "epilogue operands are not aligned (residual: 16 bytes, scale / shift: 4 bytes)");
+    MNT_CHECK(reinterpret_cast<uintptr_t>(packed_weights) % 16 == 0 && reinterpret_cast<uintptr_t>(sources) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0,
+              "operands are not 16-byte aligned");
+    check_group_offsets(group_offsets_host);
+    if (T == 0) return;
+    MNT_CHECK(sources != nullptr && packed_weights != nullptr && rank != nullptr && src != nullptr &&
+                  head != nullptr && out != nullptr,
+              "null argument");
+    const Epilogue epilogue = {channel_scale, channel_shift, residual, activation, negative_slope};
+#define MNT_GROUPS(FT)                                                                                  \
+  forward_groups_typed<FT>(static_cast<const FT *>(sources), static_cast<const FT *>(packed_weights), rank, \
+                           reinterpret_cast<const int4 *>(src), head, group_offsets_host, S, T, K, N, epilogue, \
+                           static_cast<FT *>(out), stream)
+    if (float_dtype == MNT_FLOAT16) {
+      MNT_GROUPS(half_t);
+    } else {
+      MNT_GROUPS(bf16_t);
+    }
+#undef MNT_GROUPS
   });
 }
 

@@ -65,6 +65,7 @@ class KernelMapCache(object):
         self._key_memo = dict()
         self._dense_maps_cache = dict()         # key -> (dense kernel map [O, T], number of sources)
         self._inverse_maps_cache = dict()       # key -> its inverse [O, S] (transposed layers)
+        self._offset_groups_cache = dict()      # key -> offset-group tables of the dense map (False: none)
         self._coordinates_cache = dict()
         self._bounds_cache = dict()
         self.num_map_builds = 0
@@ -110,6 +111,7 @@ class KernelMapCache(object):
         self._swapped_maps_cache.clear()
         self._dense_maps_cache.clear()
         self._inverse_maps_cache.clear()
+        self._offset_groups_cache.clear()
         self._bounds_cache.clear()
 
     def _from_ahead(self, tag, record, coordinates, stride, batch_dims):
@@ -266,6 +268,33 @@ class KernelMapCache(object):
         if not transposed:
             return entry[0]
         return self._inverse_of(key)
+
+    def get_offset_groups(self, source_coordinates: torch.Tensor, source_stride,
+                          source_batch_dims: Optional[torch.Tensor],
+                          target_coordinates: torch.Tensor, target_stride,
+                          target_batch_dims: Optional[torch.Tensor], kernel_size,
+                          kernel_dilation, transposed: bool = False):
+        """The offset-group tables of a layer whose 27 offsets form a 3 x 3 x 3 grid
+        (``_C.OffsetGroups``; None for other kernels and for transposed layers):
+        what the ``offset_groups`` dataflow reads instead of rank tables.  Made
+        from the dense kernel map in three launches; waits for nothing on the
+        device.  Not in the reference, whose kernel map has one row per offset
+        (convolutions.py:147-170)."""
+        if transposed:
+            return None
+        key, stride_key, size_key, dilation_key = self._map_key(
+            source_coordinates.shape[1], source_stride, target_stride, kernel_size, kernel_dilation, False)
+        entry = self._offset_groups_cache.get(key)
+        if entry is None:
+            offsets = self._kernel_offsets(stride_key, size_key, dilation_key)
+            entry = False
+            if offsets.shape == (27, 3) and _C.offset_group_table(offsets) is not None:
+                dense = self.get_dense_kernel_map(source_coordinates, source_stride, source_batch_dims,
+                                                  target_coordinates, target_stride, target_batch_dims,
+                                                  kernel_size, kernel_dilation)
+                entry = _C.kernel_map_offset_groups(dense, offsets) or False
+            self._offset_groups_cache[key] = entry
+        return entry or None
 
     def _inverse_of(self, key) -> torch.Tensor:
         """Dense map of the transposed layer of ``key`` ([O, S]), made on first use."""
@@ -562,23 +591,36 @@ class SparseConv(Module):
         """Times one whole layer per dataflow on the recorded kernel maps (random
         features) and keeps the faster one."""
         best = None
-        for dataflow in ("gather_gemm_scatter", "list_driven", "implicit"):
+        for dataflow in ("gather_gemm_scatter", "list_driven", "implicit", "offset_groups"):
             total = 0.0
             try:
                 for kernel_map in self._tuning_data:
-                    if dataflow == "implicit" and kernel_map.dense is None:
+                    if dataflow in ("implicit", "offset_groups") and kernel_map.dense is None:
                         raise RuntimeError("no dense kernel map")
                     if dataflow == "list_driven" and not kernel_map.ensure_row_lists():
                         raise RuntimeError("no row lists for this kernel map")
                     sources = torch.randn(kernel_map.num_sources, self.in_channels,
                                           device=self.kernel.device).to(self.kernel.dtype)
                     order = kernel_map.kernel_map_order
-                    call = lambda: F.sparse_convolution_forward(
-                        sources=sources, weights=self.kernel, kernel_map=kernel_map,
-                        gather_tile_size=self._tunable_config["gather_tile_size"],
-                        scatter_tile_size=self._tunable_config["scatter_tile_size"],
-                        allow_shortcut_matmul=self._allow_shortcut_matmul and order is not None,
-                        threshold=self._tunable_config["threshold"], dataflow=dataflow)
+                    if dataflow == "offset_groups":
+                        offsets = self._kernel_map_cache._kernel_offsets(
+                            (1,) * self.ndim, self.kernel_size, self.dilation)
+                        groups = None
+                        if (not self.transposed and sources.is_cuda and _C.offset_groups_forward_supported(
+                                self.in_channels, self.out_channels, sources.dtype)):
+                            groups = _C.kernel_map_offset_groups(kernel_map.dense, offsets)
+                        if groups is None:
+                            raise RuntimeError("no offset groups for this layer")
+                        packed = F.pack_weights(self.kernel.detach())
+                        call = lambda: _C.sparse_convolution_forward_groups(
+                            sources, self.kernel.detach(), groups, packed_weights=packed)
+                    else:
+                        call = lambda: F.sparse_convolution_forward(
+                            sources=sources, weights=self.kernel, kernel_map=kernel_map,
+                            gather_tile_size=self._tunable_config["gather_tile_size"],
+                            scatter_tile_size=self._tunable_config["scatter_tile_size"],
+                            allow_shortcut_matmul=self._allow_shortcut_matmul and order is not None,
+                            threshold=self._tunable_config["threshold"], dataflow=dataflow)
                     call()
                     start = torch.cuda.Event(enable_timing=True)
                     stop = torch.cuda.Event(enable_timing=True)
@@ -620,7 +662,8 @@ class SparseConv(Module):
         a small kernel, else a multiple of 16 bytes); 0 where they already are,
         or where that dataflow is not an option."""
         if (features.dtype == torch.float32 or not features.is_cuda
-                or self._tunable_config.get("dataflow", "auto") in ("gather_gemm_scatter", "list_driven")):
+                or self._tunable_config.get("dataflow", "auto") in ("gather_gemm_scatter", "list_driven",
+                                                                     "offset_groups")):
             return 0
         esize = features.element_size()
         row_bytes = self.in_channels * esize
@@ -634,7 +677,7 @@ class SparseConv(Module):
         """Whether this call runs the single-kernel dataflow: forced by the
         tunable ``dataflow``, or chosen where it is the faster one."""
         dataflow = self._tunable_config.get("dataflow", "auto")
-        if dataflow in ("gather_gemm_scatter", "list_driven") or not features.is_cuda:
+        if dataflow in ("gather_gemm_scatter", "list_driven", "offset_groups") or not features.is_cuda:
             return False
         if features.dtype != self.kernel.dtype:
             return False
@@ -642,6 +685,19 @@ class SparseConv(Module):
             return True
         return F.prefers_implicit(self.kernel.shape[0], self.in_channels + pad, self.out_channels,
                                   features.dtype)
+
+    def _takes_offset_groups(self, features: torch.Tensor) -> bool:
+        """Whether this call multiplies its offsets three at a time (the
+        ``offset_groups`` dataflow): forced by the tunable ``dataflow``, or, under
+        ``auto``, for the wide 16-bit 3 x 3 x 3 layers that the single-kernel form
+        does not take, whose product rows are what bounds them."""
+        dataflow = self._tunable_config.get("dataflow", "auto")
+        if dataflow not in ("auto", "offset_groups") or not features.is_cuda or self.transposed:
+            return False
+        if (features.dtype != self.kernel.dtype or self.ndim != 3 or self.kernel.shape[0] != 27
+                or not _C.offset_groups_forward_supported(self.in_channels, self.out_channels, features.dtype)):
+            return False
+        return dataflow == "offset_groups" or self.in_channels * features.element_size() >= 256
 
     def _pointwise(self, features: torch.Tensor, epilogue: Optional[F.Epilogue]) -> torch.Tensor:
         """1x1x1 kernel, stride 1: a plain ``features @ W`` (reference:
@@ -708,10 +764,17 @@ class SparseConv(Module):
             route = self._routes.get(route_key)
             if route is None:
                 pad = self._row_padding(sources)
-                route = (pad, self._takes_implicit(sources, pad))
+                implicit = self._takes_implicit(sources, pad)
+                route = (pad, implicit, not implicit and self._takes_offset_groups(sources))
                 self._routes[route_key] = route
-            pad, implicit = route
-            if implicit and self._tuning_data is None:
+            pad, implicit, grouped = route
+            groups = cache.get_offset_groups(**map_args) if grouped and self._tuning_data is None else None
+            if groups is not None:
+                # offsets multiplied three at a time: needs the dense map and its group tables only
+                weights, packed = self._packed_kernel()
+                features = _C.sparse_convolution_forward_groups(sources, weights, groups, epilogue=epilogue,
+                                                                packed_weights=packed)
+            elif implicit and self._tuning_data is None:
                 # single-kernel dataflow: the dense map is all it needs
                 dense = cache.get_dense_kernel_map(**map_args)
                 if pad:

@@ -92,6 +92,9 @@ SIGNATURES = {
     "mnt_sparse_convolution_forward_rows": (_int, [_i64, _vp, _vp, _pi64, _pi64, _vp, _vp, _vp, _i64, _i64,
                                                    _i64, _i64, _i64, _int, _vp, _vp, _vp, _int, _c.c_float,
                                                    _vp, _vp, _vp]),
+    "mnt_kernel_map_offset_groups": (_int, [_vp, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "mnt_sparse_convolution_forward_groups": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int,
+                                                     _vp, _vp, _vp, _int, _c.c_float, _vp, _vp]),
     "mnt_pack_weights": (_int, [_vp, _i64, _i64, _i64, _int, _vp, _vp]),
     "mnt_sparse_convolution_forward_implicit": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                                                        _int, _vp, _vp, _vp, _int, _c.c_float, _vp,
@@ -1170,6 +1173,112 @@ def sparse_convolution_forward_rows(sources: torch.Tensor, weights: torch.Tensor
             _ptr(ep.residual), ACTIVATION_CODES[ep.activation], float(ep.negative_slope),
             _ptr(packed_weights), _ptr(out), _stream(device)))
     del keep, keep_order
+    return out
+
+
+def offset_group_table(offsets_host: np.ndarray) -> Optional[np.ndarray]:
+    """For a kernel of 27 offsets that form a 3 x 3 x 3 grid (any dilation, any
+    order): int32 ``[3, 9, 3]``, the offset index of member m of group j along
+    axis a, where the groups along an axis are the triples of offsets that
+    differ along that axis only.  None for any other kernel."""
+    offsets = np.asarray(offsets_host, dtype=np.int64)
+    if offsets.shape != (27, 3):
+        return None
+    key = offsets.tobytes()
+    if key in _GROUP_TABLES:
+        return _GROUP_TABLES[key]
+    table = _offset_group_table(offsets)
+    if len(_GROUP_TABLES) > 64:
+        _GROUP_TABLES.clear()
+    _GROUP_TABLES[key] = table
+    return table
+
+
+_GROUP_TABLES = {}
+
+
+def _offset_group_table(offsets: np.ndarray) -> Optional[np.ndarray]:
+    table = np.zeros((3, 9, 3), dtype=np.int32)
+    for axis in range(3):
+        others = [a for a in range(3) if a != axis]
+        rest = offsets[:, others]
+        keys, group_of = np.unique(rest, axis=0, return_inverse=True)
+        group_of = np.asarray(group_of).reshape(-1)
+        if keys.shape[0] != 9:
+            return None
+        for j in range(9):
+            members = np.nonzero(group_of == j)[0]
+            if members.shape[0] != 3 or np.unique(offsets[members, axis]).shape[0] != 3:
+                return None
+            table[axis, j] = members[np.argsort(offsets[members, axis], kind="stable")]
+    return np.ascontiguousarray(table)
+
+
+class OffsetGroups:
+    """The offset-group tables of one dense kernel map (mnt_kernel_map_offset_groups):
+    ``rank`` int32 [9, T], ``src`` int32 [9 * T, 4], ``head`` int32 [16] on the
+    device and the host table ``offsets`` int32 [3, 9, 3] they were built with."""
+
+    def __init__(self, rank, src, head, offsets, num_targets):
+        self.rank, self.src, self.head, self.offsets, self.num_targets = rank, src, head, offsets, num_targets
+        self._offsets_address = offsets.ctypes.data
+
+
+def kernel_map_offset_groups(kernel_map: torch.Tensor, offsets_host: np.ndarray) -> Optional[OffsetGroups]:
+    """Offset groups of a dense int32 kernel map ``[27, T]`` whose offsets form a
+    3 x 3 x 3 grid; None for other kernels.  Waits for nothing on the device."""
+    table = offset_group_table(offsets_host)
+    if table is None or kernel_map.dim() != 2 or kernel_map.shape[0] != 27:
+        return None
+    if kernel_map.dtype != torch.int32:
+        _fail("kernel_map_offset_groups expects an int32 kernel map")
+    device = _common_device([kernel_map])
+    kernel_map = kernel_map.contiguous()
+    T = kernel_map.shape[1]
+    table = np.ascontiguousarray(table)
+    store = torch.empty((9 * T * 5 + 16,), dtype=torch.int32, device=device)
+    src, rank, head = store[:36 * T].view(9 * T, 4), store[36 * T:45 * T].view(9, T), store[45 * T:]
+    with _on(device):
+        _check(load_library().mnt_kernel_map_offset_groups(
+            _ptr(kernel_map), T, table.ctypes.data, _ptr(rank), _ptr(src), _ptr(head), _stream(device)))
+    return OffsetGroups(rank, src, head, table, T)
+
+
+def offset_groups_forward_supported(in_channels: int, out_channels: int, dtype: torch.dtype) -> bool:
+    """Whether mnt_sparse_convolution_forward_groups takes these widths."""
+    return (dtype in (torch.float16, torch.bfloat16) and (in_channels * 2) % 128 == 0
+            and out_channels % 8 == 0)
+
+
+def sparse_convolution_forward_groups(sources: torch.Tensor, weights: torch.Tensor, groups: OffsetGroups,
+                                      epilogue: Optional["Epilogue"] = None,
+                                      packed_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The forward pass over offset groups (mnt_sparse_convolution_forward_groups):
+    ``weights`` [27, Cin, Cout] in the layer's own offset order (``packed_weights``:
+    their :func:`pack_weights` form, made here when missing)."""
+    _ensure_ndim("sources", sources, 2)
+    _ensure_ndim("weights", weights, 3)
+    device = _common_device([sources, weights, groups.rank])
+    fcode = _float_code(_common_dtype([sources, weights]), "sparse_convolution_forward_groups")
+    S, K = sources.shape
+    O, K2, N = weights.shape
+    if K2 != K or O != 27:
+        _fail(f"weights are expected to be [27, {K}, C_out] but found {tuple(weights.shape)}")
+    if not offset_groups_forward_supported(K, N, sources.dtype):
+        _fail(f"the offset-group forward does not take {K} -> {N} channels of {sources.dtype}")
+    T = groups.num_targets
+    ep = Epilogue() if epilogue is None else epilogue.checked(T, N, sources.dtype, device)
+    if packed_weights is None:
+        packed_weights = pack_weights(weights.contiguous())
+    else:
+        _check_packed(packed_weights, weights)
+    sources = sources.contiguous()
+    out = torch.empty((T, N), dtype=sources.dtype, device=device)
+    with _on(device):
+        _check(load_library().mnt_sparse_convolution_forward_groups(
+            _ptr(sources), _ptr(packed_weights), _ptr(groups.rank), _ptr(groups.src), _ptr(groups.head),
+            groups._offsets_address, S, T, K, N, fcode, _ptr(ep.scale), _ptr(ep.shift), _ptr(ep.residual),
+            ACTIVATION_CODES[ep.activation], float(ep.negative_slope), _ptr(out), _stream(device)))
     return out
 
 

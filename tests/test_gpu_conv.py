@@ -897,3 +897,112 @@ def test_bf16_non_finite_features_stay_in_their_rows():
     assert np.isfinite(got[~touched]).all()
     err = np.abs(got[~touched].astype(np.float64) - ref[~touched]).max()
     assert err <= 2e-2 * np.sqrt(np.mean(ref ** 2))
+
+
+def _surface_cloud(seed, n, extent):
+    """Voxels near a few planes and one box: dense along some axes, thin along
+    others, like the levels of a LiDAR scan."""
+    rng = np.random.default_rng(seed)
+    parts = []
+    for axis in (2, 2, 0):
+        pts = rng.integers(0, extent, size=(n // 3, 3))
+        pts[:, axis] = rng.integers(0, extent) + rng.integers(0, 2, size=n // 3)
+        parts.append(pts)
+    parts.append(rng.integers(0, extent // 6, size=(n // 6, 3)) + extent // 3)
+    return np.concatenate(parts).astype(np.int32)
+
+
+@pytest.mark.parametrize("dilation", [1, 2])
+@pytest.mark.parametrize("layout", ["minuet", "torchsparse"])
+def test_offset_group_tables_match_brute_force(dilation, layout):
+    """mnt_kernel_map_offset_groups against plain NumPy on the dense map: the
+    axis with the fewest rows (lowest on a tie), the rows per group, every
+    target's rank inside its groups and every row's three source rows."""
+    from minuet_amd.utils.helpers import generate_kernel_offsets
+    for seed, n, extent in ((1, 9000, 60), (2, 700, 12), (3, 30000, 90)):
+        src, _ = sorted_unique(_surface_cloud(seed, n, extent), None)
+        off = np.ascontiguousarray(generate_kernel_offsets(3, 3, 1, dilation, layout=layout), dtype=np.int64)
+        dense, _ = _C.kernel_map_dense(dev(src), dev(src), off, None, None)
+        groups = _C.kernel_map_offset_groups(dense, off)
+        assert groups is not None
+        table = _C.offset_group_table(off)
+        for axis in range(3):
+            assert sorted(table[axis].reshape(-1).tolist()) == list(range(27))
+            for j in range(9):
+                members = off[table[axis, j]]
+                others = [a for a in range(3) if a != axis]
+                assert (members[:, others] == members[0, others]).all()
+                assert (np.diff(members[:, axis]) > 0).all()
+        m = host(dense)
+        T = m.shape[1]
+        reach = np.stack([[(m[table[a, j]] >= 0).any(0) for j in range(9)] for a in range(3)])   # [3, 9, T]
+        totals = reach.sum((1, 2))
+        axis = int(np.argmin(totals))
+        head = host(groups.head)
+        assert head[0] == axis
+        np.testing.assert_array_equal(head[1:10], reach[axis].sum(1))
+        rank, rows = host(groups.rank), host(groups.src)
+        for j in range(9):
+            hit = reach[axis, j]
+            np.testing.assert_array_equal(rank[j], np.where(hit, np.cumsum(hit) - 1, -1))
+            expect = m[table[axis, j]][:, hit].T                                # [rows, 3]
+            np.testing.assert_array_equal(rows[j * T:j * T + expect.shape[0], :3], expect)
+
+
+@pytest.mark.parametrize("kind", ["fp16", "bf16"])
+@pytest.mark.parametrize("cin,cout,n,extent", [(128, 128, 9000, 60), (256, 256, 3000, 30), (64, 64, 5000, 40),
+                                               (128, 256, 4000, 40), (192, 72, 2500, 30), (256, 128, 700, 12)])
+def test_forward_offset_groups(kind, cin, cout, n, extent):
+    """The forward pass over offset groups against the float64 oracle, with and
+    without an epilogue, and against the three-kernel dataflow."""
+    rng = np.random.default_rng(5)
+    src, _ = sorted_unique(_surface_cloud(7, n, extent), None)
+    off = orc.generate_kernel_offsets(3, 3, 1, 1)
+    feats = quantise(rng.normal(size=(src.shape[0], cin)), kind)
+    weights = quantise(rng.normal(size=(27, cin, cout)) / np.sqrt(27 * cin), kind)
+    esm, etm, eorder, esizes, _ = orc.build_kernel_map(src, None, src, None, off, reorder=True)
+    ref = orc.sparse_convolution_forward(feats, weights, esm, etm, eorder, esizes)
+    dtype = TORCH[kind]
+    f_dev, w_dev = dev(feats).to(dtype), dev(weights).to(dtype)
+    dense, _ = _C.kernel_map_dense(dev(src), dev(src), off.astype(np.int64), None, None)
+    groups = _C.kernel_map_offset_groups(dense, off.astype(np.int64))
+    out = _C.sparse_convolution_forward_groups(f_dev, w_dev, groups)
+    assert out.dtype == dtype and out.shape == ref.shape
+    assert_features_close(out, ref, kind)
+    again = _C.sparse_convolution_forward_groups(f_dev, w_dev, groups, packed_weights=F.pack_weights(w_dev))
+    assert torch.equal(again, out)                                   # no atomics: reruns are bit-equal
+    scale = rng.uniform(0.5, 1.5, size=cout).astype(np.float32)
+    shift = rng.uniform(-0.5, 0.5, size=cout).astype(np.float32)
+    residual = quantise(rng.normal(size=ref.shape), kind)
+    fused_ref = np.maximum(ref * scale.astype(np.float64) + shift.astype(np.float64) + residual, 0.0)
+    fused = _C.sparse_convolution_forward_groups(
+        f_dev, w_dev, groups, epilogue=F.Epilogue(dev(scale), dev(shift), dev(residual).to(dtype), "relu"))
+    got = host(fused.float()).astype(np.float64)
+    # the bound is taken from the sums before the ReLU, whose rounding it covers
+    pre = ref * scale.astype(np.float64) + shift.astype(np.float64) + residual
+    assert np.abs(got - fused_ref).max() <= 2e-2 * np.sqrt(np.mean(pre ** 2))
+
+
+@pytest.mark.parametrize("kind", ["fp16", "bf16"])
+def test_module_takes_offset_groups_for_wide_layers(kind):
+    """A 128 -> 128 3x3x3 layer under ``dataflow="auto"`` runs over offset groups
+    (the cache then builds the dense map and the group tables only) and agrees
+    with the same layer forced through Gather-GEMM-Scatter."""
+    dtype = TORCH[kind]
+    src, _ = sorted_unique(_surface_cloud(9, 8000, 50), None)
+    conv = minuet.nn.SparseConv3d(128, 128, 3, dtype=dtype, device="cuda")
+    x = minuet.SparseTensor(torch.randn(src.shape[0], 128, device="cuda").to(dtype), dev(src))
+    with torch.no_grad():
+        cache = minuet.nn.KernelMapCache(3, torch.int32, "cuda")
+        conv.set_kernel_map_cache(cache)
+        auto = conv(x).F
+        assert len(cache._offset_groups_cache) == 1 and not cache._kernel_maps_cache
+        conv.tunable_config["dataflow"] = "gather_gemm_scatter"
+        conv._routes.clear()
+        three = conv(x).F
+        assert len(cache._kernel_maps_cache) == 1
+    # two roundings of the same sums: 2e-2 of the RMS, or one unit in the last
+    # place of the largest value where that is more (bf16 keeps 8 bits)
+    diff = (auto.float() - three.float()).abs().max().item()
+    ulp = three.float().abs().max().item() * 2.0 ** (-7 if kind == "bf16" else -10)
+    assert diff <= max(2e-2 * three.float().pow(2).mean().sqrt().item(), ulp), diff
