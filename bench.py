@@ -253,8 +253,11 @@ def layer_stages(device, config, channels, kernel_size, dtype_name, tune=False):
                                       # rows in and out of the buffers: what bounds it at small widths
                                       **{"hbm_" + k: v for k, v in hbm(2 * nnz * channels * esize, gemm_ms).items()
                                          if k != "ms"}}
-        for flow in ("gather_gemm_scatter", "list_driven", "implicit"):
+        for flow in ("gather_gemm_scatter", "list_driven", "implicit", "offset_groups"):
             if flow == "implicit" and not _C.implicit_forward_supported(channels, channels, dtype):
+                continue
+            if flow == "offset_groups" and not (conv.kernel.shape[0] == 27 and _C.offset_groups_forward_supported(
+                    channels, channels, dtype)):
                 continue
             conv.tunable_config["dataflow"] = flow
             if flow == "list_driven":

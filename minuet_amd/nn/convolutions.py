@@ -763,9 +763,9 @@ class SparseConv(Module):
             route_key = (sources.dtype, sources.is_cuda, self._tunable_config.get("dataflow", "auto"))
             route = self._routes.get(route_key)
             if route is None:
-                pad = self._row_padding(sources)
-                implicit = self._takes_implicit(sources, pad)
-                route = (pad, implicit, not implicit and self._takes_offset_groups(sources))
+                grouped = self._takes_offset_groups(sources)
+                pad = 0 if grouped else self._row_padding(sources)
+                route = (pad, not grouped and self._takes_implicit(sources, pad), grouped)
                 self._routes[route_key] = route
             pad, implicit, grouped = route
             groups = cache.get_offset_groups(**map_args) if grouped and self._tuning_data is None else None
