@@ -233,6 +233,77 @@ __global__ __launch_bounds__(256) void scatter_wide_kernel(const TB *__restrict_
   finish_row<T, V, E, NV>(acc, ep, t, channels, lr, lanes_per_row, dst, unscale);
 }
 
+// Scatter for kernel maps of at most MAXO rank rows (offset groups, 2 x 2 x 2
+// kernels): one lane group per target reads its MAXO rank entries in one trip
+// and all of its buffer rows in a second one, sums them in row order in fp32
+// and writes the target once; no row list, no barrier.
+template <typename TB, typename T, int VB, int NV, typename IT, int MAXO>
+__global__ __launch_bounds__(256) void scatter_few_kernel(const TB *__restrict__ buffer,
+                                                          unsigned char *__restrict__ targets,
+                                                          const IT *__restrict__ target_masks,
+                                                          const int *__restrict__ row_start,
+                                                          long long num_targets, int num_offsets,
+                                                          int channels, int lanes_per_row,
+                                                          const TB *__restrict__ direct, Epilogue ep) {
+  typedef typename VecOf<VB>::type V;
+  const float unscale = 1.0f / range_scale(ep.range);            // every lane is still here
+  constexpr int E = VB / static_cast<int>(sizeof(T));
+  constexpr int BB = E * static_cast<int>(sizeof(TB));          // buffer bytes per vector
+  typedef typename VecOf<(BB > 16 ? 16 : BB)>::type BV;
+  constexpr int NBV = BB > 16 ? BB / 16 : 1;
+  const long long gtid = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const long long t = gtid / lanes_per_row;
+  const int lr = static_cast<int>(gtid % lanes_per_row);
+  if (t >= num_targets) return;
+  int d[MAXO];
+#pragma unroll
+  for (int j = 0; j < MAXO; ++j) {
+    d[j] = j < num_offsets ? static_cast<int>(target_masks[static_cast<long long>(j) * num_targets + t]) : -1;
+  }
+  BV first[NV][NBV];
+  if (direct != nullptr) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const TB *piece = direct + t * channels + (lr + i * lanes_per_row) * E;
+#pragma unroll
+      for (int v = 0; v < NBV; ++v) first[i][v] = reinterpret_cast<const BV *>(piece)[v];
+    }
+  }
+  BV raw[MAXO][NV][NBV];
+#pragma unroll
+  for (int j = 0; j < MAXO; ++j) {
+    if (d[j] >= 0) {
+      const TB *src = buffer + (static_cast<long long>(row_start[j]) + d[j]) * channels;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const TB *piece = src + (lr + i * lanes_per_row) * E;
+#pragma unroll
+        for (int v = 0; v < NBV; ++v) raw[j][i][v] = reinterpret_cast<const BV *>(piece)[v];
+      }
+    }
+  }
+  float acc[NV][E];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const TB *e = reinterpret_cast<const TB *>(first[i]);
+#pragma unroll
+    for (int k = 0; k < E; ++k) acc[i][k] = direct != nullptr ? to_float(e[k]) : 0.0f;
+  }
+#pragma unroll
+  for (int j = 0; j < MAXO; ++j) {
+    if (d[j] >= 0) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const TB *e = reinterpret_cast<const TB *>(raw[j][i]);
+#pragma unroll
+        for (int k = 0; k < E; ++k) acc[i][k] += to_float(e[k]);
+      }
+    }
+  }
+  unsigned char *dst = targets + t * channels * static_cast<long long>(sizeof(T));
+  finish_row<T, V, E, NV>(acc, ep, t, channels, lr, lanes_per_row, dst, unscale);
+}
+
 // Scatter in two phases per workgroup of `tile_targets` (a power of two)
 // consecutive targets.
 //   1. Listing: thread (part, target) reads its share of the target's rank
@@ -248,6 +319,7 @@ __global__ __launch_bounds__(256) void scatter_wide_kernel(const TB *__restrict_
 // no rank table.  Dynamic LDS: (num_offsets + 256 / tile_targets) * tile_targets
 // ints.
 constexpr int kScatterBlock = 256;
+constexpr int kScatterFewOffsets = 9;   // rank rows that scatter_few_kernel keeps in flight at once
 
 template <typename TB, typename T, int VB, int NV, typename IT>
 __global__ __launch_bounds__(kScatterBlock) void scatter_kernel(
@@ -1185,6 +1257,31 @@ static void launch_scatter(const LaneShape &sh, const TB *buffer, void *targets,
                            const int *row_start, int64_t num_targets, int num_offsets, int channels,
                            const TB *direct, const Epilogue &ep, hipStream_t stream) {
   if (num_targets == 0) return;
+  if (num_offsets <= kScatterFewOffsets && sh.nv <= 2 && sizeof(TB) <= sizeof(T)) {
+    const unsigned few_grid = static_cast<unsigned>(div_ceil(num_targets * sh.lanes_per_row, 256));
+#define MNT_F(VB, NV)                                                                                          \
+  scatter_few_kernel<TB, T, VB, NV, IT, kScatterFewOffsets><<<few_grid, 256, 0, stream>>>(                      \
+      buffer, static_cast<unsigned char *>(targets), masks, row_start, num_targets, num_offsets, channels,     \
+      sh.lanes_per_row, direct, ep)
+#define MNT_FV(VB)       \
+  if (sh.nv == 1) {      \
+    MNT_F(VB, 1);        \
+  } else {               \
+    MNT_F(VB, 2);        \
+  }
+    if (sh.vb == 16) {
+      MNT_FV(16);
+      check_launch("scatter_few_kernel");
+      return;
+    }
+    if (sh.vb == 8) {
+      MNT_FV(8);
+      check_launch("scatter_few_kernel");
+      return;
+    }
+#undef MNT_FV
+#undef MNT_F
+  }
   const bool listed = num_offsets <= kScatterListedOffsets && sh.lanes_per_row <= kScatterBlock;
   // 64 targets per workgroup (32 for large kernels, so that the row lists fit
   // in LDS); fewer when that would leave most of the chip without a workgroup,

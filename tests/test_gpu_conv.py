@@ -984,13 +984,15 @@ def test_forward_offset_groups(kind, cin, cout, n, extent):
 
 
 @pytest.mark.parametrize("kind", ["fp16", "bf16"])
-def test_module_takes_offset_groups_for_wide_layers(kind):
+@pytest.mark.parametrize("stride,n,extent", [(1, 8000, 50), (2, 6000, 40), (1, 40, 6), (1, 1, 6)])
+def test_module_takes_offset_groups_for_wide_layers(kind, stride, n, extent):
     """A 128 -> 128 3x3x3 layer under ``dataflow="auto"`` runs over offset groups
     (the cache then builds the dense map and the group tables only) and agrees
-    with the same layer forced through Gather-GEMM-Scatter."""
+    with the same layer forced through Gather-GEMM-Scatter; also strided (fewer
+    targets than sources) and on clouds smaller than a tile."""
     dtype = TORCH[kind]
-    src, _ = sorted_unique(_surface_cloud(9, 8000, 50), None)
-    conv = minuet.nn.SparseConv3d(128, 128, 3, dtype=dtype, device="cuda")
+    src, _ = sorted_unique(_surface_cloud(9, max(n, 6), extent)[:n], None)
+    conv = minuet.nn.SparseConv3d(128, 128, 3, stride=stride, dtype=dtype, device="cuda")
     x = minuet.SparseTensor(torch.randn(src.shape[0], 128, device="cuda").to(dtype), dev(src))
     with torch.no_grad():
         cache = minuet.nn.KernelMapCache(3, torch.int32, "cuda")
