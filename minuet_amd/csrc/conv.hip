@@ -1098,58 +1098,63 @@ __global__ __launch_bounds__(kGroupTile) void group_count_kernel(const int *__re
 
 __global__ __launch_bounds__(1024) void group_scan_kernel(int *__restrict__ tile_counts, int tiles,
                                                            int *__restrict__ head) {
-  __shared__ int s_part[1024 / kWave];
-  __shared__ int s_axis_total[3];
-  __shared__ int s_carry;
+  constexpr int kWaves = 1024 / kWave;
+  constexpr int kBatch = 8;                          // loads a lane keeps in flight
+  __shared__ int s_part[3][kWaves];
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-  auto block_sum = [&](int v) {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
-    __syncthreads();
-    if (lane == 0) s_part[wave] = v;
-    __syncthreads();
-    int sum = 0;
-    for (int w = 0; w < 1024 / kWave; ++w) sum += s_part[w];
-    return sum;
-  };
+  // totals per axis: every lane adds up a strided share, kBatch loads at a time
+  const int per_axis = kGroupCount * tiles;
   for (int axis = 0; axis < 3; ++axis) {
+    const int *counts = tile_counts + axis * per_axis;
     int mine = 0;
-    for (int i = tid; i < kGroupCount * tiles; i += 1024) mine += tile_counts[axis * kGroupCount * tiles + i];
-    const int total = block_sum(mine);
-    if (tid == 0) s_axis_total[axis] = total;
+    for (int base = tid; base < per_axis; base += kBatch * 1024) {
+      int v[kBatch];
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) v[k] = base + k * 1024 < per_axis ? counts[base + k * 1024] : 0;
+#pragma unroll
+      for (int k = 0; k < kBatch; ++k) mine += v[k];
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) mine += __shfl_xor(mine, d);
+    if (lane == 0) s_part[axis][wave] = mine;
   }
   __syncthreads();
+  int total[3] = {0, 0, 0};
+#pragma unroll
+  for (int axis = 0; axis < 3; ++axis) {
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) total[axis] += s_part[axis][w];
+  }
   int axis = 0;
-  if (s_axis_total[1] < s_axis_total[axis]) axis = 1;
-  if (s_axis_total[2] < s_axis_total[axis]) axis = 2;
+  if (total[1] < total[axis]) axis = 1;
+  if (total[2] < total[axis]) axis = 2;
   if (tid == 0) head[0] = axis;
-  // exclusive prefixes of the winning axis' tile counts, group by group
-  int *counts = tile_counts + axis * kGroupCount * tiles;
-  for (int j = 0; j < kGroupCount; ++j) {
-    if (tid == 0) s_carry = 0;
-    __syncthreads();
-    for (int base = 0; base < tiles; base += 1024) {
-      const int i = base + tid;
-      const int v = i < tiles ? counts[j * tiles + i] : 0;
-      int scan = v;                                              // inclusive scan inside the wavefront
+  // exclusive prefixes of the winning axis' tile counts: a wavefront per group,
+  // kBatch x 64 counts fetched at a time and scanned in registers
+  if (wave >= kGroupCount) return;
+  int *counts = tile_counts + (axis * kGroupCount + wave) * tiles;
+  int carry = 0;
+  for (int base = 0; base < tiles; base += kBatch * kWave) {
+    int v[kBatch];
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) {
+      const int i = base + k * kWave + lane;
+      v[k] = i < tiles ? counts[i] : 0;
+    }
+#pragma unroll
+    for (int k = 0; k < kBatch; ++k) {
+      int scan = v[k];                                           // inclusive scan inside the wavefront
 #pragma unroll
       for (int d = 1; d < kWave; d <<= 1) {
         const int up = __shfl_up(scan, d);
         if (lane >= d) scan += up;
       }
-      __syncthreads();
-      if (lane == kWave - 1) s_part[wave] = scan;
-      __syncthreads();
-      int before = s_carry;
-      for (int w = 0; w < wave; ++w) before += s_part[w];
-      if (i < tiles) counts[j * tiles + i] = before + scan - v;
-      __syncthreads();
-      if (tid == 1023) s_carry = before + scan;
-      __syncthreads();
+      const int i = base + k * kWave + lane;
+      if (i < tiles) counts[i] = carry + scan - v[k];
+      carry += __builtin_amdgcn_readlane(scan, kWave - 1);
     }
-    if (tid == 0) head[1 + j] = s_carry;
-    __syncthreads();
   }
+  if (lane == 0) head[1 + wave] = carry;
 }
 
 __global__ __launch_bounds__(kGroupTile) void group_emit_kernel(const int *__restrict__ dense,
