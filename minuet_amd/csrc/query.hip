@@ -1996,12 +1996,13 @@ extern "C" int mnt_sorted_kernel_map_lists(const void *coords, int64_t n, int nd
       buf.partial = scope.alloc<long long>(128 * 8);
       buf.folded = scope.alloc<long long>(2 * MNT_MAX_NDIM);
       // bucket totals, cursors, the copies of the hits per offset, the equal-rows flag
-      buf.counter_words = 2 * buckets + kMaxTotalCopies * kPlanMaxOffsets + 1;
+      // (and the sort's status words, which must start at zero like the rest)
+      buf.counter_words = 2 * buckets + kMaxTotalCopies * kPlanMaxOffsets + 1 + 4;
       buf.counters = scope.alloc<unsigned>(buf.counter_words);
       buf.info = scope.alloc<unsigned>(4);
-      buf.status = scope.alloc<unsigned>(4);
+      buf.status = buf.counters + (buf.counter_words - 4);
       buf.chunks = scope.alloc<uint4>(chain_sort_max_pairs(n));
-      buf.words = scope.alloc<unsigned long long>(n);
+      buf.words = scope.alloc<unsigned long long>(chain_sort_words(n));
       buf.plan = scope.alloc<DevicePlan>(1);
       unsigned *row_totals = buf.counters + 2 * buckets;
       int *stage = scope.alloc<int>(static_cast<size_t>(num_offsets) * n);

@@ -48,10 +48,11 @@ struct ChainSortBuffers {
   unsigned *counters;
   int counter_words;
   unsigned *info;                // [4]
-  unsigned *status;              // [4]: [0] set by the dealing kernel (non-zero: the sort declined),
-                                 // [2] number of (bucket, chunk) pairs of the ranking launch
+  unsigned *status;              // [4], inside `counters` (zero when the dealing kernel starts): [0] non-zero:
+                                 // the sort declined, [2] (bucket, chunk) pairs of the ranking launch
+                                 // (histogram form only)
   uint4 *chunks;                 // [chain_sort_max_pairs(n)]
-  unsigned long long *words;     // [n]
+  unsigned long long *words;     // [chain_sort_words(n)]
   DevicePlan *plan;              // query plan written by the ranking launch (nullable)
 };
 
@@ -62,6 +63,9 @@ bool chain_sort_takes(int64_t n, int64_t num_batches, int num_offsets);
 // (bucket, chunk) pairs its ranking launch can have.
 int chain_sort_msd_bits(int64_t n);
 int64_t chain_sort_max_pairs(int64_t n);
+// Words of ChainSortBuffers::words the chain needs for n rows (a slab per
+// bucket when the dealing launch works without a histogram).
+size_t chain_sort_words(int64_t n);
 // Enqueues bounds -> histogram -> dealing -> ranking (int32 permutation and
 // sorted rows); the ranking launch also writes the query plan for `offsets`.
 void enqueue_chain_sort(const void *coords, int64_t n, int ndim, int coord_dtype, int32_t *indices_out,

@@ -7,6 +7,7 @@
 #include "sort.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <vector>
 
 #include "device_utils.h"
@@ -1296,7 +1297,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_rank_chain_kernel(
     const unsigned long long *__restrict__ words, const uint4 *__restrict__ chunks,
     const unsigned *__restrict__ pair_count, int max_pairs, const long long *__restrict__ folded,
     int ndim, int msd_cap, int idx_bits, const unsigned *__restrict__ status, FinalSink<CT, IT> sink,
-    OffsetTable offsets, int num_offsets, DevicePlan *__restrict__ plan_out) {
+    OffsetTable offsets, int num_offsets, DevicePlan *__restrict__ plan_out, int slabs) {
   __shared__ __align__(16) unsigned long long s_words[kChainBucketCap + 128];
   __shared__ RankShared sh;
   const unsigned declined = status[0];
@@ -1320,7 +1321,191 @@ __global__ __launch_bounds__(kSortBlock) void bucket_rank_chain_kernel(
   const int key_bits = single_round_spec(bounds, ndim, 1, spec);
   const BucketLayout lay = bucket_layout(key_bits, msd_cap, idx_bits);
   const KeySink<CT, IT> key_sink{spec, sink.indices, sink.sorted};
-  rank_bucket_chunk<CT, IT>(words, entry, idx_bits, lay.shift + idx_bits, key_sink, s_words, sh);
+  // rank_bucket_chunk reads a bucket's words at words[first output row + i]: with a
+  // slab per bucket (slabs != 0) they sit at the start of the bucket's slab instead
+  const unsigned long long *from =
+      slabs != 0 ? words + static_cast<size_t>(entry.z) * kChainBucketCap - entry.x : words;
+  rank_bucket_chunk<CT, IT>(from, entry, idx_bits, lay.shift + idx_bits, key_sink, s_words, sh);
+}
+
+// The chain without its histogram launch.  The dealing launch needs to know
+// where a bucket starts only because buckets are packed end to end; when every
+// bucket gets a slab of kChainBucketCap words of its own (the most the ranking
+// launch takes anyway), a row's place is its bucket's slab plus what the
+// bucket's cursor says, and the cursors, which start at zero, end up as the
+// bucket totals.  The dealing launch then folds the bounds itself (what the
+// histogram launch did), and a one-workgroup launch turns the totals into the
+// ranking launch's list of (bucket, chunk) pairs (every ranking workgroup doing
+// that scan for itself was measured: 16 us more on 2 800 workgroups).  A slab
+// that would overflow raises status[0] (which starts at zero) like a bad key
+// layout does, and the caller takes the separate sort.
+template <typename CT, typename IT, int kBucketItems>
+__global__ __launch_bounds__(kSortBlock) void bucket_deal_slab_kernel(
+    const CT *__restrict__ coords, int ndim, long long n, const long long *__restrict__ partial,
+    int num_partials, int msd_cap, int idx_bits_, unsigned *__restrict__ cursors,
+    unsigned *__restrict__ status, long long *__restrict__ bounds_out,
+    unsigned long long *__restrict__ slabs) {
+  extern __shared__ __align__(16) unsigned s_deal[];
+  const int tid = threadIdx.x;
+  unsigned *s_hist = s_deal;
+  // the rows first: their loads wait for nothing
+  const long long base = static_cast<long long>(blockIdx.x) * (kSortBlock * kBucketItems);
+  CT c[kBucketItems][MNT_MAX_NDIM];
+#pragma unroll
+  for (int r = 0; r < kBucketItems; ++r) {
+    const long long i = base + r * kSortBlock + tid;
+    load_row_raw<CT>(coords + (i < n ? i : n - 1) * ndim, ndim, c[r]);
+  }
+  long long bounds[2 * MNT_MAX_NDIM];
+  fold_bounds(partial, num_partials, bounds);
+  if (blockIdx.x == 0 && tid == 0) {
+#pragma unroll
+    for (int slot = 0; slot < 2 * MNT_MAX_NDIM; ++slot) bounds_out[slot] = bounds[slot];
+  }
+  CoordSource<CT, IT> src;
+  const BucketLayout lay = layout_on_device<CT, IT>(coords, nullptr, 1, ndim, bounds, msd_cap, idx_bits_, src);
+  if (!lay.ok) {                                 // the same verdict in every workgroup
+    if (blockIdx.x == 0 && tid == 0) status[0] = 1u;
+    return;
+  }
+  const int buckets = 1 << lay.msd_bits;
+  for (int d = tid; d < buckets; d += kSortBlock) s_hist[d] = 0;
+  __syncthreads();
+  const int shift = lay.shift, idx_bits = lay.idx_bits;
+  const unsigned long long rest_mask = (1ull << shift) - 1ull;
+  unsigned long long key[kBucketItems];
+  unsigned row[kBucketItems], place[kBucketItems];
+#pragma unroll
+  for (int r = 0; r < kBucketItems; ++r) {
+    const long long i = base + r * kSortBlock + tid;
+    src.pack(i, c[r], key[r], row[r]);
+    place[r] = 0;
+    if (i < n) place[r] = atomicAdd(&s_hist[static_cast<unsigned>(key[r] >> shift)], 1u);
+  }
+  __syncthreads();
+  // a range of every bucket this tile has rows for
+  constexpr int kPer = kBucketMax / kSortBlock;
+  unsigned count[kPer], got[kPer];
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int d = j * kSortBlock + tid;
+    count[j] = d < buckets ? s_hist[d] : 0u;
+  }
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int d = j * kSortBlock + tid;
+    got[j] = 0;
+    if (count[j] != 0) got[j] = atomicAdd(&cursors[d], count[j]);
+  }
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int d = j * kSortBlock + tid;
+    if (count[j] != 0) s_hist[d] = got[j];
+  }
+  __syncthreads();
+  bool over = false;
+#pragma unroll
+  for (int r = 0; r < kBucketItems; ++r) {
+    const long long i = base + r * kSortBlock + tid;
+    if (i < n) {
+      const unsigned bucket = static_cast<unsigned>(key[r] >> shift);
+      const unsigned pos = s_hist[bucket] + place[r];
+      if (pos < static_cast<unsigned>(kChainBucketCap)) {
+        slabs[static_cast<size_t>(bucket) * kChainBucketCap + pos] =
+            ((key[r] & rest_mask) << idx_bits) | static_cast<unsigned long long>(row[r]);
+      } else {
+        over = true;
+      }
+    }
+  }
+  if (over) status[0] = 1u;
+}
+
+// One workgroup between the dealing and the ranking launch of the slab form:
+// from counts[d] = rows of bucket d (the dealing launch's cursors) the list of
+// (bucket, chunk) pairs of the ranking launch, numbered as bucket_scan_kernel
+// numbers them (the chunks of buckets that several workgroups share first:
+// they run longest), and their number in status[2].
+__global__ __launch_bounds__(1024) void bucket_pairs_kernel(const unsigned *__restrict__ counts, int buckets,
+                                                            uint4 *__restrict__ chunks,
+                                                            unsigned *__restrict__ status) {
+  constexpr int kPer = kBucketMax / 1024;
+  __shared__ unsigned long long wave_both[1024 / kWave];
+  __shared__ unsigned wave_shared[1024 / kWave];
+  const int t = threadIdx.x;
+  const int per = (buckets + 1023) / 1024;    // consecutive buckets of one thread
+  unsigned v[kPer];
+  unsigned sum = 0, singles = 0, shared = 0;
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int d = t * per + j;
+    v[j] = j < per && d < buckets ? counts[d] : 0u;
+    sum += v[j];
+    const unsigned mine = bucket_pieces(v[j]);
+    singles += mine == 1 ? 1u : 0u;
+    shared += mine > 1 ? mine : 0u;
+  }
+  if (status[0] != 0) return;                 // declined (a slab overflowed): the counts mean nothing
+  const unsigned long long mine_both =
+      static_cast<unsigned long long>(sum) | (static_cast<unsigned long long>(singles) << 32);
+  unsigned long long inclusive = mine_both;
+  unsigned shared_inclusive = shared;
+  for (int off = 1; off < kWave; off <<= 1) {
+    const unsigned long long u = __shfl_up(inclusive, off);
+    const unsigned u2 = __shfl_up(shared_inclusive, off);
+    if (static_cast<int>(lane_id()) >= off) {
+      inclusive += u;
+      shared_inclusive += u2;
+    }
+  }
+  if (lane_id() == kWave - 1) {
+    wave_both[t >> 6] = inclusive;
+    wave_shared[t >> 6] = shared_inclusive;
+  }
+  __syncthreads();
+  unsigned long long before = 0, all_both = 0;
+  unsigned shared_before = 0, all_shared = 0;
+#pragma unroll
+  for (int w = 0; w < 1024 / kWave; ++w) {
+    const unsigned long long x = wave_both[w];
+    const unsigned x2 = wave_shared[w];
+    before += w < (t >> 6) ? x : 0ull;
+    shared_before += w < (t >> 6) ? x2 : 0u;
+    all_both += x;
+    all_shared += x2;
+  }
+  const unsigned long long exclusive = before + inclusive - mine_both;
+  unsigned run = static_cast<unsigned>(exclusive);
+  unsigned shared_at = shared_before + shared_inclusive - shared;
+  unsigned single_at = all_shared + static_cast<unsigned>(exclusive >> 32);
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int d = t * per + j;
+    if (j < per && d < buckets) {
+      const unsigned mine = bucket_pieces(v[j]);
+      const unsigned head = v[j] | (bucket_mode(v[j]) << 13);
+      if (mine == 1) chunks[single_at++] = make_uint4(run, head, d, 0u);
+      for (unsigned c = 0; mine > 1 && c < mine; ++c) {
+        chunks[shared_at++] = make_uint4(run, head | (c << 16), d, 0u);
+      }
+    }
+    run += v[j];
+  }
+  if (t == 0) status[2] = all_shared + static_cast<unsigned>(all_both >> 32);
+}
+
+static bool chain_slabs_enabled() {
+  static const bool on = [] {
+    const char *text = std::getenv("MINUET_CHAIN_SLABS");
+    return text == nullptr || std::atoi(text) != 0;
+  }();
+  return on;
+}
+
+size_t chain_sort_words(int64_t n) {
+  const size_t packed = static_cast<size_t>(n);
+  if (!chain_slabs_enabled()) return packed;
+  return std::max(packed, (static_cast<size_t>(1) << chain_sort_msd_bits(n)) * kChainBucketCap);
 }
 
 bool chain_sort_takes(int64_t n, int64_t num_batches, int num_offsets) {
@@ -1344,6 +1529,29 @@ static void enqueue_chain_sort_typed(const CT *coords, int64_t n, int ndim, int3
   const unsigned tiles = static_cast<unsigned>(div_ceil(n, kSortBlock * (large ? 16 : 4)));
   unsigned *totals = buf.counters;
   unsigned *cursors = buf.counters + buckets;
+  if (chain_slabs_enabled()) {
+    // status starts at zero: it sits in the counters that bounds_kernel clears
+    const size_t lds = sizeof(unsigned) * static_cast<size_t>(buckets);
+    if (large) {
+      bucket_deal_slab_kernel<CT, int32_t, 16><<<tiles, kSortBlock, lds, stream>>>(
+          coords, ndim, n, buf.partial, num_partials, msd_cap, idx_bits, cursors, buf.status, buf.folded, buf.words);
+    } else {
+      bucket_deal_slab_kernel<CT, int32_t, 4><<<tiles, kSortBlock, lds, stream>>>(
+          coords, ndim, n, buf.partial, num_partials, msd_cap, idx_bits, cursors, buf.status, buf.folded, buf.words);
+    }
+    check_launch("bucket_deal_slab_kernel");
+    profile_mark("sort_deal", stream);
+    bucket_pairs_kernel<<<1, 1024, 0, stream>>>(cursors, buckets, buf.chunks, buf.status);
+    check_launch("bucket_pairs_kernel");
+    profile_mark("sort_pairs", stream);
+    const int max_pairs = static_cast<int>(chain_sort_max_pairs(n));
+    bucket_rank_chain_kernel<CT, int32_t><<<max_pairs + 1, kSortBlock, 0, stream>>>(
+        buf.words, buf.chunks, buf.status + 2, max_pairs, buf.folded, ndim, msd_cap, idx_bits, buf.status,
+        FinalSink<CT, int32_t>{coords, ndim, indices_out, sorted_out}, offsets, num_offsets, buf.plan, 1);
+    check_launch("bucket_rank_chain_kernel");
+    profile_mark("sort_rank", stream);
+    return;
+  }
   if (large) {
     bucket_hist_kernel<CT, int32_t, 16><<<tiles, kSortBlock, 0, stream>>>(
         coords, nullptr, 1, ndim, n, buf.partial, num_partials, msd_cap, idx_bits, totals, buf.info, buf.folded);
@@ -1366,7 +1574,7 @@ static void enqueue_chain_sort_typed(const CT *coords, int64_t n, int ndim, int3
   const int max_pairs = static_cast<int>(chain_sort_max_pairs(n));
   bucket_rank_chain_kernel<CT, int32_t><<<max_pairs + 1, kSortBlock, 0, stream>>>(
       buf.words, buf.chunks, buf.status + 2, max_pairs, buf.folded, ndim, msd_cap, idx_bits, buf.status,
-      FinalSink<CT, int32_t>{coords, ndim, indices_out, sorted_out}, offsets, num_offsets, buf.plan);
+      FinalSink<CT, int32_t>{coords, ndim, indices_out, sorted_out}, offsets, num_offsets, buf.plan, 0);
   check_launch("bucket_rank_chain_kernel");
   profile_mark("sort_rank", stream);
 }
