@@ -294,10 +294,10 @@ int mnt_kernel_map_lists(const void *sources, int64_t num_sources,
  * device and on the host).  bounds_host_out (8 x int64) receives the
  * coordinate minima [0..3] and maxima [4..7].
  * For clouds of 2 048 .. 2 097 152 rows and up to 64 offsets the whole step is
- * a chain of six launches (bounds, bucket histogram, dealing, ranking, query,
- * list placing) that never returns to the host in between: key layouts, bucket
- * starts and the query plan are worked out on the device, and the host waits
- * once, for the sizes.  Offsets that come in pairs d / -d are looked up once
+ * a chain of six launches (bounds, dealing into a slab per bucket, listing the
+ * ranking work, ranking, query, list placing) that never returns to the host
+ * in between: key layouts, bucket totals and the query plan are worked out on
+ * the device, and the host waits once, for the sizes.  Offsets that come in pairs d / -d are looked up once
  * per pair there: a cloud mapped onto itself has the pair list of -d equal to
  * the pair list of d with the two indices exchanged, in the same order.  A
  * cloud the chain declines (a bucket beyond 4 096 rows, keys that do not fit

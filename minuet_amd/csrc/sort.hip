@@ -1583,7 +1583,12 @@ static void enqueue_chain_sort_typed(const CT *coords, int64_t n, int ndim, int3
 int64_t chain_sort_max_pairs(int64_t n) { return (int64_t(1) << chain_sort_msd_bits(n)) + n / kSortBlock + 1; }
 
 int chain_sort_msd_bits(int64_t n) {
-  return std::max(1, std::min(kBucketMaxBits, bit_width(static_cast<unsigned long long>(n / kBucketRows))));
+  static const int rows = [] {
+    const char *text = std::getenv("MINUET_CHAIN_BUCKET_ROWS");
+    const int v = text != nullptr ? std::atoi(text) : 0;
+    return v >= 16 && v <= 2048 ? v : kBucketRows;
+  }();
+  return std::max(1, std::min(kBucketMaxBits, bit_width(static_cast<unsigned long long>(n / rows))));
 }
 
 void enqueue_chain_sort(const void *coords, int64_t n, int ndim, int coord_dtype, int32_t *indices_out,
