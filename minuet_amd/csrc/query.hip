@@ -497,12 +497,37 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
   const long long t = t0 + tid;
   const bool valid = t < t_end;
   const unsigned long long key = valid ? tgt(t, frame) : 0ull;
-  if (w < 2) {
+  // A cloud mapped onto itself under offsets of positive key delta only (halves):
+  // nothing below the tile's first target can match, and where the sort left
+  // its bucket starts the upper end is one table entry instead of a search:
+  // the end of the rows whose coordinate 0 is at most that of the last target
+  // plus the reach.  The window is then a little larger than the exact one;
+  // should it take more than one chunk, the searches are done after all.
+  const bool by_buckets = halves && device_plan->window_buckets > 0;
+  auto search_end = [&](int which) {
     const unsigned long long edge =
-        w == 0 ? tgt(t0, frame) + static_cast<unsigned long long>(delta_min)
-               : tgt(t_end - 1, frame) + static_cast<unsigned long long>(delta_max) + 1ull;
+        which == 0 ? tgt(t0, frame) + static_cast<unsigned long long>(delta_min)
+                   : tgt(t_end - 1, frame) + static_cast<unsigned long long>(delta_max) + 1ull;
     const long long pos = wave_lower_bound<CT, BT>(src, frame, edge, 0, num_sources);
-    if (lane_id() == 0) s_bounds[w] = pos;
+    if (lane_id() == 0) s_bounds[which] = pos;
+  };
+  if (w < 2) {
+    if (!by_buckets) {
+      search_end(w);
+    } else if (w == 0) {
+      if (lane_id() == 0) s_bounds[0] = t0;
+    } else {
+      const long long x = static_cast<long long>(tgt.coords[(t_end - 1) * frame.ndim]) + device_plan->window_reach;
+      long long pos = num_sources;
+      if (x < device_plan->window_hi) {
+        const int buckets = device_plan->window_buckets;
+        const int shift = device_plan->window_shift, bucket_shift = device_plan->window_bucket_shift;
+        const unsigned long long key = static_cast<unsigned long long>(x + 1 - device_plan->window_lo) << shift;
+        const unsigned long long bucket = (key >> bucket_shift) + (bucket_shift > shift ? 1ull : 0ull);
+        pos = device_plan->window_starts[bucket < static_cast<unsigned long long>(buckets) ? bucket : buckets];
+      }
+      if (lane_id() == 0) s_bounds[1] = pos;
+    }
   }
   if (halves) {
     if (lane_id() == 0) s_wave_first[w] = key;
@@ -515,6 +540,11 @@ __global__ __launch_bounds__(kQueryThreads) void query_kernel(
     const unsigned long long next_key = t + 1 >= t_end ? s_wave_first[kQueryThreads / kWave]
                                         : lane_id() == kWave - 1 ? s_wave_first[w + 1] : down;
     if (__ballot(valid && next_key == key) != 0ull && lane_id() == 0) sink.repeats[0] = 1u;
+  }
+  if (by_buckets && s_bounds[1] - s_bounds[0] > kWindowChunk) {        // the same for the whole workgroup
+    __syncthreads();
+    if (w < 2) search_end(w);
+    __syncthreads();
   }
   const long long w_lo = s_bounds[0];
   const long long w_hi = s_bounds[1] > w_lo ? s_bounds[1] : w_lo;
@@ -2003,6 +2033,7 @@ extern "C" int mnt_sorted_kernel_map_lists(const void *coords, int64_t n, int nd
       buf.status = buf.counters + (buf.counter_words - 4);
       buf.chunks = scope.alloc<uint4>(chain_sort_max_pairs(n));
       buf.words = scope.alloc<unsigned long long>(chain_sort_words(n));
+      buf.starts = scope.alloc<unsigned>(buckets + 1);
       buf.plan = scope.alloc<DevicePlan>(1);
       unsigned *row_totals = buf.counters + 2 * buckets;
       int *stage = scope.alloc<int>(static_cast<size_t>(num_offsets) * n);

@@ -85,6 +85,17 @@ struct DevicePlan {
   // the offsets that have rows of their own to write (all but the mirror
   // images), in offset order: offset | kind << 8 | (mirror + 1) << 16
   int rows[kPlanMaxOffsets];
+  // Upper end of a tile's source window from the sort's bucket starts instead
+  // of a search (a chain whose dealing launch worked by slabs; 0 buckets:
+  // search).  The sort's key has coordinate 0 in its top field, so the rows
+  // with coordinate 0 below x end where bucket ((x - lo) << shift) >> bucket_shift
+  // starts (its next bucket when a bucket holds parts of two such planes).
+  int window_buckets;
+  int window_shift;               // of coordinate 0 in the sort's key
+  int window_bucket_shift;        // sort key >> this = bucket
+  int window_reach;               // largest offset along coordinate 0
+  long long window_lo, window_hi; // range of coordinate 0 in the cloud
+  const unsigned *window_starts;  // [window_buckets + 1]
 };
 
 struct PlanScratch {        // LDS of the wavefront that builds the plan
@@ -102,7 +113,9 @@ __device__ __forceinline__ int plan_bits(unsigned long long range) {
 __device__ __forceinline__ void make_plan_on_device(const long long *__restrict__ bounds,
                                                     const OffsetTable &offsets, int num_offsets,
                                                     int ndim, unsigned declined, PlanScratch &lds,
-                                                    DevicePlan *__restrict__ out) {
+                                                    DevicePlan *__restrict__ out,
+                                                    const unsigned *__restrict__ bucket_starts = nullptr,
+                                                    int msd_cap = 0) {
   const int lane = lane_id();
   // lane o takes offset o: selects on scalar operands, no indexed access to the arguments
   int d[MNT_MAX_NDIM] = {0, 0, 0, 0};
@@ -247,6 +260,26 @@ __device__ __forceinline__ void make_plan_on_device(const long long *__restrict_
     out->groups_in_rows = in_rows ? 1 : 0;
     out->verdict = declined != 0 ? static_cast<int>(declined) : (fits && consistent ? 0 : 2);
     out->num_offsets = num_offsets;
+    // the sort's key: fields of the cloud's own ranges, coordinate 0 on top
+    int sort_bits = 0, below_top = 0;
+#pragma unroll
+    for (int k = MNT_MAX_NDIM - 1; k >= 0; --k) {
+      if (k < ndim) {
+        const int w = plan_bits(static_cast<unsigned long long>(bounds[MNT_MAX_NDIM + k]) -
+                                static_cast<unsigned long long>(bounds[k]));
+        if (k > 0) below_top += w;
+        sort_bits += w;
+      }
+    }
+    const int msd_bits = sort_bits < msd_cap ? sort_bits : msd_cap;
+    const bool usable = bucket_starts != nullptr && sort_bits >= 1 && sort_bits <= 63 && sort_bits > below_top;
+    out->window_buckets = usable ? 1 << msd_cap : 0;
+    out->window_shift = below_top;
+    out->window_bucket_shift = sort_bits - msd_bits;
+    out->window_reach = reach_hi[0];
+    out->window_lo = bounds[0];
+    out->window_hi = bounds[MNT_MAX_NDIM];
+    out->window_starts = bucket_starts;
   }
 }
 

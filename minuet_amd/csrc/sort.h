@@ -53,6 +53,7 @@ struct ChainSortBuffers {
                                  // (histogram form only)
   uint4 *chunks;                 // [chain_sort_max_pairs(n)]
   unsigned long long *words;     // [chain_sort_words(n)]
+  unsigned *starts;              // [buckets + 1] first sorted row of every bucket (slab form only)
   DevicePlan *plan;              // query plan written by the ranking launch (nullable)
 };
 

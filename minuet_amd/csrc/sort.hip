@@ -1297,7 +1297,8 @@ __global__ __launch_bounds__(kSortBlock) void bucket_rank_chain_kernel(
     const unsigned long long *__restrict__ words, const uint4 *__restrict__ chunks,
     const unsigned *__restrict__ pair_count, int max_pairs, const long long *__restrict__ folded,
     int ndim, int msd_cap, int idx_bits, const unsigned *__restrict__ status, FinalSink<CT, IT> sink,
-    OffsetTable offsets, int num_offsets, DevicePlan *__restrict__ plan_out, int slabs) {
+    OffsetTable offsets, int num_offsets, DevicePlan *__restrict__ plan_out, int slabs,
+    const unsigned *__restrict__ bucket_starts) {
   __shared__ __align__(16) unsigned long long s_words[kChainBucketCap + 128];
   __shared__ RankShared sh;
   const unsigned declined = status[0];
@@ -1306,7 +1307,7 @@ __global__ __launch_bounds__(kSortBlock) void bucket_rank_chain_kernel(
     if (plan_out != nullptr && threadIdx.x < kWave) {
       PlanScratch &scratch = *reinterpret_cast<PlanScratch *>(s_words);
       static_assert(sizeof(PlanScratch) <= sizeof(s_words), "plan scratch must fit the word staging area");
-      make_plan_on_device(folded, offsets, num_offsets, ndim, declined, scratch, plan_out);
+      make_plan_on_device(folded, offsets, num_offsets, ndim, declined, scratch, plan_out, bucket_starts, msd_cap);
     }
     return;
   }
@@ -1428,7 +1429,8 @@ __global__ __launch_bounds__(kSortBlock) void bucket_deal_slab_kernel(
 // they run longest), and their number in status[2].
 __global__ __launch_bounds__(1024) void bucket_pairs_kernel(const unsigned *__restrict__ counts, int buckets,
                                                             uint4 *__restrict__ chunks,
-                                                            unsigned *__restrict__ status) {
+                                                            unsigned *__restrict__ status,
+                                                            unsigned *__restrict__ starts) {
   constexpr int kPer = kBucketMax / 1024;
   __shared__ unsigned long long wave_both[1024 / kWave];
   __shared__ unsigned wave_shared[1024 / kWave];
@@ -1482,6 +1484,7 @@ __global__ __launch_bounds__(1024) void bucket_pairs_kernel(const unsigned *__re
   for (int j = 0; j < kPer; ++j) {
     const int d = t * per + j;
     if (j < per && d < buckets) {
+      starts[d] = run;                        // first sorted row of the bucket
       const unsigned mine = bucket_pieces(v[j]);
       const unsigned head = v[j] | (bucket_mode(v[j]) << 13);
       if (mine == 1) chunks[single_at++] = make_uint4(run, head, d, 0u);
@@ -1491,12 +1494,23 @@ __global__ __launch_bounds__(1024) void bucket_pairs_kernel(const unsigned *__re
     }
     run += v[j];
   }
-  if (t == 0) status[2] = all_shared + static_cast<unsigned>(all_both >> 32);
+  if (t == 0) {
+    status[2] = all_shared + static_cast<unsigned>(all_both >> 32);
+    starts[buckets] = static_cast<unsigned>(all_both);
+  }
 }
 
 static bool chain_slabs_enabled() {
   static const bool on = [] {
     const char *text = std::getenv("MINUET_CHAIN_SLABS");
+    return text == nullptr || std::atoi(text) != 0;
+  }();
+  return on;
+}
+
+static bool chain_windows_enabled() {
+  static const bool on = [] {
+    const char *text = std::getenv("MINUET_CHAIN_WINDOWS");
     return text == nullptr || std::atoi(text) != 0;
   }();
   return on;
@@ -1541,13 +1555,14 @@ static void enqueue_chain_sort_typed(const CT *coords, int64_t n, int ndim, int3
     }
     check_launch("bucket_deal_slab_kernel");
     profile_mark("sort_deal", stream);
-    bucket_pairs_kernel<<<1, 1024, 0, stream>>>(cursors, buckets, buf.chunks, buf.status);
+    bucket_pairs_kernel<<<1, 1024, 0, stream>>>(cursors, buckets, buf.chunks, buf.status, buf.starts);
     check_launch("bucket_pairs_kernel");
     profile_mark("sort_pairs", stream);
     const int max_pairs = static_cast<int>(chain_sort_max_pairs(n));
     bucket_rank_chain_kernel<CT, int32_t><<<max_pairs + 1, kSortBlock, 0, stream>>>(
         buf.words, buf.chunks, buf.status + 2, max_pairs, buf.folded, ndim, msd_cap, idx_bits, buf.status,
-        FinalSink<CT, int32_t>{coords, ndim, indices_out, sorted_out}, offsets, num_offsets, buf.plan, 1);
+        FinalSink<CT, int32_t>{coords, ndim, indices_out, sorted_out}, offsets, num_offsets, buf.plan, 1,
+        chain_windows_enabled() ? buf.starts : nullptr);
     check_launch("bucket_rank_chain_kernel");
     profile_mark("sort_rank", stream);
     return;
@@ -1574,7 +1589,7 @@ static void enqueue_chain_sort_typed(const CT *coords, int64_t n, int ndim, int3
   const int max_pairs = static_cast<int>(chain_sort_max_pairs(n));
   bucket_rank_chain_kernel<CT, int32_t><<<max_pairs + 1, kSortBlock, 0, stream>>>(
       buf.words, buf.chunks, buf.status + 2, max_pairs, buf.folded, ndim, msd_cap, idx_bits, buf.status,
-      FinalSink<CT, int32_t>{coords, ndim, indices_out, sorted_out}, offsets, num_offsets, buf.plan, 0);
+      FinalSink<CT, int32_t>{coords, ndim, indices_out, sorted_out}, offsets, num_offsets, buf.plan, 0, nullptr);
   check_launch("bucket_rank_chain_kernel");
   profile_mark("sort_rank", stream);
 }
