@@ -749,3 +749,16 @@ def test_cache_bounds_survive_recycled_storage():
     dense_b = cache.get_dense_kernel_map(b_dev, 2, None, b_dev, 2, None, 3, 1)
     np.testing.assert_array_equal(host(dense_b), orc.query_sorted_index_with_offsets(
         b, b, orc.generate_kernel_offsets(3, 3, 2, 1)))
+
+
+def test_sorted_kernel_map_lists_wide_planes():
+    """Planes of constant first coordinate with tens of thousands of rows: the
+    one-call Map step's shortcut for a tile's source window (from the sort's
+    bucket starts) would span more than one window chunk there, so the tiles
+    fall back to their searches; and a cloud that is a single such plane."""
+    rng = np.random.default_rng(23)
+    off = orc.generate_kernel_offsets(3, 3, 1, 1)
+    for planes, side, n in ((12, 220, 150000), (1, 300, 60000)):
+        flat = rng.choice(planes * side * side, size=n, replace=False)
+        cloud = np.stack([flat // (side * side) - 3, (flat // side) % side, flat % side - 100], 1).astype(np.int32)
+        _check_sorted_lists(cloud, off)
