@@ -76,8 +76,8 @@ SIGNATURES = {
     "mnt_sorted_kernel_map_lists": (_int, [_vp, _i64, _int, _int, _vp, _i64, _int, _vp, _vp, _vp, _vp,
                                            _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
     "mnt_kernel_map_row_lists": (_int, [_vp, _i64, _i64, _pi64, _pi64, _vp, _vp, _vp]),
-    "mnt_kernel_map_dense": (_int, [_vp, _i64, _vp, _i64, _pi64, _i64, _int, _int, _vp, _vp, _i64, _int,
-                                    _pi64, _pi64, _pi64, _vp, _vp]),
+    "mnt_kernel_map_dense": (_int, [_vp, _i64, _vp, _i64, _vp, _i64, _int, _int, _vp, _vp, _i64, _int,
+                                    _vp, _vp, _vp, _vp, _vp]),
     "mnt_kernel_map_tables": (_int, [_vp, _i64, _i64, _i64, _int, _pi64, _pi64, _vp]),
     "mnt_kernel_map_pair_lists": (_int, [_vp, _i64, _i64, _pi64, _vp, _vp, _vp]),
     "mnt_generate_padding_buckets": (_int, [_pi64, _i64, _int, _dbl, _pi64, _pi64]),
@@ -768,37 +768,51 @@ def kernel_map_dense(sources: torch.Tensor, targets: torch.Tensor, offsets_host:
     """The query alone: ``(kernel_map [O, T] int32, bounds)``.  Nothing is read
     back when both bounds are given, so the call returns without waiting for
     the device."""
-    _ensure_ndim("sources", sources, 2)
-    _ensure_ndim("targets", targets, 2)
-    ndim = sources.size(1)
-    _ensure_dim("targets", targets, 1, ndim)
-    ctype = _common_dtype([sources, targets])
-    tensors = [sources, targets]
+    if sources.dim() != 2:
+        _ensure_ndim("sources", sources, 2)
+    if targets.dim() != 2:
+        _ensure_ndim("targets", targets, 2)
+    ndim = sources.shape[1]
+    if targets.shape[1] != ndim:
+        _ensure_dim("targets", targets, 1, ndim)
+    ctype = sources.dtype
+    if targets.dtype != ctype:
+        _common_dtype([sources, targets])
     if (source_batch_dims is None) != (target_batch_dims is None):
         raise ValueError("source_batch_dims and target_batch_dims must be both provided or "
                          "neither provided")
+    device = sources.device
+    if device.type != "cuda" or targets.device != device:
+        _common_device([sources, targets])
     bcode = 0
+    num_batches = 1
     if source_batch_dims is not None:
-        tensors += [source_batch_dims, target_batch_dims]
+        if source_batch_dims.device != device or target_batch_dims.device != device:
+            _common_device([sources, source_batch_dims, target_batch_dims])
         bcode = _int_code(_common_dtype([source_batch_dims, target_batch_dims]), "index",
                           "kernel_map_dense")
-    device = _common_device(tensors)
-    ccode = _int_code(ctype, "coordinate", "kernel_map_dense")
-    offs = np.ascontiguousarray(np.asarray(offsets_host, dtype=np.int64).reshape(-1, ndim))
+        num_batches = source_batch_dims.numel() - 1
+    ccode = _INT.get(ctype)
+    if ccode is None:
+        _int_code(ctype, "coordinate", "kernel_map_dense")
+    offs = offsets_host
+    if not (isinstance(offs, np.ndarray) and offs.dtype == np.int64 and offs.ndim == 2
+            and offs.shape[1] == ndim and offs.flags.c_contiguous):
+        offs = np.ascontiguousarray(np.asarray(offsets_host, dtype=np.int64).reshape(-1, ndim))
     num_offsets = offs.shape[0]
-    dense = torch.empty((num_offsets, targets.size(0)), dtype=torch.int32, device=device)
+    dense = torch.empty((num_offsets, targets.shape[0]), dtype=torch.int32, device=device)
     bounds = np.zeros(16, dtype=np.int64)
     sb = None if source_bounds is None else np.ascontiguousarray(source_bounds, dtype=np.int64)
     tb = None if target_bounds is None else np.ascontiguousarray(target_bounds, dtype=np.int64)
     with _on(device):
-        _check(load_library().mnt_kernel_map_dense(
-            _ptr(sources), sources.size(0), _ptr(targets), targets.size(0),
-            offs.ctypes.data_as(_pi64), num_offsets, ndim, ccode, _ptr(source_batch_dims),
-            _ptr(target_batch_dims),
-            source_batch_dims.numel() - 1 if source_batch_dims is not None else 1, bcode,
-            None if sb is None else sb.ctypes.data_as(_pi64),
-            None if tb is None else tb.ctypes.data_as(_pi64), bounds.ctypes.data_as(_pi64),
-            _ptr(dense), _stream(device)))
+        status = load_library().mnt_kernel_map_dense(
+            _ptr(sources), sources.shape[0], _ptr(targets), targets.shape[0],
+            _host_address(offs), num_offsets, ndim, ccode, _ptr(source_batch_dims),
+            _ptr(target_batch_dims), num_batches, bcode,
+            None if sb is None else sb.ctypes.data, None if tb is None else tb.ctypes.data,
+            bounds.ctypes.data, _ptr(dense), _stream(device))
+    if status != 0:
+        _check(status)
     return dense, bounds
 
 
